@@ -1,0 +1,417 @@
+"""Dense numpy oracle for the Sinkhorn solver, gradient and plan products.
+
+TEST INFRASTRUCTURE ONLY: the shipped package never imports this module.
+
+All citations are into ``/root/reference/src/flash_sinkhorn`` (abbreviated FS).
+Arithmetic runs in ``dtype`` (float64 by default: the mathematical answer the
+fp32 reference approximates; pass ``np.float32`` to mimic the reference's own
+precision).  Row-chunked so that n*m never has to fit in memory at once.
+
+Pin status (what each function is checked against in tests/test_oracle_*.py):
+
+* log_weights, dampening, max_diameter, epsilon_schedule ... closed forms
+  (FS/testing/test_flashstyle_parity.py:86-190, test_unbalanced_sinkhorn.py:228-242)
+* softmin / lse_shifted / symmetric_step ... scipy.special.logsumexp, brute
+  force python loops on tiny inputs, shift invariance
+* sinkhorn_symmetric (balanced, full cost) ... golden vectors written from
+  FS/testing/reference_sinkhorn.py:119-192 (tests/golden/make_golden.py)
+* half cost ... identity 0.5|x-y|^2 = |x/sqrt2 - y/sqrt2|^2 against the golden
+  full-cost run
+* sinkhorn_alternating, OTT convention ... golden vectors from
+  FS/testing/reference_sinkhorn.py:65-82
+* sinkhorn_alternating, GeomLoss convention (balanced) ... relation to the OTT
+  convention f_ott = f + eps*log a, fixed point marginals
+* unbalanced / semi-unbalanced (symmetric and alternating) ... PARITY UNPINNED
+  by any reference-held artefact (the reference checks these against GeomLoss,
+  which is not installed); pinned only by the limits rho->inf == balanced,
+  reach_x == reach_y == reach, and the unbalanced fixed-point equation
+* grad_barycentric / grad_plan ... golden vectors from
+  FS/testing/reference_sinkhorn.py:195-233 and finite differences of the dual
+* apply_plan_vec / apply_plan_mat / mat5 ... brute-force python loops
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional, Sequence
+
+import numpy as np
+
+__all__ = [
+    "log_weights",
+    "dampening",
+    "max_diameter",
+    "epsilon_schedule",
+    "sqeuclid_cost",
+    "softmin",
+    "lse_shifted",
+    "lse_shifted_fused",
+    "symmetric_step",
+    "resolve_rho",
+    "sinkhorn_symmetric",
+    "sinkhorn_alternating",
+    "sinkhorn_cost",
+    "plan",
+    "grad_plan",
+    "grad_barycentric",
+    "apply_plan_vec",
+    "apply_plan_mat",
+    "mat5",
+]
+
+
+# ---------------------------------------------------------------------------
+# scalar / small-vector helpers  (FS/kernels/_common.py:20-90)
+# ---------------------------------------------------------------------------
+
+def log_weights(w, dtype=np.float64):
+    """log(w) with w<=0 mapped to -100000 (FS/kernels/_common.py:39-44)."""
+    w = np.asarray(w, dtype=dtype)
+    out = np.full_like(w, -100000.0)
+    pos = w > 0
+    out[pos] = np.log(w[pos])
+    return out
+
+
+def dampening(eps: float, rho: Optional[float]) -> float:
+    """1/(1+eps/rho), 1 for rho=None (FS/kernels/_common.py:20-36)."""
+    return 1.0 if rho is None else 1.0 / (1.0 + eps / rho)
+
+
+def max_diameter(x, y) -> float:
+    """Diagonal of the joint bounding box (FS/kernels/_common.py:47-53)."""
+    x = np.asarray(x, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    lo = np.minimum(x.min(axis=0), y.min(axis=0))
+    hi = np.maximum(x.max(axis=0), y.max(axis=0))
+    return float(np.linalg.norm(hi - lo))
+
+
+def epsilon_schedule(diameter: float, blur: float, scaling: float, p: float = 2.0):
+    """[D^p, exp(arange(p ln D, p ln blur, p ln s))..., blur^p]
+    (FS/kernels/_common.py:56-90)."""
+    if diameter <= 0:
+        raise ValueError("diameter must be > 0.")
+    if blur <= 0:
+        raise ValueError("blur must be > 0.")
+    if not (0.0 < scaling < 1.0):
+        raise ValueError("scaling must be in (0, 1).")
+    mid = np.arange(p * np.log(diameter), p * np.log(blur), p * np.log(scaling))
+    return [diameter ** p] + [float(np.exp(e)) for e in mid] + [blur ** p]
+
+
+# ---------------------------------------------------------------------------
+# cost and log-sum-exp building blocks
+# ---------------------------------------------------------------------------
+
+def sqeuclid_cost(x, y, cost_scale: float = 1.0, dtype=np.float64):
+    """cost_scale * (|x|^2 + |y|^2 - 2 x.y)  (FS/testing/reference_sinkhorn.py:4-9)."""
+    x = np.asarray(x, dtype=dtype)
+    y = np.asarray(y, dtype=dtype)
+    x2 = (x * x).sum(axis=1)[:, None]
+    y2 = (y * y).sum(axis=1)[None, :]
+    return cost_scale * (x2 + y2 - 2.0 * (x @ y.T))
+
+
+def _lse_rows(vals):
+    """Row-wise log-sum-exp; rows that are all -inf give -inf."""
+    mx = vals.max(axis=1)
+    safe = np.where(np.isfinite(mx), mx, 0.0)
+    s = np.exp(vals - safe[:, None]).sum(axis=1)
+    with np.errstate(divide="ignore"):
+        return safe + np.log(s)
+
+
+def _row_chunks(n: int, m: int, budget_elems: int = 32_000_000):
+    step = max(1, min(n, budget_elems // max(m, 1)))
+    for i0 in range(0, n, step):
+        yield i0, min(n, i0 + step)
+
+
+def softmin(x, y, pot_y, logw_y, eps, cost_scale=1.0, dtype=np.float64):
+    """-eps * LSE_j[(pot_j - C_ij)/eps + logw_j]
+    (FS/testing/reference_sinkhorn.py:168-174)."""
+    x = np.asarray(x, dtype=dtype)
+    y = np.asarray(y, dtype=dtype)
+    pot_y = np.asarray(pot_y, dtype=dtype)
+    logw_y = np.asarray(logw_y, dtype=dtype)
+    eps = dtype(eps)
+    out = np.empty(x.shape[0], dtype=dtype)
+    for i0, i1 in _row_chunks(x.shape[0], y.shape[0]):
+        c = sqeuclid_cost(x[i0:i1], y, cost_scale, dtype)
+        out[i0:i1] = -eps * _lse_rows((pot_y[None, :] - c) / eps + logw_y[None, :])
+    return out
+
+
+def lse_shifted(x, y, bias, eps, cost_scale=1.0, damping=1.0, dtype=np.float64):
+    """out_i = -eps*damping*LSE_j[2*cost_scale*x_i.y_j/eps + bias_j]
+    (FS/kernels/sinkhorn_flashstyle_sqeuclid.py:227, 285-306)."""
+    x = np.asarray(x, dtype=dtype)
+    y = np.asarray(y, dtype=dtype)
+    bias = np.asarray(bias, dtype=dtype)
+    out = np.empty(x.shape[0], dtype=dtype)
+    sc = dtype(2.0 * cost_scale / eps)
+    for i0, i1 in _row_chunks(x.shape[0], y.shape[0]):
+        out[i0:i1] = _lse_rows((x[i0:i1] @ y.T) * sc + bias[None, :])
+    return dtype(-eps * damping) * out
+
+
+def lse_shifted_fused(x, y, pot_hat, log_w, eps, cost_scale=1.0, damping=1.0,
+                      dtype=np.float64):
+    """Same with bias_j = pot_hat_j/eps + log_w_j formed inside
+    (FS/kernels/sinkhorn_flashstyle_sqeuclid.py:352, 399-418)."""
+    bias = np.asarray(pot_hat, dtype=dtype) / dtype(eps) + np.asarray(log_w, dtype=dtype)
+    return lse_shifted(x, y, bias, eps, cost_scale, damping, dtype)
+
+
+def symmetric_step(x, y, f_hat, g_hat, log_a, log_b, eps, cost_scale=1.0, alpha=0.5,
+                   damping_f=1.0, damping_g=1.0, dtype=np.float64):
+    """One Jacobi step on shifted potentials; both halves read the OLD potentials
+    (FS/kernels/sinkhorn_flashstyle_sqeuclid.py:508-584, 589-661)."""
+    f_hat = np.asarray(f_hat, dtype=dtype)
+    g_hat = np.asarray(g_hat, dtype=dtype)
+    f_c = lse_shifted_fused(x, y, g_hat, log_b, eps, cost_scale, damping_f, dtype)
+    g_c = lse_shifted_fused(y, x, f_hat, log_a, eps, cost_scale, damping_g, dtype)
+    return (1.0 - alpha) * f_hat + alpha * f_c, (1.0 - alpha) * g_hat + alpha * g_c
+
+
+# ---------------------------------------------------------------------------
+# solvers
+# ---------------------------------------------------------------------------
+
+def resolve_rho(rho=None, reach=None, rho_x=None, rho_y=None, reach_x=None, reach_y=None):
+    """Priority rho_x/rho_y > reach_x/reach_y > rho > reach
+    (FS/sinkhorn_solvers.py:397-419)."""
+    if rho is not None and reach is not None:
+        raise ValueError("Specify either rho or reach, not both.")
+    if reach is not None:
+        rho = reach ** 2
+    if rho is not None:
+        if rho_x is None and reach_x is None:
+            rho_x = rho
+        if rho_y is None and reach_y is None:
+            rho_y = rho
+    if reach_x is not None:
+        if rho_x is not None:
+            raise ValueError("Specify either rho_x or reach_x, not both.")
+        rho_x = reach_x ** 2
+    if reach_y is not None:
+        if rho_y is not None:
+            raise ValueError("Specify either rho_y or reach_y, not both.")
+        rho_y = reach_y ** 2
+    return rho_x, rho_y
+
+
+def sinkhorn_symmetric(
+    x, y, a, b, *,
+    blur=0.05, scaling=0.5, use_epsilon_scaling=True, last_extrapolation=True,
+    cost_scale=1.0, eps=None, n_iters=None, diameter=None, eps_list=None,
+    rho=None, reach=None, rho_x=None, rho_y=None, reach_x=None, reach_y=None,
+    threshold=None, check_every=5, return_n_iters=False, return_prelast=False,
+    f_init=None, g_init=None, dtype=np.float64,
+):
+    """GeomLoss-style symmetric solver in standard potentials.
+
+    Restates FS/sinkhorn_solvers.py:394-707 (whose balanced full-cost case is
+    FS/testing/reference_sinkhorn.py:119-192).  In standard potentials the
+    shifted update plus the unbalanced shift correction (509-517, 634-639)
+    collapse to ``f <- (1-w) f + w * damp_f * softmin_eps(g)``.
+    """
+    rho_x, rho_y = resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y)
+    if eps_list is None:
+        if use_epsilon_scaling:
+            if diameter is None:
+                diameter = max_diameter(x, y)
+            eps_list = epsilon_schedule(diameter, blur, scaling, p=2.0)
+        else:
+            if eps is None or n_iters is None:
+                raise ValueError("When use_epsilon_scaling=False, provide eps and n_iters")
+            eps_list = [float(eps)] * int(n_iters)
+    if len(eps_list) == 0:
+        raise ValueError("eps_list must be non-empty")
+    if n_iters is not None:
+        eps_list = list(eps_list)[: int(n_iters)]
+
+    log_a = log_weights(a, dtype)
+    log_b = log_weights(b, dtype)
+    n, m = np.shape(x)[0], np.shape(y)[0]
+    f = np.zeros(n, dtype) if f_init is None else np.asarray(f_init, dtype).copy()
+    g = np.zeros(m, dtype) if g_init is None else np.asarray(g_init, dtype).copy()
+
+    def jacobi(f, g, e, w):
+        df, dg = dampening(e, rho_x), dampening(e, rho_y)
+        ft = df * softmin(x, y, g, log_b, e, cost_scale, dtype)
+        gt = dg * softmin(y, x, f, log_a, e, cost_scale, dtype)
+        return (1.0 - w) * f + w * ft, (1.0 - w) * g + w * gt
+
+    used = 0
+    f, g = jacobi(f, g, eps_list[0], 1.0)
+    used += 1
+    prev = None
+    for idx, e in enumerate(eps_list):
+        f, g = jacobi(f, g, e, 0.5)
+        used += 1
+        if threshold is not None and (idx + 1) % check_every == 0:
+            if prev is None:  # first check only snapshots (FS/sinkhorn_solvers.py:521-524)
+                prev = (f.copy(), g.copy())
+            else:
+                change = max(np.abs(f - prev[0]).max(), np.abs(g - prev[1]).max())
+                if change < threshold:
+                    break
+                prev = (f.copy(), g.copy())
+    f_pre, g_pre = f, g
+    if last_extrapolation:
+        f, g = jacobi(f, g, eps_list[-1], 1.0)
+        used += 1
+
+    out = (f, g)
+    if return_prelast and last_extrapolation:
+        out = out + (f_pre, g_pre)
+    if return_n_iters:
+        out = out + (used,)
+    return out
+
+
+def sinkhorn_alternating(
+    x, y, a, b, *, eps=0.1, n_iters=100, cost_scale=1.0,
+    rho=None, reach=None, rho_x=None, rho_y=None, reach_x=None, reach_y=None,
+    threshold=None, check_every=5, return_n_iters=False, ott_convention=False,
+    dtype=np.float64,
+):
+    """Gauss-Seidel solver, restating FS/sinkhorn_solvers.py:105-287 AS WRITTEN.
+
+    GeomLoss convention (240-259): the kernel damps the whole shifted value and
+    no shift correction follows, so in standard potentials
+    ``f = damp_f*softmin(g) + (1-damp_f)*cost_scale*|x|^2`` (a quirk of the
+    reference that results parity must keep).  OTT convention (188-228): g is
+    updated first, weights sit outside the LSE, and the same damping quirk
+    applies to the LSE part only.
+    """
+    rho_x, rho_y = resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y)
+    damp_f, damp_g = dampening(eps, rho_x), dampening(eps, rho_y)
+    xx = np.asarray(x, dtype)
+    yy = np.asarray(y, dtype)
+    alpha = cost_scale * (xx * xx).sum(axis=1)
+    beta = cost_scale * (yy * yy).sum(axis=1)
+    log_a = log_weights(a, dtype)
+    log_b = log_weights(b, dtype)
+    f_hat, g_hat = -alpha.copy(), -beta.copy()
+    prev_f, prev_g = f_hat.copy(), g_hat.copy()
+    used = 0
+    for i in range(int(n_iters)):
+        if ott_convention:
+            g_hat = eps * log_b + lse_shifted(yy, xx, f_hat / eps, eps, cost_scale, damp_g, dtype)
+            f_hat = eps * log_a + lse_shifted(xx, yy, g_hat / eps, eps, cost_scale, damp_f, dtype)
+        else:
+            f_hat = lse_shifted_fused(xx, yy, g_hat, log_b, eps, cost_scale, damp_f, dtype)
+            g_hat = lse_shifted_fused(yy, xx, f_hat, log_a, eps, cost_scale, damp_g, dtype)
+        used += 1
+        if threshold is not None and (i + 1) % check_every == 0:
+            change = max(np.abs(f_hat - prev_f).max(), np.abs(g_hat - prev_g).max())
+            if change < threshold:
+                break
+            prev_f, prev_g = f_hat.copy(), g_hat.copy()
+    f, g = f_hat + alpha, g_hat + beta
+    return (f, g, used) if return_n_iters else (f, g)
+
+
+def sinkhorn_cost(a, b, f, g, eps, rho_x=None, rho_y=None, dtype=np.float64):
+    """OT cost from potentials (FS/_autograd.py:436-455): <a,f>+<b,g> unless BOTH
+    marginals are relaxed, then (rho+eps/2)*<a,1-exp(-f/rho)> + same for b."""
+    a = np.asarray(a, dtype); b = np.asarray(b, dtype)
+    f = np.asarray(f, dtype); g = np.asarray(g, dtype)
+    if rho_x is None or rho_y is None:
+        return float((a * f).sum() + (b * g).sum())
+    ca = (a * (1.0 - np.exp(-f / rho_x))).sum()
+    cb = (b * (1.0 - np.exp(-g / rho_y))).sum()
+    return float((rho_x + eps / 2) * ca + (rho_y + eps / 2) * cb)
+
+
+# ---------------------------------------------------------------------------
+# plan, gradients, plan products
+# ---------------------------------------------------------------------------
+
+def plan(x, y, a, b, f, g, eps, cost_scale=1.0, dtype=np.float64):
+    """P = a b^T * exp((f+g-C)/eps) (FS/testing/reference_sinkhorn.py:195-198)."""
+    c = sqeuclid_cost(x, y, cost_scale, dtype)
+    f = np.asarray(f, dtype); g = np.asarray(g, dtype)
+    a = np.asarray(a, dtype); b = np.asarray(b, dtype)
+    return (a[:, None] * b[None, :]) * np.exp((f[:, None] + g[None, :] - c) / eps)
+
+
+def grad_plan(x, y, a, b, f, g, eps, cost_scale=1.0, dtype=np.float64):
+    """2cs(a x - P y), 2cs(b y - P^T x) (FS/testing/reference_sinkhorn.py:201-205)."""
+    p = plan(x, y, a, b, f, g, eps, cost_scale, dtype)
+    x = np.asarray(x, dtype); y = np.asarray(y, dtype)
+    a = np.asarray(a, dtype); b = np.asarray(b, dtype)
+    return (2.0 * cost_scale * (a[:, None] * x - p @ y),
+            2.0 * cost_scale * (b[:, None] * y - p.T @ x))
+
+
+def _softmax_rows(vals):
+    mx = vals.max(axis=1, keepdims=True)
+    w = np.exp(vals - mx)
+    return w / w.sum(axis=1, keepdims=True)
+
+
+def grad_barycentric(x, y, a, b, f, g, eps, cost_scale=1.0, grad_scale=1.0,
+                     dtype=np.float64):
+    """grad_x_i = 2cs*gs*a_i(x_i - softmax_j[(g_j-C_ij)/eps+log b_j].y), grad_y
+    symmetric (FS/testing/reference_sinkhorn.py:208-233; kernel
+    FS/kernels/sinkhorn_triton_grad_sqeuclid.py:270-279).  Standard potentials."""
+    x = np.asarray(x, dtype); y = np.asarray(y, dtype)
+    a = np.asarray(a, dtype); b = np.asarray(b, dtype)
+    f = np.asarray(f, dtype); g = np.asarray(g, dtype)
+    log_a, log_b = log_weights(a, dtype), log_weights(b, dtype)
+    gx = np.empty_like(x)
+    gy = np.empty_like(y)
+    for i0, i1 in _row_chunks(x.shape[0], y.shape[0]):
+        c = sqeuclid_cost(x[i0:i1], y, cost_scale, dtype)
+        w = _softmax_rows((g[None, :] - c) / eps + log_b[None, :])
+        gx[i0:i1] = a[i0:i1, None] * (x[i0:i1] - w @ y)
+    for j0, j1 in _row_chunks(y.shape[0], x.shape[0]):
+        c = sqeuclid_cost(y[j0:j1], x, cost_scale, dtype)
+        w = _softmax_rows((f[None, :] - c) / eps + log_a[None, :])
+        gy[j0:j1] = b[j0:j1, None] * (y[j0:j1] - w @ x)
+    s = 2.0 * cost_scale * grad_scale
+    return s * gx, s * gy
+
+
+def _plan_shifted(x, y, f_hat, g_hat, log_a, log_b, eps, cost_scale, dtype):
+    """P_ij = exp(log a_i + log b_j + (f_hat_i + g_hat_j + 2cs x.y)/eps)
+    (FS/kernels/apply_flash.py:86-89)."""
+    x = np.asarray(x, dtype); y = np.asarray(y, dtype)
+    lg = (np.asarray(f_hat, dtype)[:, None] + np.asarray(g_hat, dtype)[None, :]
+          + 2.0 * cost_scale * (x @ y.T)) / eps
+    return np.exp(lg + np.asarray(log_a, dtype)[:, None] + np.asarray(log_b, dtype)[None, :])
+
+
+def apply_plan_vec(x, y, f_hat, g_hat, log_a, log_b, vec, eps, axis, cost_scale=1.0,
+                   dtype=np.float64):
+    """P@v (axis=1) or P^T@v (axis=0), shifted potentials
+    (FS/kernels/apply_flash.py:855-863)."""
+    p = _plan_shifted(x, y, f_hat, g_hat, log_a, log_b, eps, cost_scale, dtype)
+    v = np.asarray(vec, dtype)
+    return p @ v if axis == 1 else p.T @ v
+
+
+def apply_plan_mat(x, y, f_hat, g_hat, log_a, log_b, mat, eps, axis, cost_scale=1.0,
+                   scale=None, dtype=np.float64):
+    """P@V (axis=1, optional V*scale[:,None]) or P^T@V (axis=0)
+    (FS/kernels/apply_flash.py:389-393, 175-181)."""
+    p = _plan_shifted(x, y, f_hat, g_hat, log_a, log_b, eps, cost_scale, dtype)
+    v = np.asarray(mat, dtype)
+    if scale is not None:
+        if axis != 1:
+            raise ValueError("scale is only supported for axis=1.")
+        v = v * np.asarray(scale, dtype)[:, None]
+    return p @ v if axis == 1 else p.T @ v
+
+
+def mat5(x, y, f_ott, g_ott, A, eps, cost_scale=1.0, dtype=np.float64):
+    """(-4cs/eps) * sum_j P_ij (A_i.y_j) y_j, P = exp((f+g-C)/eps) with OTT
+    potentials (FS/kernels/apply_ott.py:473, 128-162, 518)."""
+    x = np.asarray(x, dtype); y = np.asarray(y, dtype); A = np.asarray(A, dtype)
+    c = sqeuclid_cost(x, y, cost_scale, dtype)
+    p = np.exp((np.asarray(f_ott, dtype)[:, None] + np.asarray(g_ott, dtype)[None, :] - c) / eps)
+    return (-4.0 * cost_scale / eps) * ((p * (A @ y.T)) @ y)

@@ -1,0 +1,238 @@
+"""Oracle vs what the mathematics fixes: closed forms, brute force, invariants."""
+import math
+
+import numpy as np
+import pytest
+from scipy.special import logsumexp
+
+import oracle
+from tests.golden.recipe import inputs
+
+
+def test_helpers_closed_forms():
+    # FS/testing/test_unbalanced_sinkhorn.py:228-242 cases
+    assert oracle.dampening(0.1, None) == 1.0
+    assert oracle.dampening(0.1, 1.0) == pytest.approx(1.0 / 1.1, rel=1e-12)
+    assert oracle.dampening(0.5, 0.25) == pytest.approx(1.0 / 3.0, rel=1e-12)
+    lw = oracle.log_weights(np.array([0.5, 0.0, -1.0, 2.0]))
+    assert lw.tolist() == [math.log(0.5), -100000.0, -100000.0, math.log(2.0)]
+    x = np.array([[0.0, 0.0], [1.0, 2.0]]); y = np.array([[-1.0, 0.5], [3.0, 1.0]])
+    assert oracle.max_diameter(x, y) == pytest.approx(math.hypot(4.0, 2.0))
+    sched = oracle.epsilon_schedule(4.0, 0.5, 0.5)
+    # 16, then 16,4,1 (geometric by 0.25 down to but excluding 0.25), then 0.25
+    assert sched == pytest.approx([16.0, 16.0, 4.0, 1.0, 0.25])
+    with pytest.raises(ValueError):
+        oracle.epsilon_schedule(1.0, 0.1, 1.0)
+
+
+def test_resolve_rho_priority():
+    assert oracle.resolve_rho(reach=2.0) == (4.0, 4.0)
+    assert oracle.resolve_rho(reach_x=3.0) == (9.0, None)
+    assert oracle.resolve_rho(rho=1.0, rho_y=5.0) == (1.0, 5.0)
+    with pytest.raises(ValueError):
+        oracle.resolve_rho(rho=1.0, reach=1.0)
+    with pytest.raises(ValueError):
+        oracle.resolve_rho(rho_x=1.0, reach_x=1.0)
+
+
+def test_lse_step_brute_force():
+    x, y, a, b = inputs(21, 7, 5, 3)
+    g = np.linspace(-1, 1, 5); eps = 0.3
+    lb = np.log(b.astype(np.float64))
+    want = np.empty(7)
+    for i in range(7):  # python loops: nothing shared with the vectorised code
+        terms = []
+        for j in range(5):
+            c = sum((float(x[i, k]) - float(y[j, k])) ** 2 for k in range(3))
+            terms.append((g[j] - c) / eps + lb[j])
+        want[i] = -eps * logsumexp(terms)
+    got = oracle.softmin(x, y, g, lb, eps)
+    np.testing.assert_allclose(got, want, rtol=1e-12)
+    # shifted form: same thing minus |x|^2 once g is shifted by |y|^2
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    al, be = (x64 ** 2).sum(1), (y64 ** 2).sum(1)
+    got_hat = oracle.lse_shifted_fused(x, y, g - be, lb, eps)
+    np.testing.assert_allclose(got_hat + al, want, rtol=1e-11)
+    bias = (g - be) / eps + lb
+    np.testing.assert_allclose(oracle.lse_shifted(x, y, bias, eps), got_hat, rtol=1e-12)
+    # bias + c  =>  out - eps*c ; damping scales the whole value
+    np.testing.assert_allclose(oracle.lse_shifted(x, y, bias + 2.0, eps), got_hat - eps * 2.0,
+                               rtol=1e-11)
+    np.testing.assert_allclose(oracle.lse_shifted(x, y, bias, eps, damping=0.25), 0.25 * got_hat,
+                               rtol=1e-12)
+    # half cost halves the cross term
+    got_half = oracle.lse_shifted(x, y, bias, eps, cost_scale=0.5)
+    np.testing.assert_allclose(
+        got_half, -eps * logsumexp((x64 @ y64.T) / eps + bias[None, :], axis=1), rtol=1e-12)
+
+
+def test_symmetric_step_uses_old_potentials():
+    x, y, a, b = inputs(22, 9, 6, 4)
+    fh = np.linspace(-2, 0, 9); gh = np.linspace(-1, 1, 6)
+    la, lb = np.log(a.astype(np.float64)), np.log(b.astype(np.float64))
+    f1, g1 = oracle.symmetric_step(x, y, fh, gh, la, lb, 0.4, alpha=0.5)
+    fc = oracle.lse_shifted_fused(x, y, gh, lb, 0.4)
+    gc = oracle.lse_shifted_fused(y, x, fh, la, 0.4)  # OLD f, not f1
+    np.testing.assert_allclose(f1, 0.5 * fh + 0.5 * fc, rtol=1e-12)
+    np.testing.assert_allclose(g1, 0.5 * gh + 0.5 * gc, rtol=1e-12)
+
+
+def test_balanced_fixed_point_has_right_marginals():
+    x, y, a, b = inputs(23, 30, 20, 2)
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=0.5, n_iters=400)
+    P = oracle.plan(x, y, a, b, f, g, 0.5)
+    np.testing.assert_allclose(P.sum(1), a, rtol=1e-6)
+    np.testing.assert_allclose(P.sum(0), b, rtol=1e-6)
+    # alternating (both conventions) reaches the same plan; OTT potentials absorb eps*log w
+    fa, ga = oracle.sinkhorn_alternating(x, y, a, b, eps=0.5, n_iters=400)
+    np.testing.assert_allclose(oracle.plan(x, y, a, b, fa, ga, 0.5), P, rtol=1e-5, atol=1e-12)
+    fo, go = oracle.sinkhorn_alternating(x, y, a, b, eps=0.5, n_iters=400, ott_convention=True)
+    Po = np.exp((fo[:, None] + go[None, :] - oracle.sqeuclid_cost(x, y)) / 0.5)
+    np.testing.assert_allclose(Po, P, rtol=1e-5, atol=1e-12)
+    # dual cost == primal transport cost + eps*KL at the optimum
+    C = oracle.sqeuclid_cost(x, y)
+    ab = a.astype(np.float64)[:, None] * b.astype(np.float64)[None, :]
+    primal = (P * C).sum() + 0.5 * (P * np.log(P / ab)).sum()
+    assert oracle.sinkhorn_cost(a, b, f, g, 0.5) == pytest.approx(primal, rel=1e-6)
+
+
+def test_unbalanced_limits_and_fixed_point():
+    x, y, a, b = inputs(24, 25, 18, 3)
+    kw = dict(use_epsilon_scaling=False, eps=0.3, n_iters=30)
+    f0, g0 = oracle.sinkhorn_symmetric(x, y, a, b, **kw)
+    f1, g1 = oracle.sinkhorn_symmetric(x, y, a, b, rho=1e12, **kw)
+    np.testing.assert_allclose(f1, f0, rtol=1e-9, atol=1e-9)
+    fa, ga = oracle.sinkhorn_symmetric(x, y, a, b, reach=1.5, **kw)
+    fb, gb = oracle.sinkhorn_symmetric(x, y, a, b, reach_x=1.5, reach_y=1.5, **kw)
+    np.testing.assert_array_equal(fa, fb)
+    # unbalanced fixed point: f = damp * softmin(g)
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, rho=2.0, use_epsilon_scaling=False, eps=0.3,
+                                     n_iters=500, last_extrapolation=False)
+    damp = 1.0 / (1.0 + 0.3 / 2.0)
+    lb = np.log(b.astype(np.float64))
+    np.testing.assert_allclose(f, damp * oracle.softmin(x, y, g, lb, 0.3), rtol=1e-8)
+    # alternating + rho keeps the reference's missing shift correction
+    fq, gq = oracle.sinkhorn_alternating(x, y, a, b, eps=0.3, n_iters=1, rho=2.0)
+    al = (x.astype(np.float64) ** 2).sum(1)
+    be = (y.astype(np.float64) ** 2).sum(1)
+    want = damp * oracle.softmin(x, y, np.zeros(18), lb, 0.3) + (1 - damp) * al
+    np.testing.assert_allclose(fq, want, rtol=1e-10)
+
+
+def test_early_stop_bookkeeping():
+    x, y, a, b = inputs(25, 20, 20, 2)
+    # first check only snapshots => earliest stop after 2*check_every averaged steps
+    out = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=5.0, n_iters=50,
+                                    threshold=1e9, check_every=3, return_n_iters=True)
+    assert out[-1] == 1 + 6 + 1
+    out = oracle.sinkhorn_alternating(x, y, a, b, eps=5.0, n_iters=50, threshold=1e9,
+                                      check_every=3, return_n_iters=True)
+    assert out[-1] == 3
+
+
+def test_gradient_is_derivative_of_dual_at_fixed_potentials():
+    x, y, a, b = inputs(26, 6, 5, 2)
+    x = x.astype(np.float64)
+    eps = 0.7
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=eps, n_iters=300,
+                                     last_extrapolation=False)
+    lb = np.log(b.astype(np.float64))
+
+    def dual(xx):  # <a, softmin(g)> with g frozen: d/dx_i gives the barycentric gradient
+        return float((a * oracle.softmin(xx, y, g, lb, eps)).sum())
+
+    gx, _ = oracle.grad_barycentric(x, y, a, b, f, g, eps)
+    fd = np.zeros_like(x)
+    for i in range(6):
+        for k in range(2):
+            e = np.zeros_like(x); e[i, k] = 1e-6
+            fd[i, k] = (dual(x + e) - dual(x - e)) / 2e-6
+    np.testing.assert_allclose(gx, fd, rtol=1e-6, atol=1e-9)
+    # at the balanced optimum the plan form agrees
+    gp, _ = oracle.grad_plan(x, y, a, b, f, g, eps)
+    np.testing.assert_allclose(gp, gx, rtol=1e-5, atol=1e-9)
+    # half cost: chain rule through the sqrt(2) rescaling
+    gh, _ = oracle.grad_barycentric(x, y, a, b, f, g, eps, cost_scale=0.5)
+    s = math.sqrt(0.5)
+    gs, _ = oracle.grad_barycentric(s * x, s * y.astype(np.float64), a, b, f, g, eps)
+    np.testing.assert_allclose(gh, s * gs, rtol=1e-10)
+
+
+def test_apply_and_mat5_brute_force():
+    x, y, a, b = inputs(27, 5, 4, 3)
+    rng = np.random.default_rng(5)
+    fh, gh = rng.standard_normal(5), rng.standard_normal(4)
+    la, lb = np.log(a.astype(np.float64)), np.log(b.astype(np.float64))
+    v = rng.standard_normal(4); V = rng.standard_normal((4, 3)); sc = rng.random(4)
+    eps, cs = 0.9, 0.5
+    P = np.zeros((5, 4))
+    for i in range(5):
+        for j in range(4):
+            dot = sum(float(x[i, k]) * float(y[j, k]) for k in range(3))
+            P[i, j] = a[i] * b[j] * math.exp((fh[i] + gh[j] + 2 * cs * dot) / eps)
+    kw = dict(eps=eps, cost_scale=cs)
+    np.testing.assert_allclose(oracle.apply_plan_vec(x, y, fh, gh, la, lb, v, axis=1, **kw), P @ v,
+                               rtol=1e-6)
+    np.testing.assert_allclose(
+        oracle.apply_plan_vec(x, y, fh, gh, la, lb, fh, axis=0, **kw), P.T @ fh, rtol=1e-6)
+    np.testing.assert_allclose(
+        oracle.apply_plan_mat(x, y, fh, gh, la, lb, V, axis=1, scale=sc, **kw),
+        P @ (V * sc[:, None]), rtol=1e-6)
+    W = rng.standard_normal((5, 3))
+    np.testing.assert_allclose(oracle.apply_plan_mat(x, y, fh, gh, la, lb, W, axis=0, **kw),
+                               P.T @ W, rtol=1e-6)
+    with pytest.raises(ValueError):
+        oracle.apply_plan_mat(x, y, fh, gh, la, lb, W, axis=0, scale=sc, **kw)
+    # mat5 with OTT potentials
+    A = rng.standard_normal((5, 3))
+    fo, go = rng.standard_normal(5), rng.standard_normal(4)
+    want = np.zeros((5, 3))
+    for i in range(5):
+        for j in range(4):
+            c = cs * sum((float(x[i, k]) - float(y[j, k])) ** 2 for k in range(3))
+            p = math.exp((fo[i] + go[j] - c) / eps)
+            ay = sum(A[i, k] * float(y[j, k]) for k in range(3))
+            want[i] += p * ay * y[j]
+    np.testing.assert_allclose(oracle.mat5(x, y, fo, go, A, eps, cs), (-4 * cs / eps) * want,
+                               rtol=1e-6)
+
+
+def test_cg_matches_dense_solve_and_bookkeeping():
+    rng = np.random.default_rng(3)
+    M = rng.standard_normal((12, 12)); M = M @ M.T + 12 * np.eye(12)
+    b = rng.standard_normal(12)
+    x, info = oracle.conjugate_gradient(lambda v: M @ v, b, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(x, np.linalg.solve(M, b), rtol=1e-9)
+    assert info.cg_converged and info.cg_iters <= 12
+    _, info = oracle.conjugate_gradient(lambda v: M @ v, b, max_iter=2, rtol=1e-14, atol=0.0)
+    assert (not info.cg_converged) and info.cg_iters == 2
+    x, info = oracle.conjugate_gradient(lambda v: M @ v, b, x0=np.linalg.solve(M, b))
+    assert info.cg_iters == 1 or info.cg_initial_residual < 1e-10
+    d = np.diag(M)
+    x, _ = oracle.conjugate_gradient(lambda v: M @ v, b, preconditioner=lambda r: r / d,
+                                     rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(x, np.linalg.solve(M, b), rtol=1e-9)
+
+
+def test_hvp_matches_finite_difference_of_gradient():
+    # Full cost, balanced: d/dt grad_x OT(x + tA, y) at a converged solve equals the HVP (up
+    # to the tau2 regularisation).  A dropped Mat term or wrong sign fails this.
+    x, y, a, b = inputs(28, 10, 8, 2)
+    x = x.astype(np.float64); y = y.astype(np.float64)
+    rng = np.random.default_rng(9)
+    A = rng.standard_normal(x.shape)
+    eps = 0.8
+
+    def grad(xx):
+        f, g = oracle.sinkhorn_symmetric(xx, y, a, b, use_epsilon_scaling=False, eps=eps,
+                                         n_iters=3000, last_extrapolation=False)
+        return oracle.grad_barycentric(xx, y, a, b, f, g, eps)[0]
+
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=eps, n_iters=3000,
+                                     last_extrapolation=False)
+    fo, go = oracle.geomloss_to_ott_potentials(f, g, a, b, eps)
+    h, info = oracle.hvp_x_from_potentials(x, y, fo, go, A, eps=eps, tau2=1e-9, cg_rtol=1e-12,
+                                           cg_atol=1e-14)
+    t = 1e-5
+    fd = (grad(x + t * A) - grad(x - t * A)) / (2 * t)
+    np.testing.assert_allclose(h, fd, rtol=2e-4, atol=1e-7)
