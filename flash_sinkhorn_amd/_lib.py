@@ -1,0 +1,98 @@
+"""ctypes binding of ``libflash_sinkhorn_hip.so`` (C ABI in include/flash_sinkhorn_hip.h).
+
+The shared object is built in-tree by ``flash_sinkhorn_amd/csrc/Makefile``.  There
+is no fallback: if it is missing, every kernel entry point raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libflash_sinkhorn_hip.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+FS_FLAG_EXP2 = 1
+FS_FLAG_REDUCED_OPERANDS = 2
+OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5 = range(6)
+
+_lib: Optional[ctypes.CDLL] = None
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int64
+_F = ctypes.c_float
+_U = ctypes.c_uint32
+_Z = ctypes.c_size_t
+_TAIL = [_U, _P, _Z, _P]  # flags, workspace, workspace_bytes, stream
+
+_SIGNATURES = {
+    "fs_version": (ctypes.c_int, []),
+    "fs_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "fs_workspace_bytes": (_Z, [ctypes.c_int, _I, _I, _I]),
+    "fs_lse": (ctypes.c_int, [_P] * 4 + [_I] * 3 + [_F] * 3 + _TAIL),
+    "fs_lse_fused": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] * 3 + _TAIL),
+    "fs_symmetric_step": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + _TAIL),
+    "fs_grad": (ctypes.c_int, [_P] * 13 + [_I] * 3 + [_F] * 2 + _TAIL),
+    "fs_apply_vec": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + [ctypes.c_int] + _TAIL),
+    "fs_apply_mat": (ctypes.c_int, [_P] * 9 + [_I] * 4 + [_F] * 2 + [ctypes.c_int] + _TAIL),
+    "fs_mat5": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + _TAIL),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", CSRC_DIR, "-j8"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("building libflash_sinkhorn_hip.so failed:\n" + res.stdout[-4000:]
+                           + res.stderr[-8000:])
+    if verbose:
+        print(res.stdout[-2000:])
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared object once; raise loudly when it is not there."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {CSRC_DIR}` "
+                "(flash_sinkhorn_amd has no non-HIP code path).")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = lib().fs_error_string(code).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {code})")
+
+
+def ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def stream_of(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def workspace(op: int, n: int, m: int, d: int, device) -> Optional[torch.Tensor]:
+    nbytes = int(lib().fs_workspace_bytes(op, n, m, d))
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def flags(use_exp2: bool, allow_tf32: bool) -> int:
+    return (FS_FLAG_EXP2 if use_exp2 else 0) | (FS_FLAG_REDUCED_OPERANDS if allow_tf32 else 0)

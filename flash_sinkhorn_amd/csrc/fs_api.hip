@@ -1,0 +1,410 @@
+// extern "C" entry points: argument checks, launch planning and kernel dispatch.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "flash_sinkhorn_hip.h"
+#include "fs_common.hpp"
+#include "fs_stream.hpp"
+
+namespace fs {
+namespace {
+
+constexpr int kMaxStreamD = 128;
+
+inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+inline int padded_d(int64_t d) {
+  if (d <= 8) return 8;
+  if (d <= 16) return 16;
+  if (d <= 32) return 32;
+  if (d <= 64) return 64;
+  return 128;
+}
+
+int env_int(const char* name, int dflt) {
+  const char* v = std::getenv(name);
+  return (v && *v) ? std::atoi(v) : dflt;
+}
+
+// Tunables (read once): blocks a launch should reach before key splitting stops.
+int target_blocks(bool has_o) {
+  static const int t_lse = env_int("FS_TARGET_BLOCKS", 2048);
+  static const int t_mat = env_int("FS_TARGET_BLOCKS_MAT", 1024);
+  return has_o ? t_mat : t_lse;
+}
+
+struct SidePlan {
+  int rb, igroups, splits, chunk;
+};
+
+// Rows per wavefront (RB blocks of 32) and the key split for one side.
+SidePlan plan_side(int mode, int64_t nq, int64_t nk, int dp) {
+  SidePlan p;
+  const bool has_o = (mode == kMat || mode == kMat5);
+  p.rb = 1;
+  if (mode == kLse || mode == kVec) p.rb = (dp <= 64 && nq >= 2048) ? 2 : 1;
+  if (mode == kMat) p.rb = (dp <= 32 && nq >= 2048) ? 2 : 1;
+  const int jt = (dp >= 128) ? 32 : 64;
+  p.igroups = ceil_div(nq, 128 * p.rb);
+  const int max_splits = (int)std::max<int64_t>(1, nk / (4 * jt));
+  const int cap = has_o ? 16 : 64;
+  int s = 1;
+  while (p.igroups * s < target_blocks(has_o) && s * 2 <= max_splits && s * 2 <= cap) s *= 2;
+  p.chunk = ceil_div(ceil_div(nk, s), jt) * jt;
+  p.splits = ceil_div(nk, p.chunk);
+  return p;
+}
+
+size_t side_ws_floats(int mode, const SidePlan& p, int64_t nq, int dp) {
+  if (p.splits <= 1) return 0;
+  size_t f = (size_t)p.splits * (size_t)nq * 2;
+  if (mode == kVec) f += (size_t)p.splits * (size_t)nq;
+  if (mode == kMat || mode == kMat5) f += (size_t)p.splits * (size_t)nq * (size_t)dp;
+  return (f + 3) & ~(size_t)3;  // keep the next region 16-byte aligned
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <int MODE, int DP, int RB, bool SEPV>
+int launch_one(const LaunchArgs& a, int blocks, hipStream_t st) {
+  hipLaunchKernelGGL((stream_kernel<MODE, DP, RB, SEPV>), dim3(blocks), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+template <int MODE, int DP, bool SEPV>
+int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
+  if constexpr (MODE == kLse || MODE == kVec) {
+    if constexpr (DP <= 64) {
+      if (rb == 2) return launch_one<MODE, DP, 2, SEPV>(a, blocks, st);
+    }
+  }
+  if constexpr (MODE == kMat) {
+    if constexpr (DP <= 32) {
+      if (rb == 2) return launch_one<MODE, DP, 2, SEPV>(a, blocks, st);
+    }
+  }
+  return launch_one<MODE, DP, 1, SEPV>(a, blocks, st);
+}
+
+template <int MODE, bool SEPV>
+int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
+  switch (dp) {
+    case 8: return launch_rb<MODE, 8, SEPV>(a, rb, blocks, st);
+    case 16: return launch_rb<MODE, 16, SEPV>(a, rb, blocks, st);
+    case 32: return launch_rb<MODE, 32, SEPV>(a, rb, blocks, st);
+    case 64: return launch_rb<MODE, 64, SEPV>(a, rb, blocks, st);
+    case 128: return launch_rb<MODE, 128, SEPV>(a, rb, blocks, st);
+  }
+  return FS_ERR_UNSUPPORTED;
+}
+
+// Plans, carves the workspace, launches the streaming kernel over one or two
+// sides and, when keys were split, the merge kernel.
+int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes,
+               hipStream_t st) {
+  if (d > kMaxStreamD) return FS_ERR_UNSUPPORTED;
+  const int dp = padded_d(d);
+  LaunchArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.d = (int)d;
+  bool vec_ok = (d % 4 == 0);
+  int rb = 2;
+  SidePlan plans[2];
+  size_t need = 0;
+  for (int s = 0; s < nsides; ++s) {
+    plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, dp);
+    rb = std::min(rb, plans[s].rb);
+  }
+  for (int s = 0; s < nsides; ++s) {
+    // both sides run in one launch and must share the rows-per-wave template
+    if (plans[s].rb != rb) {
+      plans[s].rb = rb;
+      plans[s].igroups = ceil_div(sides[s].nq, 128 * rb);
+    }
+    need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
+  }
+  if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
+  float* wsp = static_cast<float*>(ws);
+  bool any_split = false;
+  int blocks[2] = {0, 0};
+  for (int s = 0; s < nsides; ++s) {
+    Side& sd = sides[s];
+    const SidePlan& p = plans[s];
+    sd.splits = p.splits;
+    sd.chunk = p.chunk;
+    sd.igroups = p.igroups;
+    sd.part_ms = nullptr;
+    sd.part_o = nullptr;
+    if (p.splits > 1) {
+      any_split = true;
+      sd.part_ms = wsp;
+      size_t off = (size_t)p.splits * (size_t)sd.nq * 2;
+      if (mode != kLse) sd.part_o = wsp + ((off + 3) & ~(size_t)3);
+      wsp += side_ws_floats(mode, p, sd.nq, dp);
+    }
+    vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.k) && aligned16(sd.ep.out);
+    if (sd.q2) vec_ok = vec_ok && aligned16(sd.q2);
+    if (mode == kMat && sd.v) vec_ok = vec_ok && aligned16(sd.v);
+    blocks[s] = p.igroups * p.splits;
+    a.side[s] = sd;
+  }
+  if (nsides == 1) a.side[1] = a.side[0];
+  a.blocks0 = blocks[0];
+  a.vec_ok = vec_ok ? 1 : 0;
+  const int total = blocks[0] + blocks[1];
+  if (total <= 0) return FS_OK;
+
+  int rc;
+  switch (mode) {
+    case kLse: rc = launch_dp<kLse, false>(a, dp, rb, total, st); break;
+    case kVec: rc = launch_dp<kVec, false>(a, dp, rb, total, st); break;
+    case kMat:
+      rc = sepv ? launch_dp<kMat, true>(a, dp, rb, total, st)
+                : launch_dp<kMat, false>(a, dp, rb, total, st);
+      break;
+    case kMat5: rc = launch_dp<kMat5, false>(a, dp, rb, total, st); break;
+    default: rc = FS_ERR_BAD_ARGUMENT;
+  }
+  if (rc != FS_OK) return rc;
+
+  if (any_split) {
+    // sides that were not split already wrote their output; give them no items
+    const bool has_o = (mode == kMat || mode == kMat5);
+    const int per_row = has_o ? dp / 4 : 1;
+    int items[2] = {0, 0};
+    for (int s = 0; s < nsides; ++s)
+      items[s] = (a.side[s].splits > 1) ? a.side[s].nq * per_row : 0;
+    LaunchArgs f = a;
+    if (items[0] == 0 && nsides == 2) {  // only the second side needs merging
+      f.side[0] = a.side[1];
+      items[0] = items[1];
+      items[1] = 0;
+    }
+    const int tot = items[0] + items[1];
+    const int grid = ceil_div(tot, 256);
+    if (has_o)
+      hipLaunchKernelGGL((finish_kernel<true>), dim3(grid), dim3(256), 0, st, f, dp, items[0], items[1]);
+    else
+      hipLaunchKernelGGL((finish_kernel<false>), dim3(grid), dim3(256), 0, st, f, dp, items[0], items[1]);
+    if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
+  }
+  return FS_OK;
+}
+
+bool bad_sizes(int64_t n, int64_t m, int64_t d) {
+  return n <= 0 || m <= 0 || d <= 0 || n > (1 << 30) || m > (1 << 30) || d > (1 << 20);
+}
+
+Side lse_side(const float* q, const float* k, const float* kb0, float kc0, const float* kb1,
+              float kc1, int64_t nq, int64_t nk, float qscale) {
+  Side s;
+  std::memset(&s, 0, sizeof(s));
+  s.q = q; s.k = k;
+  s.kb0 = kb0; s.kc0 = kc0;
+  s.kb1 = kb1; s.kc1 = kc1;
+  s.nq = (int)nq; s.nk = (int)nk;
+  s.qscale = qscale;
+  return s;
+}
+
+void lse_epilogue(Side& s, float* out, const float* old, float alpha, float eps, float damping,
+                  const float* shift) {
+  s.ep.kind = kEpiLse;
+  s.ep.out = out;
+  s.ep.old = (alpha != 1.0f) ? old : nullptr;
+  s.ep.alpha = alpha;
+  s.ep.out_scale = -eps * damping * kLn2;
+  s.ep.shift = (shift && damping < 1.0f) ? shift : nullptr;
+  s.ep.shift_coef = alpha * (1.0f - damping);
+}
+
+}  // namespace
+}  // namespace fs
+
+using namespace fs;
+
+extern "C" {
+
+int fs_version(void) { return 1; }
+
+const char* fs_error_string(int code) {
+  switch (code) {
+    case FS_OK: return "ok";
+    case FS_ERR_NULL_POINTER: return "null pointer argument";
+    case FS_ERR_BAD_SIZE: return "size out of range";
+    case FS_ERR_BAD_ARGUMENT: return "bad argument";
+    case FS_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
+    case FS_ERR_LAUNCH_FAILED: return "kernel launch failed";
+    case FS_ERR_UNSUPPORTED: return "unsupported configuration";
+  }
+  return "unknown error";
+}
+
+size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
+  if (bad_sizes(n, m, d) || d > kMaxStreamD) return 0;
+  const int dp = padded_d(d);
+  int mode;
+  bool both = false, either = false;
+  switch (op) {
+    case FS_OP_LSE: mode = kLse; either = true; break;
+    case FS_OP_SYMMETRIC_STEP: mode = kLse; both = true; break;
+    case FS_OP_GRAD: mode = kMat; both = true; break;
+    case FS_OP_APPLY_VEC: mode = kVec; either = true; break;
+    case FS_OP_APPLY_MAT: mode = kMat; either = true; break;
+    case FS_OP_MAT5: mode = kMat5; break;
+    default: return 0;
+  }
+  // rb may be lowered when two sides share a launch: size for the rb=1 plan too
+  auto side_bytes = [&](int64_t nq, int64_t nk) {
+    SidePlan p = plan_side(mode, nq, nk, dp);
+    size_t b = side_ws_floats(mode, p, nq, dp);
+    return b * sizeof(float);
+  };
+  const size_t a = side_bytes(n, m), b = side_bytes(m, n);
+  if (both) return a + b + 64;
+  if (either) return std::max(a, b) + 64;
+  return a + 64;
+}
+
+int fs_lse(const float* x, const float* y, const float* bias, float* out, int64_t n, int64_t m,
+           int64_t d, float eps, float coord_scale, float damping, uint32_t flags,
+           void* workspace, size_t workspace_bytes, void* stream) {
+  (void)flags;
+  if (!x || !y || !bias || !out) return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
+  Side s = lse_side(x, y, bias, kLog2e, nullptr, 0.f, n, m, coord_scale / eps * kLog2e);
+  lse_epilogue(s, out, nullptr, 1.0f, eps, damping, nullptr);
+  return run_stream(kLse, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int fs_lse_fused(const float* x, const float* y, const float* pot_hat, const float* log_w,
+                 float* out, int64_t n, int64_t m, int64_t d, float eps, float coord_scale,
+                 float damping, uint32_t flags, void* workspace, size_t workspace_bytes,
+                 void* stream) {
+  (void)flags;
+  if (!x || !y || !pot_hat || !log_w || !out) return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
+  Side s = lse_side(x, y, pot_hat, kLog2e / eps, log_w, kLog2e, n, m,
+                    coord_scale / eps * kLog2e);
+  lse_epilogue(s, out, nullptr, 1.0f, eps, damping, nullptr);
+  return run_stream(kLse, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                      const float* log_a, const float* log_b, float* f_out, float* g_out,
+                      const float* shift_x, const float* shift_y, int64_t n, int64_t m,
+                      int64_t d, float eps, float alpha, float damp_f, float damp_g,
+                      float coord_scale, uint32_t flags, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  (void)flags;
+  if (!x || !y || !f_hat || !g_hat || !log_a || !log_b || !f_out || !g_out)
+    return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
+  if (f_out == f_hat || g_out == g_hat) return FS_ERR_BAD_ARGUMENT;
+  const float qs = coord_scale / eps * kLog2e;
+  Side s[2];
+  s[0] = lse_side(x, y, g_hat, kLog2e / eps, log_b, kLog2e, n, m, qs);
+  lse_epilogue(s[0], f_out, f_hat, alpha, eps, damp_f, shift_x);
+  s[1] = lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
+  lse_epilogue(s[1], g_out, g_hat, alpha, eps, damp_g, shift_y);
+  return run_stream(kLse, false, s, 2, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int fs_grad(const float* x, const float* y, const float* f, const float* g, const float* log_a,
+            const float* log_b, const float* a, const float* b, const float* x2, const float* y2,
+            const float* grad_scale, float* grad_x, float* grad_y, int64_t n, int64_t m,
+            int64_t d, float eps, float cost_scale, uint32_t flags, void* workspace,
+            size_t workspace_bytes, void* stream) {
+  (void)flags;
+  if (!x || !y || !f || !g || !log_a || !log_b || !a || !b || !x2 || !y2)
+    return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
+  const float qs = 2.0f * cost_scale / eps * kLog2e;
+  Side s[2];
+  int ns = 0;
+  if (grad_x) {
+    Side& sd = s[ns++];
+    sd = lse_side(x, y, g, kLog2e / eps, y2, -cost_scale * kLog2e / eps, n, m, qs);
+    sd.kb2 = log_b; sd.kc2 = kLog2e;
+    sd.ep.kind = kEpiGrad; sd.ep.out = grad_x; sd.ep.w = a; sd.ep.grad_scale = grad_scale;
+    sd.ep.gcoef = 2.0f * cost_scale;
+  }
+  if (grad_y) {
+    Side& sd = s[ns++];
+    sd = lse_side(y, x, f, kLog2e / eps, x2, -cost_scale * kLog2e / eps, m, n, qs);
+    sd.kb2 = log_a; sd.kc2 = kLog2e;
+    sd.ep.kind = kEpiGrad; sd.ep.out = grad_y; sd.ep.w = b; sd.ep.grad_scale = grad_scale;
+    sd.ep.gcoef = 2.0f * cost_scale;
+  }
+  if (ns == 0) return FS_OK;
+  return run_stream(kMat, false, s, ns, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int fs_apply_vec(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                 const float* log_a, const float* log_b, const float* vec, float* out,
+                 int64_t n, int64_t m, int64_t d, float eps, float coord_scale, int axis,
+                 uint32_t flags, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)flags;
+  if (!x || !y || !f_hat || !g_hat || !log_a || !log_b || !vec || !out)
+    return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f) || (axis != 0 && axis != 1)) return FS_ERR_BAD_ARGUMENT;
+  const float qs = coord_scale / eps * kLog2e;
+  Side s = (axis == 1) ? lse_side(x, y, g_hat, kLog2e / eps, log_b, kLog2e, n, m, qs)
+                       : lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
+  s.v = vec;
+  s.ep.kind = kEpiApply; s.ep.out = out; s.ep.post = 1.0f;
+  s.ep.r0 = (axis == 1) ? f_hat : g_hat; s.ep.rc0 = kLog2e / eps;
+  s.ep.r1 = (axis == 1) ? log_a : log_b; s.ep.rc1 = kLog2e;
+  return run_stream(kVec, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int fs_apply_mat(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                 const float* log_a, const float* log_b, const float* mat, const float* scale,
+                 float* out, int64_t n, int64_t m, int64_t d, int64_t dv, float eps,
+                 float coord_scale, int axis, uint32_t flags, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  (void)flags;
+  if (!x || !y || !f_hat || !g_hat || !log_a || !log_b || !mat || !out)
+    return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f) || (axis != 0 && axis != 1)) return FS_ERR_BAD_ARGUMENT;
+  if (axis == 0 && scale) return FS_ERR_BAD_ARGUMENT;
+  if (dv != d) return FS_ERR_UNSUPPORTED;
+  const float qs = coord_scale / eps * kLog2e;
+  Side s = (axis == 1) ? lse_side(x, y, g_hat, kLog2e / eps, log_b, kLog2e, n, m, qs)
+                       : lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
+  const bool sepv = !(mat == s.k && scale == nullptr);
+  s.v = sepv ? mat : nullptr;
+  s.vscale = scale;
+  s.ep.kind = kEpiApply; s.ep.out = out; s.ep.post = 1.0f;
+  s.ep.r0 = (axis == 1) ? f_hat : g_hat; s.ep.rc0 = kLog2e / eps;
+  s.ep.r1 = (axis == 1) ? log_a : log_b; s.ep.rc1 = kLog2e;
+  return run_stream(kMat, sepv, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_ott,
+            const float* A, const float* x2, const float* y2, float* out, int64_t n, int64_t m,
+            int64_t d, float eps, float cost_scale, uint32_t flags, void* workspace,
+            size_t workspace_bytes, void* stream) {
+  (void)flags;
+  if (!x || !y || !f_ott || !g_ott || !A || !x2 || !y2 || !out) return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
+  const float qs = 2.0f * cost_scale / eps * kLog2e;
+  Side s = lse_side(x, y, g_ott, kLog2e / eps, y2, -cost_scale * kLog2e / eps, n, m, qs);
+  s.q2 = A;
+  s.ep.kind = kEpiApply; s.ep.out = out; s.ep.post = -4.0f * cost_scale / eps;
+  s.ep.r0 = f_ott; s.ep.rc0 = kLog2e / eps;
+  s.ep.r1 = x2; s.ep.rc1 = -cost_scale * kLog2e / eps;
+  return run_stream(kMat5, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,81 @@
+// Shared definitions for the gfx950 FlashSinkhorn kernels.
+//
+// Every streaming kernel computes, for a block of stationary "query" rows q_i and
+// a stream of "key" rows k_j, base-2 logits
+//     L_ij = qscale * (q_i . k_j) + kbias_j
+// and reduces over j with a lane-private online soft-max.  The transport-plan
+// operations differ only in what they accumulate next to the running sum.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "flash_sinkhorn_hip.h"
+
+namespace fs {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;   // finite stand-in for -inf on masked keys
+constexpr float kLazyThresh = 16.0f;  // rescale only when the tile max exceeds 2^16
+
+enum Mode : int { kLse = 0, kVec = 1, kMat = 2, kMat5 = 3 };
+enum EpiKind : int { kEpiLse = 0, kEpiApply = 1, kEpiGrad = 2 };
+
+// What to do with a finished row (M, s, O[.]) of base-2 soft-max statistics.
+struct Epilogue {
+  int kind;
+  float* out;            // [nq] (LSE, VEC) or [nq, d] (MAT kinds)
+  // kEpiLse: out = alpha*(out_scale*(M+log2 s)) + (1-alpha)*old - shift_coef*shift
+  const float* old;
+  const float* shift;
+  float alpha, out_scale, shift_coef;
+  // kEpiApply: out = post * exp2(rc0*r0[i] + rc1*r1[i] + rc2*r2[i] + M) * O
+  const float* r0;
+  const float* r1;
+  const float* r2;
+  float rc0, rc1, rc2, post;
+  // kEpiGrad: out = gcoef * gs * w[i] * (q[i,:] - O/s)
+  const float* w;
+  const float* grad_scale;  // 1-element device array or null
+  float gcoef;
+};
+
+// One half of a launch: which rows are stationary, which are streamed.
+struct Side {
+  const float* q;       // [nq, d] stationary rows
+  const float* k;       // [nk, d] streamed rows
+  const float* q2;      // kMat5: second stationary operand [nq, d]
+  const float* v;       // kVec: [nk]; kMat: [nk, d] or null (values = k rows)
+  const float* vscale;  // kMat: optional per-key scale [nk]
+  const float* kb0;     // key bias (base 2): kc0*kb0[j] + kc1*kb1[j] + kc2*kb2[j]
+  const float* kb1;
+  const float* kb2;
+  float kc0, kc1, kc2;
+  float qscale;         // coord_scale / eps * log2(e)
+  int nq, nk;
+  int splits;           // number of key chunks
+  int chunk;            // keys per chunk (multiple of the key tile)
+  int igroups;          // ceil(nq / rows per workgroup)
+  float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
+  float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
+  Epilogue ep;
+};
+
+struct LaunchArgs {
+  Side side[2];
+  int blocks0;   // blocks belonging to side[0]; the rest belong to side[1]
+  int d;         // true feature dimension
+  int vec_ok;    // rows are 16-byte aligned (d % 4 == 0 and aligned bases)
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+__device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
+
+}  // namespace fs

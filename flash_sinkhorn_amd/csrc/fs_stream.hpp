@@ -1,0 +1,463 @@
+// Streaming plan kernels for feature dimension d <= 128 (fp32 MFMA).
+//
+// Work decomposition (one workgroup = 4 wavefronts of 64 lanes):
+//   * each wavefront owns RB blocks of 32 stationary query rows, held in VGPRs
+//     for the whole sweep, pre-multiplied by qscale;
+//   * the workgroup streams its chunk of key rows through LDS in tiles of JT
+//     rows (double buffered, one barrier per tile); all four wavefronts read the
+//     same key tile;
+//   * logits are produced TRANSPOSED, (keys x queries), by
+//     v_mfma_f32_32x32x2_f32 with the key tile as the A operand.  In that layout
+//     a lane holds ONE query column and 16 key rows, so the online soft-max over
+//     keys is lane-private: no cross-lane traffic in the inner loop.  The two
+//     half-waves of a column are merged once at the end;
+//   * one extra MFMA per tile adds kbias_j - M_i to every logit (A = [kbias, 1],
+//     B = [1, -M]), so masking, the bias and the running-max subtraction cost no
+//     VALU work.  The running max M is only moved when a tile exceeds it by
+//     more than 2^16 ("lazy rescale"), a wave-uniform rare branch;
+//   * exp'ed logits are already laid out as the B operand of a second MFMA
+//     against the value tile (keys x d), which accumulates O^T for the
+//     gradient / plan-matrix / mat5 kinds.
+//
+// The key range can be split into `splits` chunks to fill the chip; partial
+// (M, s, O) statistics are then merged by finish_kernel.
+#pragma once
+
+#include "fs_common.hpp"
+
+namespace fs {
+
+template <int DP>
+struct Geo {
+  static constexpr int JT = (DP >= 128) ? 32 : 64;  // key rows per LDS tile
+  static constexpr int NSUB = JT / 32;
+  static constexpr int LDW = DP + 4;                // padded LDS row stride (floats)
+  static constexpr int KK = DP / 2;                 // MFMAs per 32x32 logits tile
+  static constexpr int NQ8 = DP / 8;
+  static constexpr int NDB = (DP + 31) / 32;        // 32-wide output column blocks
+  static constexpr int V4_PER_ROW = DP / 4;
+  static constexpr int V4_TOTAL = JT * V4_PER_ROW;
+  static constexpr int PER_THREAD = (V4_TOTAL + 255) / 256;
+  static constexpr bool VDB = false;                // separate value tile is single buffered
+};
+
+__device__ __forceinline__ float4 load_row4(const float* __restrict__ base, int row, int nrows,
+                                            int col, int d, bool vec_ok) {
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (row < nrows && col < d) {
+    const float* p = base + (size_t)row * (size_t)d + col;
+    if (vec_ok) {
+      v = *reinterpret_cast<const float4*>(p);
+    } else {
+      v.x = p[0];
+      if (col + 1 < d) v.y = p[1];
+      if (col + 2 < d) v.z = p[2];
+      if (col + 3 < d) v.w = p[3];
+    }
+  }
+  return v;
+}
+
+__device__ __forceinline__ float key_bias(const Side& sd, int j, int j_end) {
+  float b = kNegBig;
+  if (j < j_end) {
+    b = sd.kc0 * sd.kb0[j];
+    if (sd.kb1) b += sd.kc1 * sd.kb1[j];
+    if (sd.kb2) b += sd.kc2 * sd.kb2[j];
+    b = fmaxf(b, kNegBig);
+  }
+  return b;
+}
+
+// ---- epilogues -------------------------------------------------------------
+
+__device__ __forceinline__ float apply_row_factor(const Epilogue& ep, int row, float M) {
+  float t = M + ep.rc0 * ep.r0[row];
+  if (ep.r1) t += ep.rc1 * ep.r1[row];
+  if (ep.r2) t += ep.rc2 * ep.r2[row];
+  return ep.post * exp2f(t);
+}
+
+__device__ __forceinline__ void epilogue_scalar(const Epilogue& ep, int row, float M, float s,
+                                                float o) {
+  if (ep.kind == kEpiLse) {
+    float cand = ep.out_scale * (M + log2f(fmaxf(s, 1e-40f)));
+    float r = ep.alpha * cand;
+    if (ep.old) r += (1.0f - ep.alpha) * ep.old[row];
+    if (ep.shift) r -= ep.shift_coef * ep.shift[row];
+    ep.out[row] = r;
+  } else {
+    ep.out[row] = apply_row_factor(ep, row, M) * o;
+  }
+}
+
+__device__ __forceinline__ void epilogue_vec4(const Epilogue& ep, const float* __restrict__ q,
+                                              int d, bool vec_ok, int row, int col, float M,
+                                              float s, float4 O) {
+  if (col >= d) return;
+  float4 r;
+  if (ep.kind == kEpiGrad) {
+    float gs = ep.grad_scale ? ep.grad_scale[0] : 1.0f;
+    float c = ep.gcoef * gs * ep.w[row];
+    float inv = 1.0f / fmaxf(s, 1e-40f);
+    float4 x = load_row4(q, row, row + 1, col, d, vec_ok);
+    r = make_float4(c * (x.x - O.x * inv), c * (x.y - O.y * inv), c * (x.z - O.z * inv),
+                    c * (x.w - O.w * inv));
+  } else {
+    float c = apply_row_factor(ep, row, M);
+    r = make_float4(c * O.x, c * O.y, c * O.z, c * O.w);
+  }
+  float* p = ep.out + (size_t)row * (size_t)d + col;
+  if (vec_ok) {
+    *reinterpret_cast<float4*>(p) = r;
+  } else {
+    p[0] = r.x;
+    if (col + 1 < d) p[1] = r.y;
+    if (col + 2 < d) p[2] = r.z;
+    if (col + 3 < d) p[3] = r.w;
+  }
+}
+
+// ---- main kernel -----------------------------------------------------------
+
+template <int MODE, int DP, int RB, bool SEPV>
+__global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
+  using G = Geo<DP>;
+  constexpr bool kHasO = (MODE == kMat || MODE == kMat5);
+  constexpr int NVBUF = G::VDB ? 2 : 1;
+
+  __shared__ __attribute__((aligned(16))) float lds_k[2][G::JT * G::LDW];
+  __shared__ __attribute__((aligned(16))) float lds_v[SEPV ? NVBUF : 1][SEPV ? G::JT * G::LDW : 4];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][G::JT];
+  __shared__ __attribute__((aligned(16))) float lds_x[2][MODE == kVec ? G::JT : 4];
+
+  int bid = blockIdx.x;
+  const bool second = bid >= args.blocks0;
+  if (second) bid -= args.blocks0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const int d = args.d;
+  const bool vec_ok = args.vec_ok != 0;
+
+  const int split = bid % sd.splits;
+  const int ig = bid / sd.splits;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int h = lane >> 5;
+  const int row0 = (ig * 4 + wave) * (32 * RB);
+  const int j_begin = split * sd.chunk;
+  const int j_end = min(sd.nk, j_begin + sd.chunk);
+  const int ntiles = (j_end - j_begin + G::JT - 1) / G::JT;
+
+  // ---- stationary operands: lane (li, h) keeps q[row][8q+4h+t] for all q, t ----
+  float xs[RB][G::KK];
+  float x2s[MODE == kMat5 ? RB : 1][MODE == kMat5 ? G::KK : 1];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = row0 + rb * 32 + li;
+#pragma unroll
+    for (int q = 0; q < G::NQ8; ++q) {
+      float4 v = load_row4(sd.q, row, sd.nq, 8 * q + 4 * h, d, vec_ok);
+      xs[rb][4 * q + 0] = v.x * sd.qscale;
+      xs[rb][4 * q + 1] = v.y * sd.qscale;
+      xs[rb][4 * q + 2] = v.z * sd.qscale;
+      xs[rb][4 * q + 3] = v.w * sd.qscale;
+      if constexpr (MODE == kMat5) {
+        float4 u = load_row4(sd.q2, row, sd.nq, 8 * q + 4 * h, d, vec_ok);
+        x2s[rb][4 * q + 0] = u.x;
+        x2s[rb][4 * q + 1] = u.y;
+        x2s[rb][4 * q + 2] = u.z;
+        x2s[rb][4 * q + 3] = u.w;
+      }
+    }
+  }
+
+  float run_m[RB], run_s[RB], run_o[RB];
+  f32x16 oacc[kHasO ? RB : 1][kHasO ? G::NDB : 1];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    run_m[rb] = 0.f;
+    run_s[rb] = 0.f;
+    run_o[rb] = 0.f;
+    if constexpr (kHasO) {
+#pragma unroll
+      for (int db = 0; db < G::NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[rb][db][r] = 0.f;
+    }
+  }
+
+  // ---- tile staging registers ----
+  float4 st_k[G::PER_THREAD];
+  float4 st_v[SEPV ? G::PER_THREAD : 1];
+  float st_b = 0.f, st_x = 0.f;
+
+  auto stage_load = [&](int j0) {
+#pragma unroll
+    for (int c = 0; c < G::PER_THREAD; ++c) {
+      const int idx = tid + 256 * c;
+      const int r = idx / G::V4_PER_ROW;
+      const int c4 = (idx % G::V4_PER_ROW) * 4;
+      const int j = j0 + r;
+      st_k[c] = load_row4(sd.k, j, j_end, c4, d, vec_ok);
+      if constexpr (SEPV) {
+        float4 v = load_row4(sd.v, j, j_end, c4, d, vec_ok);
+        if (sd.vscale && j < j_end) {
+          const float sc = sd.vscale[j];
+          v.x *= sc; v.y *= sc; v.z *= sc; v.w *= sc;
+        }
+        st_v[c] = v;
+      }
+    }
+    if (tid < G::JT) {
+      st_b = key_bias(sd, j0 + tid, j_end);
+    } else if (MODE == kVec && tid < 2 * G::JT) {
+      const int j = j0 + tid - G::JT;
+      st_x = (j < j_end) ? sd.v[j] : 0.f;
+    }
+  };
+  auto stage_store_k = [&](int buf) {
+#pragma unroll
+    for (int c = 0; c < G::PER_THREAD; ++c) {
+      const int idx = tid + 256 * c;
+      if (G::V4_TOTAL % 256 == 0 || idx < G::V4_TOTAL) {
+        const int r = idx / G::V4_PER_ROW;
+        const int c4 = (idx % G::V4_PER_ROW) * 4;
+        *reinterpret_cast<float4*>(&lds_k[buf][r * G::LDW + c4]) = st_k[c];
+      }
+    }
+    if (tid < G::JT) {
+      lds_b[buf][tid] = st_b;
+    } else if (MODE == kVec && tid < 2 * G::JT) {
+      lds_x[buf][tid - G::JT] = st_x;
+    }
+  };
+  auto stage_store_v = [&](int buf) {
+    if constexpr (SEPV) {
+#pragma unroll
+      for (int c = 0; c < G::PER_THREAD; ++c) {
+        const int idx = tid + 256 * c;
+        if (G::V4_TOTAL % 256 == 0 || idx < G::V4_TOTAL) {
+          const int r = idx / G::V4_PER_ROW;
+          const int c4 = (idx % G::V4_PER_ROW) * 4;
+          *reinterpret_cast<float4*>(&lds_v[buf][r * G::LDW + c4]) = st_v[c];
+        }
+      }
+    }
+  };
+
+  stage_load(j_begin);
+  stage_store_k(0);
+  stage_store_v(0);
+  __syncthreads();
+
+  for (int t = 0; t < ntiles; ++t) {
+    const int buf = t & 1;
+    const int vbuf = G::VDB ? buf : 0;
+    const bool more = (t + 1 < ntiles);
+    if (more) stage_load(j_begin + (t + 1) * G::JT);
+
+    const float* kt = lds_k[buf];
+    const float* vt = SEPV ? lds_v[vbuf] : lds_k[buf];
+
+#pragma unroll
+    for (int js = 0; js < G::NSUB; ++js) {
+      // A operand of the logits MFMAs: key row (js*32+li), columns 8q+4h+t
+      float ya[G::KK];
+      const float* yrow = kt + (js * 32 + li) * G::LDW + 4 * h;
+#pragma unroll
+      for (int q = 0; q < G::NQ8; ++q) {
+        const float4 v = *reinterpret_cast<const float4*>(yrow + 8 * q);
+        ya[4 * q + 0] = v.x;
+        ya[4 * q + 1] = v.y;
+        ya[4 * q + 2] = v.z;
+        ya[4 * q + 3] = v.w;
+      }
+      const float ab = h ? 1.0f : lds_b[buf][js * 32 + li];
+
+      float vj[MODE == kVec ? 16 : 1];
+      if constexpr (MODE == kVec) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const float4 v =
+              *reinterpret_cast<const float4*>(&lds_x[buf][js * 32 + 8 * q4 + 4 * h]);
+          vj[4 * q4 + 0] = v.x;
+          vj[4 * q4 + 1] = v.y;
+          vj[4 * q4 + 2] = v.z;
+          vj[4 * q4 + 3] = v.w;
+        }
+      }
+
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < G::KK; ++kk)
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya[kk], xs[rb][kk], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
+
+        f32x16 tacc;
+        if constexpr (MODE == kMat5) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tacc[r] = 0.f;
+#pragma unroll
+          for (int kk = 0; kk < G::KK; ++kk)
+            tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya[kk], x2s[rb][kk], tacc, 0, 0, 0);
+        }
+
+        float tmax = fmaxf(acc[0], acc[1]);
+#pragma unroll
+        for (int r = 2; r < 16; ++r) tmax = fmaxf(tmax, acc[r]);
+
+        const bool first = (t == 0 && js == 0);
+        if (first || wave_any(tmax > kLazyThresh)) {
+          const float tm = fmaxf(tmax, xor32(tmax));
+          const float delta = (first || tm > kLazyThresh) ? tm : 0.f;
+          const float resc = first ? 0.f : fast_exp2(-delta);
+          run_m[rb] += delta;
+          run_s[rb] *= resc;
+          run_o[rb] *= resc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] -= delta;
+          if constexpr (kHasO) {
+#pragma unroll
+            for (int db = 0; db < G::NDB; ++db)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) oacc[rb][db][r] *= resc;
+          }
+        }
+
+        float p[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) p[r] = fast_exp2(acc[r]);
+
+        if constexpr (MODE != kMat5) {
+          float ps = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) ps += p[r];
+          run_s[rb] += ps;
+        }
+        if constexpr (MODE == kVec) {
+          float po = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) po += p[r] * vj[r];
+          run_o[rb] += po;
+        }
+        if constexpr (MODE == kMat5) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) p[r] *= tacc[r];
+        }
+        if constexpr (kHasO) {
+          // O^T[dd][i] += V[j][dd] * P^T[j][i]; register r of p holds key row
+          // j = js*32 + 8*(r/4) + 4*h + (r%4), which is this lane's K slot.
+#pragma unroll
+          for (int db = 0; db < G::NDB; ++db) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int jr = js * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+              const int col = db * 32 + li;
+              const float va = (DP % 32 == 0 || col < DP) ? vt[jr * G::LDW + col] : 0.f;
+              oacc[rb][db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, p[r], oacc[rb][db], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+
+    if (more) {
+      if constexpr (SEPV && !G::VDB) __syncthreads();
+      stage_store_k(buf ^ 1);
+      stage_store_v(G::VDB ? (buf ^ 1) : 0);
+    }
+    __syncthreads();
+  }
+
+  // ---- merge the two half-waves of each query column, then finish or spill ----
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = row0 + rb * 32 + li;
+    const float M = run_m[rb];
+    const float s = run_s[rb] + xor32(run_s[rb]);
+    const float o = run_o[rb] + xor32(run_o[rb]);
+    const bool live = row < sd.nq;
+    if (sd.splits == 1) {
+      if constexpr (!kHasO) {
+        if (live && h == 0) epilogue_scalar(sd.ep, row, M, s, o);
+      } else {
+        if (live) {
+#pragma unroll
+          for (int db = 0; db < G::NDB; ++db)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+              const int col = db * 32 + 8 * q4 + 4 * h;
+              const float4 O = make_float4(oacc[rb][db][4 * q4], oacc[rb][db][4 * q4 + 1],
+                                           oacc[rb][db][4 * q4 + 2], oacc[rb][db][4 * q4 + 3]);
+              epilogue_vec4(sd.ep, sd.q, d, vec_ok, row, col, M, s, O);
+            }
+        }
+      }
+    } else if (live) {
+      const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+      if (h == 0) {
+        sd.part_ms[2 * pr] = M;
+        sd.part_ms[2 * pr + 1] = s;
+        if constexpr (MODE == kVec) sd.part_o[pr] = o;
+      }
+      if constexpr (kHasO) {
+#pragma unroll
+        for (int db = 0; db < G::NDB; ++db)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const int col = db * 32 + 8 * q4 + 4 * h;
+            if (DP % 32 == 0 || col < DP) {
+              *reinterpret_cast<float4*>(&sd.part_o[pr * DP + col]) =
+                  make_float4(oacc[rb][db][4 * q4], oacc[rb][db][4 * q4 + 1],
+                              oacc[rb][db][4 * q4 + 2], oacc[rb][db][4 * q4 + 3]);
+            }
+          }
+      }
+    }
+  }
+}
+
+// Merge `splits` partial rows and run the epilogue.  One thread per output row
+// (scalar kinds) or per 4 output columns (matrix kinds); grid covers both sides.
+template <bool HAS_O>
+__global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int dp, int items0,
+                                                     int items1) {
+  int it = blockIdx.x * 256 + threadIdx.x;
+  if (it >= items0 + items1) return;  // the other side may have nothing to merge
+  const bool second = it >= items0;
+  if (second) it -= items0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const int per_row = HAS_O ? dp / 4 : 1;
+  const int row = it / per_row;
+  const int col = (it % per_row) * 4;
+  if (row >= sd.nq) return;
+  float M = -3.0e38f;
+  for (int sp = 0; sp < sd.splits; ++sp)
+    M = fmaxf(M, sd.part_ms[2 * ((size_t)sp * sd.nq + row)]);
+  float s = 0.f, o = 0.f;
+  float4 O = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int sp = 0; sp < sd.splits; ++sp) {
+    const size_t pr = (size_t)sp * sd.nq + row;
+    const float w = exp2f(sd.part_ms[2 * pr] - M);
+    s += w * sd.part_ms[2 * pr + 1];
+    if constexpr (HAS_O) {
+      const float4 v = *reinterpret_cast<const float4*>(&sd.part_o[pr * dp + col]);
+      O.x += w * v.x; O.y += w * v.y; O.z += w * v.z; O.w += w * v.w;
+    } else if (sd.part_o) {
+      o += w * sd.part_o[pr];
+    }
+  }
+  if constexpr (HAS_O) {
+    epilogue_vec4(sd.ep, sd.q, args.d, args.vec_ok != 0, row, col, M, s, O);
+  } else {
+    epilogue_scalar(sd.ep, row, M, s, o);
+  }
+}
+
+}  // namespace fs

@@ -1,0 +1,162 @@
+"""Shifted-potential log-sum-exp launchers (gfx950 HIP kernels behind a C ABI).
+
+Same public surface as the reference's ``kernels/sinkhorn_flashstyle_sqeuclid.py``:
+``flashsinkhorn_lse`` (:815-955), ``flashsinkhorn_lse_fused`` (:958-1090),
+``flashsinkhorn_symmetric_step`` (:1093-1317), the precompute/bias/shift helpers
+(:68-147, :1324-1363) and re-exports of the two solvers (:1370-1373).
+
+With alpha_i = cost_scale*|x_i|^2, beta_j = cost_scale*|y_j|^2 and shifted
+potentials f_hat = f - alpha, g_hat = g - beta, one half-update is
+    f_hat_i = -eps * damping * LSE_j[ 2*cost_scale*x_i.y_j/eps + g_hat_j/eps + log b_j ].
+Triton tuning keywords (block_*, num_warps, num_stages, autotune) are accepted
+and ignored; ``use_exp2`` selects nothing (the kernels work in base 2, which is
+the same function); ``allow_tf32=False`` means strict fp32 MFMA operands.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from flash_sinkhorn_amd import _lib
+from flash_sinkhorn_amd.kernels._common import _f32c, log_weights
+
+__all__ = [
+    "precompute_flashsinkhorn_inputs", "compute_bias_f", "compute_bias_g",
+    "flashsinkhorn_lse", "flashsinkhorn_lse_fused", "flashsinkhorn_symmetric_step",
+    "shifted_to_standard_potentials", "standard_to_shifted_potentials",
+    "sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric",
+]
+
+
+def precompute_flashsinkhorn_inputs(x, y, a, b, eps: float, cost_scale: float = 1.0):
+    """(alpha, beta, gamma, delta) = (cs|x|^2, cs|y|^2, eps*log a, eps*log b)."""
+    alpha = cost_scale * (x.float() ** 2).sum(dim=1)
+    beta = cost_scale * (y.float() ** 2).sum(dim=1)
+    return alpha, beta, eps * log_weights(a), eps * log_weights(b)
+
+
+def compute_bias_f(g, beta, delta, eps: float):
+    """u = (g - beta + delta)/eps, the key bias of the f half-update."""
+    return ((g - beta) + delta) / eps
+
+
+def compute_bias_g(f, alpha, gamma, eps: float):
+    """v = (f - alpha + gamma)/eps, the key bias of the g half-update."""
+    return ((f - alpha) + gamma) / eps
+
+
+def shifted_to_standard_potentials(f_hat, g_hat, alpha, beta):
+    return f_hat + alpha, g_hat + beta
+
+
+def standard_to_shifted_potentials(f, g, alpha, beta):
+    return f - alpha, g - beta
+
+
+def flashsinkhorn_lse(
+    x: torch.Tensor, y: torch.Tensor, bias: torch.Tensor, eps: float, *,
+    cost_scale: float = 1.0, damping: float = 1.0, allow_tf32: bool = True,
+    use_exp2: bool = True, block_m: Optional[int] = None, block_n: Optional[int] = None,
+    block_k: Optional[int] = None, num_warps: Optional[int] = None, num_stages: int = 2,
+    autotune: bool = True,
+) -> torch.Tensor:
+    """out_i = -eps*damping*LSE_j[2*cost_scale*x_i.y_j/eps + bias_j]; returns fp32 [n]."""
+    if not x.is_cuda or not y.is_cuda:
+        raise ValueError("x and y must be CUDA tensors")
+    if x.ndim != 2 or y.ndim != 2:
+        raise ValueError("x and y must be 2D tensors")
+    if bias.ndim != 1:
+        raise ValueError("bias must be 1D tensor")
+    n, d = x.shape
+    m, d2 = y.shape
+    if d != d2:
+        raise ValueError("x and y must have same feature dimension")
+    if bias.shape[0] != m:
+        raise ValueError(f"bias must have length {m}, got {bias.shape[0]}")
+    x, y, bias = _f32c(x), _f32c(y), _f32c(bias)
+    out = torch.empty((n,), device=x.device, dtype=torch.float32)
+    ws = _lib.workspace(_lib.OP_LSE, n, m, d, x.device)
+    rc = _lib.lib().fs_lse(
+        x.data_ptr(), y.data_ptr(), bias.data_ptr(), out.data_ptr(), n, m, d,
+        float(eps), 2.0 * float(cost_scale), float(damping), _lib.flags(use_exp2, allow_tf32),
+        _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_of(x))
+    _lib.check(rc, "fs_lse")
+    return out
+
+
+def flashsinkhorn_lse_fused(
+    x: torch.Tensor, y: torch.Tensor, g_hat: torch.Tensor, log_w: torch.Tensor, eps: float, *,
+    cost_scale: float = 1.0, damping: float = 1.0, allow_tf32: bool = True,
+    use_exp2: bool = True, block_m: Optional[int] = None, block_n: Optional[int] = None,
+    block_k: Optional[int] = None, num_warps: Optional[int] = None, num_stages: int = 2,
+    autotune: bool = True,
+) -> torch.Tensor:
+    """Same as flashsinkhorn_lse with bias_j = g_hat_j/eps + log_w_j formed in the kernel."""
+    if not x.is_cuda or not y.is_cuda:
+        raise ValueError("x and y must be CUDA tensors")
+    n, d = x.shape
+    m, d2 = y.shape
+    if d != d2:
+        raise ValueError("x and y must have same feature dimension")
+    if g_hat.shape[0] != m or log_w.shape[0] != m:
+        raise ValueError(f"g_hat and log_w must have length {m}")
+    x, y, g_hat, log_w = _f32c(x), _f32c(y), _f32c(g_hat), _f32c(log_w)
+    out = torch.empty((n,), device=x.device, dtype=torch.float32)
+    ws = _lib.workspace(_lib.OP_LSE, n, m, d, x.device)
+    rc = _lib.lib().fs_lse_fused(
+        x.data_ptr(), y.data_ptr(), g_hat.data_ptr(), log_w.data_ptr(), out.data_ptr(), n, m, d,
+        float(eps), 2.0 * float(cost_scale), float(damping), _lib.flags(use_exp2, allow_tf32),
+        _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_of(x))
+    _lib.check(rc, "fs_lse_fused")
+    return out
+
+
+def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, alpha, damping_f,
+                        damping_g, shift_x=None, shift_y=None, allow_tf32=True, use_exp2=True):
+    """One launch on already contiguous fp32 operands.  With shift_x/shift_y the
+    unbalanced shift correction is applied inside the epilogue."""
+    n, d = x.shape
+    m = y.shape[0]
+    f_out = torch.empty((n,), device=x.device, dtype=torch.float32)
+    g_out = torch.empty((m,), device=x.device, dtype=torch.float32)
+    ws = _lib.workspace(_lib.OP_SYMMETRIC_STEP, n, m, d, x.device)
+    rc = _lib.lib().fs_symmetric_step(
+        x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
+        log_b.data_ptr(), f_out.data_ptr(), g_out.data_ptr(), _lib.ptr(shift_x),
+        _lib.ptr(shift_y), n, m, d, float(eps), float(alpha), float(damping_f), float(damping_g),
+        2.0 * float(cost_scale), _lib.flags(use_exp2, allow_tf32), _lib.ptr(ws),
+        0 if ws is None else ws.numel(), _lib.stream_of(x))
+    _lib.check(rc, "fs_symmetric_step")
+    return f_out, g_out
+
+
+def flashsinkhorn_symmetric_step(
+    x: torch.Tensor, y: torch.Tensor, f_hat: torch.Tensor, g_hat: torch.Tensor,
+    log_a: torch.Tensor, log_b: torch.Tensor, eps: float, *,
+    cost_scale: float = 1.0, alpha: float = 0.5, damping_f: float = 1.0, damping_g: float = 1.0,
+    allow_tf32: bool = True, use_exp2: bool = True, autotune: bool = True,
+    block_m: Optional[int] = None, block_n: Optional[int] = None, block_k: Optional[int] = None,
+    num_warps: Optional[int] = None, num_stages: int = 2,
+    label_x: Optional[torch.Tensor] = None, label_y: Optional[torch.Tensor] = None,
+    label_cost_matrix: Optional[torch.Tensor] = None, lambda_x: float = 1.0,
+    lambda_y: float = 0.0,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Both Jacobi half-steps in one launch, each from the OLD potentials:
+    f_new = (1-alpha) f_hat + alpha*(-eps*damping_f*LSE_j[...]), g_new likewise over i.
+    The OTDD label-cost variant (label_* with lambda_y != 0) is not built."""
+    if (label_x is not None and label_y is not None and label_cost_matrix is not None
+            and lambda_y != 0.0):
+        raise NotImplementedError("label-augmented cost is not part of this build")
+    if not x.is_cuda or not y.is_cuda:
+        raise ValueError("x and y must be CUDA tensors")
+    return _symmetric_step_raw(
+        _f32c(x), _f32c(y), _f32c(f_hat), _f32c(g_hat), _f32c(log_a), _f32c(log_b), eps,
+        cost_scale=cost_scale, alpha=alpha, damping_f=damping_f, damping_g=damping_g,
+        allow_tf32=allow_tf32, use_exp2=use_exp2)
+
+
+from flash_sinkhorn_amd.sinkhorn_solvers import (  # noqa: E402
+    sinkhorn_flashstyle_alternating,
+    sinkhorn_flashstyle_symmetric,
+)

@@ -1,0 +1,209 @@
+"""Host loops of the two Sinkhorn solvers over the HIP log-sum-exp kernels.
+
+Same signatures, defaults, return conventions and iteration bookkeeping as the
+reference's ``sinkhorn_solvers.py`` (alternating :30-287, symmetric :290-707).
+Everything device-side is one C-ABI call per step; the loops themselves are a
+few lines of Python because the averaging, damping and the unbalanced shift
+correction live in the kernel epilogue.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from flash_sinkhorn_amd.kernels._common import (
+    _f32c, dampening, epsilon_schedule, log_weights, max_diameter,
+)
+
+__all__ = ["sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric"]
+
+# Reference switches from the one-launch step to two launches at this n
+# (sinkhorn_solvers.py:463-468).  Both give the same numbers; here the one-launch
+# step is used at every size unless the caller passes fused=False.
+_FUSE_THRESHOLD = 30000
+
+
+def _resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y):
+    """rho_x/rho_y beat reach_x/reach_y beat rho beats reach; reach**2 = rho."""
+    if rho is not None and reach is not None:
+        raise ValueError("Specify either rho or reach, not both.")
+    if reach is not None:
+        rho = reach ** 2
+    if rho is not None:
+        if rho_x is None and reach_x is None:
+            rho_x = rho
+        if rho_y is None and reach_y is None:
+            rho_y = rho
+    if reach_x is not None:
+        if rho_x is not None:
+            raise ValueError("Specify either rho_x or reach_x, not both.")
+        rho_x = reach_x ** 2
+    if reach_y is not None:
+        if rho_y is not None:
+            raise ValueError("Specify either rho_y or reach_y, not both.")
+        rho_y = reach_y ** 2
+    return rho_x, rho_y
+
+
+def _max_change(f, g, prev_f, prev_g) -> float:
+    return max((f - prev_f).abs().max().item(), (g - prev_g).abs().max().item())
+
+
+def sinkhorn_flashstyle_alternating(
+    x: torch.Tensor, y: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *,
+    eps: float = 0.1, n_iters: int = 100, cost_scale: float = 1.0,
+    rho: Optional[float] = None, reach: Optional[float] = None,
+    rho_x: Optional[float] = None, rho_y: Optional[float] = None,
+    reach_x: Optional[float] = None, reach_y: Optional[float] = None,
+    allow_tf32: bool = True, use_exp2: bool = True, autotune: bool = True,
+    threshold: Optional[float] = None, check_every: int = 5, return_n_iters: bool = False,
+    ott_convention: bool = False,
+):
+    """Gauss-Seidel Sinkhorn at fixed eps: f from g, then g from the NEW f.
+
+    GeomLoss convention (default): weights inside the LSE, P = a b exp((f+g-C)/eps).
+    ``ott_convention=True``: g is updated first and eps*log(weight) sits outside the
+    LSE, P = exp((f+g-C)/eps).  With rho set, the kernel damps the whole shifted
+    value and, as in the reference (:240-259), no shift correction follows.
+    The early-stop test every ``check_every`` iterations compares against the
+    potentials of the previous check (the initial ones at the first check).
+    Returns (f, g) or (f, g, n_iters_used).
+    """
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        flashsinkhorn_lse, flashsinkhorn_lse_fused,
+    )
+
+    rho_x, rho_y = _resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y)
+    damp_f, damp_g = dampening(eps, rho_x), dampening(eps, rho_y)
+    xf, yf = x.float().contiguous(), y.float().contiguous()
+    alpha = cost_scale * (xf * xf).sum(dim=1)
+    beta = cost_scale * (yf * yf).sum(dim=1)
+    log_a, log_b = log_weights(a), log_weights(b)
+    f_hat, g_hat = -alpha, -beta
+    prev_f, prev_g = (f_hat.clone(), g_hat.clone()) if threshold is not None else (None, None)
+    kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
+
+    used = 0
+    for it in range(int(n_iters)):
+        if ott_convention:
+            g_hat = eps * log_b + flashsinkhorn_lse(yf, xf, f_hat / eps, eps, damping=damp_g, **kw)
+            f_hat = eps * log_a + flashsinkhorn_lse(xf, yf, g_hat / eps, eps, damping=damp_f, **kw)
+        else:
+            f_hat = flashsinkhorn_lse_fused(xf, yf, g_hat, log_b, eps, damping=damp_f, **kw)
+            g_hat = flashsinkhorn_lse_fused(yf, xf, f_hat, log_a, eps, damping=damp_g, **kw)
+        used += 1
+        if threshold is not None and (it + 1) % check_every == 0:
+            if _max_change(f_hat, g_hat, prev_f, prev_g) < threshold:
+                break
+            prev_f, prev_g = f_hat.clone(), g_hat.clone()
+
+    f, g = f_hat + alpha, g_hat + beta
+    return (f, g, used) if return_n_iters else (f, g)
+
+
+def sinkhorn_flashstyle_symmetric(
+    x: torch.Tensor, y: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *,
+    blur: float = 0.05, scaling: float = 0.5, use_epsilon_scaling: bool = True,
+    last_extrapolation: bool = True, cost_scale: float = 1.0,
+    eps: Optional[float] = None, n_iters: Optional[int] = None,
+    diameter: Optional[float] = None, eps_list: Optional[Sequence[float]] = None,
+    rho: Optional[float] = None, reach: Optional[float] = None,
+    rho_x: Optional[float] = None, rho_y: Optional[float] = None,
+    reach_x: Optional[float] = None, reach_y: Optional[float] = None,
+    allow_tf32: bool = True, use_exp2: bool = True, autotune: bool = True,
+    fused: Optional[bool] = None, threshold: Optional[float] = None, check_every: int = 5,
+    return_n_iters: bool = False, return_prelast: bool = False,
+    f_init: Optional[torch.Tensor] = None, g_init: Optional[torch.Tensor] = None,
+    label_x: Optional[torch.Tensor] = None, label_y: Optional[torch.Tensor] = None,
+    label_cost_matrix: Optional[torch.Tensor] = None, lambda_x: float = 1.0,
+    lambda_y: float = 0.0,
+):
+    """GeomLoss-style symmetric (Jacobi, averaged) Sinkhorn with an eps schedule.
+
+    Steps: one full step at eps_list[0]; one averaged step (weight 1/2) per entry
+    of eps_list; if ``last_extrapolation`` one more full step at eps_list[-1].
+    Unbalanced marginals (rho_x / rho_y) enter as the per-step damping
+    1/(1+eps/rho) of the soft-min, i.e. in standard potentials
+    f <- (1-w) f + w*damp_f*softmin_eps(g).
+    Early stop: every ``check_every`` averaged steps; the first check only takes a
+    snapshot.  ``f_init``/``g_init`` warm-start (standard potentials).
+    Returns (f, g[, f_prelast, g_prelast][, n_iters_used]); the prelast pair is
+    only returned when ``return_prelast and last_extrapolation``.
+    """
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        _symmetric_step_raw, flashsinkhorn_lse,
+    )
+
+    if (label_x is not None and label_y is not None and label_cost_matrix is not None
+            and lambda_y != 0.0):
+        raise NotImplementedError("label-augmented cost is not part of this build")
+    rho_x, rho_y = _resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y)
+
+    if eps_list is None:
+        if use_epsilon_scaling:
+            if diameter is None:
+                diameter = max_diameter(x, y)
+            eps_list = epsilon_schedule(diameter, blur, scaling, p=2.0)
+        else:
+            if eps is None or n_iters is None:
+                raise ValueError("When use_epsilon_scaling=False, provide eps and n_iters")
+            eps_list = [float(eps)] * int(n_iters)
+    if len(eps_list) == 0:
+        raise ValueError("eps_list must be non-empty")
+    if n_iters is not None:
+        eps_list = list(eps_list)[: int(n_iters)]
+
+    xf, yf = x.float().contiguous(), y.float().contiguous()
+    alpha = (cost_scale * (xf * xf).sum(dim=1)).contiguous()
+    beta = (cost_scale * (yf * yf).sum(dim=1)).contiguous()
+    log_a, log_b = _f32c(log_weights(a)), _f32c(log_weights(b))
+    f_hat = -alpha if f_init is None else _f32c(f_init) - alpha
+    g_hat = -beta if g_init is None else _f32c(g_init) - beta
+    if fused is None:
+        fused = True
+
+    def jacobi(f_hat, g_hat, e, w):
+        damp_f, damp_g = dampening(e, rho_x), dampening(e, rho_y)
+        if fused:
+            return _symmetric_step_raw(
+                xf, yf, f_hat, g_hat, log_a, log_b, e, cost_scale=cost_scale, alpha=w,
+                damping_f=damp_f, damping_g=damp_g,
+                shift_x=alpha if damp_f < 1.0 else None, shift_y=beta if damp_g < 1.0 else None,
+                allow_tf32=allow_tf32, use_exp2=use_exp2)
+        # two launches, raw-bias kernel, averaging and shift correction on the host
+        kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
+        f_c = flashsinkhorn_lse(xf, yf, (g_hat + e * log_b) / e, e, damping=damp_f, **kw)
+        g_c = flashsinkhorn_lse(yf, xf, (f_hat + e * log_a) / e, e, damping=damp_g, **kw)
+        if damp_f < 1.0:
+            f_c = f_c - alpha * (1.0 - damp_f)
+        if damp_g < 1.0:
+            g_c = g_c - beta * (1.0 - damp_g)
+        if w == 1.0:
+            return f_c, g_c
+        return (1.0 - w) * f_hat + w * f_c, (1.0 - w) * g_hat + w * g_c
+
+    used = 0
+    f_hat, g_hat = jacobi(f_hat, g_hat, eps_list[0], 1.0)
+    used += 1
+    prev_f = prev_g = None
+    for idx, e in enumerate(eps_list):
+        f_hat, g_hat = jacobi(f_hat, g_hat, e, 0.5)
+        used += 1
+        if threshold is not None and (idx + 1) % check_every == 0:
+            if prev_f is not None and _max_change(f_hat, g_hat, prev_f, prev_g) < threshold:
+                break
+            prev_f, prev_g = f_hat.clone(), g_hat.clone()
+
+    f_prelast = g_prelast = None
+    if last_extrapolation:
+        f_prelast, g_prelast = f_hat + alpha, g_hat + beta
+        f_hat, g_hat = jacobi(f_hat, g_hat, eps_list[-1], 1.0)
+        used += 1
+
+    out = (f_hat + alpha, g_hat + beta)
+    if return_prelast and last_extrapolation:
+        out = out + (f_prelast, g_prelast)
+    if return_n_iters:
+        out = out + (used,)
+    return out

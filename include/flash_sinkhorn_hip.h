@@ -1,0 +1,143 @@
+/*
+ * C ABI of the MI355X (gfx950) FlashSinkhorn kernels.
+ *
+ * The reference (ot-triton-lab/flash-sinkhorn) has no FFI layer: its device
+ * boundary is the set of Python launcher functions in flash_sinkhorn/kernels/
+ * that call Triton kernels.  Each entry point below replaces one of those
+ * launchers (cited per function, paths relative to src/flash_sinkhorn/).
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer to contiguous row-major fp32 unless
+ *    stated otherwise; sizes are element counts
+ *  - nothing here allocates or frees device memory; the caller owns inputs,
+ *    outputs and the workspace (size from fs_workspace_bytes)
+ *  - all work is enqueued on `stream` (a hipStream_t passed as void*) and
+ *    returns without synchronising; the library keeps no mutable global state
+ *  - return value: FS_OK or a negative FS_ERR_* code (fs_error_string names it)
+ *  - flags: FS_FLAG_EXP2 is accepted for interface parity (the kernels always
+ *    work in base 2, which is the same function); FS_FLAG_REDUCED_OPERANDS
+ *    permits split-bf16 MFMA operands (the counterpart of allow_tf32=True)
+ */
+#ifndef FLASH_SINKHORN_HIP_H
+#define FLASH_SINKHORN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FS_OK 0
+#define FS_ERR_NULL_POINTER (-1)
+#define FS_ERR_BAD_SIZE (-2)
+#define FS_ERR_BAD_ARGUMENT (-3)
+#define FS_ERR_WORKSPACE_TOO_SMALL (-4)
+#define FS_ERR_LAUNCH_FAILED (-5)
+#define FS_ERR_UNSUPPORTED (-6)
+
+#define FS_FLAG_EXP2 1u
+#define FS_FLAG_REDUCED_OPERANDS 2u
+
+/* operation ids for fs_workspace_bytes */
+#define FS_OP_LSE 0
+#define FS_OP_SYMMETRIC_STEP 1
+#define FS_OP_GRAD 2
+#define FS_OP_APPLY_VEC 3
+#define FS_OP_APPLY_MAT 4
+#define FS_OP_MAT5 5
+
+int fs_version(void);
+const char* fs_error_string(int code);
+
+/* Bytes of device scratch the given operation needs for an (n, m, d) problem. */
+size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d);
+
+/*
+ * out[i] = -eps*damping * LSE_j[ coord_scale * x_i.y_j / eps + bias[j] ]
+ * Replaces flashsinkhorn_lse (kernels/sinkhorn_flashstyle_sqeuclid.py:815-955,
+ * kernel 194-307).  x:[n,d] y:[m,d] bias:[m] out:[n].
+ */
+int fs_lse(const float* x, const float* y, const float* bias, float* out,
+           int64_t n, int64_t m, int64_t d, float eps, float coord_scale, float damping,
+           uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Same with bias[j] = pot_hat[j]/eps + log_w[j] formed inside the kernel.
+ * Replaces flashsinkhorn_lse_fused (kernels/sinkhorn_flashstyle_sqeuclid.py:958-1090,
+ * kernel 317-419).
+ */
+int fs_lse_fused(const float* x, const float* y, const float* pot_hat, const float* log_w,
+                 float* out, int64_t n, int64_t m, int64_t d, float eps, float coord_scale,
+                 float damping, uint32_t flags, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/*
+ * One Jacobi step on shifted potentials, both halves from the OLD potentials:
+ *   f_out = (1-alpha) f_hat + alpha * (-eps*damp_f * LSE_j[(cs2 x.y + g_hat_j)/eps + log_b_j])
+ *           - alpha*(1-damp_f)*shift_x      (only when shift_x != NULL)
+ *   g_out likewise over i.
+ * Replaces flashsinkhorn_symmetric_step (kernels/sinkhorn_flashstyle_sqeuclid.py:1093-1317,
+ * kernel 433-661).  shift_x/shift_y (= cost_scale*|x|^2, cost_scale*|y|^2, may be NULL)
+ * fold in the unbalanced shift correction the reference's solver applies on the
+ * host right after the launch (sinkhorn_solvers.py:509-517).  Outputs must not
+ * alias inputs.
+ */
+int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                      const float* log_a, const float* log_b, float* f_out, float* g_out,
+                      const float* shift_x, const float* shift_y,
+                      int64_t n, int64_t m, int64_t d, float eps, float alpha, float damp_f,
+                      float damp_g, float coord_scale, uint32_t flags, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/*
+ * Analytic gradient: grad_x[i,:] = 2*cost_scale*gs*a_i*(x_i - sum_j w_ij y_j),
+ * w_i. = softmax_j[(g_j - C_ij)/eps + log_b_j]; grad_y symmetric over i.
+ * Standard (unshifted) potentials f, g; x2, y2 = row squared norms; gs is read
+ * from the 1-element device array grad_scale (NULL means 1).  Either output may
+ * be NULL.  Picks the large-d variant internally.
+ * Replaces sinkhorn_geomloss_online_grad_sqeuclid
+ * (kernels/sinkhorn_triton_grad_sqeuclid.py:891-1207, kernels 101-402 and 405-791).
+ */
+int fs_grad(const float* x, const float* y, const float* f, const float* g, const float* log_a,
+            const float* log_b, const float* a, const float* b, const float* x2, const float* y2,
+            const float* grad_scale, float* grad_x, float* grad_y, int64_t n, int64_t m,
+            int64_t d, float eps, float cost_scale, uint32_t flags, void* workspace,
+            size_t workspace_bytes, void* stream);
+
+/*
+ * axis=1: out[i] = sum_j P_ij vec[j];  axis=0: out[j] = sum_i P_ij vec[i], with
+ * P_ij = exp(log_a_i + log_b_j + (f_hat_i + g_hat_j + coord_scale x_i.y_j)/eps).
+ * Replaces apply_plan_vec_flashstyle (kernels/apply_flash.py:835-951, kernels 594-832).
+ */
+int fs_apply_vec(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                 const float* log_a, const float* log_b, const float* vec, float* out,
+                 int64_t n, int64_t m, int64_t d, float eps, float coord_scale, int axis,
+                 uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * axis=1: out = P @ (mat * scale[:,None]) (mat:[m,dv], scale:[m] or NULL);
+ * axis=0: out = P^T @ mat (mat:[n,dv], scale must be NULL).  out:[n|m, dv].
+ * Replaces apply_plan_mat_flashstyle (kernels/apply_flash.py:360-579, kernels 49-343);
+ * the reference fixes dv == d.
+ */
+int fs_apply_mat(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                 const float* log_a, const float* log_b, const float* mat, const float* scale,
+                 float* out, int64_t n, int64_t m, int64_t d, int64_t dv, float eps,
+                 float coord_scale, int axis, uint32_t flags, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
+/*
+ * out[i,:] = (-4*cost_scale/eps) * sum_j P_ij (A_i.y_j) y_j with
+ * P_ij = exp((f_ott_i + g_ott_j - cost_scale*|x_i-y_j|^2)/eps).
+ * Replaces mat5_sqeuclid (kernels/apply_ott.py:453-566, kernel 34-168).
+ */
+int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_ott,
+            const float* A, const float* x2, const float* y2, float* out, int64_t n, int64_t m,
+            int64_t d, float eps, float cost_scale, uint32_t flags, void* workspace,
+            size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_SINKHORN_HIP_H */

@@ -1,0 +1,154 @@
+"""HIP kernels (through the C ABI) vs the fp64 oracle on seeded inputs.
+
+Tolerance: north-star bar is rel 1e-4 on potentials and gradients for fp32;
+errors are measured relative to the largest magnitude of the expected output.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.golden.recipe import inputs
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-4
+
+SHAPES = [  # (n, m, d): ragged tiles, d not a multiple of 4/8, every padded width
+    (64, 48, 32), (300, 257, 64), (129, 1000, 3), (1000, 130, 20), (257, 300, 128),
+    (70, 65, 100), (4500, 3000, 64), (33, 5, 8), (1, 1, 1),
+]
+
+
+def dev(*arrs):
+    return [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in arrs]
+
+
+def rel_err(got, want):
+    got = got.detach().cpu().numpy().astype(np.float64)
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def problem(n, m, d, seed=0, eps=0.3):
+    x, y, a, b = inputs(100 + seed, n, m, d, scale=1.0 / np.sqrt(max(d, 1)) * 2.0)
+    rng = np.random.default_rng(seed + 7)
+    f_hat = rng.standard_normal(n).astype(np.float32) * 0.3
+    g_hat = rng.standard_normal(m).astype(np.float32) * 0.3
+    return x, y, a, b, f_hat, g_hat
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_lse_raw_and_fused(n, m, d):
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        flashsinkhorn_lse, flashsinkhorn_lse_fused)
+    x, y, a, b, f_hat, g_hat = problem(n, m, d)
+    eps = 0.3
+    lb = np.log(b)
+    bias = (g_hat / eps + lb).astype(np.float32)
+    X, Y, B, G, LB = dev(x, y, bias, g_hat, lb)
+    for cs, damp in ((1.0, 1.0), (0.5, 0.7)):
+        want = oracle.lse_shifted(x, y, bias, eps, cs, damp)
+        got = flashsinkhorn_lse(X, Y, B, eps, cost_scale=cs, damping=damp, allow_tf32=False)
+        assert rel_err(got, want) < RTOL
+        want = oracle.lse_shifted_fused(x, y, g_hat, lb, eps, cs, damp)
+        got = flashsinkhorn_lse_fused(X, Y, G, LB, eps, cost_scale=cs, damping=damp,
+                                      allow_tf32=False)
+        assert rel_err(got, want) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_symmetric_step(n, m, d):
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        flashsinkhorn_symmetric_step)
+    x, y, a, b, f_hat, g_hat = problem(n, m, d, seed=1)
+    la, lb = np.log(a), np.log(b)
+    X, Y, F, G, LA, LB = dev(x, y, f_hat, g_hat, la, lb)
+    for alpha, df, dg in ((0.5, 1.0, 1.0), (1.0, 0.8, 0.6)):
+        wf, wg = oracle.symmetric_step(x, y, f_hat, g_hat, la, lb, 0.25, 0.5, alpha, df, dg)
+        gf, gg = flashsinkhorn_symmetric_step(X, Y, F, G, LA, LB, 0.25, cost_scale=0.5,
+                                              alpha=alpha, damping_f=df, damping_g=dg,
+                                              allow_tf32=False)
+        assert rel_err(gf, wf) < RTOL and rel_err(gg, wg) < RTOL
+
+
+def test_lse_small_eps_large_logits():
+    # eps = 0.01 with |x.y| ~ 50: logits of order 1e4, the regime of the headline config
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import flashsinkhorn_lse_fused
+    x, y, a, b = inputs(5, 700, 900, 64, y_shift=0.5)
+    be = (y.astype(np.float64) ** 2).sum(1)
+    g_hat = (-be).astype(np.float32)
+    lb = np.log(b)
+    want = oracle.lse_shifted_fused(x, y, g_hat, lb, 0.01)
+    got = flashsinkhorn_lse_fused(*dev(x, y, g_hat, lb), 0.01, allow_tf32=False)
+    assert rel_err(got, want) < RTOL
+
+
+def test_zero_weight_and_masked_bias():
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        flashsinkhorn_lse, flashsinkhorn_lse_fused)
+    from flash_sinkhorn_amd.kernels._common import log_weights
+    x, y, a, b, f_hat, g_hat = problem(90, 70, 16)
+    b = b.copy(); b[::3] = 0.0
+    LB = log_weights(torch.from_numpy(b).cuda())
+    want = oracle.lse_shifted_fused(x, y, g_hat, oracle.log_weights(b), 0.3)
+    got = flashsinkhorn_lse_fused(*dev(x, y, g_hat), LB, 0.3, allow_tf32=False)
+    assert rel_err(got, want) < RTOL
+    bias = (g_hat / 0.3).astype(np.float32); bias[5:] = -np.inf  # only 5 live keys
+    want = oracle.lse_shifted(x, y, bias, 0.3)
+    got = flashsinkhorn_lse(*dev(x, y, bias), 0.3, allow_tf32=False)
+    assert rel_err(got, want) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_gradient(n, m, d):
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    x, y, a, b, f, g = problem(n, m, d, seed=2)
+    gs = np.array([0.7], np.float32)
+    wx, wy = oracle.grad_barycentric(x, y, a, b, f, g, 0.3, cost_scale=0.5, grad_scale=0.7)
+    X, Y, A, B, F, G, GS = dev(x, y, a, b, f, g, gs)
+    gx, gy = grad(X, Y, A, B, F, G, eps=0.3, cost_scale=0.5, grad_scale=GS, allow_tf32=False)
+    assert rel_err(gx, wx) < RTOL and rel_err(gy, wy) < RTOL
+    gx, gy = grad(X, Y, A, B, F, G, eps=0.3, cost_scale=0.5, grad_scale=GS, allow_tf32=False,
+                  compute_grad_y=False)
+    assert gy is None and rel_err(gx, wx) < RTOL
+    gx, gy = grad(X, Y, A, B, F, G, eps=0.3, cost_scale=0.5, grad_scale=GS, allow_tf32=False,
+                  compute_grad_x=False)
+    assert gx is None and rel_err(gy, wy) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_apply_vec_and_mat(n, m, d):
+    from flash_sinkhorn_amd.kernels.apply_flash import (
+        apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
+    x, y, a, b, f_hat, g_hat = problem(n, m, d, seed=3)
+    la, lb = np.log(a), np.log(b)
+    rng = np.random.default_rng(4)
+    vm, vn = rng.standard_normal(m).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    Vm = rng.standard_normal((m, d)).astype(np.float32)
+    Vn = rng.standard_normal((n, d)).astype(np.float32)
+    sc = rng.random(m).astype(np.float32)
+    X, Y, F, G, LA, LB = dev(x, y, f_hat, g_hat, la, lb)
+    kw = dict(eps=0.4, cost_scale=0.5)
+    okw = dict(eps=0.4, cost_scale=0.5)
+    got = apply_plan_vec_flashstyle(X, Y, F, G, LA, LB, dev(vm)[0], axis=1, **kw)
+    assert rel_err(got, oracle.apply_plan_vec(x, y, f_hat, g_hat, la, lb, vm, axis=1, **okw)) < RTOL
+    got = apply_plan_vec_flashstyle(X, Y, F, G, LA, LB, dev(vn)[0], axis=0, **kw)
+    assert rel_err(got, oracle.apply_plan_vec(x, y, f_hat, g_hat, la, lb, vn, axis=0, **okw)) < RTOL
+    got = apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, dev(Vm)[0], axis=1, scale=dev(sc)[0], **kw)
+    want = oracle.apply_plan_mat(x, y, f_hat, g_hat, la, lb, Vm, axis=1, scale=sc, **okw)
+    assert rel_err(got, want) < RTOL
+    got = apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, Y, axis=1, **kw)  # values = key rows
+    assert rel_err(got, oracle.apply_plan_mat(x, y, f_hat, g_hat, la, lb, y, axis=1, **okw)) < RTOL
+    got = apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, dev(Vn)[0], axis=0, **kw)
+    assert rel_err(got, oracle.apply_plan_mat(x, y, f_hat, g_hat, la, lb, Vn, axis=0, **okw)) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_mat5(n, m, d):
+    from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
+    x, y, a, b, f, g = problem(n, m, d, seed=5)
+    A = np.random.default_rng(6).standard_normal((n, d)).astype(np.float32)
+    f = f - 2.0  # keep exp((f+g-C)/eps) in a tame range
+    want = oracle.mat5(x, y, f, g, A, 0.5, 0.5)
+    got = mat5_sqeuclid(*dev(x, y, f, g, A), eps=0.5, cost_scale=0.5)
+    assert rel_err(got, want) < RTOL
