@@ -1,0 +1,170 @@
+"""Headline benchmark: ms per 100 symmetric Sinkhorn iterations, n=m=50,000, d=64, fp32.
+
+One "step" is one full solve, ``sinkhorn_flashstyle_symmetric(use_epsilon_scaling=False,
+eps=0.01, n_iters=100, last_extrapolation=True, allow_tf32=False)`` = 102 double
+log-sum-exp launches, on a seeded 8-component Gaussian mixture per cloud with
+uniform weights, inputs already resident in HBM.  Prints ONE JSON line.
+
+roofline: the symmetric-step kernel does 4*n*m*d matrix flop per launch (both
+half-updates), priced against the MI355X fp32 MFMA peak of 157.3 TFLOP/s; its
+launch duration is measured here with HIP events on the launch stream.
+cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores
+on a bounded sample and scaled to the metric's unit.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+N, M, D = 50_000, 50_000, 64
+EPS = 0.01
+ITERS = 100
+FP32_MFMA_PEAK_TFLOPS = 157.3
+EXP_PEAK_PER_S = 256 * 16 * 2.4e9  # quarter-rate transcendental: 16 lanes/clk/CU
+
+
+def gmm_cloud(rng, n, d, k=8):
+    import numpy as np
+
+    means = rng.standard_normal((k, d)) * 2.0
+    comp = rng.integers(0, k, size=n)
+    return (means[comp] + rng.standard_normal((n, d))).astype(np.float32)
+
+
+def make_inputs(n, m, d, seed=3):
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    x = gmm_cloud(rng, n, d)
+    y = gmm_cloud(rng, m, d)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    return x, y, a, b
+
+
+def cpu_baseline(x, y, a, b, budget_s=20.0):
+    """Oracle symmetric steps (fp32 numpy) on a row sample, scaled to ms/100 iterations."""
+    import numpy as np
+
+    import oracle
+
+    n, m = x.shape[0], y.shape[0]
+    rows = min(n, 4096)
+    la, lb = np.log(a), np.log(b)
+    fh = -(x.astype(np.float32) ** 2).sum(1)
+    gh = -(y.astype(np.float32) ** 2).sum(1)
+    done, t0 = 0, time.perf_counter()
+    while True:
+        i0 = (done * rows) % max(1, n - rows + 1)
+        # one half-update for `rows` query rows against all m keys, and the mirrored one
+        oracle.lse_shifted_fused(x[i0:i0 + rows], y, gh, lb, EPS, dtype=np.float32)
+        oracle.lse_shifted_fused(y[i0:i0 + rows], x, fh, la, EPS, dtype=np.float32)
+        done += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or done * rows >= n:
+            break
+    frac = done * rows / n  # fraction of one full symmetric iteration that was timed
+    ms_per_100 = el / frac * (ITERS + 2) * 1e3
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    return {
+        "value": ms_per_100, "unit": "ms/100 symmetric iters", "cores": cores, "kind": "port",
+        "sample": f"{done * rows} of {n} query rows of each half-update against all {m} keys "
+                  f"({el:.1f} s of numpy fp32 oracle), scaled to 102 steps",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--n", type=int, default=N)
+    ap.add_argument("--m", type=int, default=M)
+    ap.add_argument("--d", type=int, default=D)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--reduced", action="store_true",
+                    help="time the split-bf16 operand path (allow_tf32=True) instead")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric
+    from flash_sinkhorn_amd.kernels._common import log_weights
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+
+    n, m, d = args.n, args.m, args.d
+    x, y, a, b = make_inputs(n, m, d)
+    dev = torch.device("cuda:0")
+    X, Y, A, B = (torch.from_numpy(t).to(dev) for t in (x, y, a, b))
+    strict = not args.reduced
+
+    def solve():
+        return sinkhorn_flashstyle_symmetric(
+            X, Y, A, B, use_epsilon_scaling=False, eps=EPS, n_iters=ITERS,
+            last_extrapolation=True, allow_tf32=not strict)
+
+    for _ in range(args.warmup):
+        solve()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        f, g = solve()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # dominant kernel: one symmetric-step launch, timed with events on the launch stream
+    alpha = (X * X).sum(1).contiguous()
+    beta = (Y * Y).sum(1).contiguous()
+    la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
+    fh, gh = f - alpha, g - beta
+    reps = 20
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, cost_scale=1.0, alpha=0.5, damping_f=1.0,
+                        damping_g=1.0, allow_tf32=not strict)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, cost_scale=1.0, alpha=0.5, damping_f=1.0,
+                            damping_g=1.0, allow_tf32=not strict)
+    e1.record()
+    torch.cuda.synchronize()
+    launch_ms = e0.elapsed_time(e1) / reps
+    flop = 4.0 * n * m * d
+    achieved = flop / (launch_ms * 1e-3) / 1e12
+    exp_rate = 2.0 * n * m / (launch_ms * 1e-3)
+
+    loss = float((A * f).sum() + (B * g).sum())
+    line = {
+        "metric": "ms per 100 symmetric Sinkhorn iterations (n=m=50k, d=64, fp32)",
+        "value": ms_per_step, "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32" if strict else "bf16x3",
+        "data": "synthetic",
+        "config": {"workload": f"balanced symmetric FlashSinkhorn, n={n}, m={m}, d={d}, seeded "
+                               "8-component Gaussian mixtures, uniform weights, eps=0.01, "
+                               "100 iterations + init + extrapolation = 102 steps",
+                   "loss": loss},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "kernel": "stream_kernel<lse> (one symmetric step, both half-updates)",
+                     "launch_ms": launch_ms, "exp_per_s": exp_rate,
+                     "exp_frac_of_peak": exp_rate / EXP_PEAK_PER_S,
+                     "serial_mfma_plus_exp_ms_per_step": (flop / (FP32_MFMA_PEAK_TFLOPS * 1e12)
+                                                          + 2.0 * n * m / EXP_PEAK_PER_S) * 1e3},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(x, y, a, b)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
