@@ -1,2 +1,15 @@
-"""MI355X-native FlashSinkhorn: streaming entropic OT on hand-written gfx950 kernels."""
+"""MI355X-native FlashSinkhorn: streaming entropic optimal transport on hand-written
+gfx950 kernels, behind the public names of the reference package (``flash_sinkhorn``)."""
+from flash_sinkhorn_amd.samples_loss import SamplesLoss
+from flash_sinkhorn_amd.cg import CGInfo, conjugate_gradient
+from flash_sinkhorn_amd.hvp import (
+    HvpInfo,
+    geomloss_to_ott_potentials,
+    hvp_x_sqeuclid,
+    hvp_x_sqeuclid_from_potentials,
+)
+
+__all__ = ["SamplesLoss", "CGInfo", "conjugate_gradient", "HvpInfo",
+           "geomloss_to_ott_potentials", "hvp_x_sqeuclid", "hvp_x_sqeuclid_from_potentials",
+           "__version__"]
 __version__ = "0.1.0"
