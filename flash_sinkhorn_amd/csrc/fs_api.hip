@@ -7,12 +7,14 @@
 
 #include "flash_sinkhorn_hip.h"
 #include "fs_common.hpp"
+#include "fs_dispatch.hpp"
 #include "fs_stream.hpp"
 
 namespace fs {
 namespace {
 
-constexpr int kMaxStreamD = 128;
+constexpr int kMaxStreamD = 128;    // register-stationary streaming kernels
+constexpr int kMaxSlicedD = 1536;   // column-sliced kernels
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
@@ -40,19 +42,52 @@ struct SidePlan {
   int rb, igroups, splits, chunk;
 };
 
+// Which kernel family serves feature dimension d, and its tile geometry.
+struct Family {
+  bool sliced;
+  int dp;        // padded feature width (also the width of partial O rows)
+  int jt;        // keys per tile
+  int nw, nsl;   // sliced only: wavefronts per workgroup, 32-column blocks per wavefront
+};
+
+Family family_for(int64_t d) {
+  Family f;
+  f.sliced = d > kMaxStreamD;
+  f.nw = f.nsl = 0;
+  if (!f.sliced) {
+    f.dp = padded_d(d);
+    f.jt = (f.dp >= 128) ? 32 : 64;
+    return f;
+  }
+  if (d <= 256) { f.nw = 4; f.nsl = 2; }
+  else if (d <= 512) { f.nw = 8; f.nsl = 2; }
+  else if (d <= 1024) { f.nw = 8; f.nsl = 4; }
+  else { f.nw = 8; f.nsl = 6; }
+  f.dp = f.nw * f.nsl * 32;
+  f.jt = 32;
+  return f;
+}
+
 // Rows per wavefront (RB blocks of 32) and the key split for one side.
-SidePlan plan_side(int mode, int64_t nq, int64_t nk, int dp) {
+SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam) {
   SidePlan p;
   const bool has_o = (mode == kMat || mode == kMat5);
+  const int dp = fam.dp;
+  const int jt = fam.jt;
   p.rb = 1;
-  if (mode == kLse || mode == kVec) p.rb = (dp <= 64 && nq >= 2048) ? 2 : 1;
-  if (mode == kMat) p.rb = (dp <= 32 && nq >= 2048) ? 2 : 1;
-  const int jt = (dp >= 128) ? 32 : 64;
-  p.igroups = ceil_div(nq, 128 * p.rb);
+  int target = target_blocks(has_o);
+  if (fam.sliced) {
+    p.igroups = ceil_div(nq, 32);
+    target = 512;  // one workgroup of nw wavefronts per CU, two rounds
+  } else {
+    if (mode == kLse || mode == kVec) p.rb = (dp <= 64 && nq >= 2048) ? 2 : 1;
+    if (mode == kMat) p.rb = (dp <= 32 && nq >= 2048) ? 2 : 1;
+    p.igroups = ceil_div(nq, 128 * p.rb);
+  }
   const int max_splits = (int)std::max<int64_t>(1, nk / (4 * jt));
   const int cap = has_o ? 16 : 64;
   int s = 1;
-  while (p.igroups * s < target_blocks(has_o) && s * 2 <= max_splits && s * 2 <= cap) s *= 2;
+  while (p.igroups * s < target && s * 2 <= max_splits && s * 2 <= cap) s *= 2;
   p.chunk = ceil_div(ceil_div(nk, s), jt) * jt;
   p.splits = ceil_div(nk, p.chunk);
   return p;
@@ -105,8 +140,9 @@ int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
 // sides and, when keys were split, the merge kernel.
 int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes,
                hipStream_t st) {
-  if (d > kMaxStreamD) return FS_ERR_UNSUPPORTED;
-  const int dp = padded_d(d);
+  if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
+  const Family fam = family_for(d);
+  const int dp = fam.dp;
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -115,12 +151,12 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   SidePlan plans[2];
   size_t need = 0;
   for (int s = 0; s < nsides; ++s) {
-    plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, dp);
+    plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam);
     rb = std::min(rb, plans[s].rb);
   }
   for (int s = 0; s < nsides; ++s) {
     // both sides run in one launch and must share the rows-per-wave template
-    if (plans[s].rb != rb) {
+    if (!fam.sliced && plans[s].rb != rb) {
       plans[s].rb = rb;
       plans[s].igroups = ceil_div(sides[s].nq, 128 * rb);
     }
@@ -158,6 +194,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (total <= 0) return FS_OK;
 
   int rc;
+  if (fam.sliced) {
+    rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
+  } else
   switch (mode) {
     case kLse: rc = launch_dp<kLse, false>(a, dp, rb, total, st); break;
     case kVec: rc = launch_dp<kVec, false>(a, dp, rb, total, st); break;
@@ -244,8 +283,9 @@ const char* fs_error_string(int code) {
 }
 
 size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
-  if (bad_sizes(n, m, d) || d > kMaxStreamD) return 0;
-  const int dp = padded_d(d);
+  if (bad_sizes(n, m, d) || d > kMaxSlicedD) return 0;
+  const Family fam = family_for(d);
+  const int dp = fam.dp;
   int mode;
   bool both = false, either = false;
   switch (op) {
@@ -259,7 +299,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   }
   // rb may be lowered when two sides share a launch: size for the rb=1 plan too
   auto side_bytes = [&](int64_t nq, int64_t nk) {
-    SidePlan p = plan_side(mode, nq, nk, dp);
+    SidePlan p = plan_side(mode, nq, nk, fam);
     size_t b = side_ws_floats(mode, p, nq, dp);
     return b * sizeof(float);
   };
