@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libflash_sinkhorn_hip.so")
+LIB_PATH = os.environ.get("FLASH_SINKHORN_HIP_LIB", os.path.join(_HERE, "libflash_sinkhorn_hip.so"))
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 FS_FLAG_EXP2 = 1

@@ -139,7 +139,7 @@ int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
 // Plans, carves the workspace, launches the streaming kernel over one or two
 // sides and, when keys were split, the merge kernel.
 int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes,
-               hipStream_t st) {
+               hipStream_t st, uint32_t flags = 0) {
   if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
   const Family fam = family_for(d);
   const int dp = fam.dp;
@@ -154,6 +154,41 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam);
     rb = std::min(rb, plans[s].rb);
   }
+  static const int use_v2 = env_int("FS_LSE2", 1);
+  static const int strict_prec = env_int("FS_STRICT_PREC", 2);    // 2: three bf16 planes, 0: fp32 MFMA
+  static const int reduced_prec = env_int("FS_REDUCED_PREC", 1);  // 1: two bf16 planes, 0: fp32 MFMA
+  static const int rb_override = env_int("FS_RB", 0);
+  bool aligned = (d % 4 == 0);
+  for (int s = 0; s < nsides; ++s) aligned = aligned && aligned16(sides[s].q) && aligned16(sides[s].k);
+  const int prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec : strict_prec;
+  // pipelined LSE kernel: the bf16-plane modes take any d <= 128, the fp32 mode needs aligned rows
+  const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
+  const int dp2 = std::max(dp, 16);
+  const int np = (prec == 1) ? 2 : 3;
+  if (lse2 && rb_override > 0 && dp <= 64) rb = (rb_override == 4 && prec == 0) ? 2 : rb_override;
+  // distinct operand matrices that need bf16 planes (x and y, whichever roles they play)
+  const float* plane_src[4];
+  int plane_rows[4];
+  size_t plane_off[4];
+  int nplanes = 0;
+  if (lse2 && prec != 0) {
+    for (int s = 0; s < nsides; ++s) {
+      const float* ptrs[2] = {sides[s].q, sides[s].k};
+      const int rows[2] = {sides[s].nq, sides[s].nk};
+      for (int k = 0; k < 2; ++k) {
+        bool seen = false;
+        for (int i = 0; i < nplanes; ++i) seen = seen || (plane_src[i] == ptrs[k] && plane_rows[i] == rows[k]);
+        if (!seen) {
+          plane_src[nplanes] = ptrs[k];
+          plane_rows[nplanes] = rows[k];
+          plane_off[nplanes] = need;
+          need += (((size_t)rows[k] * np * (dp2 / 2) * 4) + 15) & ~(size_t)15;
+          ++nplanes;
+        }
+      }
+    }
+  }
+  const size_t need_planes_end = need;
   for (int s = 0; s < nsides; ++s) {
     // both sides run in one launch and must share the rows-per-wave template
     if (!fam.sliced && plans[s].rb != rb) {
@@ -163,7 +198,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
   }
   if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
-  float* wsp = static_cast<float*>(ws);
+  float* wsp = reinterpret_cast<float*>(static_cast<char*>(ws) + need_planes_end);
   bool any_split = false;
   int blocks[2] = {0, 0};
   for (int s = 0; s < nsides; ++s) {
@@ -185,6 +220,11 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     if (sd.q2) vec_ok = vec_ok && aligned16(sd.q2);
     if (mode == kMat && sd.v) vec_ok = vec_ok && aligned16(sd.v);
     blocks[s] = p.igroups * p.splits;
+    for (int i = 0; i < nplanes; ++i) {
+      const unsigned* base = reinterpret_cast<const unsigned*>(static_cast<char*>(ws) + plane_off[i]);
+      if (plane_src[i] == sd.q && plane_rows[i] == sd.nq) sd.qplanes = base;
+      if (plane_src[i] == sd.k && plane_rows[i] == sd.nk) sd.kplanes = base;
+    }
     a.side[s] = sd;
   }
   if (nsides == 1) a.side[1] = a.side[0];
@@ -196,6 +236,13 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   int rc;
   if (fam.sliced) {
     rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
+  } else if (lse2) {
+    rc = FS_OK;
+    for (int i = 0; i < nplanes && rc == FS_OK; ++i)
+      rc = launch_split_planes(plane_src[i],
+                               reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
+                               plane_rows[i], (int)d, dp2, np, st);
+    if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, total, st);
   } else
   switch (mode) {
     case kLse: rc = launch_dp<kLse, false>(a, dp, rb, total, st); break;
@@ -303,8 +350,11 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     size_t b = side_ws_floats(mode, p, nq, dp);
     return b * sizeof(float);
   };
-  const size_t a = side_bytes(n, m), b = side_bytes(m, n);
-  if (both) return a + b + 64;
+  size_t planes = 0;  // bf16 planes of x and y for the pipelined LSE kernel (three planes at most)
+  if (mode == kLse && !fam.sliced)
+    planes = (size_t)(n + m) * 3 * (std::max(dp, 16) / 2) * 4 + 64;
+  const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
+  if (both) return a + b - planes + 64;
   if (either) return std::max(a, b) + 64;
   return a + 64;
 }
@@ -318,7 +368,7 @@ int fs_lse(const float* x, const float* y, const float* bias, float* out, int64_
   if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
   Side s = lse_side(x, y, bias, kLog2e, nullptr, 0.f, n, m, coord_scale / eps * kLog2e);
   lse_epilogue(s, out, nullptr, 1.0f, eps, damping, nullptr);
-  return run_stream(kLse, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kLse, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 int fs_lse_fused(const float* x, const float* y, const float* pot_hat, const float* log_w,
@@ -332,7 +382,7 @@ int fs_lse_fused(const float* x, const float* y, const float* pot_hat, const flo
   Side s = lse_side(x, y, pot_hat, kLog2e / eps, log_w, kLog2e, n, m,
                     coord_scale / eps * kLog2e);
   lse_epilogue(s, out, nullptr, 1.0f, eps, damping, nullptr);
-  return run_stream(kLse, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kLse, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const float* g_hat,
@@ -353,7 +403,7 @@ int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const 
   lse_epilogue(s[0], f_out, f_hat, alpha, eps, damp_f, shift_x);
   s[1] = lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
   lse_epilogue(s[1], g_out, g_hat, alpha, eps, damp_g, shift_y);
-  return run_stream(kLse, false, s, 2, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kLse, false, s, 2, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 int fs_grad(const float* x, const float* y, const float* f, const float* g, const float* log_a,

@@ -60,6 +60,8 @@ struct Side {
   int splits;           // number of key chunks
   int chunk;            // keys per chunk (multiple of the key tile)
   int igroups;          // ceil(nq / rows per workgroup)
+  const unsigned* qplanes;  // split-bf16 kernels: query rows as packed bf16 planes [nq][NP][DP/2]
+  const unsigned* kplanes;  // same for the key rows [nk][NP][DP/2]
   float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;

@@ -1,0 +1,54 @@
+// Instantiations and dispatch of the software-pipelined log-sum-exp kernel.
+#include "fs_lse2.hpp"
+
+#include "fs_dispatch.hpp"
+
+namespace fs {
+
+template <int DP, int RB, int PREC>
+static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
+  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC>), dim3(blocks), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+template <int DP, int PREC>
+static int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
+  if constexpr (DP <= 64) {
+    if (rb == 4 && PREC != kF32) return launch_cfg<DP, (PREC != kF32 ? 4 : 2), PREC>(a, blocks, st);
+    if (rb >= 2) return launch_cfg<DP, 2, PREC>(a, blocks, st);
+  }
+  return launch_cfg<DP, 1, PREC>(a, blocks, st);
+}
+
+template <int PREC>
+static int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
+  switch (dp) {
+    case 16: return launch_rb<16, PREC>(a, rb, blocks, st);
+    case 32: return launch_rb<32, PREC>(a, rb, blocks, st);
+    case 64: return launch_rb<64, PREC>(a, rb, blocks, st);
+    case 128: return launch_rb<128, PREC>(a, rb, blocks, st);
+  }
+  return FS_ERR_UNSUPPORTED;
+}
+
+int launch_split_planes(const float* src, unsigned* dst, int rows, int d, int dp, int np,
+                        hipStream_t st) {
+  const long long items = (long long)rows * (dp / 4);
+  const int grid = (int)((items + 255) / 256);
+  if (np == 2)
+    hipLaunchKernelGGL((split_planes_kernel<2>), dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp);
+  else
+    hipLaunchKernelGGL((split_planes_kernel<3>), dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, int blocks, hipStream_t st) {
+  switch (prec) {
+    case kF32: return launch_dp<kF32>(a, dp, rb, blocks, st);
+    case kBf3: return launch_dp<kBf3>(a, dp, rb, blocks, st);
+    case kBf6: return launch_dp<kBf6>(a, dp, rb, blocks, st);
+  }
+  return FS_ERR_BAD_ARGUMENT;
+}
+
+}  // namespace fs
