@@ -18,6 +18,10 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 
 FS_FLAG_EXP2 = 1
 FS_FLAG_REDUCED_OPERANDS = 2
+FS_FLAG_FP32_MFMA = 4
+# allow_tf32=False normally runs the three-plane split-bf16 operands (fp32-grade accuracy);
+# set this (or FLASH_SINKHORN_FP32_MFMA=1) to run fp32 MFMA operands instead.
+STRICT_FP32_MFMA = os.environ.get("FLASH_SINKHORN_FP32_MFMA", "0") == "1"
 OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5 = range(6)
 
 _lib: Optional[ctypes.CDLL] = None
@@ -95,4 +99,7 @@ def workspace(op: int, n: int, m: int, d: int, device) -> Optional[torch.Tensor]
 
 
 def flags(use_exp2: bool, allow_tf32: bool) -> int:
-    return (FS_FLAG_EXP2 if use_exp2 else 0) | (FS_FLAG_REDUCED_OPERANDS if allow_tf32 else 0)
+    f = FS_FLAG_EXP2 if use_exp2 else 0
+    if allow_tf32:
+        return f | FS_FLAG_REDUCED_OPERANDS
+    return f | (FS_FLAG_FP32_MFMA if STRICT_FP32_MFMA else 0)

@@ -160,12 +160,13 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   static const int rb_override = env_int("FS_RB", 0);
   bool aligned = (d % 4 == 0);
   for (int s = 0; s < nsides; ++s) aligned = aligned && aligned16(sides[s].q) && aligned16(sides[s].k);
-  const int prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec : strict_prec;
+  const int prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec
+                   : ((flags & FS_FLAG_FP32_MFMA) ? 0 : strict_prec);
   // pipelined LSE kernel: the bf16-plane modes take any d <= 128, the fp32 mode needs aligned rows
   const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = std::max(dp, 16);
   const int np = (prec == 1) ? 2 : 3;
-  if (lse2 && rb_override > 0 && dp <= 64) rb = (rb_override == 4 && prec == 0) ? 2 : rb_override;
+  if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
   // distinct operand matrices that need bf16 planes (x and y, whichever roles they play)
   const float* plane_src[4];
   int plane_rows[4];

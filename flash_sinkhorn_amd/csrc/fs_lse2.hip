@@ -14,7 +14,6 @@ static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
 template <int DP, int PREC>
 static int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
   if constexpr (DP <= 64) {
-    if (rb == 4 && PREC != kF32) return launch_cfg<DP, (PREC != kF32 ? 4 : 2), PREC>(a, blocks, st);
     if (rb >= 2) return launch_cfg<DP, 2, PREC>(a, blocks, st);
   }
   return launch_cfg<DP, 1, PREC>(a, blocks, st);

@@ -116,7 +116,7 @@ struct Geo2 {
 };
 
 template <int DP, int RB, int PREC>
-__global__ __launch_bounds__(256) void lse2_kernel(const LaunchArgs args) {
+__global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   using G = Geo2<DP, PREC>;
   constexpr int NP = G::NP;
   constexpr bool kBf = (PREC != kF32);

@@ -15,8 +15,14 @@
  *    returns without synchronising; the library keeps no mutable global state
  *  - return value: FS_OK or a negative FS_ERR_* code (fs_error_string names it)
  *  - flags: FS_FLAG_EXP2 is accepted for interface parity (the kernels always
- *    work in base 2, which is the same function); FS_FLAG_REDUCED_OPERANDS
- *    permits split-bf16 MFMA operands (the counterpart of allow_tf32=True)
+ *    work in base 2, which is the same function).  Operand precision of the
+ *    log-sum-exp kernels for d <= 128 (everything accumulates in fp32):
+ *      default                    operands as three bf16 planes, six MFMA products:
+ *                                 error at or below that of fp32 MFMA operands
+ *      FS_FLAG_FP32_MFMA          fp32 operands on v_mfma_f32_32x32x2_f32
+ *      FS_FLAG_REDUCED_OPERANDS   two bf16 planes, three products (~2^-17 relative
+ *                                 per product): the counterpart of allow_tf32=True
+ *    The gradient / plan-product / large-d kernels always use fp32 MFMA operands.
  */
 #ifndef FLASH_SINKHORN_HIP_H
 #define FLASH_SINKHORN_HIP_H
@@ -38,6 +44,7 @@ extern "C" {
 
 #define FS_FLAG_EXP2 1u
 #define FS_FLAG_REDUCED_OPERANDS 2u
+#define FS_FLAG_FP32_MFMA 4u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0
