@@ -5,11 +5,20 @@ eps=0.01, n_iters=100, last_extrapolation=True, allow_tf32=False)`` = 102 double
 log-sum-exp launches, on a seeded 8-component Gaussian mixture per cloud with
 uniform weights, inputs already resident in HBM.  Prints ONE JSON line.
 
-roofline: the symmetric-step kernel does 4*n*m*d matrix flop per launch (both
-half-updates), priced against the MI355X fp32 MFMA peak of 157.3 TFLOP/s; its
-launch duration is measured here with HIP events on the launch stream.
-cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores
-on a bounded sample and scaled to the metric's unit.
+Operand modes of the log-sum-exp kernel (results are fp32 in all of them):
+  strict (default, allow_tf32=False)  three bf16 planes per operand, six MFMA products,
+                                      fp32 accumulate: error <= that of fp32 MFMA operands
+  fp32_mfma (--mode fp32_mfma)        fp32 operands on v_mfma_f32_32x32x2_f32
+  reduced (--mode reduced)            two bf16 planes, three products (allow_tf32=True)
+
+roofline: one symmetric-step launch does 4*n*m*d algorithmic matrix flop (both
+half-updates) plus 2*n*m exp2; its duration is measured here with HIP events on the
+launch stream.  The algorithmic rate is priced against the fp32 MFMA peak (157.3 TFLOP/s,
+the pipe an fp32 implementation is bound by); the split-bf16 modes execute 6 (3) bf16 MFMA
+products plus one fp32 bias MFMA per algorithmic product, and that executed rate is
+reported against the 2516.6 TFLOP/s bf16 peak next to it.
+cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores on a
+bounded sample and scaled to the metric's unit.
 """
 import argparse
 import json
@@ -25,7 +34,13 @@ N, M, D = 50_000, 50_000, 64
 EPS = 0.01
 ITERS = 100
 FP32_MFMA_PEAK_TFLOPS = 157.3
-EXP_PEAK_PER_S = 256 * 16 * 2.4e9  # quarter-rate transcendental: 16 lanes/clk/CU
+BF16_MFMA_PEAK_TFLOPS = 2516.6
+EXP_PEAK_PER_S = 256 * 16 * 2.4e9  # quarter-rate transcendental assumption: 16 lanes/clk/CU
+# Memory-side bytes per lse2_kernel launch of the default workload in strict mode, from two
+# rocprofv3 --pmc runs (FETCH_SIZE 286,269 KiB x 2.0, WRITE_SIZE 105,622 KiB x 1.0; the factors
+# are what the same counters read for a 256 MiB copy kernel).  Not measured for the other modes.
+MEASURED_TRAFFIC_BYTES = {"strict": int((286269 * 2.0 + 105622) * 1024), "fp32_mfma": None,
+                          "reduced": None}
 
 
 def gmm_cloud(rng, n, d, k=8):
@@ -72,9 +87,11 @@ def cpu_baseline(x, y, a, b, budget_s=20.0):
     ms_per_100 = el / frac * (ITERS + 2) * 1e3
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
     return {
-        "value": ms_per_100, "unit": "ms/100 symmetric iters", "cores": cores, "kind": "port",
+        "value": ms_per_100, "unit": "ms per 100 symmetric iterations", "cores": cores,
+        "kind": "port",
         "sample": f"{done * rows} of {n} query rows of each half-update against all {m} keys "
-                  f"({el:.1f} s of numpy fp32 oracle), scaled to 102 steps",
+                  f"({el:.1f} s of the numpy fp32 oracle, BLAS threads = host default), scaled "
+                  "to 102 steps",
     }
 
 
@@ -86,9 +103,10 @@ def main():
     ap.add_argument("--n", type=int, default=N)
     ap.add_argument("--m", type=int, default=M)
     ap.add_argument("--d", type=int, default=D)
+    ap.add_argument("--mode", choices=["strict", "fp32_mfma", "reduced"], default="strict")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--reduced", action="store_true",
-                    help="time the split-bf16 operand path (allow_tf32=True) instead")
+    ap.add_argument("--no-other-modes", action="store_true",
+                    help="skip the one-launch timings of the two other operand modes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported",
@@ -97,6 +115,7 @@ def main():
 
     import torch
 
+    from flash_sinkhorn_amd import _lib
     from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric
     from flash_sinkhorn_amd.kernels._common import log_weights
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
@@ -105,19 +124,23 @@ def main():
     x, y, a, b = make_inputs(n, m, d)
     dev = torch.device("cuda:0")
     X, Y, A, B = (torch.from_numpy(t).to(dev) for t in (x, y, a, b))
-    strict = not args.reduced
 
-    def solve():
+    def set_mode(mode):
+        _lib.STRICT_FP32_MFMA = (mode == "fp32_mfma")
+        return mode == "reduced"  # allow_tf32
+
+    def solve(mode):
+        tf32 = set_mode(mode)
         return sinkhorn_flashstyle_symmetric(
             X, Y, A, B, use_epsilon_scaling=False, eps=EPS, n_iters=ITERS,
-            last_extrapolation=True, allow_tf32=not strict)
+            last_extrapolation=True, allow_tf32=tf32)
 
     for _ in range(args.warmup):
-        solve()
+        solve(args.mode)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        f, g = solve()
+        f, g = solve(args.mode)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
@@ -125,42 +148,66 @@ def main():
     alpha = (X * X).sum(1).contiguous()
     beta = (Y * Y).sum(1).contiguous()
     la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
-    fh, gh = f - alpha, g - beta
-    reps = 20
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, cost_scale=1.0, alpha=0.5, damping_f=1.0,
-                        damping_g=1.0, allow_tf32=not strict)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(reps):
-        _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, cost_scale=1.0, alpha=0.5, damping_f=1.0,
-                            damping_g=1.0, allow_tf32=not strict)
-    e1.record()
-    torch.cuda.synchronize()
-    launch_ms = e0.elapsed_time(e1) / reps
-    flop = 4.0 * n * m * d
-    achieved = flop / (launch_ms * 1e-3) / 1e12
-    exp_rate = 2.0 * n * m / (launch_ms * 1e-3)
+    fh, gh = (f - alpha).contiguous(), (g - beta).contiguous()
 
-    loss = float((A * f).sum() + (B * g).sum())
+    def launch_ms(mode, reps=20):
+        tf32 = set_mode(mode)
+        kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=tf32)
+        _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, **kw)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, **kw)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    flop = 4.0 * n * m * d
+    products = {"strict": 6, "reduced": 3, "fp32_mfma": 0}
+    dtypes = {"strict": "bf16x3-planes/fp32-accumulate (fp32-grade)", "fp32_mfma": "f32",
+              "reduced": "bf16x2-planes/fp32-accumulate"}
+
+    def roofline_for(mode, ms):
+        achieved = flop / (ms * 1e-3) / 1e12
+        r = {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+             "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+             "traffic": MEASURED_TRAFFIC_BYTES.get(mode) if (n, m, d) == (N, M, D) else None,
+             "kernel": "one symmetric step (both half-updates) = split_planes + lse2_kernel + "
+                       "finish_kernel; 4*n*m*d algorithmic flop",
+             "launch_ms": ms, "exp_per_s": 2.0 * n * m / (ms * 1e-3)}
+        if products[mode]:
+            r["executed_bf16_mfma_tflops"] = achieved * products[mode]
+            r["executed_frac_of_bf16_peak"] = achieved * products[mode] / BF16_MFMA_PEAK_TFLOPS
+            r["note"] = (f"{products[mode]} bf16 MFMA products per algorithmic product; "
+                         "algorithmic rate priced against the fp32 MFMA peak, executed rate "
+                         "against the bf16 peak")
+        return r
+
+    main_ms = launch_ms(args.mode)
     line = {
         "metric": "ms per 100 symmetric Sinkhorn iterations (n=m=50k, d=64, fp32)",
         "value": ms_per_step, "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32" if strict else "bf16x3",
+        "scaling": "weak", "vs_baseline": None, "dtype": dtypes[args.mode],
         "data": "synthetic",
         "config": {"workload": f"balanced symmetric FlashSinkhorn, n={n}, m={m}, d={d}, seeded "
                                "8-component Gaussian mixtures, uniform weights, eps=0.01, "
                                "100 iterations + init + extrapolation = 102 steps",
-                   "loss": loss},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "stream_kernel<lse> (one symmetric step, both half-updates)",
-                     "launch_ms": launch_ms, "exp_per_s": exp_rate,
-                     "exp_frac_of_peak": exp_rate / EXP_PEAK_PER_S,
-                     "serial_mfma_plus_exp_ms_per_step": (flop / (FP32_MFMA_PEAK_TFLOPS * 1e12)
-                                                          + 2.0 * n * m / EXP_PEAK_PER_S) * 1e3},
+                   "operand_mode": args.mode,
+                   "loss": float((A * f).sum() + (B * g).sum())},
+        "roofline": roofline_for(args.mode, main_ms),
     }
+    if not args.no_other_modes:
+        others = {}
+        for mode in ("strict", "fp32_mfma", "reduced"):
+            if mode != args.mode:
+                ms = launch_ms(mode, reps=10)
+                rf = roofline_for(mode, ms)
+                others[mode] = {"launch_ms": ms, "ms_per_100_iters_est": ms * (ITERS + 2),
+                                "achieved": rf["achieved"], "frac_of_fp32_peak": rf["frac"]}
+        line["other_operand_modes"] = others
+        set_mode(args.mode)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(x, y, a, b)
     print(json.dumps(line))

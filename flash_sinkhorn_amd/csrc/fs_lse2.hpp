@@ -380,8 +380,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         epilogue_scalar(sd.ep, row, M2, s, 0.f);
       } else {
         const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
-        sd.part_ms[2 * pr] = M2;
-        sd.part_ms[2 * pr + 1] = s;
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
       }
     }
   }

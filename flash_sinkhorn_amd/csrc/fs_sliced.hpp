@@ -242,8 +242,7 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
   } else if (live) {
     const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
     if (wave == 0 && h == 0) {
-      sd.part_ms[2 * pr] = M;
-      sd.part_ms[2 * pr + 1] = s;
+      *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M, s);
       if constexpr (MODE == kVec) sd.part_o[pr] = o;
     }
     if constexpr (kHasO) {

@@ -402,8 +402,7 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
     } else if (live) {
       const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
       if (h == 0) {
-        sd.part_ms[2 * pr] = M;
-        sd.part_ms[2 * pr + 1] = s;
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M, s);
         if constexpr (MODE == kVec) sd.part_o[pr] = o;
       }
       if constexpr (kHasO) {
