@@ -6,17 +6,19 @@ log-sum-exp launches, on a seeded 8-component Gaussian mixture per cloud with
 uniform weights, inputs already resident in HBM.  Prints ONE JSON line.
 
 Operand modes of the log-sum-exp kernel (results are fp32 in all of them):
-  strict (default, allow_tf32=False)  three bf16 planes per operand, six MFMA products,
-                                      fp32 accumulate: error <= that of fp32 MFMA operands
+  strict (default, allow_tf32=False)  two fp16 planes per operand (22 significand bits) of the
+                                      power-of-two scaled matrix, three MFMA products, fp32
+                                      accumulate: error <= that of fp32 MFMA operands
+  bf16x3 (--mode bf16x3)              three bf16 planes, six products: same accuracy class
   fp32_mfma (--mode fp32_mfma)        fp32 operands on v_mfma_f32_32x32x2_f32
   reduced (--mode reduced)            two bf16 planes, three products (allow_tf32=True)
 
 roofline: one symmetric-step launch does 4*n*m*d algorithmic matrix flop (both
 half-updates) plus 2*n*m exp2; its duration is measured here with HIP events on the
 launch stream.  The algorithmic rate is priced against the fp32 MFMA peak (157.3 TFLOP/s,
-the pipe an fp32 implementation is bound by); the split-bf16 modes execute 6 (3) bf16 MFMA
-products plus one fp32 bias MFMA per algorithmic product, and that executed rate is
-reported against the 2516.6 TFLOP/s bf16 peak next to it.
+the pipe an fp32 implementation is bound by); the split modes execute 3 (fp16x2, reduced) or
+6 (bf16x3) 16-bit MFMA products plus one fp32 bias MFMA per algorithmic product, and that
+executed rate is reported against the 2516.6 TFLOP/s fp16/bf16 peak next to it.
 cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores on a
 bounded sample and scaled to the metric's unit.
 """
@@ -33,14 +35,14 @@ if ROOT not in sys.path:
 N, M, D = 50_000, 50_000, 64
 EPS = 0.01
 ITERS = 100
+MODES = ["strict", "bf16x3", "fp32_mfma", "reduced"]
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2516.6
 EXP_PEAK_PER_S = 256 * 16 * 2.4e9  # quarter-rate transcendental assumption: 16 lanes/clk/CU
-# Memory-side bytes per lse2_kernel launch of the default workload in strict mode, from two
+# Memory-side bytes per lse2_kernel launch of the default workload, per operand mode, from two
 # rocprofv3 --pmc runs (FETCH_SIZE 286,269 KiB x 2.0, WRITE_SIZE 105,622 KiB x 1.0; the factors
 # are what the same counters read for a 256 MiB copy kernel).  Not measured for the other modes.
-MEASURED_TRAFFIC_BYTES = {"strict": int((286269 * 2.0 + 105622) * 1024), "fp32_mfma": None,
-                          "reduced": None}
+MEASURED_TRAFFIC_BYTES = {"strict": None, "bf16x3": int((286269 * 2.0 + 105622) * 1024)}
 
 
 def gmm_cloud(rng, n, d, k=8):
@@ -103,7 +105,7 @@ def main():
     ap.add_argument("--n", type=int, default=N)
     ap.add_argument("--m", type=int, default=M)
     ap.add_argument("--d", type=int, default=D)
-    ap.add_argument("--mode", choices=["strict", "fp32_mfma", "reduced"], default="strict")
+    ap.add_argument("--mode", choices=MODES, default="strict")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-modes", action="store_true",
                     help="skip the one-launch timings of the two other operand modes")
@@ -126,7 +128,7 @@ def main():
     X, Y, A, B = (torch.from_numpy(t).to(dev) for t in (x, y, a, b))
 
     def set_mode(mode):
-        _lib.STRICT_FP32_MFMA = (mode == "fp32_mfma")
+        _lib.STRICT_OPERANDS = {"fp32_mfma": "fp32_mfma", "bf16x3": "bf16x3"}.get(mode, "fp16x2")
         return mode == "reduced"  # allow_tf32
 
     def solve(mode):
@@ -164,8 +166,9 @@ def main():
         return e0.elapsed_time(e1) / reps
 
     flop = 4.0 * n * m * d
-    products = {"strict": 6, "reduced": 3, "fp32_mfma": 0}
-    dtypes = {"strict": "bf16x3-planes/fp32-accumulate (fp32-grade)", "fp32_mfma": "f32",
+    products = {"strict": 3, "bf16x3": 6, "reduced": 3, "fp32_mfma": 0}
+    dtypes = {"strict": "fp16x2-planes/fp32-accumulate (fp32-grade)",
+              "bf16x3": "bf16x3-planes/fp32-accumulate (fp32-grade)", "fp32_mfma": "f32",
               "reduced": "bf16x2-planes/fp32-accumulate"}
 
     def roofline_for(mode, ms):
@@ -177,11 +180,11 @@ def main():
                        "finish_kernel; 4*n*m*d algorithmic flop",
              "launch_ms": ms, "exp_per_s": 2.0 * n * m / (ms * 1e-3)}
         if products[mode]:
-            r["executed_bf16_mfma_tflops"] = achieved * products[mode]
-            r["executed_frac_of_bf16_peak"] = achieved * products[mode] / BF16_MFMA_PEAK_TFLOPS
-            r["note"] = (f"{products[mode]} bf16 MFMA products per algorithmic product; "
+            r["executed_16bit_mfma_tflops"] = achieved * products[mode]
+            r["executed_frac_of_16bit_peak"] = achieved * products[mode] / BF16_MFMA_PEAK_TFLOPS
+            r["note"] = (f"{products[mode]} 16-bit MFMA products per algorithmic product; "
                          "algorithmic rate priced against the fp32 MFMA peak, executed rate "
-                         "against the bf16 peak")
+                         "against the fp16/bf16 peak")
         return r
 
     main_ms = launch_ms(args.mode)
@@ -200,7 +203,7 @@ def main():
     }
     if not args.no_other_modes:
         others = {}
-        for mode in ("strict", "fp32_mfma", "reduced"):
+        for mode in MODES:
             if mode != args.mode:
                 ms = launch_ms(mode, reps=10)
                 rf = roofline_for(mode, ms)

@@ -19,9 +19,11 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 FS_FLAG_EXP2 = 1
 FS_FLAG_REDUCED_OPERANDS = 2
 FS_FLAG_FP32_MFMA = 4
-# allow_tf32=False normally runs the three-plane split-bf16 operands (fp32-grade accuracy);
-# set this (or FLASH_SINKHORN_FP32_MFMA=1) to run fp32 MFMA operands instead.
-STRICT_FP32_MFMA = os.environ.get("FLASH_SINKHORN_FP32_MFMA", "0") == "1"
+FS_FLAG_BF16X3_OPERANDS = 8
+# allow_tf32=False normally runs the two-plane fp16 operands (fp32-grade accuracy).
+# STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" runs fp32 MFMA
+# operands, "bf16x3" the three-plane bf16 split instead.
+STRICT_OPERANDS = os.environ.get("FLASH_SINKHORN_STRICT_OPERANDS", "fp16x2")
 OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5 = range(6)
 
 _lib: Optional[ctypes.CDLL] = None
@@ -102,4 +104,9 @@ def flags(use_exp2: bool, allow_tf32: bool) -> int:
     f = FS_FLAG_EXP2 if use_exp2 else 0
     if allow_tf32:
         return f | FS_FLAG_REDUCED_OPERANDS
-    return f | (FS_FLAG_FP32_MFMA if STRICT_FP32_MFMA else 0)
+    if STRICT_OPERANDS not in _STRICT_FLAGS:
+        raise ValueError(f"STRICT_OPERANDS must be one of {sorted(_STRICT_FLAGS)}")
+    return f | _STRICT_FLAGS[STRICT_OPERANDS]
+
+
+_STRICT_FLAGS = {"fp16x2": 0, "fp32_mfma": FS_FLAG_FP32_MFMA, "bf16x3": FS_FLAG_BF16X3_OPERANDS}

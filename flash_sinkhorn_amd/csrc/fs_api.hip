@@ -15,6 +15,8 @@ namespace {
 
 constexpr int kMaxStreamD = 128;    // register-stationary streaming kernels
 constexpr int kMaxSlicedD = 1536;   // column-sliced kernels
+constexpr int kPlanePadRowsApi = 256;  // must match kPlanePadRows of the plane-splitting kernels
+constexpr size_t kPlaneAuxBytes = (2 * 256 + 4) * sizeof(float);  // absmax partials + plane scales
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
@@ -155,19 +157,21 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     rb = std::min(rb, plans[s].rb);
   }
   static const int use_v2 = env_int("FS_LSE2", 1);
-  static const int strict_prec = env_int("FS_STRICT_PREC", 2);    // 2: three bf16 planes, 0: fp32 MFMA
+  static const int strict_prec = env_int("FS_STRICT_PREC", 3);    // 3: two fp16 planes, 2: three bf16 planes, 0: fp32 MFMA
   static const int reduced_prec = env_int("FS_REDUCED_PREC", 1);  // 1: two bf16 planes, 0: fp32 MFMA
   static const int rb_override = env_int("FS_RB", 0);
   bool aligned = (d % 4 == 0);
   for (int s = 0; s < nsides; ++s) aligned = aligned && aligned16(sides[s].q) && aligned16(sides[s].k);
   const int prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec
-                   : ((flags & FS_FLAG_FP32_MFMA) ? 0 : strict_prec);
-  // pipelined LSE kernel: the bf16-plane modes take any d <= 128, the fp32 mode needs aligned rows
+                   : ((flags & FS_FLAG_FP32_MFMA) ? 0
+                      : ((flags & FS_FLAG_BF16X3_OPERANDS) ? 2 : strict_prec));
+  // pipelined LSE kernel: the 16-bit plane modes take any d <= 128, the fp32 mode needs aligned rows
   const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = std::max(dp, 16);
-  const int np = (prec == 1) ? 2 : 3;
+  const int np = (prec == 2) ? 3 : 2;
   if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
-  // distinct operand matrices that need bf16 planes (x and y, whichever roles they play)
+  if (lse2 && prec == 2 && dp >= 64) rb = 1;  // three planes of 64 columns x two row blocks spill
+  // distinct operand matrices that need 16-bit planes (x and y, whichever roles they play)
   const float* plane_src[4];
   int plane_rows[4];
   size_t plane_off[4];
@@ -183,11 +187,18 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
           plane_src[nplanes] = ptrs[k];
           plane_rows[nplanes] = rows[k];
           plane_off[nplanes] = need;
-          need += (((size_t)rows[k] * np * (dp2 / 2) * 4) + 15) & ~(size_t)15;
+          need += (((size_t)(rows[k] + kPlanePadRowsApi) * np * (dp2 / 2) * 4) + 15) & ~(size_t)15;
           ++nplanes;
         }
       }
     }
+  }
+  // fp16 planes: partial maxima [2][256] and the two power-of-two scales
+  size_t aux_off = 0;
+  if (lse2 && prec == 3) {
+    if (nplanes > 2) return FS_ERR_BAD_ARGUMENT;
+    aux_off = need;
+    need += kPlaneAuxBytes;
   }
   const size_t need_planes_end = need;
   for (int s = 0; s < nsides; ++s) {
@@ -226,6 +237,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       if (plane_src[i] == sd.q && plane_rows[i] == sd.nq) sd.qplanes = base;
       if (plane_src[i] == sd.k && plane_rows[i] == sd.nk) sd.kplanes = base;
     }
+    if (lse2 && prec == 3)
+      sd.plane_scale = reinterpret_cast<const float*>(static_cast<char*>(ws) + aux_off) + 2 * 256;
     a.side[s] = sd;
   }
   if (nsides == 1) a.side[1] = a.side[0];
@@ -239,10 +252,23 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
   } else if (lse2) {
     rc = FS_OK;
-    for (int i = 0; i < nplanes && rc == FS_OK; ++i)
-      rc = launch_split_planes(plane_src[i],
-                               reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
-                               plane_rows[i], (int)d, dp2, np, st);
+    if (prec == 3) {
+      float* partial = reinterpret_cast<float*>(static_cast<char*>(ws) + aux_off);
+      float* scales = partial + 2 * 256;
+      const bool two = nplanes > 1;
+      rc = launch_absmax(plane_src[0], (long long)plane_rows[0] * d, two ? plane_src[1] : plane_src[0],
+                         two ? (long long)plane_rows[1] * d : 0, partial, st);
+      for (int i = 0; i < nplanes && rc == FS_OK; ++i)
+        rc = launch_split_planes_f16(
+            plane_src[i], reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
+            plane_rows[i], (int)d, dp2, partial + 256 * i, scales + i,
+            two ? nullptr : scales + 1, st);
+    } else {
+      for (int i = 0; i < nplanes && rc == FS_OK; ++i)
+        rc = launch_split_planes(plane_src[i],
+                                 reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
+                                 plane_rows[i], (int)d, dp2, np, st);
+    }
     if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, total, st);
   } else
   switch (mode) {
@@ -353,7 +379,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   };
   size_t planes = 0;  // bf16 planes of x and y for the pipelined LSE kernel (three planes at most)
   if (mode == kLse && !fam.sliced)
-    planes = (size_t)(n + m) * 3 * (std::max(dp, 16) / 2) * 4 + 64;
+    planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   if (both) return a + b - planes + 64;
   if (either) return std::max(a, b) + 64;

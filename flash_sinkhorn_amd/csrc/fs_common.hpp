@@ -62,6 +62,7 @@ struct Side {
   int igroups;          // ceil(nq / rows per workgroup)
   const unsigned* qplanes;  // split-bf16 kernels: query rows as packed bf16 planes [nq][NP][DP/2]
   const unsigned* kplanes;  // same for the key rows [nk][NP][DP/2]
+  const float* plane_scale; // fp16 planes: power-of-two scales of the two operand matrices [2]
   float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;

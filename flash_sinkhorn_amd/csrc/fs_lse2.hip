@@ -13,7 +13,7 @@ static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
 
 template <int DP, int PREC>
 static int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
-  if constexpr (DP <= 64) {
+  if constexpr (DP <= 64 && !(PREC == kBf6 && DP == 64)) {
     if (rb >= 2) return launch_cfg<DP, 2, PREC>(a, blocks, st);
   }
   return launch_cfg<DP, 1, PREC>(a, blocks, st);
@@ -32,7 +32,7 @@ static int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_
 
 int launch_split_planes(const float* src, unsigned* dst, int rows, int d, int dp, int np,
                         hipStream_t st) {
-  const long long items = (long long)rows * (dp / 4);
+  const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
   const int grid = (int)((items + 255) / 256);
   if (np == 2)
     hipLaunchKernelGGL((split_planes_kernel<2>), dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp);
@@ -41,11 +41,28 @@ int launch_split_planes(const float* src, unsigned* dst, int rows, int d, int dp
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
+int launch_absmax(const float* a, long long na, const float* b, long long nb, float* partial,
+                  hipStream_t st) {
+  hipLaunchKernelGGL(absmax_kernel, dim3(2 * kAbsmaxBlocks), dim3(256), 0, st, a, na, b, nb, partial);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
+                            const float* partial_max, float* scale_out, float* scale_out2,
+                            hipStream_t st) {
+  const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
+  const int grid = (int)((items + 255) / 256);
+  hipLaunchKernelGGL(split_planes_f16_kernel, dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp,
+                     partial_max, scale_out, scale_out2);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
 int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, int blocks, hipStream_t st) {
   switch (prec) {
     case kF32: return launch_dp<kF32>(a, dp, rb, blocks, st);
     case kBf3: return launch_dp<kBf3>(a, dp, rb, blocks, st);
     case kBf6: return launch_dp<kBf6>(a, dp, rb, blocks, st);
+    case kH3: return launch_dp<kH3>(a, dp, rb, blocks, st);
   }
   return FS_ERR_BAD_ARGUMENT;
 }

@@ -24,6 +24,11 @@
 //   kBf6   three bf16 planes, the six products whose weight is >= 2^-16: same
 //          accuracy class as fp32 operands (the planes sum to the fp32 value exactly)
 //          at 6/16 of the fp32 MFMA time.
+//   kH3    two fp16 planes (hi, lo) of the operand times a power of two that brings the
+//          matrix's largest magnitude to [2^14, 2^15); hi*hi + hi*lo + lo*hi on
+//          v_mfma_f32_32x32x16_f16.  The planes carry 22 significand bits and the dropped
+//          lo*lo term weighs 2^-22, so a dot product is as accurate as one accumulated in
+//          fp32 from exact products, at the MFMA cost of kBf3.
 #pragma once
 
 #include "fs_common.hpp"
@@ -31,10 +36,15 @@
 
 namespace fs {
 
-enum Prec : int { kF32 = 0, kBf3 = 1, kBf6 = 2 };
+enum Prec : int { kF32 = 0, kBf3 = 1, kBf6 = 2, kH3 = 3 };
+
+constexpr int kPlanePadRows = 256;  // zero rows after the last row of a plane buffer
+constexpr int kAbsmaxBlocks = 256;  // partial maxima per matrix written by absmax_kernel
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
@@ -62,21 +72,22 @@ __device__ __forceinline__ void split_pair(float a, float b, unsigned (&out)[NP]
   }
 }
 
-// x[rows, d] (fp32) -> packed bf16 planes [rows][NP][DP/2] (32-bit words), zero padded to DP
-// columns; plane p holds the p-th round-to-nearest bf16 piece, so the planes sum to x.
+// x[rows, d] (fp32) -> packed bf16 planes [rows + kPlanePadRows][NP][DP/2] (32-bit words), zero
+// padded to DP columns and in the trailing rows; plane p holds the p-th round-to-nearest bf16
+// piece, so the planes sum to x.
 template <int NP>
 __global__ __launch_bounds__(256) void split_planes_kernel(const float* __restrict__ src,
                                                            unsigned* __restrict__ dst, int rows,
                                                            int d, int dp) {
   const int per_row = dp / 4;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (long long)rows * per_row) return;
+  if (idx >= (long long)(rows + kPlanePadRows) * per_row) return;
   const int r = (int)(idx / per_row);
   const int c4 = (int)(idx % per_row) * 4;
-  const float* p = src + (size_t)r * (size_t)d;
+  const float* p = src + (size_t)min(r, rows - 1) * (size_t)d;
   float v[4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) v[t] = (c4 + t < d) ? p[c4 + t] : 0.f;
+  for (int t = 0; t < 4; ++t) v[t] = (c4 + t < d && r < rows) ? p[c4 + t] : 0.f;
   unsigned p01[NP], p23[NP];
   split_pair<NP>(v[0], v[1], p01);
   split_pair<NP>(v[2], v[3], p23);
@@ -86,44 +97,117 @@ __global__ __launch_bounds__(256) void split_planes_kernel(const float* __restri
     *reinterpret_cast<uint2*>(o + pl * (dp / 2) + c4 / 2) = make_uint2(p01[pl], p23[pl]);
 }
 
-// Scheduling hint for one pipelined unit: N MFMAs in a row, with the 17 exp2 and ~44 plain
-// VALU ops of the lagging soft-max spread evenly between them.
-template <int I, int N>
-struct SpreadSoftmax {
-  static __device__ __forceinline__ void emit() {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                       // MFMA
-    __builtin_amdgcn_sched_group_barrier(0x400, (17 * (I + 1)) / N - (17 * I) / N, 0);       // exp2
-    __builtin_amdgcn_sched_group_barrier(0x002, (44 * (I + 1)) / N - (44 * I) / N, 0);       // VALU
-    SpreadSoftmax<I + 1, N>::emit();
+// Largest |value| of two matrices: blocks [0, kAbsmaxBlocks) scan a, the rest scan b; one
+// partial maximum per block goes to partial[2][kAbsmaxBlocks].
+__global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ a, long long na,
+                                                     const float* __restrict__ b, long long nb,
+                                                     float* __restrict__ partial) {
+  __shared__ float red[4];
+  const bool second = blockIdx.x >= kAbsmaxBlocks;
+  const float* src = second ? b : a;
+  const long long cnt = second ? nb : na;
+  const int blk = second ? blockIdx.x - kAbsmaxBlocks : blockIdx.x;
+  float m = 0.f;
+  for (long long i = (long long)blk * 256 + threadIdx.x; i < cnt; i += 256LL * kAbsmaxBlocks)
+    m = fmaxf(m, fabsf(src[i]));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    partial[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// Power of two that maps a largest magnitude `mx` into [2^14, 2^15); 1 for zero / denormal
+// / non-finite maxima, exponent clamped to +-40.
+__device__ __forceinline__ float f16_plane_scale(float mx) {
+  const int e = (int)((__builtin_bit_cast(unsigned, mx) >> 23) & 255u);
+  if (e == 0 || e == 255) return 1.0f;
+  int se = 14 - (e - 127);
+  se = max(-40, min(40, se));
+  return __builtin_bit_cast(float, (unsigned)(127 + se) << 23);
+}
+
+__device__ __forceinline__ unsigned pack_f16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2));
+}
+
+// x[rows, d] (fp32) -> two packed fp16 planes [rows + kPlanePadRows][2][DP/2] of scale*x, zero
+// padded to DP columns and in the trailing rows.  scale is derived from the partial maxima of
+// absmax_kernel; block 0 also
+// publishes it in *scale_out for the consuming kernel.
+__global__ __launch_bounds__(256) void split_planes_f16_kernel(
+    const float* __restrict__ src, unsigned* __restrict__ dst, int rows, int d, int dp,
+    const float* __restrict__ partial_max, float* __restrict__ scale_out,
+    float* __restrict__ scale_out2) {
+  __shared__ float red[4];
+  float m = partial_max[threadIdx.x];  // kAbsmaxBlocks == blockDim.x
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  const float sc = f16_plane_scale(fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *scale_out = sc;
+    if (scale_out2) *scale_out2 = sc;  // the same matrix plays both roles
   }
-};
-template <int N>
-struct SpreadSoftmax<N, N> {
-  static __device__ __forceinline__ void emit() {}
-};
+
+  const int per_row = dp / 4;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)(rows + kPlanePadRows) * per_row) return;
+  const int r = (int)(idx / per_row);
+  const int c4 = (int)(idx % per_row) * 4;
+  const float* p = src + (size_t)min(r, rows - 1) * (size_t)d;
+  float v[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) v[t] = (c4 + t < d && r < rows) ? p[c4 + t] * sc : 0.f;
+  const unsigned h01 = pack_f16(v[0], v[1]), h23 = pack_f16(v[2], v[3]);
+  const f16x2 a = __builtin_bit_cast(f16x2, h01), b = __builtin_bit_cast(f16x2, h23);
+  const unsigned l01 = pack_f16(v[0] - (float)a[0], v[1] - (float)a[1]);
+  const unsigned l23 = pack_f16(v[2] - (float)b[0], v[3] - (float)b[1]);
+  unsigned* o = dst + (size_t)r * (size_t)dp;  // two planes of dp/2 words
+  *reinterpret_cast<uint2*>(o + c4 / 2) = make_uint2(h01, h23);
+  *reinterpret_cast<uint2*>(o + dp / 2 + c4 / 2) = make_uint2(l01, l23);
+}
 
 template <int DP, int PREC>
 struct Geo2 {
-  static constexpr int NP = (PREC == kF32) ? 1 : (PREC == kBf3 ? 2 : 3);
+  static constexpr int NP = (PREC == kF32) ? 1 : (PREC == kBf6 ? 3 : 2);
   static constexpr int JT = (DP >= 128) ? 32 : 64;
   static constexpr int NSUB = JT / 32;
-  // LDS row stride in 32-bit words: fp32 row + 4, or NP bf16 planes + 4
+  // LDS row stride in 32-bit words: fp32 row + 4, or NP 16-bit planes + 4
   static constexpr int LDW = (PREC == kF32) ? (DP + 4) : (NP * DP / 2 + 4);
-  static constexpr int V4_PER_ROW = DP / 4;
-  static constexpr int V4_TOTAL = JT * V4_PER_ROW;
-  static constexpr int PER_THREAD = (V4_TOTAL + 255) / 256;
-  static constexpr int KK16 = DP / 16;  // bf16 MFMAs per plane pair
+  static constexpr int KK16 = DP / 16;  // 16-bit MFMAs per plane pair
+  // MFMAs of one logits tile, the bias one excluded
+  static constexpr int NMAIN = (PREC == kF32) ? DP / 2 : (NP == 2 ? 3 : 6) * KK16;
+};
+
+#define FS_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Soft-max of one logits tile cut into kPieces program-order pieces, so that the caller can
+// place a piece after every few MFMAs of the NEXT tile: a wavefront issues in order, and only
+// VALU work that sits between the MFMAs in program order runs in their shadow.
+constexpr int kPieces = 12;
+struct SoftmaxStage {
+  float m[6], aa, bb, c, ps0, ps1;
+  float t[16], e[16];
 };
 
 template <int DP, int RB, int PREC>
 __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   using G = Geo2<DP, PREC>;
   constexpr int NP = G::NP;
+  constexpr int NSUB = G::NSUB;
+  constexpr int NMAIN = G::NMAIN;
   constexpr bool kBf = (PREC != kF32);
   constexpr int ROWW = kBf ? NP * DP / 2 : DP;  // 32-bit words per operand row in global memory
+  // Key-register prefetch (A operands of the next 32-key sub-tile are read from LDS while the
+  // current one is multiplied) and the early LDS store it needs; off where registers are short.
+  constexpr bool KPF = (NSUB == 2) && !(PREC == kBf6 && RB == 2);
 
   __shared__ __attribute__((aligned(16))) unsigned lds_k[2][G::JT * G::LDW];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][G::JT];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][256];  // [buf][thread]; first JT used
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;
@@ -144,10 +228,12 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   const int ntiles = (j_end - j_begin + G::JT - 1) / G::JT;
 
   // fp32 mode: logits come out of the MFMAs already in base-2 units (queries pre-scaled).
-  // bf16 modes: MFMAs produce raw dot products; lscale turns them into base-2 logits inside
-  // the exp2 argument, and the bias / running max are kept in dot-product units.
-  const float lscale = kBf ? sd.qscale : 1.0f;
-  const float inv_lscale = kBf ? 1.0f / sd.qscale : 1.0f;
+  // 16-bit plane modes: MFMAs produce raw dot products; lscale turns them into base-2 logits
+  // inside the exp2 argument, and the bias / running max are kept in dot-product units.
+  // fp16 planes carry a power-of-two scale per matrix, which lscale takes out again.
+  float lscale = kBf ? sd.qscale : 1.0f;
+  if constexpr (PREC == kH3) lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  const float inv_lscale = kBf ? 1.0f / lscale : 1.0f;
 
   // ---- stationary query operands ----
   float xs[kBf ? 1 : RB][kBf ? 1 : DP / 2];
@@ -189,22 +275,48 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int C16_TOTAL = G::JT * C16_PER_ROW;
   constexpr int PER_THREAD = (C16_TOTAL + 255) / 256;
   u32x4 st_k[PER_THREAD];
-  float st_b = 0.f;
+  float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f, st_pen = 0.f;
   const unsigned* krows = kBf ? sd.kplanes : reinterpret_cast<const unsigned*>(sd.k);
   const int krow_words = kBf ? ROWW : d;
+  const float* kb1p = sd.kb1 ? sd.kb1 : sd.kb0;  // always loadable; unused terms are dropped
+  const float* kb2p = sd.kb2 ? sd.kb2 : sd.kb0;
+  // Plane buffers end with kPlanePadRows zero rows, so the 16-bit modes walk them with plain
+  // running pointers (tiles up to two past the chunk are fetched and masked by the bias);
+  // the fp32 mode reads the caller's matrix and clamps the row instead.
+  const unsigned* kp[PER_THREAD];
+#pragma unroll
+  for (int c = 0; c < PER_THREAD; ++c) {
+    const int idx = tid + 256 * c;
+    kp[c] = krows + (size_t)(j_begin + idx / C16_PER_ROW) * (size_t)krow_words +
+            (idx % C16_PER_ROW) * 4;
+  }
+  // No branches anywhere in the main loop: a branch would split the basic block and let the
+  // compiler sink the soft-max pieces out from between the MFMAs.
   auto stage_load = [&](int j0) {
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
-      const int idx = tid + 256 * c;
-      const int r = idx / C16_PER_ROW;
-      const int c4 = (idx % C16_PER_ROW) * 4;
-      const int j = min(j0 + r, j_end - 1);
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (kBf || c4 < d)
-        v = *reinterpret_cast<const u32x4*>(krows + (size_t)j * (size_t)krow_words + c4);
-      st_k[c] = v;
+      if constexpr (kBf) {
+        st_k[c] = *reinterpret_cast<const u32x4*>(kp[c]);
+        kp[c] += G::JT * ROWW;
+      } else {
+        const int idx = tid + 256 * c;
+        const int r = idx / C16_PER_ROW;
+        const int c4 = (idx % C16_PER_ROW) * 4;
+        const int j = max(0, min(j0 + r, j_end - 1));
+        u32x4 v = *reinterpret_cast<const u32x4*>(krows + (size_t)j * (size_t)krow_words +
+                                                  min(c4, d - 4));
+        if (c4 >= d) v = u32x4{0u, 0u, 0u, 0u};
+        st_k[c] = v;
+      }
     }
-    if (tid < G::JT) st_b = key_bias(sd, j0 + tid, j_end) * inv_lscale;
+    {  // raw key-bias terms of row j0 + tid; combined at store time so that nothing here
+       // waits for the loads (threads beyond the tile fetch a clamped, unused row)
+      const int j = max(0, min(j0 + tid, j_end - 1));
+      st_b0 = sd.kb0[j];
+      st_b1 = kb1p[j];
+      st_b2 = kb2p[j];
+      st_pen = (j0 + tid < j_end) ? 0.f : 2.0f * kNegBig;
+    }
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
@@ -216,9 +328,18 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         *reinterpret_cast<u32x4*>(&lds_k[buf][r * G::LDW + c4]) = st_k[c];
       }
     }
-    if (tid < G::JT) lds_b[buf][tid] = st_b;
+    // masked rows get a penalty ADDED (not selected), so the loads stay unconditional
+    float b = sd.kc0 * st_b0 + (sd.kb1 ? sd.kc1 * st_b1 : 0.f);
+    b += (sd.kb2 ? sd.kc2 * st_b2 : 0.f);
+    lds_b[buf][tid] = (fmaxf(b, kNegBig) + st_pen) * inv_lscale;
   };
 
+  // v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its
+  // second, so (a, b) = (t, t) becomes (low half twice, high half twice).  Issued as inline
+  // asm: this compiler models the builtin's two results as one register.
+  auto swap_halves = [&](float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  };
   // max over the 16 key rows this lane holds and over the other half-wave of the column
   auto column_max = [&](const f32x16& acc) {
     const float m0 = fmaxf(fmaxf(acc[0], acc[1]), acc[2]);
@@ -228,17 +349,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     const float m4 = fmaxf(fmaxf(acc[12], acc[13]), acc[14]);
     const float m5 = fmaxf(fmaxf(m0, m1), acc[15]);
     const float m6 = fmaxf(fmaxf(m2, m3), m4);
-    const float tmax = fmaxf(m5, m6);
-#ifdef FS_DBG_XOR32
-    return fmaxf(tmax, xor32(tmax));
-#else
-    // v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its
-    // second, so (a, b) = (tmax, tmax) becomes (low half twice, high half twice).  Issued as
-    // inline asm: this compiler models the builtin's two results as one register.
-    float a = tmax, b = tmax;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    float a = fmaxf(m5, m6), b = a;
+    swap_halves(a, b);
     return fmaxf(a, b);
-#endif
   };
   // classic online soft-max step; acc holds (logit - M)/lscale for the current M = run_m[rb]
   auto softmax = [&](const f32x16& acc, int rb) {
@@ -263,6 +376,51 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     for (int r = 0; r < 16; ++r) ps += fast_exp2(__builtin_fmaf(acc[r], lscale, c));
     run_s[rb] = ps;
     run_m[rb] = delta;
+  };
+  // The same step as `softmax`, piece p of kPieces; fma / exp2 / add of a value sit in
+  // consecutive pieces so that no piece waits on its own results.
+  auto softmax_piece = [&](int p, SoftmaxStage& s, const f32x16& a, int rb) {
+    if (p == 0) {
+      s.m[0] = fmaxf(fmaxf(a[0], a[1]), a[2]);
+      s.m[1] = fmaxf(fmaxf(a[3], a[4]), a[5]);
+      s.m[2] = fmaxf(fmaxf(a[6], a[7]), a[8]);
+    }
+    if (p == 1) {
+      s.m[3] = fmaxf(fmaxf(a[9], a[10]), a[11]);
+      s.m[4] = fmaxf(fmaxf(a[12], a[13]), a[14]);
+      s.m[5] = fmaxf(fmaxf(s.m[0], s.m[1]), a[15]);
+    }
+    if (p == 2) {
+      s.aa = fmaxf(s.m[5], fmaxf(fmaxf(s.m[2], s.m[3]), s.m[4]));
+      s.bb = s.aa;
+      swap_halves(s.aa, s.bb);
+    }
+    if (p == 3) {
+      const float delta = fmaxf(fmaxf(s.aa, s.bb), 0.f);
+      const float m_new = run_m[rb] + delta;
+      s.c = -(m_new - run_m[rb]) * lscale;
+      run_m[rb] = m_new;
+      s.ps0 = 0.f;
+      s.ps1 = 0.f;
+    }
+    const int q = p - 3;  // two values per piece: fma at q, exp2 at q + 1, add at q + 2
+    if (q >= 0 && q < 8) {
+      s.t[2 * q] = __builtin_fmaf(a[2 * q], lscale, s.c);
+      s.t[2 * q + 1] = __builtin_fmaf(a[2 * q + 1], lscale, s.c);
+    }
+    if (q >= 1 && q < 9) {
+      s.e[2 * q - 2] = fast_exp2(s.t[2 * q - 2]);
+      s.e[2 * q - 1] = fast_exp2(s.t[2 * q - 1]);
+    }
+    if (q >= 2 && q < 10) {
+      s.ps0 += s.e[2 * q - 4];
+      s.ps1 += s.e[2 * q - 3];
+    }
+  };
+  auto softmax_tail = [&](SoftmaxStage& s, int rb) {  // what pieces 0..11 left undone
+    s.ps0 += s.e[14];
+    s.ps1 += s.e[15];
+    run_s[rb] = run_s[rb] * fast_exp2(s.c) + (s.ps0 + s.ps1);
   };
 
   // A operands (one 32-key sub-tile) from LDS
@@ -289,84 +447,135 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         for (int kk = 0; kk < G::KK16; ++kk)
           kr.yq[p][kk] = *reinterpret_cast<const u32x4*>(yrow + p * (DP / 2) + 8 * kk + 4 * h);
     }
-    kr.ab = h ? 1.0f : lds_b[buf][js * 32 + li];
+    const float b = lds_b[buf][js * 32 + li];
+    kr.ab = h ? 1.0f : b;
   };
-  // One logits tile (32 keys x 32 queries) of query block rb: all MFMAs except the bias one.
+  // MFMA number k (0 <= k < NMAIN) of one logits tile (32 keys x 32 queries) of query block
+  // rb.  Plane products run from the lowest weight to hi*hi; those below 2^-16 (2^-24 with
+  // three planes) are skipped.
+  auto mfma_k = [&](int k, f32x16 acc, const KeyRegs& kr, int rb) {
+    if constexpr (!kBf) {
+      return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ya[k], xs[rb][k], acc, 0, 0, 0);
+    } else {
+      const int prod = k / G::KK16, kk = k % G::KK16;
+      // NP == 2: (1,0) (0,1) (0,0);  NP == 3: (2,0) (1,1) (0,2) (1,0) (0,1) (0,0)
+      int pa, pb;
+      if (NP == 2) {
+        pa = (prod == 0) ? 1 : 0;
+        pb = (prod == 1) ? 1 : 0;
+      } else {
+        pa = (prod == 0) ? 2 : ((prod == 1 || prod == 3) ? 1 : 0);
+        pb = (prod == 2) ? 2 : ((prod == 1 || prod == 4) ? 1 : 0);
+      }
+      if constexpr (PREC == kH3)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr.yq[pa][kk]),
+                                                      __builtin_bit_cast(f16x8, xq[rb][pb][kk]),
+                                                      acc, 0, 0, 0);
+      else
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kr.yq[pa][kk]),
+                                                       __builtin_bit_cast(bf16x8, xq[rb][pb][kk]),
+                                                       acc, 0, 0, 0);
+    }
+  };
   auto chain = [&](const KeyRegs& kr, int rb) {
     f32x16 acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-    if constexpr (!kBf) {
 #pragma unroll
-      for (int kk = 0; kk < DP / 2; ++kk)
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ya[kk], xs[rb][kk], acc, 0, 0, 0);
-    } else {
-      // low-order products first, hi*hi last
-#pragma unroll
-      for (int pa = NP - 1; pa >= 0; --pa)
-#pragma unroll
-        for (int pb = NP - 1; pb >= 0; --pb) {
-          if (pa + pb > NP - 1) continue;  // weight below 2^-16 (2^-24 for three planes)
-#pragma unroll
-          for (int kk = 0; kk < G::KK16; ++kk)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                __builtin_bit_cast(bf16x8, kr.yq[pa][kk]),
-                __builtin_bit_cast(bf16x8, xq[rb][pb][kk]), acc, 0, 0, 0);
-        }
-    }
+    for (int k = 0; k < NMAIN; ++k) acc = mfma_k(k, acc, kr, rb);
     return acc;
   };
   // The bias MFMA (fp32 operands in every mode): adds kbias_j - M_i with the freshest M.
   auto add_bias = [&](f32x16 acc, const KeyRegs& kr, int rb) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
   };
-  constexpr int kMain = kBf ? (NP == 2 ? 3 : 6) * G::KK16 : DP / 2;  // MFMAs per chain
 
+  KeyRegs K[KPF ? 2 : 1];
+
+  // ---- prologue: tile 0 into LDS buffer 0; with KPF tile 1 is already on its way ----
   stage_load(j_begin);
   stage_store(0);
+  if constexpr (KPF) stage_load(j_begin + G::JT);
   __syncthreads();
+  if constexpr (KPF) load_keys(K[0], 0, 0);
+
+  // ---- tile 0: establishes the running max, no soft-max pipelining ----
+  {
+    if constexpr (KPF) {
+      stage_store(1);
+      stage_load(j_begin + 2 * G::JT);
+    } else {
+      stage_load(j_begin + G::JT);
+    }
+#pragma unroll
+    for (int js = 0; js < NSUB; ++js) {
+      if constexpr (!KPF) load_keys(K[0], 0, js);
+      KeyRegs& kr = K[KPF ? (js & 1) : 0];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        if (KPF && rb == RB - 1) {
+          if (js + 1 < NSUB) {
+            load_keys(K[(js + 1) & 1], 0, js + 1);
+          } else {
+            __syncthreads();  // tile 1 is in buffer 1; every wave is done reading buffer 0
+            load_keys(K[0], 1, 0);
+          }
+        }
+        const f32x16 acc = add_bias(chain(kr, rb), kr, rb);
+        if (js == 0) softmax_first(acc, rb); else softmax(acc, rb);
+      }
+    }
+    if constexpr (!KPF) {
+      stage_store(1);
+      __syncthreads();
+    }
+  }
 
   f32x16 acc_prev;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc_prev[r] = kNegBig;
 
-  for (int t = 0; t < ntiles; ++t) {
+  // ---- steady state: the soft-max of the previous logits tile rides between the MFMAs ----
+  for (int t = 1; t < ntiles; ++t) {
     const int buf = t & 1;
-    const bool more = (t + 1 < ntiles);
-    if (more) stage_load(j_begin + (t + 1) * G::JT);
-
-    if (t == 0) {
-      // first tile of the block: establish the running max, no pipelining
+    if constexpr (!KPF) stage_load(j_begin + (t + 1) * G::JT);
 #pragma unroll
-      for (int js = 0; js < G::NSUB; ++js) {
-        KeyRegs kr;
-        load_keys(kr, buf, js);
+    for (int js = 0; js < NSUB; ++js) {
+      if constexpr (!KPF) load_keys(K[0], buf, js);
+      KeyRegs& kr = K[KPF ? (js & 1) : 0];
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          const f32x16 acc = add_bias(chain(kr, rb), kr, rb);
-          if (js == 0) softmax_first(acc, rb); else softmax(acc, rb);
+      for (int rb = 0; rb < RB; ++rb) {
+        const int prev_rb = (rb + RB - 1) % RB;
+        SoftmaxStage st;
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        FS_SCHED_FENCE();
+#pragma unroll
+        for (int p = 0; p < kPieces; ++p) {
+#pragma unroll
+          for (int k = (p * NMAIN) / kPieces; k < ((p + 1) * NMAIN) / kPieces; ++k)
+            acc = mfma_k(k, acc, kr, rb);
+          if constexpr (KPF) {
+            // LDS / global traffic of the pipeline, placed where it has the whole unit to land
+            if (js == 0 && rb == 0 && p == 0) stage_store(buf ^ 1);              // tile t+1
+            if (js == 0 && rb == 0 && p == 1) stage_load(j_begin + (t + 2) * G::JT);
+            if (rb == RB - 1 && js + 1 < NSUB && p == 1) load_keys(K[(js + 1) & 1], buf, js + 1);
+            if (rb == RB - 1 && js + 1 == NSUB && p == 1) __syncthreads();
+            if (rb == RB - 1 && js + 1 == NSUB && p == 2) load_keys(K[0], buf ^ 1, 0);
+          }
+          softmax_piece(p, st, acc_prev, prev_rb);
+          FS_SCHED_FENCE();
         }
-      }
-    } else {
-#pragma unroll
-      for (int js = 0; js < G::NSUB; ++js) {
-        KeyRegs kr;
-        load_keys(kr, buf, js);
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          f32x16 acc = chain(kr, rb);
-          // the soft-max of the previous tile runs in the shadow of the MFMAs above
-          softmax(acc_prev, (rb + RB - 1) % RB);
-#ifndef FS_DBG_NOSCHED
-          SpreadSoftmax<0, kMain>::emit();
-#endif
-          acc_prev = add_bias(acc, kr, rb);
-        }
+        softmax_tail(st, prev_rb);
+        acc_prev = add_bias(acc, kr, rb);
+        FS_SCHED_FENCE();
       }
     }
-
-    if (more) stage_store(buf ^ 1);
-    __syncthreads();
+    if constexpr (!KPF) {
+      stage_store(buf ^ 1);
+      __syncthreads();
+    }
   }
   softmax(acc_prev, RB - 1);
 

@@ -17,8 +17,11 @@
  *  - flags: FS_FLAG_EXP2 is accepted for interface parity (the kernels always
  *    work in base 2, which is the same function).  Operand precision of the
  *    log-sum-exp kernels for d <= 128 (everything accumulates in fp32):
- *      default                    operands as three bf16 planes, six MFMA products:
- *                                 error at or below that of fp32 MFMA operands
+ *      default                    operands as two fp16 planes (22 significand bits) of
+ *                                 the matrix scaled by a power of two, three MFMA
+ *                                 products: error at or below that of fp32 MFMA operands
+ *      FS_FLAG_BF16X3_OPERANDS    three bf16 planes, six products: same accuracy class,
+ *                                 no dependence on the dynamic range inside a matrix
  *      FS_FLAG_FP32_MFMA          fp32 operands on v_mfma_f32_32x32x2_f32
  *      FS_FLAG_REDUCED_OPERANDS   two bf16 planes, three products (~2^-17 relative
  *                                 per product): the counterpart of allow_tf32=True
@@ -45,6 +48,7 @@ extern "C" {
 #define FS_FLAG_EXP2 1u
 #define FS_FLAG_REDUCED_OPERANDS 2u
 #define FS_FLAG_FP32_MFMA 4u
+#define FS_FLAG_BF16X3_OPERANDS 8u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0
