@@ -96,3 +96,79 @@ def test_config2_loss_and_potentials():
     assert rel_err(fp.cpu().numpy(), fix["f_prelast"]) < 1e-4
     loss = float((A.double() * f.double()).sum() + (A.double() * g.double()).sum())
     assert abs(loss - float(fix["loss"])) < 1e-4 * abs(float(fix["loss"]))
+
+
+def _fixture(name):
+    import os
+    return np.load(os.path.join(os.path.dirname(__file__), "golden", name))
+
+
+def test_config1_debiased_loss_and_gradient():
+    """BASELINE config 1 at full size (n=m=2000, d=3, half cost, debiased, eps=0.01, 100
+    iterations) against the fp64 oracle cached in tests/golden/oracle_config1.npz."""
+    from flash_sinkhorn_amd import SamplesLoss
+    from tests.golden.make_oracle_fixtures import config1_inputs
+    x, y, _ = config1_inputs()
+    fix = _fixture("oracle_config1.npz")
+    X = torch.from_numpy(x).cuda().requires_grad_(True)
+    Y = torch.from_numpy(y).cuda()
+    loss = SamplesLoss("sinkhorn", blur=0.1, half_cost=True, debias=True,
+                       use_epsilon_scaling=False, eps=0.01, n_iters=100, allow_tf32=False)(X, Y)
+    (gx,) = torch.autograd.grad(loss, X)
+    want = float(fix["loss"])
+    # the debiased loss is a difference of three O(1) costs: 1e-4 of it plus fp32 round-off
+    # of the undebiased terms
+    assert abs(float(loss.detach()) - want) <= 1e-4 * abs(want) + 2e-6
+    assert rel_err(gx.detach().cpu().numpy(), fix["grad_x"]) < 2e-4
+
+
+@pytest.mark.parametrize("tag,kw", [("reach", dict(reach=1.0)),
+                                    ("semi", dict(reach_x=1.0, reach_y=None))])
+def test_config4_unbalanced_alternating(tag, kw):
+    """BASELINE config 4 (n=20,000, m=30,000, d=128, eps=0.05^2, Dirichlet weights of mass
+    1.0 / 1.3, 10 alternating iterations with the early-stop check at 10) against the fp64
+    oracle cached in tests/golden/oracle_config4.npz, all rows."""
+    from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating
+    from tests.golden.make_oracle_fixtures import config4_inputs
+    x, y, a, b = config4_inputs()
+    fix = _fixture("oracle_config4.npz")
+    X, Y, A, B = [torch.from_numpy(t).cuda() for t in (x, y, a, b)]
+    f, g, used = sinkhorn_flashstyle_alternating(
+        X, Y, A, B, eps=0.05 ** 2, n_iters=10, threshold=1e-3, check_every=10,
+        return_n_iters=True, allow_tf32=False, **kw)
+    assert used == int(fix[f"used_{tag}"])
+    assert rel_err(f.cpu().numpy(), fix[f"f_{tag}"]) < 1e-4
+    assert rel_err(g.cpu().numpy(), fix[f"g_{tag}"]) < 1e-4
+
+
+def test_config5_large_d_loss_gradient_and_hvp():
+    """BASELINE config 5 (n=m=8192, d=1536, eps=0.25, 50 iterations): debiased loss and
+    grad_x through the column-sliced kernels, then the Hessian-vector product of the xy term
+    by double backward (streaming CG, at most 20 iterations), against the fp64 oracle cached
+    in tests/golden/oracle_config5.npz (48 sampled rows plus Frobenius norms)."""
+    from flash_sinkhorn_amd import SamplesLoss
+    from tests.golden.make_oracle_fixtures import config5_inputs
+    x, y, _, v = config5_inputs()
+    fix = _fixture("oracle_config5.npz")
+    rows = fix["rows"]
+    X = torch.from_numpy(x).cuda().requires_grad_(True)
+    Y, V = torch.from_numpy(y).cuda(), torch.from_numpy(v).cuda()
+    kw = dict(blur=0.5, use_epsilon_scaling=False, eps=0.25, n_iters=50, allow_tf32=False)
+    loss = SamplesLoss("sinkhorn", debias=True, **kw)(X, Y)
+    (gx,) = torch.autograd.grad(loss, X)
+    want = float(fix["loss_debiased"])
+    assert abs(float(loss.detach()) - want) <= 1e-4 * abs(want) + 1e-6 * float(fix["loss_xy"])
+    g = gx.detach().cpu().numpy().astype(np.float64)
+    assert rel_err(g[rows], fix["grad_x_debiased_rows"].astype(np.float64)) < 2e-4
+    assert abs(np.linalg.norm(g) - float(fix["grad_x_norm"])) < 1e-4 * float(fix["grad_x_norm"])
+
+    X2 = torch.from_numpy(x).cuda().requires_grad_(True)
+    loss_xy = SamplesLoss("sinkhorn", debias=False, hvp_max_cg_iter=20, **kw)(X2, Y)
+    assert abs(float(loss_xy.detach()) - float(fix["loss_xy"])) < 1e-4 * float(fix["loss_xy"])
+    (g1,) = torch.autograd.grad(loss_xy, X2, create_graph=True)
+    assert rel_err(g1.detach().cpu().numpy()[rows],
+                   fix["grad_x_xy_rows"].astype(np.float64)) < 1e-4
+    (hv,) = torch.autograd.grad((g1 * V).sum(), X2)
+    h = hv.cpu().numpy().astype(np.float64)
+    assert rel_err(h[rows], fix["hvp_rows"].astype(np.float64)) < 2e-4
+    assert abs(np.linalg.norm(h) - float(fix["hvp_norm"])) < 1e-4 * float(fix["hvp_norm"])
