@@ -38,11 +38,11 @@ ITERS = 100
 MODES = ["strict", "bf16x3", "fp32_mfma", "reduced"]
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2516.6
-EXP_PEAK_PER_S = 256 * 16 * 2.4e9  # quarter-rate transcendental assumption: 16 lanes/clk/CU
 # Memory-side bytes per lse2_kernel launch of the default workload, per operand mode, from two
-# rocprofv3 --pmc runs (FETCH_SIZE 286,269 KiB x 2.0, WRITE_SIZE 105,622 KiB x 1.0; the factors
-# are what the same counters read for a 256 MiB copy kernel).  Not measured for the other modes.
-MEASURED_TRAFFIC_BYTES = {"strict": None, "bf16x3": int((286269 * 2.0 + 105622) * 1024)}
+# rocprofv3 --pmc runs (FETCH_SIZE 112,324 KiB x 2.0, WRITE_SIZE 12,511 KiB x 1.0; the factors
+# are what the same counters read for the 256 MiB copy of --copy-calibration: 131,094 and
+# 262,144 KiB).  Not measured for the other modes.
+MEASURED_TRAFFIC_BYTES = {"strict": int((112324 * 2.0 + 12511) * 1024)}
 
 
 def gmm_cloud(rng, n, d, k=8):
@@ -76,22 +76,22 @@ def cpu_baseline(x, y, a, b, budget_s=20.0):
     fh = -(x.astype(np.float32) ** 2).sum(1)
     gh = -(y.astype(np.float32) ** 2).sum(1)
     done, t0 = 0, time.perf_counter()
-    while True:
-        i0 = (done * rows) % max(1, n - rows + 1)
-        # one half-update for `rows` query rows against all m keys, and the mirrored one
-        oracle.lse_shifted_fused(x[i0:i0 + rows], y, gh, lb, EPS, dtype=np.float32)
-        oracle.lse_shifted_fused(y[i0:i0 + rows], x, fh, la, EPS, dtype=np.float32)
-        done += 1
+    for i0 in range(0, n, rows):
+        i1 = min(n, i0 + rows)
+        # one half-update for these query rows against all m keys, and the mirrored one
+        oracle.lse_shifted_fused(x[i0:i1], y, gh, lb, EPS, dtype=np.float32)
+        oracle.lse_shifted_fused(y[i0:i1], x, fh, la, EPS, dtype=np.float32)
+        done += i1 - i0
         el = time.perf_counter() - t0
-        if el > budget_s or done * rows >= n:
+        if el > budget_s:
             break
-    frac = done * rows / n  # fraction of one full symmetric iteration that was timed
+    frac = done / n  # fraction of one full symmetric iteration that was timed
     ms_per_100 = el / frac * (ITERS + 2) * 1e3
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
     return {
         "value": ms_per_100, "unit": "ms per 100 symmetric iterations", "cores": cores,
         "kind": "port",
-        "sample": f"{done * rows} of {n} query rows of each half-update against all {m} keys "
+        "sample": f"{done} of {n} query rows of each half-update against all {m} keys "
                   f"({el:.1f} s of the numpy fp32 oracle, BLAS threads = host default), scaled "
                   "to 102 steps",
     }
@@ -108,7 +108,10 @@ def main():
     ap.add_argument("--mode", choices=MODES, default="strict")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-modes", action="store_true",
-                    help="skip the one-launch timings of the two other operand modes")
+                    help="skip the one-launch timings of the other operand modes")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 256 MiB device copy: under rocprofv3 --pmc its "
+                         "FETCH_SIZE / WRITE_SIZE give the counters' scale factors")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported",
@@ -211,6 +214,12 @@ def main():
                                 "achieved": rf["achieved"], "frac_of_fp32_peak": rf["frac"]}
         line["other_operand_modes"] = others
         set_mode(args.mode)
+    if args.copy_calibration:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(x, y, a, b)
     print(json.dumps(line))
