@@ -424,10 +424,17 @@ int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const 
   if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
   if (!(eps > 0.f)) return FS_ERR_BAD_ARGUMENT;
   if (f_out == f_hat || g_out == g_hat) return FS_ERR_BAD_ARGUMENT;
+  // Self problem OT(x, x): when every paired argument aliases, the two half-updates are the
+  // same computation and it is done once (f_out == g_out receives it).
+  const bool self = (x == y && f_hat == g_hat && log_a == log_b && f_out == g_out &&
+                     shift_x == shift_y && n == m && damp_f == damp_g);
+  if (f_out == g_out && !self) return FS_ERR_BAD_ARGUMENT;
   const float qs = coord_scale / eps * kLog2e;
   Side s[2];
   s[0] = lse_side(x, y, g_hat, kLog2e / eps, log_b, kLog2e, n, m, qs);
   lse_epilogue(s[0], f_out, f_hat, alpha, eps, damp_f, shift_x);
+  if (self)
+    return run_stream(kLse, false, s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
   s[1] = lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
   lse_epilogue(s[1], g_out, g_hat, alpha, eps, damp_g, shift_y);
   return run_stream(kLse, false, s, 2, d, workspace, workspace_bytes, (hipStream_t)stream, flags);

@@ -115,11 +115,15 @@ def flashsinkhorn_lse_fused(
 def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, alpha, damping_f,
                         damping_g, shift_x=None, shift_y=None, allow_tf32=True, use_exp2=True):
     """One launch on already contiguous fp32 operands.  With shift_x/shift_y the
-    unbalanced shift correction is applied inside the epilogue."""
+    unbalanced shift correction is applied inside the epilogue.  When every paired argument
+    is the same tensor (the self problem OT(x, x)) the library computes the one distinct
+    half-update and the same tensor is returned twice."""
     n, d = x.shape
     m = y.shape[0]
     f_out = torch.empty((n,), device=x.device, dtype=torch.float32)
-    g_out = torch.empty((m,), device=x.device, dtype=torch.float32)
+    self_problem = (y is x and g_hat is f_hat and log_b is log_a and shift_y is shift_x
+                    and damping_f == damping_g)
+    g_out = f_out if self_problem else torch.empty((m,), device=x.device, dtype=torch.float32)
     ws = _lib.workspace(_lib.OP_SYMMETRIC_STEP, n, m, d, x.device)
     rc = _lib.lib().fs_symmetric_step(
         x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),

@@ -1,0 +1,138 @@
+"""Per-operation timings at the BASELINE shapes: ``python -m flash_sinkhorn_amd.op_timings [c1 c2 c3 c4 c5]``.
+
+Prints one JSON line per shape with the average launch time (HIP events on the current
+stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop),
+one LSE half-update (2nmd), gradient of one side (4nmd), plan-vector (2nmd), plan-matrix
+(4nmd) and mat5 (6nmd), followed by end-to-end wall times of the five configurations
+through the public API (solver loops, autograd, CG included).
+"""
+from __future__ import annotations
+
+import json
+import sys
+import time
+
+import torch
+
+from flash_sinkhorn_amd import SamplesLoss
+from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating
+from flash_sinkhorn_amd.kernels.apply_flash import (apply_plan_mat_flashstyle,
+                                                    apply_plan_vec_flashstyle)
+from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
+from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (_symmetric_step_raw,
+                                                                     flashsinkhorn_lse_fused)
+from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+    sinkhorn_geomloss_online_grad_sqeuclid)
+
+SHAPES = {"c1": (2000, 2000, 3, 0.01), "c2": (10000, 10000, 64, 0.01),
+          "c3": (50000, 50000, 64, 0.01), "c4": (20000, 30000, 128, 0.0025),
+          "c5": (8192, 8192, 1536, 0.25)}
+
+
+def _avg_ms(fn, reps=5):
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def _wall_ms(fn, reps=2):
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / reps
+
+
+def kernel_timings(name):
+    n, m, d, eps = SHAPES[name]
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    sc = 2.0 / d ** 0.5
+    X = torch.randn(n, d, device="cuda", generator=gen) * sc
+    Y = torch.randn(m, d, device="cuda", generator=gen) * sc
+    A = torch.full((n,), 1.0 / n, device="cuda")
+    B = torch.full((m,), 1.0 / m, device="cuda")
+    la, lb = A.log(), B.log()
+    al, be = (X * X).sum(1), (Y * Y).sum(1)
+    fh, gh = -al, -be
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    for _ in range(3):  # a few iterations so that the plan is not degenerate
+        fh, gh = _symmetric_step_raw(X, Y, fh, gh, la, lb, eps, **kw)
+    f, g = fh + al, gh + be
+    v = torch.randn(m, device="cuda", generator=gen)
+    V = torch.randn(m, d, device="cuda", generator=gen)
+    Am = torch.randn(n, d, device="cuda", generator=gen)
+    fo, go = f + eps * la, g + eps * lb
+    nmd = float(n) * m * d
+    ops = {
+        "symmetric_step": (4, lambda: _symmetric_step_raw(X, Y, fh, gh, la, lb, eps, **kw)),
+        "lse_half": (2, lambda: flashsinkhorn_lse_fused(X, Y, gh, lb, eps, allow_tf32=False)),
+        "grad_x": (4, lambda: sinkhorn_geomloss_online_grad_sqeuclid(
+            X, Y, A, B, f, g, eps=eps, allow_tf32=False, compute_grad_y=False)),
+        "apply_vec": (2, lambda: apply_plan_vec_flashstyle(X, Y, fh, gh, la, lb, v, eps=eps,
+                                                           axis=1)),
+        "apply_mat": (4, lambda: apply_plan_mat_flashstyle(X, Y, fh, gh, la, lb, V, eps=eps,
+                                                           axis=1)),
+        "mat5": (6, lambda: mat5_sqeuclid(X, Y, fo, go, Am, eps=eps)),
+    }
+    out = {"shape": name, "n": n, "m": m, "d": d}
+    for op, (k, fn) in ops.items():
+        ms = _avg_ms(fn)
+        out[op] = {"ms": round(ms, 4), "algorithmic_TFLOPs": round(k * nmd / ms / 1e9, 1)}
+    return out
+
+
+def end_to_end(name):
+    n, m, d, eps = SHAPES[name]
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    X = torch.randn(n, d, device="cuda", generator=gen)
+    Y = torch.randn(m, d, device="cuda", generator=gen)
+    if name == "c5":
+        X, Y = X / d ** 0.5, Y / d ** 0.5
+    out = {"config": name}
+    if name in ("c1", "c2", "c3", "c5"):
+        kw = dict(blur=eps ** 0.5, use_epsilon_scaling=False, eps=eps,
+                  n_iters=50 if name == "c5" else 100, allow_tf32=False,
+                  half_cost=(name == "c1"), debias=(name != "c3"))
+        Xg = X.clone().requires_grad_(True)
+
+        def loss_and_grad():
+            loss = SamplesLoss("sinkhorn", **kw)(Xg, Y)
+            return torch.autograd.grad(loss, Xg)
+        out["loss_and_grad_x_ms"] = round(_wall_ms(loss_and_grad), 2)
+        if name == "c5":
+            Vv = torch.randn(n, d, device="cuda", generator=gen)
+            kw2 = dict(kw, debias=False, hvp_max_cg_iter=20)
+
+            def hvp():
+                loss = SamplesLoss("sinkhorn", **kw2)(Xg, Y)
+                (g1,) = torch.autograd.grad(loss, Xg, create_graph=True)
+                return torch.autograd.grad((g1 * Vv).sum(), Xg)
+            out["loss_grad_hvp_ms"] = round(_wall_ms(hvp), 2)
+    else:
+        A = torch.rand(n, device="cuda", generator=gen)
+        B = torch.rand(m, device="cuda", generator=gen)
+        A, B = A / A.sum(), 1.3 * B / B.sum()
+        out["alternating_10_iters_ms"] = round(_wall_ms(lambda: sinkhorn_flashstyle_alternating(
+            X, Y, A, B, eps=eps, n_iters=10, reach=1.0, threshold=1e-3, check_every=10,
+            allow_tf32=False)), 2)
+    return out
+
+
+def main(argv):
+    names = [a for a in argv if a in SHAPES] or list(SHAPES)
+    for name in names:
+        print(json.dumps(kernel_timings(name)), flush=True)
+    for name in names:
+        print(json.dumps(end_to_end(name)), flush=True)
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

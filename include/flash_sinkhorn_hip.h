@@ -92,7 +92,10 @@ int fs_lse_fused(const float* x, const float* y, const float* pot_hat, const flo
  * kernel 433-661).  shift_x/shift_y (= cost_scale*|x|^2, cost_scale*|y|^2, may be NULL)
  * fold in the unbalanced shift correction the reference's solver applies on the
  * host right after the launch (sinkhorn_solvers.py:509-517).  Outputs must not
- * alias inputs.
+ * alias inputs.  Self problem OT(x, x): when x == y, f_hat == g_hat, log_a == log_b,
+ * shift_x == shift_y, f_out == g_out (same pointers), n == m and damp_f == damp_g, the two
+ * half-updates are the same numbers and are computed once; f_out == g_out otherwise is an
+ * error.
  */
 int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const float* g_hat,
                       const float* log_a, const float* log_b, float* f_out, float* g_out,

@@ -201,3 +201,23 @@ def test_double_backward_equals_direct_hvp():
         Yg = Y.clone().requires_grad_(True)
         gx, gy = torch.autograd.grad(L(A, X, B, Yg), [X, Yg], create_graph=True)
         torch.autograd.grad((gy * gy).sum(), Yg)
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(reach=0.8)])
+def test_self_problem_shortcut_equals_generic_path(kw):
+    """OT(x, x) with aliased arguments runs one half-update per step; a copy of x (no
+    aliasing) takes the two-sided path.  Same numbers either way."""
+    from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric as solve
+    x, _, a, _ = inputs(37, 700, 700, 16)
+    X, A = dev(x, a)
+    args = dict(use_epsilon_scaling=False, eps=0.05, n_iters=20, allow_tf32=False,
+                return_prelast=True, **kw)
+    fs, gs, fps, gps = solve(X, X, A, A, **args)
+    fg, gg, fpg, gpg = solve(X, X.clone(), A, A.clone(), **args)
+    assert torch.equal(fs, gs) and torch.equal(fps, gps)
+    assert float((fs - fg).abs().max()) <= 1e-6 * float(fg.abs().max())
+    assert float((gs - gg).abs().max()) <= 1e-6 * float(gg.abs().max())
+    assert float((fps - fpg).abs().max()) <= 1e-6 * float(fpg.abs().max())
+    want = oracle.sinkhorn_symmetric(x, x, a, a, use_epsilon_scaling=False, eps=0.05, n_iters=20,
+                                     **kw)
+    assert rel_err(fs, want[0]) < RTOL and rel_err(gs, want[1]) < RTOL
