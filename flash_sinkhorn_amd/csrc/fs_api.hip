@@ -138,6 +138,123 @@ int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
   return FS_ERR_UNSUPPORTED;
 }
 
+
+// ---- large-d LSE on chunked fp16 planes (lse_gemm_kernel) ----
+constexpr int kGemmTile = 256;  // query rows per workgroup and keys per tile
+
+struct GemmPlan {
+  int igroups, bsplits, chunk;
+};
+
+GemmPlan gemm_plan(int64_t nq, int64_t nk, int total_igroups) {
+  GemmPlan p;
+  p.igroups = ceil_div(nq, kGemmTile);
+  int s = 1;
+  while ((int64_t)total_igroups * s < 512 && nk / (2 * s) >= kGemmTile && s < 32) s *= 2;
+  p.chunk = ceil_div(ceil_div(nk, s), kGemmTile) * kGemmTile;
+  p.bsplits = ceil_div(nk, p.chunk);
+  return p;
+}
+
+inline int gemm_dp(int64_t d) { return ceil_div(d, 32) * 32; }
+
+size_t gemm_plane_bytes(int64_t rows, int dp) {
+  return (((size_t)(rows + kPlanePadRowsApi) * (size_t)dp * 4) + 15) & ~(size_t)15;
+}
+
+// Workspace: planes of the distinct operand matrices, absmax partials and scales, then per
+// side 2*bsplits partial (M, s) rows.
+int run_lse_gemm(Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes, hipStream_t st) {
+  const int dp = gemm_dp(d);
+  const float* plane_src[2];
+  int plane_rows[2];
+  size_t plane_off[2];
+  int nplanes = 0;
+  size_t need = 0;
+  for (int s = 0; s < nsides; ++s) {
+    const float* ptrs[2] = {sides[s].q, sides[s].k};
+    const int rows[2] = {sides[s].nq, sides[s].nk};
+    for (int k = 0; k < 2; ++k) {
+      bool seen = false;
+      for (int i = 0; i < nplanes; ++i) seen = seen || (plane_src[i] == ptrs[k] && plane_rows[i] == rows[k]);
+      if (seen) continue;
+      if (nplanes == 2) return FS_ERR_BAD_ARGUMENT;
+      plane_src[nplanes] = ptrs[k];
+      plane_rows[nplanes] = rows[k];
+      plane_off[nplanes] = need;
+      need += gemm_plane_bytes(rows[k], dp);
+      ++nplanes;
+    }
+  }
+  const size_t aux_off = need;
+  need += kPlaneAuxBytes;
+  int total_ig = 0;
+  for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kGemmTile);
+  GemmPlan plans[2];
+  size_t part_off[2];
+  for (int s = 0; s < nsides; ++s) {
+    plans[s] = gemm_plan(sides[s].nq, sides[s].nk, total_ig);
+    part_off[s] = need;
+    need += (((size_t)2 * plans[s].bsplits * (size_t)sides[s].nq * 2 * sizeof(float)) + 15) & ~(size_t)15;
+  }
+  if (need > ws_bytes || ws == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(ws);
+  float* partial = reinterpret_cast<float*>(base + aux_off);
+  float* scales = partial + 2 * 256;
+
+  LaunchArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.d = (int)d;
+  int blocks[2] = {0, 0};
+  for (int s = 0; s < nsides; ++s) {
+    Side& sd = sides[s];
+    sd.splits = 2 * plans[s].bsplits;
+    sd.chunk = plans[s].chunk;
+    sd.igroups = plans[s].igroups;
+    sd.part_ms = reinterpret_cast<float*>(base + part_off[s]);
+    sd.part_o = nullptr;
+    sd.plane_scale = scales;
+    for (int i = 0; i < nplanes; ++i) {
+      const unsigned* pb = reinterpret_cast<const unsigned*>(base + plane_off[i]);
+      if (plane_src[i] == sd.q && plane_rows[i] == sd.nq) sd.qplanes = pb;
+      if (plane_src[i] == sd.k && plane_rows[i] == sd.nk) sd.kplanes = pb;
+    }
+    blocks[s] = plans[s].igroups * plans[s].bsplits;
+    a.side[s] = sd;
+  }
+  if (nsides == 1) a.side[1] = a.side[0];
+  a.blocks0 = blocks[0];
+  const int total = blocks[0] + blocks[1];
+  if (total <= 0) return FS_OK;
+
+  const bool two = nplanes > 1;
+  int rc = launch_absmax(plane_src[0], (long long)plane_rows[0] * d, two ? plane_src[1] : plane_src[0],
+                         two ? (long long)plane_rows[1] * d : 0, partial, st);
+  for (int i = 0; i < nplanes && rc == FS_OK; ++i)
+    rc = launch_split_planes_f16(plane_src[i], reinterpret_cast<unsigned*>(base + plane_off[i]),
+                                 plane_rows[i], (int)d, dp, partial + 256 * i, scales + i,
+                                 two ? nullptr : scales + 1, 1, st);
+  if (rc == FS_OK) rc = launch_lse_gemm(a, total, st);
+  if (rc != FS_OK) return rc;
+  const int items0 = a.side[0].nq, items1 = (nsides == 2) ? a.side[1].nq : 0;
+  hipLaunchKernelGGL((finish_kernel<false>), dim3(ceil_div(items0 + items1, 256)), dim3(256), 0, st,
+                     a, dp, items0, items1);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
+  const int dp = gemm_dp(d);
+  size_t planes = gemm_plane_bytes(n, dp) + gemm_plane_bytes(m, dp) + kPlaneAuxBytes;
+  auto part = [&](int64_t nq, int64_t nk, int total_ig) {
+    const GemmPlan p = gemm_plan(nq, nk, total_ig);
+    return (size_t)2 * p.bsplits * (size_t)nq * 2 * sizeof(float) + 16;
+  };
+  const int ig_n = ceil_div(n, kGemmTile), ig_m = ceil_div(m, kGemmTile);
+  if (both) return planes + part(n, m, ig_n + ig_m) + part(m, n, ig_n + ig_m) + 64;
+  if (either) return planes + std::max(part(n, m, ig_n), part(m, n, ig_m)) + 64;
+  return planes + part(n, m, ig_n) + 64;
+}
+
 // Plans, carves the workspace, launches the streaming kernel over one or two
 // sides and, when keys were split, the merge kernel.
 int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes,
@@ -145,6 +262,10 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
   const Family fam = family_for(d);
   const int dp = fam.dp;
+  static const int use_gemm = env_int("FS_LSEGEMM", 1);
+  if (mode == kLse && fam.sliced && use_gemm &&
+      !(flags & (FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS)))
+    return run_lse_gemm(sides, nsides, d, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -262,7 +383,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
         rc = launch_split_planes_f16(
             plane_src[i], reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
             plane_rows[i], (int)d, dp2, partial + 256 * i, scales + i,
-            two ? nullptr : scales + 1, st);
+            two ? nullptr : scales + 1, 0, st);
     } else {
       for (int i = 0; i < nplanes && rc == FS_OK; ++i)
         rc = launch_split_planes(plane_src[i],
@@ -381,9 +502,10 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   if (mode == kLse && !fam.sliced)
     planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
-  if (both) return a + b - planes + 64;
-  if (either) return std::max(a, b) + 64;
-  return a + 64;
+  const size_t gemm = (mode == kLse && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
+  if (both) return std::max(a + b - planes + 64, gemm);
+  if (either) return std::max(std::max(a, b) + 64, gemm);
+  return std::max(a + 64, gemm);
 }
 
 int fs_lse(const float* x, const float* y, const float* bias, float* out, int64_t n, int64_t m,

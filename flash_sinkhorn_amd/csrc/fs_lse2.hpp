@@ -41,12 +41,6 @@ enum Prec : int { kF32 = 0, kBf3 = 1, kBf6 = 2, kH3 = 3 };
 constexpr int kPlanePadRows = 256;  // zero rows after the last row of a plane buffer
 constexpr int kAbsmaxBlocks = 256;  // partial maxima per matrix written by absmax_kernel
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ unsigned pack_bf16(float a, float b) {
   f32x2 v = {a, b};
@@ -135,12 +129,12 @@ __device__ __forceinline__ unsigned pack_f16(float a, float b) {
 
 // x[rows, d] (fp32) -> two packed fp16 planes [rows + kPlanePadRows][2][DP/2] of scale*x, zero
 // padded to DP columns and in the trailing rows.  scale is derived from the partial maxima of
-// absmax_kernel; block 0 also
-// publishes it in *scale_out for the consuming kernel.
+// absmax_kernel; block 0 also publishes it in *scale_out for the consuming kernel.  With
+// `chunked` the two planes are interleaved per 32 columns (layout of lse_gemm_kernel).
 __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     const float* __restrict__ src, unsigned* __restrict__ dst, int rows, int d, int dp,
     const float* __restrict__ partial_max, float* __restrict__ scale_out,
-    float* __restrict__ scale_out2) {
+    float* __restrict__ scale_out2, int chunked) {
   __shared__ float red[4];
   float m = partial_max[threadIdx.x];  // kAbsmaxBlocks == blockDim.x
 #pragma unroll
@@ -167,8 +161,15 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
   const unsigned l01 = pack_f16(v[0] - (float)a[0], v[1] - (float)a[1]);
   const unsigned l23 = pack_f16(v[2] - (float)b[0], v[3] - (float)b[1]);
   unsigned* o = dst + (size_t)r * (size_t)dp;  // two planes of dp/2 words
-  *reinterpret_cast<uint2*>(o + c4 / 2) = make_uint2(h01, h23);
-  *reinterpret_cast<uint2*>(o + dp / 2 + c4 / 2) = make_uint2(l01, l23);
+  if (chunked) {
+    // per 32 columns: 16 words of the hi plane, then 16 words of the lo plane (dp % 32 == 0)
+    unsigned* oc = o + (c4 / 32) * 32 + (c4 % 32) / 2;
+    *reinterpret_cast<uint2*>(oc) = make_uint2(h01, h23);
+    *reinterpret_cast<uint2*>(oc + 16) = make_uint2(l01, l23);
+  } else {
+    *reinterpret_cast<uint2*>(o + c4 / 2) = make_uint2(h01, h23);
+    *reinterpret_cast<uint2*>(o + dp / 2 + c4 / 2) = make_uint2(l01, l23);
+  }
 }
 
 template <int DP, int PREC>

@@ -1,0 +1,203 @@
+// Log-sum-exp kernel for large feature dimension (128 < d <= 1536) on fp16 planes.
+//
+// With d in the hundreds a block of query rows no longer fits in registers, so the sweep is
+// organised like a GEMM: a workgroup of 8 wavefronts owns 256 query rows, walks its key
+// chunk in tiles of 256 keys and, per tile, runs a k-loop over the feature axis in chunks of
+// 32 columns.  Each k-step brings the 32-column slice of the 256 query rows and of the 256
+// key rows into LDS (128 bytes per row: 16 words of the hi plane, 16 of the lo plane, which
+// the chunked plane layout stores contiguously) with direct global->LDS loads, double
+// buffered, one barrier per k-step.  Wavefront (qg, kg) accumulates the logits of query rows
+// [64 qg, 64 qg + 64) against keys [128 kg, 128 kg + 128) of the tile: 2 x 4 MFMA tiles of
+// 32 keys x 32 queries = 128 accumulator registers, three fp16 products per tile and
+// 16 columns.  After the k-loop the bias / running-max fold and the lane-private online
+// soft-max run once per tile, which is noise next to 3*d/16 MFMAs per tile.  The two key
+// groups of a workgroup write separate partial statistics, so the merge kernel sees twice
+// the workgroup-level split count.
+//
+// LDS rows are 128 bytes with no padding (a direct load deposits 64 lanes x 16 bytes
+// contiguously); 16-byte piece p of local row r sits in slot p ^ ((r >> 1) & 7), which
+// makes the ds_read_b128 of 16 consecutive rows at one piece index conflict free.
+#pragma once
+
+#include "fs_common.hpp"
+#include "fs_stream.hpp"
+
+namespace fs {
+
+constexpr int kGemmRows = 256;   // query rows per workgroup = keys per tile
+constexpr int kGemmCols = 32;    // feature columns per k-step
+
+__global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args) {
+  __shared__ __attribute__((aligned(16))) unsigned lds[2][2 * kGemmRows * 32];
+
+  int bid = blockIdx.x;
+  const bool second = bid >= args.blocks0;
+  if (second) bid -= args.blocks0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const int dp = (args.d + kGemmCols - 1) / kGemmCols * kGemmCols;  // words per plane row pair
+  const int nch = dp / kGemmCols;
+
+  const int bsplits = sd.splits >> 1;  // workgroup-level key splits
+  const int split = bid % bsplits;
+  const int ig = bid / bsplits;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int h = lane >> 5;
+  const int qg = wave & 3;
+  const int kg = wave >> 2;
+  const int row0 = ig * kGemmRows;
+  const int j_begin = split * sd.chunk;
+  const int j_end = min(sd.nk, j_begin + sd.chunk);
+  const int ntiles = (j_end - j_begin + kGemmRows - 1) / kGemmRows;
+
+  const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  const float inv_lscale = 1.0f / lscale;
+
+  // ---- loader role: wavefronts 0-3 bring query rows, 4-7 key rows (64 rows each) ----
+  // instruction i of a k-step covers local rows 8 i .. 8 i + 7 of this wavefront's 64
+  const bool load_q = wave < 4;
+  int loff[8];  // word offset of this lane's 16-byte piece inside the wavefront's row block
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int lr = i * 8 + (lane >> 3);                 // row inside the 64-row block
+    const int piece = (lane & 7) ^ ((lr >> 1) & 7);     // (64 w) >> 1 has no low bits
+    loff[i] = lr * dp + piece * 4;
+  }
+  const unsigned* qbase = sd.qplanes + (size_t)(row0 + (wave & 3) * 64) * (size_t)dp;
+  auto issue_loads = [&](int buf, int j0, int c) {
+    const unsigned* base =
+        load_q ? qbase : sd.kplanes + (size_t)(j0 + (wave & 3) * 64) * (size_t)dp;
+    unsigned* dst = &lds[buf][(wave * 64) * 32];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(base + loff[i] + c * kGemmCols),
+          (__attribute__((address_space(3))) void*)(dst + i * 8 * 32), 16, 0, 0);
+  };
+
+  // ---- reader addresses (words): piece p of local row r at r*32 + ((p ^ ((r>>1)&7)) * 4) ----
+  auto lds_piece = [&](const unsigned* stage, int r, int p) {
+    return *reinterpret_cast<const u32x4*>(stage + r * 32 + ((p ^ ((r >> 1) & 7)) << 2));
+  };
+
+  f32x16 acc[2][4];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[qb][st][r] = 0.f;
+  float run_m[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f};
+
+  auto swap_halves = [&](float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  };
+
+  issue_loads(0, j_begin, 0);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+
+  int buf = 0;
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = j_begin + t * kGemmRows;
+    for (int c = 0; c < nch; ++c) {
+      // next k-step (or the first one of the next tile) goes into the other buffer
+      const bool wrap = (c + 1 == nch);
+      if (!wrap || t + 1 < ntiles) issue_loads(buf ^ 1, wrap ? j0 + kGemmRows : j0, wrap ? 0 : c + 1);
+
+      const unsigned* stage = lds[buf];
+      u32x4 qreg[2][2][2];  // [query block][plane][16-column half]
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+            qreg[qb][p][kk] = lds_piece(stage, qg * 64 + qb * 32 + li, p * 4 + kk * 2 + h);
+#pragma unroll
+      for (int sp = 0; sp < 2; ++sp) {
+        u32x4 kreg[2][2][2];  // [sub-tile of the pair][plane][half]
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+              kreg[s2][p][kk] = lds_piece(stage, kGemmRows + kg * 128 + (sp * 2 + s2) * 32 + li,
+                                          p * 4 + kk * 2 + h);
+        // products lo*hi, hi*lo, hi*hi; four independent accumulators between dependent MFMAs
+#pragma unroll
+        for (int prod = 0; prod < 3; ++prod)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+              for (int qb = 0; qb < 2; ++qb) {
+                const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
+                acc[qb][sp * 2 + s2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                    __builtin_bit_cast(f16x8, kreg[s2][pk][kk]),
+                    __builtin_bit_cast(f16x8, qreg[qb][pq][kk]), acc[qb][sp * 2 + s2], 0, 0, 0);
+              }
+      }
+      __builtin_amdgcn_s_waitcnt(0);  // this wavefront's direct loads have landed
+      __syncthreads();
+      buf ^= 1;
+    }
+
+    // ---- tile done: fold bias - M, lane-private online soft-max over the 4 sub-tiles ----
+    float ab[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+      ab[st] = h ? 1.0f : key_bias(sd, j0 + kg * 128 + st * 32 + li, j_end) * inv_lscale;
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const float negm = h ? -run_m[qb] : 1.0f;
+      float m = -3.0e38f;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        acc[qb][st] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[st], negm, acc[qb][st], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) m = fmaxf(m, acc[qb][st][r]);
+      }
+      float a = m, b = m;
+      swap_halves(a, b);
+      m = fmaxf(a, b);
+      const bool first = (t == 0);
+      const float delta = first ? m : fmaxf(m, 0.f);
+      const float m_new = run_m[qb] + delta;
+      const float cc = -(m_new - run_m[qb]) * lscale;
+      float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          ps0 += fast_exp2(__builtin_fmaf(acc[qb][st][r], lscale, cc));
+          ps1 += fast_exp2(__builtin_fmaf(acc[qb][st][r + 1], lscale, cc));
+        }
+      run_s[qb] = (first ? 0.f : run_s[qb] * fast_exp2(cc)) + (ps0 + ps1);
+      run_m[qb] = m_new;
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[qb][st][r] = 0.f;
+    }
+  }
+
+  // ---- partial statistics of this (query group, key group) ----
+  const bool has_keys = (j_begin + kg * 128) < j_end;  // else every key this wave saw was masked
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int row = row0 + qg * 64 + qb * 32 + li;
+    const float s = run_s[qb] + xor32(run_s[qb]);
+    if (row < sd.nq && h == 0) {
+      const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;
+      *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =
+          has_keys ? make_float2(run_m[qb] * lscale, s) : make_float2(kNegBig, 0.f);
+    }
+  }
+}
+
+}  // namespace fs
