@@ -20,6 +20,7 @@ FS_FLAG_EXP2 = 1
 FS_FLAG_REDUCED_OPERANDS = 2
 FS_FLAG_FP32_MFMA = 4
 FS_FLAG_BF16X3_OPERANDS = 8
+FS_FLAG_OPERANDS_PREPARED = 16
 # allow_tf32=False normally runs the two-plane fp16 operands (fp32-grade accuracy).
 # STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" runs fp32 MFMA
 # operands, "bf16x3" the three-plane bf16 split instead.
@@ -39,6 +40,7 @@ _SIGNATURES = {
     "fs_version": (ctypes.c_int, []),
     "fs_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "fs_workspace_bytes": (_Z, [ctypes.c_int, _I, _I, _I]),
+    "fs_prepare_operands": (ctypes.c_int, [_P] * 2 + [_I] * 3 + _TAIL),
     "fs_lse": (ctypes.c_int, [_P] * 4 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_lse_fused": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_symmetric_step": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + _TAIL),
@@ -110,3 +112,42 @@ def flags(use_exp2: bool, allow_tf32: bool) -> int:
 
 
 _STRICT_FLAGS = {"fp16x2": 0, "fp32_mfma": FS_FLAG_FP32_MFMA, "bf16x3": FS_FLAG_BF16X3_OPERANDS}
+
+
+class PreparedOperands:
+    """16-bit operand planes of (x, y), written once into a workspace that every LSE call
+    of a solver loop then shares (``fs_prepare_operands`` + ``FS_FLAG_OPERANDS_PREPARED``).
+
+    x and y must stay alive and unchanged while the object is in use, and the calls must
+    run on the stream current at construction.
+    """
+
+    def __init__(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int):
+        n, d = x.shape
+        m = y.shape[0]
+        L = lib()
+        nbytes = max(int(L.fs_workspace_bytes(op, n, m, d))
+                     for op in (OP_LSE, OP_SYMMETRIC_STEP))
+        self.ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+        self.nbytes = nbytes
+        self.flag_bits = flag_bits
+        self.keys = {(x.data_ptr(), n), (y.data_ptr(), m)}
+        self.d = d
+        check(L.fs_prepare_operands(x.data_ptr(), y.data_ptr(), n, m, d, flag_bits,
+                                    self.ws.data_ptr(), nbytes, stream_of(x)),
+              "fs_prepare_operands")
+
+    def serves(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int) -> bool:
+        return (flag_bits == self.flag_bits and x.shape[1] == self.d
+                and (x.data_ptr(), x.shape[0]) in self.keys
+                and (y.data_ptr(), y.shape[0]) in self.keys)
+
+
+def lse_workspace(op: int, x: torch.Tensor, y: torch.Tensor, flag_bits: int,
+                  prepared: Optional[PreparedOperands]):
+    """(workspace pointer, bytes, flags, keep-alive) for an LSE-type call."""
+    if prepared is not None and prepared.serves(x, y, flag_bits):
+        return (prepared.ws.data_ptr(), prepared.nbytes,
+                flag_bits | FS_FLAG_OPERANDS_PREPARED, prepared.ws)
+    ws = workspace(op, x.shape[0], y.shape[0], x.shape[1], x.device)
+    return ptr(ws), 0 if ws is None else ws.numel(), flag_bits, ws

@@ -139,6 +139,133 @@ int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
 }
 
 
+// ---- 16-bit operand planes of the LSE kernels ----
+// The workspace of an LSE operation starts with the planes of its distinct operand matrices in
+// canonical order (ascending address), then the absmax partials and plane scales.  The layout
+// depends only on (matrices, d, precision), never on which matrix is the stationary one, so
+// planes written once by fs_prepare_operands serve every later step on the same operands.
+struct LseConfig {
+  bool gemm;    // lse_gemm_kernel (128 < d <= 1536, fp16 planes)
+  int prec;     // Prec of lse2_kernel: 0 fp32, 1 two bf16, 2 three bf16, 3 two fp16 planes
+  int dp;       // padded columns of a plane row
+  int np;       // planes per operand
+};
+
+int strict_prec_default() {
+  static const int v = env_int("FS_STRICT_PREC", 3);  // 3: two fp16 planes, 2: three bf16 planes, 0: fp32 MFMA
+  return v;
+}
+int reduced_prec_default() {
+  static const int v = env_int("FS_REDUCED_PREC", 1);  // 1: two bf16 planes, 0: fp32 MFMA
+  return v;
+}
+
+LseConfig lse_config(int64_t d, uint32_t flags) {
+  static const int use_gemm = env_int("FS_LSEGEMM", 1);
+  LseConfig c;
+  c.prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec_default()
+           : ((flags & FS_FLAG_FP32_MFMA) ? 0
+              : ((flags & FS_FLAG_BF16X3_OPERANDS) ? 2 : strict_prec_default()));
+  const bool sliced = d > kMaxStreamD;
+  c.gemm = sliced && use_gemm && !(flags & (FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS));
+  if (c.gemm) {
+    c.prec = 3;
+    c.dp = ceil_div(d, 32) * 32;
+    c.np = 2;
+  } else {
+    c.dp = std::max(padded_d(d), 16);
+    c.np = (c.prec == 2) ? 3 : 2;
+    if (sliced) c.prec = 0;  // column-sliced fp32 kernels: no planes
+  }
+  return c;
+}
+
+struct PlaneSet {
+  int n;  // distinct matrices, 0 when the configuration uses no planes
+  const float* src[2];
+  int rows[2];
+  size_t off[2];
+  size_t aux_off, end;
+};
+
+size_t plane_bytes(int64_t rows, const LseConfig& c) {
+  return (((size_t)(rows + kPlanePadRowsApi) * (size_t)c.np * (size_t)(c.dp / 2) * 4) + 15) & ~(size_t)15;
+}
+
+// Distinct (pointer, rows) operands among up to four candidates, in canonical order.
+int make_plane_set(const float* const* ptrs, const int* rows, int count, const LseConfig& c,
+                   PlaneSet& ps) {
+  ps.n = 0;
+  ps.aux_off = ps.end = 0;
+  if (c.prec == 0) return FS_OK;
+  for (int k = 0; k < count; ++k) {
+    bool seen = false;
+    for (int i = 0; i < ps.n; ++i) seen = seen || (ps.src[i] == ptrs[k] && ps.rows[i] == rows[k]);
+    if (seen) continue;
+    if (ps.n == 2) return FS_ERR_BAD_ARGUMENT;
+    ps.src[ps.n] = ptrs[k];
+    ps.rows[ps.n] = rows[k];
+    ++ps.n;
+  }
+  if (ps.n == 2 && (ps.src[1] < ps.src[0] || (ps.src[1] == ps.src[0] && ps.rows[1] < ps.rows[0]))) {
+    std::swap(ps.src[0], ps.src[1]);
+    std::swap(ps.rows[0], ps.rows[1]);
+  }
+  size_t need = 0;
+  for (int i = 0; i < ps.n; ++i) {
+    ps.off[i] = need;
+    need += plane_bytes(ps.rows[i], c);
+  }
+  ps.aux_off = need;
+  ps.end = need + kPlaneAuxBytes;
+  return FS_OK;
+}
+
+const float* plane_scales(const PlaneSet& ps, void* ws) {
+  return reinterpret_cast<const float*>(static_cast<char*>(ws) + ps.aux_off) + 2 * 256;
+}
+
+const unsigned* plane_of(const PlaneSet& ps, void* ws, const float* src, int rows) {
+  for (int i = 0; i < ps.n; ++i)
+    if (ps.src[i] == src && ps.rows[i] == rows)
+      return reinterpret_cast<const unsigned*>(static_cast<char*>(ws) + ps.off[i]);
+  return nullptr;
+}
+
+// Writes the planes (and, for fp16, the scales) of every matrix of the set.
+int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws, hipStream_t st) {
+  if (ps.n == 0) return FS_OK;
+  char* base = static_cast<char*>(ws);
+  int rc = FS_OK;
+  if (c.prec == 3) {
+    float* partial = reinterpret_cast<float*>(base + ps.aux_off);
+    float* scales = partial + 2 * 256;
+    const bool two = ps.n > 1;
+    rc = launch_absmax(ps.src[0], (long long)ps.rows[0] * d, two ? ps.src[1] : ps.src[0],
+                       two ? (long long)ps.rows[1] * d : 0, partial, st);
+    for (int i = 0; i < ps.n && rc == FS_OK; ++i)
+      rc = launch_split_planes_f16(ps.src[i], reinterpret_cast<unsigned*>(base + ps.off[i]),
+                                   ps.rows[i], (int)d, c.dp, partial + 256 * i, scales + i,
+                                   two ? nullptr : scales + 1, c.gemm ? 1 : 0, st);
+  } else {
+    for (int i = 0; i < ps.n && rc == FS_OK; ++i)
+      rc = launch_split_planes(ps.src[i], reinterpret_cast<unsigned*>(base + ps.off[i]),
+                               ps.rows[i], (int)d, c.dp, c.np, st);
+  }
+  return rc;
+}
+
+int side_plane_set(const Side* sides, int nsides, const LseConfig& c, PlaneSet& ps) {
+  const float* ptrs[4];
+  int rows[4];
+  int cnt = 0;
+  for (int s = 0; s < nsides; ++s) {
+    ptrs[cnt] = sides[s].q; rows[cnt++] = sides[s].nq;
+    ptrs[cnt] = sides[s].k; rows[cnt++] = sides[s].nk;
+  }
+  return make_plane_set(ptrs, rows, cnt, c, ps);
+}
+
 // ---- large-d LSE on chunked fp16 planes (lse_gemm_kernel) ----
 constexpr int kGemmTile = 256;  // query rows per workgroup and keys per tile
 
@@ -156,38 +283,13 @@ GemmPlan gemm_plan(int64_t nq, int64_t nk, int total_igroups) {
   return p;
 }
 
-inline int gemm_dp(int64_t d) { return ceil_div(d, 32) * 32; }
-
-size_t gemm_plane_bytes(int64_t rows, int dp) {
-  return (((size_t)(rows + kPlanePadRowsApi) * (size_t)dp * 4) + 15) & ~(size_t)15;
-}
-
-// Workspace: planes of the distinct operand matrices, absmax partials and scales, then per
-// side 2*bsplits partial (M, s) rows.
-int run_lse_gemm(Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes, hipStream_t st) {
-  const int dp = gemm_dp(d);
-  const float* plane_src[2];
-  int plane_rows[2];
-  size_t plane_off[2];
-  int nplanes = 0;
-  size_t need = 0;
-  for (int s = 0; s < nsides; ++s) {
-    const float* ptrs[2] = {sides[s].q, sides[s].k};
-    const int rows[2] = {sides[s].nq, sides[s].nk};
-    for (int k = 0; k < 2; ++k) {
-      bool seen = false;
-      for (int i = 0; i < nplanes; ++i) seen = seen || (plane_src[i] == ptrs[k] && plane_rows[i] == rows[k]);
-      if (seen) continue;
-      if (nplanes == 2) return FS_ERR_BAD_ARGUMENT;
-      plane_src[nplanes] = ptrs[k];
-      plane_rows[nplanes] = rows[k];
-      plane_off[nplanes] = need;
-      need += gemm_plane_bytes(rows[k], dp);
-      ++nplanes;
-    }
-  }
-  const size_t aux_off = need;
-  need += kPlaneAuxBytes;
+// Workspace: plane region (see above), then per side 2*bsplits partial (M, s) rows.
+int run_lse_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared, void* ws,
+                 size_t ws_bytes, hipStream_t st) {
+  PlaneSet ps;
+  int rc = side_plane_set(sides, nsides, cfg, ps);
+  if (rc != FS_OK) return rc;
+  size_t need = ps.end;
   int total_ig = 0;
   for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kGemmTile);
   GemmPlan plans[2];
@@ -199,8 +301,6 @@ int run_lse_gemm(Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes, 
   }
   if (need > ws_bytes || ws == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
   char* base = static_cast<char*>(ws);
-  float* partial = reinterpret_cast<float*>(base + aux_off);
-  float* scales = partial + 2 * 256;
 
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
@@ -213,12 +313,9 @@ int run_lse_gemm(Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes, 
     sd.igroups = plans[s].igroups;
     sd.part_ms = reinterpret_cast<float*>(base + part_off[s]);
     sd.part_o = nullptr;
-    sd.plane_scale = scales;
-    for (int i = 0; i < nplanes; ++i) {
-      const unsigned* pb = reinterpret_cast<const unsigned*>(base + plane_off[i]);
-      if (plane_src[i] == sd.q && plane_rows[i] == sd.nq) sd.qplanes = pb;
-      if (plane_src[i] == sd.k && plane_rows[i] == sd.nk) sd.kplanes = pb;
-    }
+    sd.plane_scale = plane_scales(ps, ws);
+    sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
+    sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
     blocks[s] = plans[s].igroups * plans[s].bsplits;
     a.side[s] = sd;
   }
@@ -227,24 +324,19 @@ int run_lse_gemm(Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes, 
   const int total = blocks[0] + blocks[1];
   if (total <= 0) return FS_OK;
 
-  const bool two = nplanes > 1;
-  int rc = launch_absmax(plane_src[0], (long long)plane_rows[0] * d, two ? plane_src[1] : plane_src[0],
-                         two ? (long long)plane_rows[1] * d : 0, partial, st);
-  for (int i = 0; i < nplanes && rc == FS_OK; ++i)
-    rc = launch_split_planes_f16(plane_src[i], reinterpret_cast<unsigned*>(base + plane_off[i]),
-                                 plane_rows[i], (int)d, dp, partial + 256 * i, scales + i,
-                                 two ? nullptr : scales + 1, 1, st);
+  if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
   if (rc == FS_OK) rc = launch_lse_gemm(a, total, st);
   if (rc != FS_OK) return rc;
   const int items0 = a.side[0].nq, items1 = (nsides == 2) ? a.side[1].nq : 0;
   hipLaunchKernelGGL((finish_kernel<false>), dim3(ceil_div(items0 + items1, 256)), dim3(256), 0, st,
-                     a, dp, items0, items1);
+                     a, cfg.dp, items0, items1);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
 size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
-  const int dp = gemm_dp(d);
-  size_t planes = gemm_plane_bytes(n, dp) + gemm_plane_bytes(m, dp) + kPlaneAuxBytes;
+  LseConfig c;
+  c.gemm = true; c.prec = 3; c.dp = ceil_div(d, 32) * 32; c.np = 2;
+  size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
   auto part = [&](int64_t nq, int64_t nk, int total_ig) {
     const GemmPlan p = gemm_plan(nq, nk, total_ig);
     return (size_t)2 * p.bsplits * (size_t)nq * 2 * sizeof(float) + 16;
@@ -262,10 +354,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
   const Family fam = family_for(d);
   const int dp = fam.dp;
-  static const int use_gemm = env_int("FS_LSEGEMM", 1);
-  if (mode == kLse && fam.sliced && use_gemm &&
-      !(flags & (FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS)))
-    return run_lse_gemm(sides, nsides, d, ws, ws_bytes, st);
+  const LseConfig cfg = lse_config(d, flags);
+  const bool prepared = (flags & FS_FLAG_OPERANDS_PREPARED) != 0;
+  if (mode == kLse && cfg.gemm) return run_lse_gemm(sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -278,48 +369,22 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     rb = std::min(rb, plans[s].rb);
   }
   static const int use_v2 = env_int("FS_LSE2", 1);
-  static const int strict_prec = env_int("FS_STRICT_PREC", 3);    // 3: two fp16 planes, 2: three bf16 planes, 0: fp32 MFMA
-  static const int reduced_prec = env_int("FS_REDUCED_PREC", 1);  // 1: two bf16 planes, 0: fp32 MFMA
   static const int rb_override = env_int("FS_RB", 0);
   bool aligned = (d % 4 == 0);
   for (int s = 0; s < nsides; ++s) aligned = aligned && aligned16(sides[s].q) && aligned16(sides[s].k);
-  const int prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec
-                   : ((flags & FS_FLAG_FP32_MFMA) ? 0
-                      : ((flags & FS_FLAG_BF16X3_OPERANDS) ? 2 : strict_prec));
+  const int prec = cfg.prec;
   // pipelined LSE kernel: the 16-bit plane modes take any d <= 128, the fp32 mode needs aligned rows
   const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
-  const int dp2 = std::max(dp, 16);
-  const int np = (prec == 2) ? 3 : 2;
+  const int dp2 = cfg.dp;
   if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
   if (lse2 && prec == 2 && dp >= 64) rb = 1;  // three planes of 64 columns x two row blocks spill
-  // distinct operand matrices that need 16-bit planes (x and y, whichever roles they play)
-  const float* plane_src[4];
-  int plane_rows[4];
-  size_t plane_off[4];
-  int nplanes = 0;
+  PlaneSet ps;
+  ps.n = 0;
+  ps.end = 0;
   if (lse2 && prec != 0) {
-    for (int s = 0; s < nsides; ++s) {
-      const float* ptrs[2] = {sides[s].q, sides[s].k};
-      const int rows[2] = {sides[s].nq, sides[s].nk};
-      for (int k = 0; k < 2; ++k) {
-        bool seen = false;
-        for (int i = 0; i < nplanes; ++i) seen = seen || (plane_src[i] == ptrs[k] && plane_rows[i] == rows[k]);
-        if (!seen) {
-          plane_src[nplanes] = ptrs[k];
-          plane_rows[nplanes] = rows[k];
-          plane_off[nplanes] = need;
-          need += (((size_t)(rows[k] + kPlanePadRowsApi) * np * (dp2 / 2) * 4) + 15) & ~(size_t)15;
-          ++nplanes;
-        }
-      }
-    }
-  }
-  // fp16 planes: partial maxima [2][256] and the two power-of-two scales
-  size_t aux_off = 0;
-  if (lse2 && prec == 3) {
-    if (nplanes > 2) return FS_ERR_BAD_ARGUMENT;
-    aux_off = need;
-    need += kPlaneAuxBytes;
+    const int prc = side_plane_set(sides, nsides, cfg, ps);
+    if (prc != FS_OK) return prc;
+    need = ps.end;
   }
   const size_t need_planes_end = need;
   for (int s = 0; s < nsides; ++s) {
@@ -353,13 +418,11 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     if (sd.q2) vec_ok = vec_ok && aligned16(sd.q2);
     if (mode == kMat && sd.v) vec_ok = vec_ok && aligned16(sd.v);
     blocks[s] = p.igroups * p.splits;
-    for (int i = 0; i < nplanes; ++i) {
-      const unsigned* base = reinterpret_cast<const unsigned*>(static_cast<char*>(ws) + plane_off[i]);
-      if (plane_src[i] == sd.q && plane_rows[i] == sd.nq) sd.qplanes = base;
-      if (plane_src[i] == sd.k && plane_rows[i] == sd.nk) sd.kplanes = base;
+    if (ps.n > 0) {
+      sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
+      sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
+      sd.plane_scale = plane_scales(ps, ws);
     }
-    if (lse2 && prec == 3)
-      sd.plane_scale = reinterpret_cast<const float*>(static_cast<char*>(ws) + aux_off) + 2 * 256;
     a.side[s] = sd;
   }
   if (nsides == 1) a.side[1] = a.side[0];
@@ -372,24 +435,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (fam.sliced) {
     rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
   } else if (lse2) {
-    rc = FS_OK;
-    if (prec == 3) {
-      float* partial = reinterpret_cast<float*>(static_cast<char*>(ws) + aux_off);
-      float* scales = partial + 2 * 256;
-      const bool two = nplanes > 1;
-      rc = launch_absmax(plane_src[0], (long long)plane_rows[0] * d, two ? plane_src[1] : plane_src[0],
-                         two ? (long long)plane_rows[1] * d : 0, partial, st);
-      for (int i = 0; i < nplanes && rc == FS_OK; ++i)
-        rc = launch_split_planes_f16(
-            plane_src[i], reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
-            plane_rows[i], (int)d, dp2, partial + 256 * i, scales + i,
-            two ? nullptr : scales + 1, 0, st);
-    } else {
-      for (int i = 0; i < nplanes && rc == FS_OK; ++i)
-        rc = launch_split_planes(plane_src[i],
-                                 reinterpret_cast<unsigned*>(static_cast<char*>(ws) + plane_off[i]),
-                                 plane_rows[i], (int)d, dp2, np, st);
-    }
+    rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
     if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, total, st);
   } else
   switch (mode) {
@@ -506,6 +552,21 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);
   return std::max(a + 64, gemm);
+}
+
+int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
+                        uint32_t flags, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !y) return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
+  const LseConfig cfg = lse_config(d, flags);
+  const float* ptrs[2] = {x, y};
+  const int rows[2] = {(int)n, (int)m};
+  PlaneSet ps;
+  const int rc = make_plane_set(ptrs, rows, 2, cfg, ps);
+  if (rc != FS_OK || ps.n == 0) return rc;
+  if (ps.end > workspace_bytes || workspace == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
+  return launch_plane_set(ps, cfg, d, workspace, (hipStream_t)stream);
 }
 
 int fs_lse(const float* x, const float* y, const float* bias, float* out, int64_t n, int64_t m,

@@ -59,7 +59,7 @@ def flashsinkhorn_lse(
     cost_scale: float = 1.0, damping: float = 1.0, allow_tf32: bool = True,
     use_exp2: bool = True, block_m: Optional[int] = None, block_n: Optional[int] = None,
     block_k: Optional[int] = None, num_warps: Optional[int] = None, num_stages: int = 2,
-    autotune: bool = True,
+    autotune: bool = True, _prepared: Optional[_lib.PreparedOperands] = None,
 ) -> torch.Tensor:
     """out_i = -eps*damping*LSE_j[2*cost_scale*x_i.y_j/eps + bias_j]; returns fp32 [n]."""
     if not x.is_cuda or not y.is_cuda:
@@ -76,11 +76,11 @@ def flashsinkhorn_lse(
         raise ValueError(f"bias must have length {m}, got {bias.shape[0]}")
     x, y, bias = _f32c(x), _f32c(y), _f32c(bias)
     out = torch.empty((n,), device=x.device, dtype=torch.float32)
-    ws = _lib.workspace(_lib.OP_LSE, n, m, d, x.device)
+    wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_LSE, x, y, _lib.flags(use_exp2, allow_tf32),
+                                           _prepared)
     rc = _lib.lib().fs_lse(
         x.data_ptr(), y.data_ptr(), bias.data_ptr(), out.data_ptr(), n, m, d,
-        float(eps), 2.0 * float(cost_scale), float(damping), _lib.flags(use_exp2, allow_tf32),
-        _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_of(x))
+        float(eps), 2.0 * float(cost_scale), float(damping), fl, wp, wn, _lib.stream_of(x))
     _lib.check(rc, "fs_lse")
     return out
 
@@ -90,7 +90,7 @@ def flashsinkhorn_lse_fused(
     cost_scale: float = 1.0, damping: float = 1.0, allow_tf32: bool = True,
     use_exp2: bool = True, block_m: Optional[int] = None, block_n: Optional[int] = None,
     block_k: Optional[int] = None, num_warps: Optional[int] = None, num_stages: int = 2,
-    autotune: bool = True,
+    autotune: bool = True, _prepared: Optional[_lib.PreparedOperands] = None,
 ) -> torch.Tensor:
     """Same as flashsinkhorn_lse with bias_j = g_hat_j/eps + log_w_j formed in the kernel."""
     if not x.is_cuda or not y.is_cuda:
@@ -103,17 +103,18 @@ def flashsinkhorn_lse_fused(
         raise ValueError(f"g_hat and log_w must have length {m}")
     x, y, g_hat, log_w = _f32c(x), _f32c(y), _f32c(g_hat), _f32c(log_w)
     out = torch.empty((n,), device=x.device, dtype=torch.float32)
-    ws = _lib.workspace(_lib.OP_LSE, n, m, d, x.device)
+    wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_LSE, x, y, _lib.flags(use_exp2, allow_tf32),
+                                           _prepared)
     rc = _lib.lib().fs_lse_fused(
         x.data_ptr(), y.data_ptr(), g_hat.data_ptr(), log_w.data_ptr(), out.data_ptr(), n, m, d,
-        float(eps), 2.0 * float(cost_scale), float(damping), _lib.flags(use_exp2, allow_tf32),
-        _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_of(x))
+        float(eps), 2.0 * float(cost_scale), float(damping), fl, wp, wn, _lib.stream_of(x))
     _lib.check(rc, "fs_lse_fused")
     return out
 
 
 def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, alpha, damping_f,
-                        damping_g, shift_x=None, shift_y=None, allow_tf32=True, use_exp2=True):
+                        damping_g, shift_x=None, shift_y=None, allow_tf32=True, use_exp2=True,
+                        prepared=None):
     """One launch on already contiguous fp32 operands.  With shift_x/shift_y the
     unbalanced shift correction is applied inside the epilogue.  When every paired argument
     is the same tensor (the self problem OT(x, x)) the library computes the one distinct
@@ -124,13 +125,13 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
     self_problem = (y is x and g_hat is f_hat and log_b is log_a and shift_y is shift_x
                     and damping_f == damping_g)
     g_out = f_out if self_problem else torch.empty((m,), device=x.device, dtype=torch.float32)
-    ws = _lib.workspace(_lib.OP_SYMMETRIC_STEP, n, m, d, x.device)
+    wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_SYMMETRIC_STEP, x, y,
+                                           _lib.flags(use_exp2, allow_tf32), prepared)
     rc = _lib.lib().fs_symmetric_step(
         x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), f_out.data_ptr(), g_out.data_ptr(), _lib.ptr(shift_x),
         _lib.ptr(shift_y), n, m, d, float(eps), float(alpha), float(damping_f), float(damping_g),
-        2.0 * float(cost_scale), _lib.flags(use_exp2, allow_tf32), _lib.ptr(ws),
-        0 if ws is None else ws.numel(), _lib.stream_of(x))
+        2.0 * float(cost_scale), fl, wp, wn, _lib.stream_of(x))
     _lib.check(rc, "fs_symmetric_step")
     return f_out, g_out
 

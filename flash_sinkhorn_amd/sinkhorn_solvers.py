@@ -12,6 +12,7 @@ from typing import Optional, Sequence, Tuple
 
 import torch
 
+from flash_sinkhorn_amd import _lib
 from flash_sinkhorn_amd.kernels._common import (
     _f32c, dampening, epsilon_schedule, log_weights, max_diameter,
 )
@@ -82,7 +83,10 @@ def sinkhorn_flashstyle_alternating(
     log_a, log_b = log_weights(a), log_weights(b)
     f_hat, g_hat = -alpha, -beta
     prev_f, prev_g = (f_hat.clone(), g_hat.clone()) if threshold is not None else (None, None)
-    kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
+    # operand planes are converted once for the whole loop
+    prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32))
+    kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
+              _prepared=prepared)
 
     used = 0
     for it in range(int(n_iters)):
@@ -169,6 +173,9 @@ def sinkhorn_flashstyle_symmetric(
             and (a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape))):
         yf, beta, log_b, g_hat = xf, alpha, log_a, f_hat
 
+    # operand planes are converted once for the whole loop
+    prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32))
+
     def jacobi(f_hat, g_hat, e, w):
         damp_f, damp_g = dampening(e, rho_x), dampening(e, rho_y)
         if fused:
@@ -176,9 +183,10 @@ def sinkhorn_flashstyle_symmetric(
                 xf, yf, f_hat, g_hat, log_a, log_b, e, cost_scale=cost_scale, alpha=w,
                 damping_f=damp_f, damping_g=damp_g,
                 shift_x=alpha if damp_f < 1.0 else None, shift_y=beta if damp_g < 1.0 else None,
-                allow_tf32=allow_tf32, use_exp2=use_exp2)
+                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared)
         # two launches, raw-bias kernel, averaging and shift correction on the host
-        kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
+        kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
+                  _prepared=prepared)
         f_c = flashsinkhorn_lse(xf, yf, (g_hat + e * log_b) / e, e, damping=damp_f, **kw)
         g_c = flashsinkhorn_lse(yf, xf, (f_hat + e * log_a) / e, e, damping=damp_g, **kw)
         if damp_f < 1.0:

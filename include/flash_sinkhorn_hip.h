@@ -49,6 +49,7 @@ extern "C" {
 #define FS_FLAG_REDUCED_OPERANDS 2u
 #define FS_FLAG_FP32_MFMA 4u
 #define FS_FLAG_BF16X3_OPERANDS 8u
+#define FS_FLAG_OPERANDS_PREPARED 16u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0
@@ -63,6 +64,19 @@ const char* fs_error_string(int code);
 
 /* Bytes of device scratch the given operation needs for an (n, m, d) problem. */
 size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d);
+
+/*
+ * Optional: writes the 16-bit operand planes of x:[n,d] and y:[m,d] that the log-sum-exp
+ * kernels multiply (see the precision notes above) into the head of `workspace`.  A solver
+ * loop calls it once and then passes FS_FLAG_OPERANDS_PREPARED, the same workspace, the same
+ * x / y pointers (in either role) and the same precision flags to every fs_lse,
+ * fs_lse_fused and fs_symmetric_step of the loop, which then skip the conversion.  The
+ * workspace must be sized for the largest of those operations; without the flag every call
+ * converts its operands itself.  No counterpart in the reference: its Triton kernels read
+ * the fp32 operands directly (kernels/sinkhorn_flashstyle_sqeuclid.py:194-661).
+ */
+int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
+                        uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * out[i] = -eps*damping * LSE_j[ coord_scale * x_i.y_j / eps + bias[j] ]

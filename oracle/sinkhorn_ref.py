@@ -33,6 +33,7 @@ Pin status (what each function is checked against in tests/test_oracle_*.py):
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional, Sequence
 
 import numpy as np
@@ -122,10 +123,29 @@ def _lse_rows(vals):
         return safe + np.log(s)
 
 
+# Row chunks of the dense sweeps may run on a thread pool (numpy releases the GIL inside
+# matmul and exp); results do not depend on it.  Only the fixture writers raise it.
+THREADS = int(os.environ.get("ORACLE_THREADS", "1"))
+
+
 def _row_chunks(n: int, m: int, budget_elems: int = 32_000_000):
+    if THREADS > 1 and n * m > 4_000_000:
+        budget_elems = min(budget_elems, max(m, (n * m) // (2 * THREADS)))
     step = max(1, min(n, budget_elems // max(m, 1)))
     for i0 in range(0, n, step):
         yield i0, min(n, i0 + step)
+
+
+def _for_chunks(fn, n: int, m: int):
+    """fn(i0, i1) for every row chunk, in threads when THREADS > 1."""
+    chunks = list(_row_chunks(n, m))
+    if THREADS > 1 and len(chunks) > 1:
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(THREADS) as pool:
+            list(pool.map(lambda c: fn(*c), chunks))
+    else:
+        for c in chunks:
+            fn(*c)
 
 
 def softmin(x, y, pot_y, logw_y, eps, cost_scale=1.0, dtype=np.float64):
@@ -137,9 +157,12 @@ def softmin(x, y, pot_y, logw_y, eps, cost_scale=1.0, dtype=np.float64):
     logw_y = np.asarray(logw_y, dtype=dtype)
     eps = dtype(eps)
     out = np.empty(x.shape[0], dtype=dtype)
-    for i0, i1 in _row_chunks(x.shape[0], y.shape[0]):
+
+    def chunk(i0, i1):
         c = sqeuclid_cost(x[i0:i1], y, cost_scale, dtype)
         out[i0:i1] = -eps * _lse_rows((pot_y[None, :] - c) / eps + logw_y[None, :])
+
+    _for_chunks(chunk, x.shape[0], y.shape[0])
     return out
 
 
@@ -151,8 +174,11 @@ def lse_shifted(x, y, bias, eps, cost_scale=1.0, damping=1.0, dtype=np.float64):
     bias = np.asarray(bias, dtype=dtype)
     out = np.empty(x.shape[0], dtype=dtype)
     sc = dtype(2.0 * cost_scale / eps)
-    for i0, i1 in _row_chunks(x.shape[0], y.shape[0]):
+
+    def chunk(i0, i1):
         out[i0:i1] = _lse_rows((x[i0:i1] @ y.T) * sc + bias[None, :])
+
+    _for_chunks(chunk, x.shape[0], y.shape[0])
     return dtype(-eps * damping) * out
 
 

@@ -221,3 +221,30 @@ def test_self_problem_shortcut_equals_generic_path(kw):
     want = oracle.sinkhorn_symmetric(x, x, a, a, use_epsilon_scaling=False, eps=0.05, n_iters=20,
                                      **kw)
     assert rel_err(fs, want[0]) < RTOL and rel_err(gs, want[1]) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", [(700, 500, 64), (300, 260, 200)])
+def test_prepared_operands_give_identical_results(n, m, d):
+    """Planes written once by fs_prepare_operands serve the symmetric step and both roles of
+    the one-sided LSE; results are bit-identical to calls that convert their operands."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        _symmetric_step_raw, flashsinkhorn_lse_fused)
+    x, y, a, b = inputs(41, n, m, d, scale=2.0 / np.sqrt(d))
+    rng = np.random.default_rng(3)
+    fh = (rng.standard_normal(n) * 0.3).astype(np.float32)
+    gh = (rng.standard_normal(m) * 0.3).astype(np.float32)
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, np.log(a), np.log(b))
+    prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    f0, g0 = _symmetric_step_raw(X, Y, F, G, LA, LB, 0.2, **kw)
+    f1, g1 = _symmetric_step_raw(X, Y, F, G, LA, LB, 0.2, prepared=prep, **kw)
+    assert torch.equal(f0, f1) and torch.equal(g0, g1)
+    for q, k, pot, lw in ((X, Y, G, LB), (Y, X, F, LA)):
+        o0 = flashsinkhorn_lse_fused(q, k, pot, lw, 0.2, allow_tf32=False)
+        o1 = flashsinkhorn_lse_fused(q, k, pot, lw, 0.2, allow_tf32=False, _prepared=prep)
+        assert torch.equal(o0, o1)
+    # a different precision request does not match the prepared planes: falls back to converting
+    o2 = flashsinkhorn_lse_fused(X, Y, G, LB, 0.2, allow_tf32=True, _prepared=prep)
+    want = oracle.lse_shifted_fused(x, y, gh, np.log(b), 0.2)
+    assert rel_err(o2, want) < 1e-3
