@@ -31,6 +31,8 @@
 //          fp32 from exact products, at the MFMA cost of kBf3.
 #pragma once
 
+#include <type_traits>
+
 #include "fs_common.hpp"
 #include "fs_stream.hpp"
 
@@ -206,9 +208,17 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // Key-register prefetch (A operands of the next 32-key sub-tile are read from LDS while the
   // current one is multiplied) and the early LDS store it needs; off where registers are short.
   constexpr bool KPF = (NSUB == 2) && !(PREC == kBf6 && RB == 2);
+  // Two-plane modes bring key tiles into LDS with direct global->LDS loads (no staging
+  // registers, no ds_write): rows are unpadded and 16-byte piece p of row r sits in slot
+  // p ^ swz(r), which keeps the b128 reads of 16 consecutive rows conflict free.  With the
+  // key-register prefetch the tile two ahead is in flight, hence three buffers.
+  constexpr bool DIRECT = kBf && NP == 2;
+  constexpr int NBUF = (DIRECT && KPF) ? 3 : 2;
+  constexpr int LDWK = DIRECT ? ROWW : G::LDW;  // LDS row stride in words
+  constexpr int PPR = ROWW / 4;                 // 16-byte pieces per row
 
-  __shared__ __attribute__((aligned(16))) unsigned lds_k[2][G::JT * G::LDW];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][256];  // [buf][thread]; first JT used
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][G::JT * LDWK];
+  __shared__ __attribute__((aligned(16))) float lds_b[NBUF][256];  // [buf][thread]; first JT used
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;
@@ -275,7 +285,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int C16_PER_ROW = ROWW / 4;  // 16-byte chunks per operand row
   constexpr int C16_TOTAL = G::JT * C16_PER_ROW;
   constexpr int PER_THREAD = (C16_TOTAL + 255) / 256;
-  u32x4 st_k[PER_THREAD];
+  u32x4 st_k[DIRECT ? 1 : PER_THREAD];
   float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f, st_pen = 0.f;
   const unsigned* krows = kBf ? sd.kplanes : reinterpret_cast<const unsigned*>(sd.k);
   const int krow_words = kBf ? ROWW : d;
@@ -284,19 +294,30 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // Plane buffers end with kPlanePadRows zero rows, so the 16-bit modes walk them with plain
   // running pointers (tiles up to two past the chunk are fetched and masked by the bias);
   // the fp32 mode reads the caller's matrix and clamps the row instead.
+  auto swz = [&](int r) {  // slot permutation of LDS row r (direct mode)
+    return PPR >= 16 ? (r & 15) : (PPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3));
+  };
   const unsigned* kp[PER_THREAD];
 #pragma unroll
   for (int c = 0; c < PER_THREAD; ++c) {
     const int idx = tid + 256 * c;
-    kp[c] = krows + (size_t)(j_begin + idx / C16_PER_ROW) * (size_t)krow_words +
-            (idx % C16_PER_ROW) * 4;
+    const int r = idx / C16_PER_ROW;
+    int piece = idx % C16_PER_ROW;
+    if constexpr (DIRECT) piece ^= swz(r);  // lane idx fills LDS slot idx; it fetches this piece
+    kp[c] = krows + (size_t)(j_begin + r) * (size_t)krow_words + piece * 4;
   }
   // No branches anywhere in the main loop: a branch would split the basic block and let the
   // compiler sink the soft-max pieces out from between the MFMAs.
-  auto stage_load = [&](int j0) {
+  auto stage_load = [&](int j0, int dbuf) {  // dbuf: LDS buffer of the direct loads
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
-      if constexpr (kBf) {
+      if constexpr (DIRECT) {
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)kp[c],
+            (__attribute__((address_space(3))) void*)(&lds_k[dbuf][(c * 256 + wave * 64) * 4]),
+            16, 0, 0);
+        kp[c] += G::JT * ROWW;
+      } else if constexpr (kBf) {
         st_k[c] = *reinterpret_cast<const u32x4*>(kp[c]);
         kp[c] += G::JT * ROWW;
       } else {
@@ -320,13 +341,15 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     }
   };
   auto stage_store = [&](int buf) {
+    if constexpr (!DIRECT) {
 #pragma unroll
-    for (int c = 0; c < PER_THREAD; ++c) {
-      const int idx = tid + 256 * c;
-      if (C16_TOTAL % 256 == 0 || idx < C16_TOTAL) {
-        const int r = idx / C16_PER_ROW;
-        const int c4 = (idx % C16_PER_ROW) * 4;
-        *reinterpret_cast<u32x4*>(&lds_k[buf][r * G::LDW + c4]) = st_k[c];
+      for (int c = 0; c < PER_THREAD; ++c) {
+        const int idx = tid + 256 * c;
+        if (C16_TOTAL % 256 == 0 || idx < C16_TOTAL) {
+          const int r = idx / C16_PER_ROW;
+          const int c4 = (idx % C16_PER_ROW) * 4;
+          *reinterpret_cast<u32x4*>(&lds_k[buf][r * LDWK + c4]) = st_k[c];
+        }
       }
     }
     // masked rows get a penalty ADDED (not selected), so the loads stay unconditional
@@ -431,7 +454,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     float ab;
   };
   auto load_keys = [&](KeyRegs& kr, int buf, int js) {
-    const unsigned* yrow = lds_k[buf] + (js * 32 + li) * G::LDW;
+    const unsigned* yrow = lds_k[buf] + (js * 32 + li) * LDWK;
     if constexpr (!kBf) {
 #pragma unroll
       for (int q = 0; q < DP / 8; ++q) {
@@ -445,8 +468,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 #pragma unroll
       for (int p = 0; p < NP; ++p)
 #pragma unroll
-        for (int kk = 0; kk < G::KK16; ++kk)
-          kr.yq[p][kk] = *reinterpret_cast<const u32x4*>(yrow + p * (DP / 2) + 8 * kk + 4 * h);
+        for (int kk = 0; kk < G::KK16; ++kk) {
+          const int piece = p * (DP / 8) + 2 * kk + h;
+          const int slot = DIRECT ? (piece ^ swz(li)) : piece;  // swz(js*32 + li) == swz(li)
+          kr.yq[p][kk] = *reinterpret_cast<const u32x4*>(yrow + slot * 4);
+        }
     }
     const float b = lds_b[buf][js * 32 + li];
     kr.ab = h ? 1.0f : b;
@@ -493,33 +519,56 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 
   KeyRegs K[KPF ? 2 : 1];
 
-  // ---- prologue: tile 0 into LDS buffer 0; with KPF tile 1 is already on its way ----
-  stage_load(j_begin);
+  // Wait until at most `newer` of this wavefront's vector-memory operations are outstanding
+  // (the direct loads write LDS behind the compiler's back, so their waits are explicit).
+  auto wait_vm = [&](auto newer) {
+    constexpr int n = decltype(newer)::value;
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (n & 15) | ((n >> 4) << 14));
+  };
+  constexpr int kLoadsPerTile = (DIRECT ? PER_THREAD : 0) + 3;  // direct loads + bias terms
+  auto wait_all_vm = [&]() { wait_vm(std::integral_constant<int, 0>{}); };
+  auto wait_older_tiles = [&]() { wait_vm(std::integral_constant<int, kLoadsPerTile>{}); };
+
+  // LDS buffers rotate: cur holds the tile being multiplied, nxt the next one, nx2 (direct
+  // mode with three buffers) the one after that; with two buffers nx2 is cur.
+  int cur = 0, nxt = 1 % NBUF, nx2 = 2 % NBUF;
+  auto rotate = [&]() {
+    const int c = cur;
+    cur = nxt;
+    nxt = nx2;
+    nx2 = (NBUF == 3) ? c : cur;
+    if (NBUF == 2) nxt = c;
+  };
+
+  // ---- prologue: tile 0 into buffer 0; with KPF tile 1 is already on its way ----
+  stage_load(j_begin, 0);
   stage_store(0);
-  if constexpr (KPF) stage_load(j_begin + G::JT);
+  if constexpr (KPF) stage_load(j_begin + G::JT, 1);
+  if constexpr (DIRECT) wait_all_vm();
   __syncthreads();
   if constexpr (KPF) load_keys(K[0], 0, 0);
 
   // ---- tile 0: establishes the running max, no soft-max pipelining ----
   {
     if constexpr (KPF) {
-      stage_store(1);
-      stage_load(j_begin + 2 * G::JT);
+      stage_store(nxt);                               // bias (and registers) of tile 1
+      stage_load(j_begin + 2 * G::JT, nx2);           // tile 2
     } else {
-      stage_load(j_begin + G::JT);
+      stage_load(j_begin + G::JT, nxt);
     }
 #pragma unroll
     for (int js = 0; js < NSUB; ++js) {
-      if constexpr (!KPF) load_keys(K[0], 0, js);
+      if constexpr (!KPF) load_keys(K[0], cur, js);
       KeyRegs& kr = K[KPF ? (js & 1) : 0];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         if (KPF && rb == RB - 1) {
           if (js + 1 < NSUB) {
-            load_keys(K[(js + 1) & 1], 0, js + 1);
+            load_keys(K[(js + 1) & 1], cur, js + 1);
           } else {
-            __syncthreads();  // tile 1 is in buffer 1; every wave is done reading buffer 0
-            load_keys(K[0], 1, 0);
+            if constexpr (DIRECT) wait_older_tiles();  // tile 1 has landed
+            __syncthreads();  // tile 1 is visible; every wave is done reading buffer cur
+            load_keys(K[0], nxt, 0);
           }
         }
         const f32x16 acc = add_bias(chain(kr, rb), kr, rb);
@@ -527,9 +576,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       }
     }
     if constexpr (!KPF) {
-      stage_store(1);
+      stage_store(nxt);
+      if constexpr (DIRECT) wait_all_vm();
       __syncthreads();
     }
+    rotate();
   }
 
   f32x16 acc_prev;
@@ -538,11 +589,10 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 
   // ---- steady state: the soft-max of the previous logits tile rides between the MFMAs ----
   for (int t = 1; t < ntiles; ++t) {
-    const int buf = t & 1;
-    if constexpr (!KPF) stage_load(j_begin + (t + 1) * G::JT);
+    if constexpr (!KPF) stage_load(j_begin + (t + 1) * G::JT, nxt);
 #pragma unroll
     for (int js = 0; js < NSUB; ++js) {
-      if constexpr (!KPF) load_keys(K[0], buf, js);
+      if constexpr (!KPF) load_keys(K[0], cur, js);
       KeyRegs& kr = K[KPF ? (js & 1) : 0];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
@@ -559,11 +609,14 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             acc = mfma_k(k, acc, kr, rb);
           if constexpr (KPF) {
             // LDS / global traffic of the pipeline, placed where it has the whole unit to land
-            if (js == 0 && rb == 0 && p == 0) stage_store(buf ^ 1);              // tile t+1
-            if (js == 0 && rb == 0 && p == 1) stage_load(j_begin + (t + 2) * G::JT);
-            if (rb == RB - 1 && js + 1 < NSUB && p == 1) load_keys(K[(js + 1) & 1], buf, js + 1);
-            if (rb == RB - 1 && js + 1 == NSUB && p == 1) __syncthreads();
-            if (rb == RB - 1 && js + 1 == NSUB && p == 2) load_keys(K[0], buf ^ 1, 0);
+            if (js == 0 && rb == 0 && p == 0) stage_store(nxt);                   // tile t+1
+            if (js == 0 && rb == 0 && p == 1) stage_load(j_begin + (t + 2) * G::JT, nx2);
+            if (rb == RB - 1 && js + 1 < NSUB && p == 1) load_keys(K[(js + 1) & 1], cur, js + 1);
+            if (rb == RB - 1 && js + 1 == NSUB && p == 1) {
+              if constexpr (DIRECT) wait_older_tiles();  // tile t+1 has landed
+              __syncthreads();
+            }
+            if (rb == RB - 1 && js + 1 == NSUB && p == 2) load_keys(K[0], nxt, 0);
           }
           softmax_piece(p, st, acc_prev, prev_rb);
           FS_SCHED_FENCE();
@@ -574,9 +627,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       }
     }
     if constexpr (!KPF) {
-      stage_store(buf ^ 1);
+      stage_store(nxt);
+      if constexpr (DIRECT) wait_all_vm();
       __syncthreads();
     }
+    rotate();
   }
   softmax(acc_prev, RB - 1);
 
