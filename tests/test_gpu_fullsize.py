@@ -96,6 +96,11 @@ def test_config2_loss_and_potentials():
     assert rel_err(fp.cpu().numpy(), fix["f_prelast"]) < 1e-4
     loss = float((A.double() * f.double()).sum() + (A.double() * g.double()).sum())
     assert abs(loss - float(fix["loss"])) < 1e-4 * abs(float(fix["loss"]))
+    # the configuration as stated: debiased loss through the public API
+    from flash_sinkhorn_amd import SamplesLoss
+    deb = SamplesLoss("sinkhorn", blur=0.1, debias=True, use_epsilon_scaling=False, eps=0.01,
+                      n_iters=100, allow_tf32=False)(X, Y)
+    assert abs(float(deb) - float(fix["loss_debiased"])) < 1e-4 * abs(float(fix["loss_debiased"]))
 
 
 def _fixture(name):
