@@ -14,7 +14,8 @@ namespace fs {
 namespace {
 
 constexpr int kMaxStreamD = 128;    // register-stationary streaming kernels
-constexpr int kMaxSlicedD = 1536;   // column-sliced kernels
+constexpr int kMaxSlicedD = 16384;  // widest supported rows
+constexpr int kSlicedSpan = 1536;   // columns one workgroup of the column-sliced kernels spans
 constexpr int kPlanePadRowsApi = 256;  // must match kPlanePadRows of the plane-splitting kernels
 constexpr size_t kPlaneAuxBytes = (2 * 256 + 4) * sizeof(float);  // absmax partials + plane scales
 
@@ -46,6 +47,7 @@ struct SidePlan {
 
 // Which kernel family serves feature dimension d, and its tile geometry.
 struct Family {
+  int nss;       // sliced only: super-slices of kSlicedSpan columns
   bool sliced;
   int dp;        // padded feature width (also the width of partial O rows)
   int jt;        // keys per tile
@@ -56,6 +58,7 @@ Family family_for(int64_t d) {
   Family f;
   f.sliced = d > kMaxStreamD;
   f.nw = f.nsl = 0;
+  f.nss = 1;
   if (!f.sliced) {
     f.dp = padded_d(d);
     f.jt = (f.dp >= 128) ? 32 : 64;
@@ -64,8 +67,8 @@ Family family_for(int64_t d) {
   if (d <= 256) { f.nw = 4; f.nsl = 2; }
   else if (d <= 512) { f.nw = 8; f.nsl = 2; }
   else if (d <= 1024) { f.nw = 8; f.nsl = 4; }
-  else { f.nw = 8; f.nsl = 6; }
-  f.dp = f.nw * f.nsl * 32;
+  else { f.nw = 8; f.nsl = 6; f.nss = ceil_div(d, kSlicedSpan); }
+  f.dp = f.nss * f.nw * f.nsl * 32;
   f.jt = 32;
   return f;
 }
@@ -417,7 +420,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.k) && aligned16(sd.ep.out);
     if (sd.q2) vec_ok = vec_ok && aligned16(sd.q2);
     if (mode == kMat && sd.v) vec_ok = vec_ok && aligned16(sd.v);
-    blocks[s] = p.igroups * p.splits;
+    blocks[s] = p.igroups * p.splits * ((fam.sliced && (mode == kMat || mode == kMat5)) ? fam.nss : 1);
     if (ps.n > 0) {
       sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
       sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
@@ -428,6 +431,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (nsides == 1) a.side[1] = a.side[0];
   a.blocks0 = blocks[0];
   a.vec_ok = vec_ok ? 1 : 0;
+  a.nss = fam.nss;
   const int total = blocks[0] + blocks[1];
   if (total <= 0) return FS_OK;
 

@@ -79,6 +79,7 @@ struct LaunchArgs {
   int blocks0;   // blocks belonging to side[0]; the rest belong to side[1]
   int d;         // true feature dimension
   int vec_ok;    // rows are 16-byte aligned (d % 4 == 0 and aligned bases)
+  int nss;       // column-sliced kernels: super-slices of 1536 columns (1 unless d > 1536)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

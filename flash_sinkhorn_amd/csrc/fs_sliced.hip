@@ -8,7 +8,15 @@ namespace fs {
 template <int MODE, int NW, int NSL>
 static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
   constexpr bool stat = (MODE != kMat5);
-  hipLaunchKernelGGL((sliced_kernel<MODE, NW, NSL, stat>), dim3(blocks), dim3(NW * 64), 0, st, a);
+  if constexpr (NW == 8 && NSL == 6) {
+    if (a.nss > 1) {  // rows wider than one workgroup's span
+      hipLaunchKernelGGL((sliced_kernel<MODE, NW, NSL, stat, true>), dim3(blocks), dim3(NW * 64), 0,
+                         st, a);
+      return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+    }
+  }
+  hipLaunchKernelGGL((sliced_kernel<MODE, NW, NSL, stat, false>), dim3(blocks), dim3(NW * 64), 0, st,
+                     a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

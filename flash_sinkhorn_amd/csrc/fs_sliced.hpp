@@ -1,4 +1,4 @@
-// Plan kernels for large feature dimension (128 < d <= 1536, fp32 MFMA).
+// Plan kernels for large feature dimension (d > 128, fp32 MFMA).
 //
 // A workgroup of NW wavefronts owns ONE block of 32 query rows and splits the
 // feature axis into NW column slices of NSL*32 columns.  Wavefront w keeps its
@@ -14,6 +14,11 @@
 // soft-max work is replicated NW times, which is noise next to d/2 MFMAs.
 // Key and value rows are read straight from global memory (L2-resident across
 // the workgroups of an XCD, which sweep the keys in the same order).
+// A workgroup spans NW*NSL*32 columns (1536 at most).  Wider rows are cut into `nss`
+// super-slices of that width: every workgroup contracts ALL super-slices for the logits
+// (its own one from registers, the others with the query rows re-read per tile), and for the
+// matrix kinds the grid is multiplied by nss, workgroup ss accumulating and writing the
+// output columns of super-slice ss only.
 #pragma once
 
 #include "fs_common.hpp"
@@ -21,7 +26,7 @@
 
 namespace fs {
 
-template <int MODE, int NW, int NSL, bool STAT>
+template <int MODE, int NW, int NSL, bool STAT, bool MULTI>
 __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) {
   constexpr bool kHasO = (MODE == kMat || MODE == kMat5);
   constexpr int SW = NSL * 32;  // slice width in columns
@@ -39,6 +44,9 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
   const int d = args.d;
   const bool vec_ok = args.vec_ok != 0;
 
+  const int nss = MULTI ? args.nss : 1;      // column super-slices of the logits contraction
+  const int ss_own = kHasO ? bid % nss : 0;  // the one whose output columns this workgroup owns
+  if (kHasO) bid /= nss;
   const int split = bid % sd.splits;
   const int ig = bid / sd.splits;
   const int tid = threadIdx.x;
@@ -47,7 +55,7 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
   const int li = lane & 31;
   const int h = lane >> 5;
   const int row = ig * 32 + li;
-  const int c0 = wave * SW;
+  const int c0 = ss_own * (NW * SW) + wave * SW;
   const int j_begin = split * sd.chunk;
   const int j_end = min(sd.nk, j_begin + sd.chunk);
   const int ntiles = (j_end - j_begin + 31) / 32;
@@ -85,30 +93,34 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
       acc[r] = 0.f;
       tacc[r] = 0.f;
     }
+    for (int ss = 0; ss < nss; ++ss) {
+      const int cs0 = ss * (NW * SW) + wave * SW;
+      const bool own = (ss == ss_own);
 #pragma unroll
-    for (int q = 0; q < NQ8; ++q) {
-      const int col = c0 + 8 * q + 4 * h;
-      const float4 ya = load_row4(sd.k, j0 + li, j_end, col, d, vec_ok);
-      float4 xb;
-      if constexpr (STAT) {
-        xb = make_float4(qs[4 * q], qs[4 * q + 1], qs[4 * q + 2], qs[4 * q + 3]);
-      } else {
-        const float4 v = load_row4(sd.q, row, sd.nq, col, d, vec_ok);
-        xb = make_float4(v.x * sd.qscale, v.y * sd.qscale, v.z * sd.qscale, v.w * sd.qscale);
+      for (int q = 0; q < NQ8; ++q) {
+        const int col = cs0 + 8 * q + 4 * h;
+        const float4 ya = load_row4(sd.k, j0 + li, j_end, col, d, vec_ok);
+        float4 xb;
+        if (STAT && own) {
+          xb = make_float4(qs[4 * q], qs[4 * q + 1], qs[4 * q + 2], qs[4 * q + 3]);
+        } else {
+          const float4 v = load_row4(sd.q, row, sd.nq, col, d, vec_ok);
+          xb = make_float4(v.x * sd.qscale, v.y * sd.qscale, v.z * sd.qscale, v.w * sd.qscale);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.x, xb.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.y, xb.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.z, xb.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.w, xb.w, acc, 0, 0, 0);
+        if constexpr (MODE == kMat5) {
+          const float4 u = load_row4(sd.q2, row, sd.nq, col, d, vec_ok);
+          tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.x, u.x, tacc, 0, 0, 0);
+          tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.y, u.y, tacc, 0, 0, 0);
+          tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.z, u.z, tacc, 0, 0, 0);
+          tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.w, u.w, tacc, 0, 0, 0);
+        }
+        // keep at most a few row loads in flight: the slice is register-heavy already
+        if (q % 4 == 3) __builtin_amdgcn_sched_barrier(0);
       }
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.x, xb.x, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.y, xb.y, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.z, xb.z, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.w, xb.w, acc, 0, 0, 0);
-      if constexpr (MODE == kMat5) {
-        const float4 u = load_row4(sd.q2, row, sd.nq, col, d, vec_ok);
-        tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.x, u.x, tacc, 0, 0, 0);
-        tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.y, u.y, tacc, 0, 0, 0);
-        tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.z, u.z, tacc, 0, 0, 0);
-        tacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya.w, u.w, tacc, 0, 0, 0);
-      }
-      // keep at most a few row loads in flight: the slice is register-heavy already
-      if (q % 4 == 3) __builtin_amdgcn_sched_barrier(0);
     }
     if (wave == 0) {
       const float ab = h ? 1.0f : key_bias(sd, j0 + li, j_end);
@@ -224,7 +236,7 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
   const float s = run_s + xor32(run_s);
   const float o = run_o + xor32(run_o);
   const bool live = row < sd.nq;
-  constexpr int DPF = NW * SW;  // padded feature width of the partial buffers
+  const int DPF = nss * NW * SW;  // padded feature width of the partial buffers
   if (sd.splits == 1) {
     if constexpr (!kHasO) {
       if (live && wave == 0 && h == 0) epilogue_scalar(sd.ep, row, M, s, o);
@@ -241,7 +253,7 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
     }
   } else if (live) {
     const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
-    if (wave == 0 && h == 0) {
+    if (wave == 0 && h == 0 && ss_own == 0) {
       *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M, s);
       if constexpr (MODE == kVec) sd.part_o[pr] = o;
     }
@@ -251,7 +263,7 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
           const int col = c0 + db * 32 + 8 * q4 + 4 * h;
-          *reinterpret_cast<float4*>(&sd.part_o[pr * DPF + col]) =
+          *reinterpret_cast<float4*>(&sd.part_o[pr * (size_t)DPF + col]) =
               make_float4(oacc[db][4 * q4], oacc[db][4 * q4 + 1], oacc[db][4 * q4 + 2],
                           oacc[db][4 * q4 + 3]);
         }

@@ -19,6 +19,8 @@ SHAPES = [  # (n, m, d): ragged tiles, d not a multiple of 4/8, every padded wid
     # column-sliced kernels (d > 128): every (wavefronts, slice) configuration, ragged d
     (100, 90, 200), (64, 70, 512), (50, 140, 700), (40, 33, 1536), (33, 20, 1030), (70, 300, 130),
     (600, 2000, 256),
+    # wider than one workgroup's 1536 columns: super-slices
+    (40, 50, 2048), (33, 70, 3100),
 ]
 
 
