@@ -157,3 +157,28 @@ def test_mat5(n, m, d):
     want = oracle.mat5(x, y, f, g, A, 0.5, 0.5)
     got = mat5_sqeuclid(*dev(x, y, f, g, A), eps=0.5, cost_scale=0.5)
     assert rel_err(got, want) < RTOL
+
+
+@pytest.mark.parametrize("scale", [1e-4, 1.0, 3e4])
+@pytest.mark.parametrize("d", [64, 200])
+def test_symmetric_step_is_scale_robust(scale, d):
+    """The default operand mode multiplies fp16 planes of the matrix scaled by a power of two
+    taken from its largest magnitude: results must not depend on the units of the clouds, on
+    rows far below that maximum, or on a single outlier coordinate far above the rest."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    n, m = 300, 257
+    x, y, a, b = inputs(101, n, m, d, scale=2.0 / np.sqrt(d))
+    x = (x * scale).astype(np.float32)
+    y = (y * scale).astype(np.float32)
+    x[5] *= 1e-6          # a row 2^-20 below the maximum
+    y[7, 3] *= 300.0      # one coordinate far above everything else
+    eps = 0.05 * scale * scale
+    rng = np.random.default_rng(8)
+    fh = (rng.standard_normal(n) * 0.3 * scale * scale).astype(np.float32)
+    gh = (rng.standard_normal(m) * 0.3 * scale * scale).astype(np.float32)
+    la, lb = np.log(a), np.log(b)
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, la, lb)
+    wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, eps, 1.0, 0.5, 1.0, 1.0)
+    gf, gg = _symmetric_step_raw(X, Y, F, G, LA, LB, eps, cost_scale=1.0, alpha=0.5,
+                                 damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    assert rel_err(gf, wf) < RTOL and rel_err(gg, wg) < RTOL
