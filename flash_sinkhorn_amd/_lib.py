@@ -52,9 +52,10 @@ _SIGNATURES = {
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 
-def build(verbose: bool = False) -> str:
-    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
-    cmd = ["make", "-C", CSRC_DIR, "-j8"]
+def build(verbose: bool = False, force: bool = False) -> str:
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU); with
+    ``force`` also the ones whose objects are up to date."""
+    cmd = ["make", "-C", CSRC_DIR, "-j8"] + (["-B"] if force else [])
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("building libflash_sinkhorn_hip.so failed:\n" + res.stdout[-4000:]
