@@ -1,23 +1,27 @@
-// Software-pipelined log-sum-exp kernel (d <= 128, d % 4 == 0, aligned rows).
+// Software-pipelined log-sum-exp kernel (d <= 128).
 //
 // Same decomposition as stream_kernel<kLse> (stationary query blocks in VGPRs,
 // key tiles through LDS, transposed logits, lane-private online soft-max, bias
-// and running max folded into one extra MFMA), with two changes that matter for
+// and running max folded into one extra MFMA), with these changes that matter for
 // speed:
-//   * the soft-max of logits tile u-1 is placed in program order BETWEEN the
-//     MFMAs of tile u.  A chain of dependent MFMAs blocks a wavefront's issue
-//     slot, so only VALU work interleaved this way runs in the MFMA shadow;
+//   * the soft-max of logits tile u-1 is cut into pieces that sit in program order BETWEEN
+//     the MFMAs of tile u, fenced with sched_barrier so the compiler keeps them there.  A
+//     wavefront issues in order and a chain of dependent MFMAs blocks its issue slot, so
+//     only VALU work interleaved this way runs in the MFMA shadow.  The loop body is one
+//     basic block: a branch would let the compiler sink the pieces past the MFMAs;
 //   * the online soft-max is branch free (per-lane max, rescale by exp2(-delta) every
 //     tile).  With the keys split into chunks every chunk is short, new running
 //     maxima are frequent, and a wave-wide "does any lane need a rescale" branch
-//     would be taken on almost every tile; ~60 VALU ops per tile hide under the
-//     MFMAs instead.  Only the very first tile of a block is handled apart.
+//     would be taken on almost every tile.  Only the first tile of a block is handled apart;
+//   * the A operands of the next 32-key sub-tile are read from LDS while the current one is
+//     multiplied, and key tiles are fetched two tiles ahead (direct global->LDS loads in the
+//     two-plane modes, through registers otherwise), with one barrier per 64 keys.
 //
 // Operand precision (PREC):
-//   kF32   v_mfma_f32_32x32x2_f32 on fp32 operands.
-//          (bf16 modes read operands that split_planes_kernel has already split into packed
-//          bf16 planes, unscaled; the logit scale is applied in the exp2 argument's FMA and
-//          the bias / running-max fold uses one fp32 MFMA, so no per-tile conversion work.)
+//   kF32   v_mfma_f32_32x32x2_f32 on fp32 operands (needs d % 4 == 0 and aligned rows).
+//          (The 16-bit modes read operands that the split kernels have already cut into
+//          packed planes; the logit scale is applied in the exp2 argument's FMA and the
+//          bias / running-max fold uses one fp32 MFMA, so no per-tile conversion work.)
 //   kBf3   operands split into two bf16 planes (hi, lo); hi*hi + hi*lo + lo*hi on
 //          v_mfma_f32_32x32x16_bf16, fp32 accumulate: ~2^-17 relative per product,
 //          the counterpart of the reference's allow_tf32=True.
