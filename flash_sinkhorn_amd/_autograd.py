@@ -62,15 +62,20 @@ class _SinkhornGradFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, y, a, b, f_grad, g_grad, grad_scale, eps: float,
-                config: _SinkhornConfig, compute_grad_x: bool, compute_grad_y: bool):
+                config: _SinkhornConfig, compute_grad_x: bool, compute_grad_y: bool,
+                label_x=None, label_y=None, label_cost_matrix=None):
         gx, gy = sinkhorn_geomloss_online_grad_sqeuclid(
             x, y, a, b, f_grad, g_grad, eps=float(eps), allow_tf32=config.allow_tf32,
             use_exp2=config.use_exp2, grad_scale=grad_scale,
             compute_grad_x=bool(compute_grad_x), compute_grad_y=bool(compute_grad_y),
-            cost_scale=config.cost_scale)
+            cost_scale=config.cost_scale, label_x=label_x, label_y=label_y,
+            label_cost_matrix=label_cost_matrix, lambda_x=config.lambda_x,
+            lambda_y=config.lambda_y)
         ctx.save_for_backward(x, y, a, b, f_grad, g_grad, grad_scale)
         ctx.eps = float(eps)
         ctx.config = config
+        ctx.use_label_cost = (label_x is not None and label_y is not None
+                              and label_cost_matrix is not None and config.lambda_y != 0.0)
         return gx, gy
 
     @staticmethod
@@ -79,6 +84,9 @@ class _SinkhornGradFn(torch.autograd.Function):
         cfg = ctx.config
         if grad_grad_y is not None:
             raise NotImplementedError("Double backward w.r.t y is not implemented yet.")
+        if ctx.use_label_cost:
+            raise NotImplementedError(
+                "Double backward (HVP) is not supported with OTDD label-augmented cost.")
         out_x = None
         if grad_grad_x is not None:
             if grad_grad_x.shape != x.shape:
@@ -97,7 +105,7 @@ class _SinkhornGradFn(torch.autograd.Function):
                     allow_tf32=False,  # second order needs full fp32 operands
                     use_exp2=cfg.use_exp2)
                 out_x = hvp * grad_scale
-        return (out_x,) + (None,) * 10
+        return (out_x,) + (None,) * 13
 
 
 class _SinkhornCostFn(torch.autograd.Function):
@@ -106,9 +114,6 @@ class _SinkhornCostFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, y, a, b, eps_list: Tuple[float, ...], config: _SinkhornConfig,
                 label_x, label_y, label_cost_matrix):
-        if (label_x is not None and label_y is not None and label_cost_matrix is not None
-                and config.lambda_y != 0.0):
-            raise NotImplementedError("label-augmented cost is not part of this build")
         eps_last = float(eps_list[-1])
         if config.backend == "alternating":
             f_cost, g_cost = sinkhorn_flashstyle_alternating(
@@ -125,7 +130,9 @@ class _SinkhornCostFn(torch.autograd.Function):
                 cost_scale=config.cost_scale, rho_x=config.rho_x, rho_y=config.rho_y,
                 last_extrapolation=config.last_extrapolation,
                 return_prelast=config.last_extrapolation, threshold=config.threshold,
-                check_every=config.inner_iterations)
+                check_every=config.inner_iterations, label_x=label_x, label_y=label_y,
+                label_cost_matrix=label_cost_matrix, lambda_x=config.lambda_x,
+                lambda_y=config.lambda_y)
             if config.last_extrapolation:
                 f_cost, g_cost, f_grad, g_grad = out
             else:
@@ -137,6 +144,8 @@ class _SinkhornCostFn(torch.autograd.Function):
         ctx.save_for_backward(x, y, a, b, f_cost, g_cost, f_grad, g_grad)
         ctx.eps = eps_last
         ctx.config = config
+        labelled = config.backend != "alternating"  # the alternating backend takes no labels
+        ctx.labels = (label_x, label_y, label_cost_matrix) if labelled else (None, None, None)
         if balanced_formula:
             return (a * f_cost).sum() + (b * g_cost).sum()
         wx = config.rho_x + eps_last / 2
@@ -150,7 +159,8 @@ class _SinkhornCostFn(torch.autograd.Function):
         grad_x = grad_y = grad_a = grad_b = None
         if x.requires_grad or y.requires_grad:
             gx, gy = _SinkhornGradFn.apply(x, y, a, b, f_grad, g_grad, grad_out, ctx.eps,
-                                           ctx.config, x.requires_grad, y.requires_grad)
+                                           ctx.config, x.requires_grad, y.requires_grad,
+                                           *ctx.labels)
             grad_x = gx if x.requires_grad else None
             grad_y = gy if y.requires_grad else None
         if a.requires_grad:

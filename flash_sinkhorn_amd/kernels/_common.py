@@ -12,6 +12,7 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 __all__ = ["dampening", "log_weights", "max_diameter", "epsilon_schedule"]
+# label_cost_active / augment_label_cost are shared by the launchers that take OTDD labels
 
 
 def dampening(eps: float, rho: Optional[float]) -> float:
@@ -60,3 +61,46 @@ def _validate_device(x: torch.Tensor, others: Sequence[Tuple[str, Optional[torch
 def _f32c(t: torch.Tensor) -> torch.Tensor:
     """Contiguous fp32 view/copy of t (what every launcher hands to the C ABI)."""
     return t.contiguous().float()
+
+
+def label_cost_active(label_x, label_y, label_cost_matrix, lambda_y: float) -> bool:
+    """The reference's switch (kernels/sinkhorn_flashstyle_sqeuclid.py:1184-1189)."""
+    return (label_x is not None and label_y is not None and label_cost_matrix is not None
+            and lambda_y != 0.0)
+
+
+def augment_label_cost(x: torch.Tensor, y: torch.Tensor, label_x: torch.Tensor,
+                       label_y: torch.Tensor, label_cost_matrix: torch.Tensor,
+                       lambda_x: float, lambda_y: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """OTDD label cost as V extra feature columns, so that the plain kernels apply.
+
+    The reference adds ``- lambda_y*cs*W[label_i, label_j]`` to ``lambda_x*2cs*x_i.y_j`` with a
+    per-element gather from W (kernels/sinkhorn_flashstyle_sqeuclid.py:546-560).  The same
+    number is a dot product of augmented rows,
+        x'_i = [lambda_x*x_i, -(lambda_y/2)*W[label_i, :]],   y'_j = [y_j, onehot(label_j)],
+    since 2cs*x'_i.y'_j = lambda_x*2cs*x_i.y_j - lambda_y*cs*W[label_i, label_j]; the matrix
+    cores then do the gather.  Validation and messages follow the reference (:1191-1210).
+    Returns contiguous fp32 (x' [n, d+V], y' [m, d+V]).
+    """
+    n, m = x.shape[0], y.shape[0]
+    if label_x.shape[0] != n:
+        raise ValueError(f"label_x must have length n={n}, got {label_x.shape[0]}")
+    if label_y.shape[0] != m:
+        raise ValueError(f"label_y must have length m={m}, got {label_y.shape[0]}")
+    if label_cost_matrix.ndim != 2:
+        raise ValueError("label_cost_matrix must be 2D (V, V)")
+    if label_cost_matrix.shape[0] != label_cost_matrix.shape[1]:
+        raise ValueError("label_cost_matrix must be square (V, V)")
+    V = label_cost_matrix.shape[0]
+    if label_x.max() >= V or label_x.min() < 0:
+        raise ValueError(f"label_x values must be in [0, {V}), got range "
+                         f"[{label_x.min()}, {label_x.max()}]")
+    if label_y.max() >= V or label_y.min() < 0:
+        raise ValueError(f"label_y values must be in [0, {V}), got range "
+                         f"[{label_y.min()}, {label_y.max()}]")
+    lx = label_x.to(device=x.device, dtype=torch.long)
+    ly = label_y.to(device=x.device, dtype=torch.long)
+    W = label_cost_matrix.to(dtype=torch.float32, device=x.device)
+    xa = torch.cat([float(lambda_x) * x.float(), (-0.5 * float(lambda_y)) * W[lx]], dim=1)
+    ya = torch.cat([y.float(), torch.nn.functional.one_hot(ly, V).to(torch.float32)], dim=1)
+    return xa.contiguous(), ya.contiguous()

@@ -19,7 +19,8 @@ from typing import Optional, Tuple
 import torch
 
 from flash_sinkhorn_amd import _lib
-from flash_sinkhorn_amd.kernels._common import _f32c, log_weights
+from flash_sinkhorn_amd.kernels._common import (_f32c, augment_label_cost, label_cost_active,
+                                                log_weights)
 
 __all__ = [
     "precompute_flashsinkhorn_inputs", "compute_bias_f", "compute_bias_g",
@@ -149,12 +150,12 @@ def flashsinkhorn_symmetric_step(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Both Jacobi half-steps in one launch, each from the OLD potentials:
     f_new = (1-alpha) f_hat + alpha*(-eps*damping_f*LSE_j[...]), g_new likewise over i.
-    The OTDD label-cost variant (label_* with lambda_y != 0) is not built."""
-    if (label_x is not None and label_y is not None and label_cost_matrix is not None
-            and lambda_y != 0.0):
-        raise NotImplementedError("label-augmented cost is not part of this build")
+    With labels (OTDD) the dot-product term becomes lambda_x*2cs*x.y - lambda_y*cs*W[l_i, l_j],
+    realised as extra feature columns (``augment_label_cost``)."""
     if not x.is_cuda or not y.is_cuda:
         raise ValueError("x and y must be CUDA tensors")
+    if label_cost_active(label_x, label_y, label_cost_matrix, lambda_y):
+        x, y = augment_label_cost(x, y, label_x, label_y, label_cost_matrix, lambda_x, lambda_y)
     return _symmetric_step_raw(
         _f32c(x), _f32c(y), _f32c(f_hat), _f32c(g_hat), _f32c(log_a), _f32c(log_b), eps,
         cost_scale=cost_scale, alpha=alpha, damping_f=damping_f, damping_g=damping_g,

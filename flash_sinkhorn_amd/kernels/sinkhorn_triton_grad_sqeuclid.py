@@ -15,7 +15,8 @@ from typing import Optional, Tuple
 import torch
 
 from flash_sinkhorn_amd import _lib
-from flash_sinkhorn_amd.kernels._common import _f32c, log_weights
+from flash_sinkhorn_amd.kernels._common import (_f32c, augment_label_cost, label_cost_active,
+                                                log_weights)
 
 __all__ = ["sinkhorn_geomloss_online_grad_sqeuclid"]
 
@@ -52,9 +53,7 @@ def sinkhorn_geomloss_online_grad_sqeuclid(
         raise ValueError("b and g shapes must match y.")
     if x.dtype not in (torch.float16, torch.bfloat16, torch.float32):
         raise ValueError(f"Unsupported dtype for x/y: {x.dtype}")
-    if (label_x is not None and label_y is not None and label_cost_matrix is not None
-            and lambda_y != 0.0):
-        raise NotImplementedError("label-augmented cost is not part of this build")
+    use_labels = label_cost_active(label_x, label_y, label_cost_matrix, lambda_y)
     compute_grad_x, compute_grad_y = bool(compute_grad_x), bool(compute_grad_y)
     if not compute_grad_x and not compute_grad_y:
         return None, None
@@ -68,6 +67,14 @@ def sinkhorn_geomloss_online_grad_sqeuclid(
     xf, yf = _f32c(x.detach()), _f32c(y.detach())
     x2 = (xf * xf).sum(dim=1).contiguous()
     y2 = (yf * yf).sum(dim=1).contiguous()
+    x_plain, y_plain, d_plain = xf, yf, d
+    if use_labels:
+        # C = lambda_x*cs*|x-y|^2 + lambda_y*cs*W (reference :222-238): the weighted dot product
+        # and the label term come from the augmented rows, the norms are weighted here
+        xf, yf = augment_label_cost(xf, yf, label_x, label_y, label_cost_matrix, lambda_x,
+                                    lambda_y)
+        x2, y2 = float(lambda_x) * x2, float(lambda_x) * y2
+        d = xf.shape[1]
     af, bf = _f32c(a.detach()), _f32c(b.detach())
     log_a, log_b = _f32c(log_weights(af)), _f32c(log_weights(bf))
     ff, gf = _f32c(f.detach()), _f32c(g.detach())
@@ -81,4 +88,20 @@ def sinkhorn_geomloss_online_grad_sqeuclid(
         _lib.flags(use_exp2, allow_tf32), _lib.ptr(ws), 0 if ws is None else ws.numel(),
         _lib.stream_of(x))
     _lib.check(rc, "fs_grad")
+    if use_labels:
+        # The kernel returned 2cs*gs*w*(q' - bar(k')) on the augmented rows.  The reference's
+        # result is 2*lambda_x*cs*gs*w*(q - bar(k)) on the first d columns (:277-283); with
+        # x' = lambda_x*x and y' = y the two differ by a multiple of the row itself.
+        lam = float(lambda_x)
+        gs = 1.0 if grad_scale is None else grad_scale
+        if gx is not None:
+            gx = gx[:, :d_plain]
+            if lam != 1.0:
+                gx = lam * gx + (2.0 * cost_scale * lam * (1.0 - lam)) * gs * af[:, None] * x_plain
+            gx = gx.contiguous()
+        if gy is not None:
+            gy = gy[:, :d_plain]
+            if lam != 1.0:
+                gy = gy + (2.0 * cost_scale * (lam - 1.0)) * gs * bf[:, None] * y_plain
+            gy = gy.contiguous()
     return gx, gy

@@ -3,7 +3,7 @@
 Same constructor arguments, call forms ``(x, y)`` / ``(a, x, b, y)``, batching,
 debiasing and ``potentials=True`` behaviour as the reference's
 ``samples_loss.py:199-597`` (argument parsing :73-191, weight normalisation :50-70).
-Squared-Euclidean cost only; the OTDD label-cost variant is not built.
+Squared-Euclidean cost, optionally with the OTDD label term lambda_y*W[label_i, label_j].
 """
 from __future__ import annotations
 

@@ -14,7 +14,8 @@ import torch
 
 from flash_sinkhorn_amd import _lib
 from flash_sinkhorn_amd.kernels._common import (
-    _f32c, dampening, epsilon_schedule, log_weights, max_diameter,
+    _f32c, augment_label_cost, dampening, epsilon_schedule, label_cost_active, log_weights,
+    max_diameter,
 )
 
 __all__ = ["sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric"]
@@ -139,9 +140,10 @@ def sinkhorn_flashstyle_symmetric(
         _symmetric_step_raw, flashsinkhorn_lse,
     )
 
-    if (label_x is not None and label_y is not None and label_cost_matrix is not None
-            and lambda_y != 0.0):
-        raise NotImplementedError("label-augmented cost is not part of this build")
+    use_labels = label_cost_active(label_x, label_y, label_cost_matrix, lambda_y)
+    if use_labels and fused is not None and not fused:
+        raise ValueError("OTDD label cost requires fused=True (default). Set fused=True or omit "
+                         "label_cost_matrix.")
     rho_x, rho_y = _resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y)
 
     if eps_list is None:
@@ -166,9 +168,13 @@ def sinkhorn_flashstyle_symmetric(
     g_hat = -beta if g_init is None else _f32c(g_init) - beta
     if fused is None:
         fused = True
+    if use_labels:
+        # the label term rides in V extra feature columns; alpha / beta keep the plain norms
+        xf, yf = augment_label_cost(xf, yf, label_x, label_y, label_cost_matrix, lambda_x,
+                                    lambda_y)
     # Self problem OT(x, x) with one weight vector (the debiasing terms): both potentials
     # stay equal under the Jacobi iteration, so every step computes one half-update.
-    if (fused and f_init is None and g_init is None and rho_x == rho_y
+    if (fused and not use_labels and f_init is None and g_init is None and rho_x == rho_y
             and xf.data_ptr() == yf.data_ptr() and xf.shape == yf.shape
             and (a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape))):
         yf, beta, log_b, g_hat = xf, alpha, log_a, f_hat

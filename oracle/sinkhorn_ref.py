@@ -28,6 +28,9 @@ Pin status (what each function is checked against in tests/test_oracle_*.py):
 * grad_barycentric / grad_plan ... golden vectors from
   FS/testing/reference_sinkhorn.py:195-233 and finite differences of the dual
 * apply_plan_vec / apply_plan_mat / mat5 ... brute-force python loops
+* LabelCost (OTDD label-augmented cost) ... PARITY UNPINNED: no test or vector in the
+  reference covers it; restated from the kernels as written and checked against a brute
+  force evaluation of the same formulas
 """
 
 from __future__ import annotations
@@ -39,6 +42,7 @@ from typing import Optional, Sequence
 import numpy as np
 
 __all__ = [
+    "LabelCost",
     "log_weights",
     "dampening",
     "max_diameter",
@@ -114,6 +118,40 @@ def sqeuclid_cost(x, y, cost_scale: float = 1.0, dtype=np.float64):
     return cost_scale * (x2 + y2 - 2.0 * (x @ y.T))
 
 
+class LabelCost:
+    """OTDD label-augmented ground cost (lambda_x, lambda_y, W[label_i, label_j]).
+
+    The reference uses two slightly different formulas, restated AS WRITTEN (they agree
+    for lambda_x = 1, its default):
+      * solver step (FS/kernels/sinkhorn_flashstyle_sqeuclid.py:546-560): the dot product
+        term alone is weighted, C = cs(|x|^2 + |y|^2) - lambda_x*2cs*x.y + lambda_y*cs*W;
+      * gradient (FS/kernels/sinkhorn_triton_grad_sqeuclid.py:222-238, 277-283):
+        C = lambda_x*cs*|x-y|^2 + lambda_y*cs*W and the result carries 2*lambda_x*cs.
+    PARITY UNPINNED: the reference holds no test or vector for the label cost.
+    """
+
+    def __init__(self, label_x, label_y, W, lambda_x=1.0, lambda_y=1.0):
+        self.lx = np.asarray(label_x, dtype=np.int64)
+        self.ly = np.asarray(label_y, dtype=np.int64)
+        self.W = np.asarray(W, dtype=np.float64)
+        self.lambda_x, self.lambda_y = float(lambda_x), float(lambda_y)
+
+    def swapped(self):
+        return LabelCost(self.ly, self.lx, self.W.T, self.lambda_x, self.lambda_y)
+
+    def step_cost(self, x, y, i0, i1, cost_scale, dtype):
+        x = np.asarray(x, dtype); y = np.asarray(y, dtype)
+        x2 = (x[i0:i1] * x[i0:i1]).sum(axis=1)[:, None]
+        y2 = (y * y).sum(axis=1)[None, :]
+        w = self.W[self.lx[i0:i1]][:, self.ly].astype(dtype)
+        return (cost_scale * (x2 + y2) - self.lambda_x * 2.0 * cost_scale * (x[i0:i1] @ y.T)
+                + self.lambda_y * cost_scale * w)
+
+    def grad_cost(self, x, y, cost_scale, dtype):
+        w = self.W[self.lx][:, self.ly].astype(dtype)
+        return self.lambda_x * sqeuclid_cost(x, y, cost_scale, dtype) + self.lambda_y * cost_scale * w
+
+
 def _lse_rows(vals):
     """Row-wise log-sum-exp; rows that are all -inf give -inf."""
     mx = vals.max(axis=1)
@@ -148,9 +186,9 @@ def _for_chunks(fn, n: int, m: int):
             fn(*c)
 
 
-def softmin(x, y, pot_y, logw_y, eps, cost_scale=1.0, dtype=np.float64):
+def softmin(x, y, pot_y, logw_y, eps, cost_scale=1.0, dtype=np.float64, label=None):
     """-eps * LSE_j[(pot_j - C_ij)/eps + logw_j]
-    (FS/testing/reference_sinkhorn.py:168-174)."""
+    (FS/testing/reference_sinkhorn.py:168-174); ``label``: a LabelCost whose rows index x."""
     x = np.asarray(x, dtype=dtype)
     y = np.asarray(y, dtype=dtype)
     pot_y = np.asarray(pot_y, dtype=dtype)
@@ -159,7 +197,8 @@ def softmin(x, y, pot_y, logw_y, eps, cost_scale=1.0, dtype=np.float64):
     out = np.empty(x.shape[0], dtype=dtype)
 
     def chunk(i0, i1):
-        c = sqeuclid_cost(x[i0:i1], y, cost_scale, dtype)
+        c = (sqeuclid_cost(x[i0:i1], y, cost_scale, dtype) if label is None
+             else label.step_cost(x, y, i0, i1, cost_scale, dtype))
         out[i0:i1] = -eps * _lse_rows((pot_y[None, :] - c) / eps + logw_y[None, :])
 
     _for_chunks(chunk, x.shape[0], y.shape[0])
@@ -234,7 +273,7 @@ def sinkhorn_symmetric(
     cost_scale=1.0, eps=None, n_iters=None, diameter=None, eps_list=None,
     rho=None, reach=None, rho_x=None, rho_y=None, reach_x=None, reach_y=None,
     threshold=None, check_every=5, return_n_iters=False, return_prelast=False,
-    f_init=None, g_init=None, dtype=np.float64,
+    f_init=None, g_init=None, dtype=np.float64, label=None,
 ):
     """GeomLoss-style symmetric solver in standard potentials.
 
@@ -266,8 +305,9 @@ def sinkhorn_symmetric(
 
     def jacobi(f, g, e, w):
         df, dg = dampening(e, rho_x), dampening(e, rho_y)
-        ft = df * softmin(x, y, g, log_b, e, cost_scale, dtype)
-        gt = dg * softmin(y, x, f, log_a, e, cost_scale, dtype)
+        ft = df * softmin(x, y, g, log_b, e, cost_scale, dtype, label)
+        gt = dg * softmin(y, x, f, log_a, e, cost_scale, dtype,
+                          None if label is None else label.swapped())
         return (1.0 - w) * f + w * ft, (1.0 - w) * g + w * gt
 
     used = 0
@@ -381,10 +421,20 @@ def _softmax_rows(vals):
 
 
 def grad_barycentric(x, y, a, b, f, g, eps, cost_scale=1.0, grad_scale=1.0,
-                     dtype=np.float64):
+                     dtype=np.float64, label=None):
     """grad_x_i = 2cs*gs*a_i(x_i - softmax_j[(g_j-C_ij)/eps+log b_j].y), grad_y
     symmetric (FS/testing/reference_sinkhorn.py:208-233; kernel
-    FS/kernels/sinkhorn_triton_grad_sqeuclid.py:270-279).  Standard potentials."""
+    FS/kernels/sinkhorn_triton_grad_sqeuclid.py:270-279).  Standard potentials.
+    With a LabelCost the weights use its gradient-side cost and the result carries
+    lambda_x (dense, small inputs only)."""
+    if label is not None:
+        x = np.asarray(x, dtype); y = np.asarray(y, dtype)
+        a = np.asarray(a, dtype); b = np.asarray(b, dtype)
+        c = label.grad_cost(x, y, cost_scale, dtype)
+        wx = _softmax_rows((np.asarray(g, dtype)[None, :] - c) / eps + log_weights(b, dtype)[None, :])
+        wy = _softmax_rows((np.asarray(f, dtype)[None, :] - c.T) / eps + log_weights(a, dtype)[None, :])
+        s = 2.0 * label.lambda_x * cost_scale * grad_scale
+        return s * a[:, None] * (x - wx @ y), s * b[:, None] * (y - wy @ x)
     x = np.asarray(x, dtype); y = np.asarray(y, dtype)
     a = np.asarray(a, dtype); b = np.asarray(b, dtype)
     f = np.asarray(f, dtype); g = np.asarray(g, dtype)

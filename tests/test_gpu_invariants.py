@@ -102,3 +102,50 @@ def test_input_forms_dtype_and_layout():
     assert torch.equal(f0, f2)
     with pytest.raises(ValueError):
         solve(X.cpu(), Y, A, B, **kw)
+
+
+@pytest.mark.parametrize("lam_x,d", [(1.0, 16), (0.6, 16), (1.0, 200)])
+def test_otdd_label_cost_solver_loss_and_gradient(lam_x, d):
+    """Label-augmented cost (extra feature columns on the GPU) against the oracle's
+    restatement of the reference formulas: potentials, debiased loss, grad_x and grad_y."""
+    from flash_sinkhorn_amd import SamplesLoss
+    from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric as solve
+    rng = np.random.default_rng(61)
+    n, m, V = 220, 190, 5
+    x, y, a, b = inputs(62, n, m, d, uniform=True, scale=1.5 / np.sqrt(d))
+    lx, ly = rng.integers(0, V, n), rng.integers(0, V, m)
+    W = rng.random((V, V)).astype(np.float32)
+    W = (W + W.T) * 0.5
+    np.fill_diagonal(W, 0.0)
+    X, Y, A, B = dev(x, y, a, b)
+    LX, LY, WT = torch.from_numpy(lx).cuda(), torch.from_numpy(ly).cuda(), torch.from_numpy(W).cuda()
+    kw = dict(use_epsilon_scaling=False, eps=0.1, n_iters=25)
+    lab = oracle.LabelCost(lx, ly, W, lam_x, 0.8)
+    f, g, fp, gp = solve(X, Y, A, B, allow_tf32=False, return_prelast=True, label_x=LX,
+                         label_y=LY, label_cost_matrix=WT, lambda_x=lam_x, lambda_y=0.8, **kw)
+    wf, wg, wfp, wgp = oracle.sinkhorn_symmetric(x, y, a, b, return_prelast=True, label=lab, **kw)
+    assert rel_err(f, wf) < 1e-4 and rel_err(g, wg) < 1e-4 and rel_err(fp, wfp) < 1e-4
+
+    X.requires_grad_(True)
+    Y.requires_grad_(True)
+    L = SamplesLoss("sinkhorn", debias=True, label_cost_matrix=WT, lambda_x=lam_x, lambda_y=0.8,
+                    allow_tf32=False, **kw)
+    loss = L(X, Y, label_x=LX, label_y=LY)
+    gx, gy = torch.autograd.grad(loss, (X, Y))
+
+    def ot(p, q, wa, wb, lp, lq):
+        lb_ = oracle.LabelCost(lp, lq, W, lam_x, 0.8)
+        f_, g_, fp_, gp_ = oracle.sinkhorn_symmetric(p, q, wa, wb, return_prelast=True,
+                                                     label=lb_, **kw)
+        gp_x, gp_y = oracle.grad_barycentric(p, q, wa, wb, fp_, gp_, 0.1, label=lb_)
+        return oracle.sinkhorn_cost(wa, wb, f_, g_, 0.1), gp_x, gp_y
+    c_xy, gx_xy, gy_xy = ot(x, y, a, b, lx, ly)
+    c_xx, gxx_1, gxx_2 = ot(x, x, a, a, lx, lx)
+    c_yy, gyy_1, gyy_2 = ot(y, y, b, b, ly, ly)
+    want = c_xy - 0.5 * c_xx - 0.5 * c_yy
+    assert abs(float(loss.detach()) - want) < 1e-4 * max(abs(want), abs(c_xy) * 1e-2)
+    assert rel_err(gx, gx_xy - 0.5 * (gxx_1 + gxx_2)) < 3e-4
+    assert rel_err(gy, gy_xy - 0.5 * (gyy_1 + gyy_2)) < 3e-4
+    with pytest.raises(NotImplementedError):
+        (g1,) = torch.autograd.grad(L(X, Y, label_x=LX, label_y=LY), X, create_graph=True)
+        torch.autograd.grad(g1.sum(), X)

@@ -236,3 +236,35 @@ def test_hvp_matches_finite_difference_of_gradient():
     t = 1e-5
     fd = (grad(x + t * A) - grad(x - t * A)) / (2 * t)
     np.testing.assert_allclose(h, fd, rtol=2e-4, atol=1e-7)
+
+
+def test_label_cost_formulas_brute_force():
+    """LabelCost restates two reference formulas; check both against python loops and the
+    solver against a dense iteration written out independently."""
+    rng = np.random.default_rng(21)
+    n, m, d, V = 7, 6, 3, 4
+    x, y = rng.standard_normal((n, d)), rng.standard_normal((m, d))
+    lx, ly = rng.integers(0, V, n), rng.integers(0, V, m)
+    W = rng.random((V, V)) * 2.0
+    lab = oracle.LabelCost(lx, ly, W, lambda_x=0.7, lambda_y=1.3)
+    cs = 0.5
+    step = lab.step_cost(x, y, 0, n, cs, np.float64)
+    grad = lab.grad_cost(x, y, cs, np.float64)
+    for i in range(n):
+        for j in range(m):
+            dot = float(x[i] @ y[j])
+            want_step = cs * (x[i] @ x[i] + y[j] @ y[j]) - 0.7 * 2 * cs * dot + 1.3 * cs * W[lx[i], ly[j]]
+            want_grad = 0.7 * cs * float(((x[i] - y[j]) ** 2).sum()) + 1.3 * cs * W[lx[i], ly[j]]
+            assert abs(step[i, j] - want_step) < 1e-12 and abs(grad[i, j] - want_grad) < 1e-12
+    np.testing.assert_allclose(lab.swapped().step_cost(y, x, 0, m, cs, np.float64), step.T, atol=1e-12)
+    # solver: with lambda_x = 1 the label problem is the plain problem on cost C + lambda_y*cs*W
+    a, b = np.full(n, 1 / n), np.full(m, 1 / m)
+    lab1 = oracle.LabelCost(lx, ly, W, 1.0, 1.3)
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=0.3, n_iters=200,
+                                     cost_scale=cs, label=lab1)
+    C = lab1.grad_cost(x, y, cs, np.float64)
+    P = a[:, None] * b[None, :] * np.exp((f[:, None] + g[None, :] - C) / 0.3)
+    np.testing.assert_allclose(P.sum(1), a, rtol=1e-6)
+    np.testing.assert_allclose(P.sum(0), b, rtol=1e-6)
+    gx, gy = oracle.grad_barycentric(x, y, a, b, f, g, 0.3, cs, label=lab1)
+    np.testing.assert_allclose(gx, 2 * cs * (a[:, None] * x - P @ y), rtol=1e-5, atol=1e-9)
