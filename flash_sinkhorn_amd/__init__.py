@@ -7,9 +7,16 @@ from flash_sinkhorn_amd.hvp import (
     geomloss_to_ott_potentials,
     hvp_x_sqeuclid,
     hvp_x_sqeuclid_from_potentials,
+    inverse_hvp_x_sqeuclid_from_potentials,
+)
+from flash_sinkhorn_amd.implicit_grad import (
+    ImplicitGradInfo,
+    implicit_grad_x,
+    implicit_grad_x_from_potentials,
 )
 
 __all__ = ["SamplesLoss", "CGInfo", "conjugate_gradient", "HvpInfo",
            "geomloss_to_ott_potentials", "hvp_x_sqeuclid", "hvp_x_sqeuclid_from_potentials",
-           "__version__"]
+           "inverse_hvp_x_sqeuclid_from_potentials", "ImplicitGradInfo", "implicit_grad_x",
+           "implicit_grad_x_from_potentials", "__version__"]
 __version__ = "0.1.0"

@@ -30,7 +30,7 @@ from flash_sinkhorn_amd.sinkhorn_solvers import sinkhorn_flashstyle_symmetric
 
 __all__ = ["HvpInfo", "geomloss_to_ott_potentials", "ott_to_geomloss_potentials",
            "sinkhorn_prelast_potentials_sqeuclid", "hvp_x_sqeuclid",
-           "hvp_x_sqeuclid_from_potentials"]
+           "hvp_x_sqeuclid_from_potentials", "inverse_hvp_x_sqeuclid_from_potentials"]
 
 
 @dataclass(frozen=True)
@@ -204,3 +204,42 @@ def hvp_x_sqeuclid(
         cg_atol=cg_atol, cg_stabilise_every=cg_stabilise_every, preconditioner=preconditioner,
         precond_terms=precond_terms, use_preconditioner=use_preconditioner,
         allow_tf32=allow_tf32, use_exp2=use_exp2)
+
+
+def inverse_hvp_x_sqeuclid_from_potentials(
+    x, y, f_hat, g_hat, gr, *, eps: float, rho_x: Optional[float] = None,
+    rho_y: Optional[float] = None, tau2: float = 1e-5, max_outer_iter: int = 100,
+    outer_rtol: float = 1e-6, outer_atol: float = 1e-6, max_inner_iter: int = 100,
+    inner_rtol: float = 1e-8, inner_atol: float = 1e-8, cg_stabilise_every: int = 0,
+    preconditioner: str = "none", precond_terms: int = 3, use_preconditioner: bool = True,
+    allow_tf32: bool = False, use_exp2: bool = True, block_m=None, block_n=None, block_k=None,
+    num_warps: int = 4, num_stages: int = 2,
+) -> Tuple[torch.Tensor, HvpInfo]:
+    """z with H z = gr, H the Hessian w.r.t. x at the given OTT potentials: an outer CG on the
+    flattened (n*d) vector whose matvec is ``hvp_x_sqeuclid_from_potentials`` (itself an inner
+    CG on the Schur complement).  Same signature and bookkeeping as the reference's
+    ``hvp.py:696-835``; ``HvpInfo`` reports the OUTER solve."""
+    if x.ndim != 2 or y.ndim != 2 or gr.ndim != 2:
+        raise ValueError("x, y, gr must be 2D tensors.")
+    if not x.is_cuda or not y.is_cuda or not f_hat.is_cuda or not g_hat.is_cuda:
+        raise ValueError("inverse_hvp_x_sqeuclid_from_potentials requires CUDA tensors.")
+    n, d = x.shape
+    m, d2 = y.shape
+    if d != d2 or gr.shape != (n, d):
+        raise ValueError("Shapes must satisfy x:(n,d), y:(m,d), gr:(n,d).")
+
+    def matvec(v_flat: torch.Tensor) -> torch.Tensor:
+        out, _ = hvp_x_sqeuclid_from_potentials(
+            x, y, f_hat, g_hat, v_flat.reshape(n, d), eps=eps, rho_x=rho_x, rho_y=rho_y,
+            tau2=tau2, max_cg_iter=max_inner_iter, cg_rtol=inner_rtol, cg_atol=inner_atol,
+            cg_stabilise_every=cg_stabilise_every, preconditioner=preconditioner,
+            precond_terms=precond_terms, use_preconditioner=use_preconditioner,
+            allow_tf32=allow_tf32, use_exp2=use_exp2)
+        return out.reshape(-1)
+
+    z, info = conjugate_gradient(matvec, gr.float().reshape(-1), max_iter=max_outer_iter,
+                                 rtol=outer_rtol, atol=outer_atol, preconditioner=None,
+                                 stabilise_every=cg_stabilise_every)
+    return z.reshape(n, d), HvpInfo(
+        cg_converged=bool(info.cg_converged), cg_iters=int(info.cg_iters),
+        cg_residual=float(info.cg_residual), cg_initial_residual=float(info.cg_initial_residual))

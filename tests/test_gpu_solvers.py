@@ -248,3 +248,50 @@ def test_prepared_operands_give_identical_results(n, m, d):
     o2 = flashsinkhorn_lse_fused(X, Y, G, LB, 0.2, allow_tf32=True, _prepared=prep)
     want = oracle.lse_shifted_fused(x, y, gh, np.log(b), 0.2)
     assert rel_err(o2, want) < 1e-3
+
+
+def test_inverse_hvp_against_dense_oracle():
+    """Outer CG on the streaming HVP against a dense solve with the oracle's Hessian."""
+    from flash_sinkhorn_amd import (geomloss_to_ott_potentials, hvp_x_sqeuclid_from_potentials,
+                                    inverse_hvp_x_sqeuclid_from_potentials)
+    rng = np.random.default_rng(5)
+    n, m, d, eps = 12, 10, 3, 0.4
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = rng.standard_normal((m, d)).astype(np.float32)
+    a, b = np.full(n, 1 / n, np.float32), np.full(m, 1 / m, np.float32)
+    _, _, fp, gp = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=eps,
+                                             n_iters=40, return_prelast=True)
+    fo, go = oracle.geomloss_to_ott_potentials(fp, gp, a, b, eps)
+    gr = rng.standard_normal((n, d)).astype(np.float32)
+    want, H = oracle.inverse_hvp_x_from_potentials(x, y, fo, go, gr, eps=eps)
+    X, Y, FO, GO, GR = dev(x, y, fo.astype(np.float32), go.astype(np.float32), gr)
+    z, info = inverse_hvp_x_sqeuclid_from_potentials(X, Y, FO, GO, GR, eps=eps)
+    # fp32 CG on a system of condition number cond(H): the bar scales with it
+    cond = np.linalg.cond(H)
+    assert rel_err(z, want) < max(2e-3, 1e-6 * cond)
+    back, _ = hvp_x_sqeuclid_from_potentials(X, Y, FO, GO, z, eps=eps)
+    assert rel_err(back, gr) < 1e-3
+
+
+@pytest.mark.parametrize("cs", [1.0, 0.5])
+def test_implicit_gradient_against_oracle(cs):
+    from flash_sinkhorn_amd import implicit_grad_x, implicit_grad_x_from_potentials
+    x, y, a, b = inputs(71, 300, 260, 6)
+    rng = np.random.default_rng(6)
+    gf = rng.standard_normal(300).astype(np.float32)
+    gg = rng.standard_normal(260).astype(np.float32)
+    eps = 0.3
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=eps, n_iters=60,
+                                     cost_scale=cs)
+    fh = f - cs * (x.astype(np.float64) ** 2).sum(1)
+    gh = g - cs * (y.astype(np.float64) ** 2).sum(1)
+    want = oracle.implicit_grad_x_from_potentials(x, y, fh, gh, gf, gg, eps=eps, log_a=np.log(a),
+                                                  log_b=np.log(b), cost_scale=cs)
+    X, Y, A, B, FH, GH, GF, GG = dev(x, y, a, b, fh.astype(np.float32), gh.astype(np.float32),
+                                     gf, gg)
+    got, info = implicit_grad_x_from_potentials(X, Y, FH, GH, GF, GG, eps=eps, log_a=A.log(),
+                                                log_b=B.log(), cost_scale=cs, max_cg_iter=300)
+    assert info.cg_converged and rel_err(got, want) < 2e-3
+    got2, _ = implicit_grad_x(X, Y, A, B, GF, GG, eps=eps, cost_scale=cs, n_iters=60,
+                              max_cg_iter=300)
+    assert rel_err(got2, want) < 2e-3

@@ -268,3 +268,51 @@ def test_label_cost_formulas_brute_force():
     np.testing.assert_allclose(P.sum(0), b, rtol=1e-6)
     gx, gy = oracle.grad_barycentric(x, y, a, b, f, g, 0.3, cs, label=lab1)
     np.testing.assert_allclose(gx, 2 * cs * (a[:, None] * x - P @ y), rtol=1e-5, atol=1e-9)
+
+
+def test_implicit_gradient_matches_finite_differences():
+    """The implicit-function-theorem gradient (full cost) is the derivative of
+    <gf, f*(x)> + <gg, g*(x)> through the converged potentials, for a loss that does not see
+    the (c, -c) gauge of the potentials."""
+    rng = np.random.default_rng(0)
+    n, m, d, eps = 6, 5, 2, 0.5
+    x, y = rng.standard_normal((n, d)), rng.standard_normal((m, d))
+    a = rng.random(n) + 0.5; a /= a.sum()
+    b = rng.random(m) + 0.5; b /= b.sum()
+    gf, gg = rng.standard_normal(n), rng.standard_normal(m)
+    gg += (gf.sum() - gg.sum()) / m
+
+    def potentials(xx):
+        return oracle.sinkhorn_symmetric(xx, y, a, b, use_epsilon_scaling=False, eps=eps,
+                                         n_iters=2000)
+
+    def loss(xx):
+        f, g = potentials(xx)
+        return gf @ f + gg @ g
+
+    f, g = potentials(x)
+    got = oracle.implicit_grad_x_from_potentials(
+        x, y, f - (x ** 2).sum(1), g - (y ** 2).sum(1), gf, gg, eps=eps, log_a=np.log(a),
+        log_b=np.log(b), tau2=1e-9)
+    h = 1e-5
+    for i in range(n):
+        for k in range(d):
+            xp, xm = x.copy(), x.copy()
+            xp[i, k] += h; xm[i, k] -= h
+            assert abs(got[i, k] - (loss(xp) - loss(xm)) / (2 * h)) < 1e-5 * (1 + abs(got[i, k]))
+
+
+def test_inverse_hvp_inverts_the_hvp():
+    rng = np.random.default_rng(1)
+    n, m, d, eps = 7, 6, 2, 0.4
+    x, y = rng.standard_normal((n, d)), rng.standard_normal((m, d))
+    a, b = np.full(n, 1 / n), np.full(m, 1 / m)
+    _, _, fp, gp = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=eps,
+                                             n_iters=50, return_prelast=True)
+    fo, go = oracle.geomloss_to_ott_potentials(fp, gp, a, b, eps)
+    gr = rng.standard_normal((n, d))
+    z, H = oracle.inverse_hvp_x_from_potentials(x, y, fo, go, gr, eps=eps)
+    back, _ = oracle.hvp_x_from_potentials(x, y, fo, go, z, eps=eps, max_cg_iter=2000,
+                                           cg_rtol=1e-13, cg_atol=1e-14)
+    np.testing.assert_allclose(back, gr, rtol=1e-7, atol=1e-9)
+    np.testing.assert_allclose(H, H.T, rtol=1e-6, atol=1e-9)  # a Hessian
