@@ -74,7 +74,7 @@ Family family_for(int64_t d) {
 }
 
 // Rows per wavefront (RB blocks of 32) and the key split for one side.
-SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam) {
+SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam, int rb_force = 0) {
   SidePlan p;
   const bool has_o = (mode == kMat || mode == kMat5);
   const int dp = fam.dp;
@@ -87,6 +87,7 @@ SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam) {
   } else {
     if (mode == kLse || mode == kVec) p.rb = (dp <= 64 && nq >= 2048) ? 2 : 1;
     if (mode == kMat) p.rb = (dp <= 32 && nq >= 2048) ? 2 : 1;
+    if (rb_force > 0) p.rb = rb_force;
     p.igroups = ceil_div(nq, 128 * p.rb);
   }
   const int max_splits = (int)std::max<int64_t>(1, nk / (4 * jt));
@@ -379,8 +380,14 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   // pipelined LSE kernel: the 16-bit plane modes take any d <= 128, the fp32 mode needs aligned rows
   const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = cfg.dp;
-  if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
   if (lse2 && prec == 2 && dp >= 64) rb = 1;  // three planes of 64 columns x two row blocks spill
+  if (lse2 && prec == 3 && dp == 64) {
+    // three row blocks per wavefront amortise key reads and staging a little further
+    bool big = true;
+    for (int s = 0; s < nsides; ++s) big = big && sides[s].nq >= 8192;
+    if (big) rb = 3;
+  }
+  if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, (dp == 64 && prec == 3) ? 3 : 2);
   PlaneSet ps;
   ps.n = 0;
   ps.end = 0;
@@ -392,10 +399,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const size_t need_planes_end = need;
   for (int s = 0; s < nsides; ++s) {
     // both sides run in one launch and must share the rows-per-wave template
-    if (!fam.sliced && plans[s].rb != rb) {
-      plans[s].rb = rb;
-      plans[s].igroups = ceil_div(sides[s].nq, 128 * rb);
-    }
+    if (!fam.sliced && plans[s].rb != rb) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam, rb);
     need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
   }
   if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
@@ -544,8 +548,9 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   }
   // rb may be lowered when two sides share a launch: size for the rb=1 plan too
   auto side_bytes = [&](int64_t nq, int64_t nk) {
-    SidePlan p = plan_side(mode, nq, nk, fam);
-    size_t b = side_ws_floats(mode, p, nq, dp);
+    size_t b = 0;  // the launch may settle on any rows-per-wave count: size for the largest
+    for (int rb = 0; rb <= 3; ++rb)
+      b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dp));
     return b * sizeof(float);
   };
   size_t planes = 0;  // bf16 planes of x and y for the pipelined LSE kernel (three planes at most)
