@@ -288,8 +288,9 @@ GemmPlan gemm_plan(int64_t nq, int64_t nk, int total_igroups) {
 }
 
 // Workspace: plane region (see above), then per side 2*bsplits partial (M, s) rows.
-int run_lse_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared, void* ws,
-                 size_t ws_bytes, hipStream_t st) {
+int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared,
+                 void* ws, size_t ws_bytes, hipStream_t st) {
+  const bool vec = (mode == kVec);
   PlaneSet ps;
   int rc = side_plane_set(sides, nsides, cfg, ps);
   if (rc != FS_OK) return rc;
@@ -297,11 +298,15 @@ int run_lse_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool 
   int total_ig = 0;
   for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kGemmTile);
   GemmPlan plans[2];
-  size_t part_off[2];
+  size_t part_off[2], part_o_off[2] = {0, 0};
   for (int s = 0; s < nsides; ++s) {
     plans[s] = gemm_plan(sides[s].nq, sides[s].nk, total_ig);
     part_off[s] = need;
     need += (((size_t)2 * plans[s].bsplits * (size_t)sides[s].nq * 2 * sizeof(float)) + 15) & ~(size_t)15;
+    if (vec) {  // one weighted sum per partial row
+      part_o_off[s] = need;
+      need += (((size_t)2 * plans[s].bsplits * (size_t)sides[s].nq * sizeof(float)) + 15) & ~(size_t)15;
+    }
   }
   if (need > ws_bytes || ws == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
   char* base = static_cast<char*>(ws);
@@ -316,7 +321,7 @@ int run_lse_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool 
     sd.chunk = plans[s].chunk;
     sd.igroups = plans[s].igroups;
     sd.part_ms = reinterpret_cast<float*>(base + part_off[s]);
-    sd.part_o = nullptr;
+    sd.part_o = vec ? reinterpret_cast<float*>(base + part_o_off[s]) : nullptr;
     sd.plane_scale = plane_scales(ps, ws);
     sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
     sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
@@ -329,7 +334,7 @@ int run_lse_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool 
   if (total <= 0) return FS_OK;
 
   if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
-  if (rc == FS_OK) rc = launch_lse_gemm(a, total, st);
+  if (rc == FS_OK) rc = launch_lse_gemm(a, vec, total, st);
   if (rc != FS_OK) return rc;
   const int items0 = a.side[0].nq, items1 = (nsides == 2) ? a.side[1].nq : 0;
   hipLaunchKernelGGL((finish_kernel<false>), dim3(ceil_div(items0 + items1, 256)), dim3(256), 0, st,
@@ -343,7 +348,7 @@ size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
   size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
   auto part = [&](int64_t nq, int64_t nk, int total_ig) {
     const GemmPlan p = gemm_plan(nq, nk, total_ig);
-    return (size_t)2 * p.bsplits * (size_t)nq * 2 * sizeof(float) + 16;
+    return (size_t)2 * p.bsplits * (size_t)nq * 3 * sizeof(float) + 32;  // (M, s) and a weighted sum
   };
   const int ig_n = ceil_div(n, kGemmTile), ig_m = ceil_div(m, kGemmTile);
   if (both) return planes + part(n, m, ig_n + ig_m) + part(m, n, ig_n + ig_m) + 64;
@@ -360,7 +365,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const int dp = fam.dp;
   const LseConfig cfg = lse_config(d, flags);
   const bool prepared = (flags & FS_FLAG_OPERANDS_PREPARED) != 0;
-  if (mode == kLse && cfg.gemm) return run_lse_gemm(sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
+  if ((mode == kLse || mode == kVec) && cfg.gemm)
+    return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -557,7 +563,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   if (mode == kLse && !fam.sliced)
     planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
-  const size_t gemm = (mode == kLse && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
+  const size_t gemm = ((mode == kLse || mode == kVec) && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);
   return std::max(a + 64, gemm);
@@ -660,7 +666,7 @@ int fs_grad(const float* x, const float* y, const float* f, const float* g, cons
     sd.ep.gcoef = 2.0f * cost_scale;
   }
   if (ns == 0) return FS_OK;
-  return run_stream(kMat, false, s, ns, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kMat, false, s, ns, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 int fs_apply_vec(const float* x, const float* y, const float* f_hat, const float* g_hat,
@@ -679,7 +685,7 @@ int fs_apply_vec(const float* x, const float* y, const float* f_hat, const float
   s.ep.kind = kEpiApply; s.ep.out = out; s.ep.post = 1.0f;
   s.ep.r0 = (axis == 1) ? f_hat : g_hat; s.ep.rc0 = kLog2e / eps;
   s.ep.r1 = (axis == 1) ? log_a : log_b; s.ep.rc1 = kLog2e;
-  return run_stream(kVec, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kVec, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 int fs_apply_mat(const float* x, const float* y, const float* f_hat, const float* g_hat,
@@ -703,7 +709,7 @@ int fs_apply_mat(const float* x, const float* y, const float* f_hat, const float
   s.ep.kind = kEpiApply; s.ep.out = out; s.ep.post = 1.0f;
   s.ep.r0 = (axis == 1) ? f_hat : g_hat; s.ep.rc0 = kLog2e / eps;
   s.ep.r1 = (axis == 1) ? log_a : log_b; s.ep.rc1 = kLog2e;
-  return run_stream(kMat, sepv, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kMat, sepv, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_ott,
@@ -720,7 +726,7 @@ int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_o
   s.ep.kind = kEpiApply; s.ep.out = out; s.ep.post = -4.0f * cost_scale / eps;
   s.ep.r0 = f_ott; s.ep.rc0 = kLog2e / eps;
   s.ep.r1 = x2; s.ep.rc1 = -cost_scale * kLog2e / eps;
-  return run_stream(kMat5, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream);
+  return run_stream(kMat5, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
 }  // extern "C"

@@ -23,7 +23,7 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
                             int chunked, hipStream_t st);
 // GEMM-style LSE kernel for 128 < d <= 1536 on chunked fp16 planes; Side::splits counts
 // partial rows (twice the workgroup-level key splits).
-int launch_lse_gemm(const LaunchArgs& a, int blocks, hipStream_t st);
+int launch_lse_gemm(const LaunchArgs& a, bool vec, int blocks, hipStream_t st);
 int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, int blocks, hipStream_t st);
 
 }  // namespace fs

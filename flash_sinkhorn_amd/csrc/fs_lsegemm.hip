@@ -5,8 +5,11 @@
 
 namespace fs {
 
-int launch_lse_gemm(const LaunchArgs& a, int blocks, hipStream_t st) {
-  hipLaunchKernelGGL(lse_gemm_kernel, dim3(blocks), dim3(512), 0, st, a);
+int launch_lse_gemm(const LaunchArgs& a, bool vec, int blocks, hipStream_t st) {
+  if (vec)
+    hipLaunchKernelGGL(lse_gemm_kernel<true>, dim3(blocks), dim3(512), 0, st, a);
+  else
+    hipLaunchKernelGGL(lse_gemm_kernel<false>, dim3(blocks), dim3(512), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

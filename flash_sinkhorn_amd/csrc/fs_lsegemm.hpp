@@ -1,4 +1,6 @@
-// Log-sum-exp kernel for large feature dimension (128 < d <= 1536) on fp16 planes.
+// Log-sum-exp and plan-times-vector kernel for large feature dimension (d > 128) on fp16
+// planes.  VEC adds the weighted sum  sum_j p_ij v_j  next to  sum_j p_ij  in the soft-max of
+// each tile (plan-vector products); everything else is shared.
 //
 // With d in the hundreds a block of query rows no longer fits in registers, so the sweep is
 // organised like a GEMM: a workgroup of 8 wavefronts owns 256 query rows, walks its key
@@ -27,8 +29,10 @@ namespace fs {
 constexpr int kGemmRows = 256;   // query rows per workgroup = keys per tile
 constexpr int kGemmCols = 32;    // feature columns per k-step
 
+template <bool VEC>
 __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args) {
   __shared__ __attribute__((aligned(16))) unsigned lds[2][2 * kGemmRows * 32];
+  __shared__ __attribute__((aligned(16))) float lds_v[2][VEC ? kGemmRows : 4];  // v of a key tile
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;
@@ -89,7 +93,7 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
     for (int st = 0; st < 4; ++st)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[qb][st][r] = 0.f;
-  float run_m[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f};
+  float run_m[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f}, run_o[2] = {0.f, 0.f};
 
   auto swap_halves = [&](float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
@@ -102,6 +106,11 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   int buf = 0;
   for (int t = 0; t < ntiles; ++t) {
     const int j0 = j_begin + t * kGemmRows;
+    if constexpr (VEC) {
+      // the barriers of the k-loop publish it; tile t + 2 overwrites it after every wavefront
+      // has passed a barrier of tile t + 1, hence finished the soft-max of tile t
+      if (tid < kGemmRows) lds_v[t & 1][tid] = (j0 + tid < j_end) ? sd.v[j0 + tid] : 0.f;
+    }
     for (int c = 0; c < nch; ++c) {
       // next k-step (or the first one of the next tile) goes into the other buffer
       const bool wrap = (c + 1 == nch);
@@ -169,15 +178,35 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
       const float delta = first ? m : fmaxf(m, 0.f);
       const float m_new = run_m[qb] + delta;
       const float cc = -(m_new - run_m[qb]) * lscale;
-      float ps0 = 0.f, ps1 = 0.f;
+      float ps0 = 0.f, ps1 = 0.f, po0 = 0.f, po1 = 0.f;
 #pragma unroll
-      for (int st = 0; st < 4; ++st)
+      for (int st = 0; st < 4; ++st) {
+        if constexpr (VEC) {
+          // accumulator register 4 g + i of a lane holds key 8 g + 4 h + i of the sub-tile
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          ps0 += fast_exp2(__builtin_fmaf(acc[qb][st][r], lscale, cc));
-          ps1 += fast_exp2(__builtin_fmaf(acc[qb][st][r + 1], lscale, cc));
+          for (int g = 0; g < 4; ++g) {
+            const float4 vv = *reinterpret_cast<const float4*>(
+                &lds_v[t & 1][kg * 128 + st * 32 + 8 * g + 4 * h]);
+            const float e0 = fast_exp2(__builtin_fmaf(acc[qb][st][4 * g], lscale, cc));
+            const float e1 = fast_exp2(__builtin_fmaf(acc[qb][st][4 * g + 1], lscale, cc));
+            const float e2 = fast_exp2(__builtin_fmaf(acc[qb][st][4 * g + 2], lscale, cc));
+            const float e3 = fast_exp2(__builtin_fmaf(acc[qb][st][4 * g + 3], lscale, cc));
+            ps0 += e0 + e2;
+            ps1 += e1 + e3;
+            po0 = __builtin_fmaf(e0, vv.x, __builtin_fmaf(e2, vv.z, po0));
+            po1 = __builtin_fmaf(e1, vv.y, __builtin_fmaf(e3, vv.w, po1));
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            ps0 += fast_exp2(__builtin_fmaf(acc[qb][st][r], lscale, cc));
+            ps1 += fast_exp2(__builtin_fmaf(acc[qb][st][r + 1], lscale, cc));
+          }
         }
-      run_s[qb] = (first ? 0.f : run_s[qb] * fast_exp2(cc)) + (ps0 + ps1);
+      }
+      const float resc = first ? 0.f : fast_exp2(cc);
+      run_s[qb] = run_s[qb] * resc + (ps0 + ps1);
+      if constexpr (VEC) run_o[qb] = run_o[qb] * resc + (po0 + po1);
       run_m[qb] = m_new;
 #pragma unroll
       for (int st = 0; st < 4; ++st)
@@ -196,6 +225,11 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
       const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;
       *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =
           has_keys ? make_float2(run_m[qb] * lscale, s) : make_float2(kNegBig, 0.f);
+    }
+    if constexpr (VEC) {
+      const float o = run_o[qb] + xor32(run_o[qb]);
+      if (row < sd.nq && h == 0)
+        sd.part_o[(size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row] = has_keys ? o : 0.f;
     }
   }
 }
