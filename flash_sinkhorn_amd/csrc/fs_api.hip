@@ -356,6 +356,146 @@ size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
   return planes + part(n, m, ig_n) + 64;
 }
 
+// ---- large-d plan-matrix products on fp16 planes (plan_gemm_kernel) ----
+constexpr int kPgTile = 256;       // keys per tile
+constexpr int kPgRowsApi = 32;     // query rows per workgroup
+constexpr size_t kPgAuxBytes = 2048;  // 256 partial maxima + the scale of a value matrix
+
+struct PgPlan {
+  int igroups, splits, chunk;
+};
+
+// Column blocks per wavefront, column groups and the row stride of partial outputs.
+void pg_columns(int64_t d, int& cb, int& ncg, int& dpo) {
+  const int ncb = ceil_div(d, 32);
+  cb = (ncb <= 16) ? 2 : ((ncb <= 32) ? 4 : 6);
+  ncg = ceil_div(ncb, 8 * cb);
+  dpo = ncg * 8 * cb * 32;
+}
+
+PgPlan pg_plan(int64_t nq, int64_t nk, int ncg, int total_igroups) {
+  PgPlan p;
+  p.igroups = ceil_div(nq, kPgRowsApi);
+  int s = 1;
+  while ((int64_t)total_igroups * ncg * s < 512 && nk / (2 * s) >= kPgTile && s < 64) s *= 2;
+  p.chunk = ceil_div(ceil_div(nk, s), kPgTile) * kPgTile;
+  p.splits = ceil_div(nk, p.chunk);
+  return p;
+}
+
+size_t pg_vt_bytes(int64_t nk, int64_t d) {
+  return (size_t)ceil_div(nk, kPgTile) * kPgTile * (size_t)ceil_div(d, 32) * 32 * 4;
+}
+
+size_t pg_partial_bytes(const PgPlan& p, int64_t nq, int dpo) {
+  if (p.splits <= 1) return 0;
+  return (size_t)p.splits * (size_t)nq * (size_t)(2 + dpo) * sizeof(float) + 32;
+}
+
+// Workspace: plane region of x and y (as for lse_gemm_kernel), then per side the transposed
+// value planes with their aux block, then per side the partial (M, s) and O rows.
+int run_plan_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared, void* ws,
+                  size_t ws_bytes, hipStream_t st) {
+  PlaneSet ps;
+  int rc = side_plane_set(sides, nsides, cfg, ps);
+  if (rc != FS_OK) return rc;
+  int cb, ncg, dpo;
+  pg_columns(d, cb, ncg, dpo);
+  size_t need = ps.end;
+  int total_ig = 0;
+  for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kPgRowsApi);
+  PgPlan plans[2];
+  size_t vt_off[2], part_off[2];
+  for (int s = 0; s < nsides; ++s) {
+    plans[s] = pg_plan(sides[s].nq, sides[s].nk, ncg, total_ig);
+    vt_off[s] = need;
+    need += pg_vt_bytes(sides[s].nk, d) + kPgAuxBytes;
+  }
+  for (int s = 0; s < nsides; ++s) {
+    part_off[s] = need;
+    need += (pg_partial_bytes(plans[s], sides[s].nq, dpo) + 15) & ~(size_t)15;
+  }
+  if (need > ws_bytes || ws == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(ws);
+
+  LaunchArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.d = (int)d;
+  a.nss = ncg;
+  bool vec_ok = (d % 4 == 0);
+  bool any_split = false;
+  int blocks[2] = {0, 0};
+  for (int s = 0; s < nsides; ++s) {
+    Side& sd = sides[s];
+    sd.splits = plans[s].splits;
+    sd.chunk = plans[s].chunk;
+    sd.igroups = plans[s].igroups;
+    sd.part_ms = nullptr;
+    sd.part_o = nullptr;
+    if (sd.splits > 1) {
+      any_split = true;
+      sd.part_ms = reinterpret_cast<float*>(base + part_off[s]);
+      sd.part_o = sd.part_ms + (((size_t)sd.splits * (size_t)sd.nq * 2 + 3) & ~(size_t)3);
+    }
+    sd.plane_scale = plane_scales(ps, ws);
+    sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
+    sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
+    sd.vplanes = reinterpret_cast<const unsigned*>(base + vt_off[s]);
+    sd.vplane_scale =
+        reinterpret_cast<const float*>(base + vt_off[s] + pg_vt_bytes(sd.nk, d)) + 256;
+    vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.ep.out);
+    blocks[s] = plans[s].igroups * plans[s].splits * ncg;
+    a.side[s] = sd;
+  }
+  if (nsides == 1) a.side[1] = a.side[0];
+  a.blocks0 = blocks[0];
+  a.vec_ok = vec_ok ? 1 : 0;
+  const int total = blocks[0] + blocks[1];
+  if (total <= 0) return FS_OK;
+
+  if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
+  for (int s = 0; s < nsides && rc == FS_OK; ++s) {
+    const Side& sd = sides[s];
+    float* aux = reinterpret_cast<float*>(base + vt_off[s] + pg_vt_bytes(sd.nk, d));
+    rc = launch_transpose_planes(sd.v ? sd.v : sd.k, sd.vscale,
+                                 reinterpret_cast<unsigned*>(base + vt_off[s]), sd.nk, (int)d,
+                                 ceil_div(sd.nk, kPgTile) * 8, ceil_div(d, 32), aux, aux + 256, st);
+  }
+  if (rc == FS_OK) rc = launch_plan_gemm(a, cb, total, st);
+  if (rc != FS_OK) return rc;
+  if (any_split) {
+    int items[2] = {0, 0};
+    for (int s = 0; s < nsides; ++s)
+      items[s] = (a.side[s].splits > 1) ? a.side[s].nq * (dpo / 4) : 0;
+    LaunchArgs f = a;
+    if (items[0] == 0 && nsides == 2) {  // only the second side needs merging
+      f.side[0] = a.side[1];
+      items[0] = items[1];
+      items[1] = 0;
+    }
+    hipLaunchKernelGGL((finish_kernel<true>), dim3(ceil_div(items[0] + items[1], 256)), dim3(256), 0,
+                       st, f, dpo, items[0], items[1]);
+    if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
+  }
+  return FS_OK;
+}
+
+size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
+  LseConfig c;
+  c.gemm = true; c.prec = 3; c.dp = ceil_div(d, 32) * 32; c.np = 2;
+  const size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
+  int cb, ncg, dpo;
+  pg_columns(d, cb, ncg, dpo);
+  // planned alone a side gets the most key splits: an upper bound for shared launches
+  auto side = [&](int64_t nq, int64_t nk) {
+    const PgPlan p = pg_plan(nq, nk, ncg, ceil_div(nq, kPgRowsApi));
+    return pg_vt_bytes(nk, d) + kPgAuxBytes + pg_partial_bytes(p, nq, dpo) + 16;
+  };
+  if (both) return planes + side(n, m) + side(m, n) + 64;
+  if (either) return planes + std::max(side(n, m), side(m, n)) + 64;
+  return planes + side(n, m) + 64;
+}
+
 // Plans, carves the workspace, launches the streaming kernel over one or two
 // sides and, when keys were split, the merge kernel.
 int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes,
@@ -367,6 +507,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const bool prepared = (flags & FS_FLAG_OPERANDS_PREPARED) != 0;
   if ((mode == kLse || mode == kVec) && cfg.gemm)
     return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
+  static const int use_plan_gemm = env_int("FS_PLANGEMM", 1);
+  if (mode == kMat && cfg.gemm && use_plan_gemm)
+    return run_plan_gemm(sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -563,7 +706,8 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   if (mode == kLse && !fam.sliced)
     planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
-  const size_t gemm = ((mode == kLse || mode == kVec) && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
+  size_t gemm = ((mode == kLse || mode == kVec) && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
+  if (mode == kMat && fam.sliced) gemm = pg_ws_bytes(n, m, d, both, either);
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);
   return std::max(a + 64, gemm);

@@ -69,6 +69,8 @@ struct Side {
   const unsigned* qplanes;  // split-bf16 kernels: query rows as packed bf16 planes [nq][NP][DP/2]
   const unsigned* kplanes;  // same for the key rows [nk][NP][DP/2]
   const float* plane_scale; // fp16 planes: power-of-two scales of the two operand matrices [2]
+  const unsigned* vplanes;  // plan_gemm_kernel: fp16 planes of the value matrix in operand order
+  const float* vplane_scale;  // their power-of-two scale [1]
   float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;
@@ -87,5 +89,20 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
 __device__ __forceinline__ bool wave_any(bool p) { return __builtin_amdgcn_ballot_w64(p) != 0ull; }
+
+// Power of two that maps a largest magnitude `mx` into [2^14, 2^15); 1 for zero / denormal
+// / non-finite maxima, exponent clamped to +-40.
+__device__ __forceinline__ float f16_plane_scale(float mx) {
+  const int e = (int)((__builtin_bit_cast(unsigned, mx) >> 23) & 255u);
+  if (e == 0 || e == 255) return 1.0f;
+  int se = 14 - (e - 127);
+  se = max(-40, min(40, se));
+  return __builtin_bit_cast(float, (unsigned)(127 + se) << 23);
+}
+
+__device__ __forceinline__ unsigned pack_f16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2));
+}
 
 }  // namespace fs

@@ -118,21 +118,6 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ a
     partial[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 }
 
-// Power of two that maps a largest magnitude `mx` into [2^14, 2^15); 1 for zero / denormal
-// / non-finite maxima, exponent clamped to +-40.
-__device__ __forceinline__ float f16_plane_scale(float mx) {
-  const int e = (int)((__builtin_bit_cast(unsigned, mx) >> 23) & 255u);
-  if (e == 0 || e == 255) return 1.0f;
-  int se = 14 - (e - 127);
-  se = max(-40, min(40, se));
-  return __builtin_bit_cast(float, (unsigned)(127 + se) << 23);
-}
-
-__device__ __forceinline__ unsigned pack_f16(float a, float b) {
-  f32x2 v = {a, b};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, f16x2));
-}
-
 // x[rows, d] (fp32) -> two packed fp16 planes [rows + kPlanePadRows][2][DP/2] of scale*x, zero
 // padded to DP columns and in the trailing rows.  scale is derived from the partial maxima of
 // absmax_kernel; block 0 also publishes it in *scale_out for the consuming kernel.  With

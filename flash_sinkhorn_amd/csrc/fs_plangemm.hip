@@ -1,0 +1,29 @@
+// Launches of the large-d plan-matrix kernel and of the value-plane transposition.
+#include "fs_plangemm.hpp"
+
+#include "fs_dispatch.hpp"
+
+namespace fs {
+
+int launch_plan_gemm(const LaunchArgs& a, int cb, int blocks, hipStream_t st) {
+  switch (cb) {
+    case 2: hipLaunchKernelGGL(plan_gemm_kernel<2>, dim3(blocks), dim3(512), 0, st, a); break;
+    case 4: hipLaunchKernelGGL(plan_gemm_kernel<4>, dim3(blocks), dim3(512), 0, st, a); break;
+    case 6: hipLaunchKernelGGL(plan_gemm_kernel<6>, dim3(blocks), dim3(512), 0, st, a); break;
+    default: return FS_ERR_BAD_ARGUMENT;
+  }
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+int launch_transpose_planes(const float* src, const float* rowscale, unsigned* dst, int rows, int d,
+                            int nkb, int ncb, float* partial, float* scale_out, hipStream_t st) {
+  hipLaunchKernelGGL(absmax_rows_kernel, dim3(256), dim3(256), 0, st, src, (long long)rows, d,
+                     rowscale, partial);
+  if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
+  const long long units = (long long)nkb * ncb * 2;
+  hipLaunchKernelGGL(transpose_planes_f16_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0,
+                     st, src, rowscale, dst, rows, d, nkb, ncb, partial, scale_out);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
+}  // namespace fs
