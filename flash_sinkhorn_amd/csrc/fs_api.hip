@@ -225,6 +225,12 @@ int make_plane_set(const float* const* ptrs, const int* rows, int count, const L
   return FS_OK;
 }
 
+int plane_index(const PlaneSet& ps, const float* src, int rows) {
+  for (int i = 0; i < ps.n; ++i)
+    if (ps.src[i] == src && ps.rows[i] == rows) return i;
+  return 0;
+}
+
 const float* plane_scales(const PlaneSet& ps, void* ws) {
   return reinterpret_cast<const float*>(static_cast<char*>(ws) + ps.aux_off) + 2 * 256;
 }
@@ -394,8 +400,9 @@ size_t pg_partial_bytes(const PgPlan& p, int64_t nq, int dpo) {
 
 // Workspace: plane region of x and y (as for lse_gemm_kernel), then per side the transposed
 // value planes with their aux block, then per side the partial (M, s) and O rows.
-int run_plan_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared, void* ws,
-                  size_t ws_bytes, hipStream_t st) {
+int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared,
+                  void* ws, size_t ws_bytes, hipStream_t st) {
+  const bool mat5 = (mode == kMat5);
   PlaneSet ps;
   int rc = side_plane_set(sides, nsides, cfg, ps);
   if (rc != FS_OK) return rc;
@@ -405,11 +412,15 @@ int run_plan_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool
   int total_ig = 0;
   for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kPgRowsApi);
   PgPlan plans[2];
-  size_t vt_off[2], part_off[2];
+  size_t vt_off[2], part_off[2], q2_off = 0;
   for (int s = 0; s < nsides; ++s) {
     plans[s] = pg_plan(sides[s].nq, sides[s].nk, ncg, total_ig);
     vt_off[s] = need;
     need += pg_vt_bytes(sides[s].nk, d) + kPgAuxBytes;
+  }
+  if (mat5) {  // chunked planes of the second stationary operand and their aux block
+    q2_off = need;
+    need += plane_bytes(sides[0].nq, cfg) + kPlaneAuxBytes;
   }
   for (int s = 0; s < nsides; ++s) {
     part_off[s] = need;
@@ -443,6 +454,13 @@ int run_plan_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool
     sd.vplanes = reinterpret_cast<const unsigned*>(base + vt_off[s]);
     sd.vplane_scale =
         reinterpret_cast<const float*>(base + vt_off[s] + pg_vt_bytes(sd.nk, d)) + 256;
+    sd.kplane_scale = sd.plane_scale + plane_index(ps, sd.k, sd.nk);
+    if (mat5) {
+      sd.q2planes = reinterpret_cast<const unsigned*>(base + q2_off);
+      sd.q2plane_scale =
+          reinterpret_cast<const float*>(base + q2_off + plane_bytes(sd.nq, cfg)) + 2 * 256;
+      vec_ok = vec_ok && aligned16(sd.q2);
+    }
     vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.ep.out);
     blocks[s] = plans[s].igroups * plans[s].splits * ncg;
     a.side[s] = sd;
@@ -461,7 +479,15 @@ int run_plan_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool
                                  reinterpret_cast<unsigned*>(base + vt_off[s]), sd.nk, (int)d,
                                  ceil_div(sd.nk, kPgTile) * 8, ceil_div(d, 32), aux, aux + 256, st);
   }
-  if (rc == FS_OK) rc = launch_plan_gemm(a, cb, total, st);
+  if (mat5 && rc == FS_OK) {
+    const Side& sd = sides[0];
+    float* partial = reinterpret_cast<float*>(base + q2_off + plane_bytes(sd.nq, cfg));
+    rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
+    if (rc == FS_OK)
+      rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, st);
+  }
+  if (rc == FS_OK) rc = launch_plan_gemm(a, mat5, cb, total, st);
   if (rc != FS_OK) return rc;
   if (any_split) {
     int items[2] = {0, 0};
@@ -480,10 +506,11 @@ int run_plan_gemm(Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool
   return FS_OK;
 }
 
-size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
+size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bool mat5) {
   LseConfig c;
   c.gemm = true; c.prec = 3; c.dp = ceil_div(d, 32) * 32; c.np = 2;
-  const size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
+  size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
+  if (mat5) planes += plane_bytes(n, c) + kPlaneAuxBytes;
   int cb, ncg, dpo;
   pg_columns(d, cb, ncg, dpo);
   // planned alone a side gets the most key splits: an upper bound for shared launches
@@ -508,8 +535,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if ((mode == kLse || mode == kVec) && cfg.gemm)
     return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   static const int use_plan_gemm = env_int("FS_PLANGEMM", 1);
-  if (mode == kMat && cfg.gemm && use_plan_gemm)
-    return run_plan_gemm(sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
+  if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
+    return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -707,7 +734,8 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec) && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
-  if (mode == kMat && fam.sliced) gemm = pg_ws_bytes(n, m, d, both, either);
+  if ((mode == kMat || mode == kMat5) && fam.sliced)
+    gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);
   return std::max(a + 64, gemm);

@@ -71,6 +71,9 @@ struct Side {
   const float* plane_scale; // fp16 planes: power-of-two scales of the two operand matrices [2]
   const unsigned* vplanes;  // plan_gemm_kernel: fp16 planes of the value matrix in operand order
   const float* vplane_scale;  // their power-of-two scale [1]
+  const unsigned* q2planes; // plan_gemm_kernel, mat5: chunked fp16 planes of q2
+  const float* q2plane_scale;  // scale of q2's planes [1]
+  const float* kplane_scale;   // scale of the key matrix alone [1]
   float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;

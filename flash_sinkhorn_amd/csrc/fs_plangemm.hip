@@ -5,13 +5,20 @@
 
 namespace fs {
 
-int launch_plan_gemm(const LaunchArgs& a, int cb, int blocks, hipStream_t st) {
+template <bool MAT5>
+static int launch_cb(const LaunchArgs& a, int cb, int blocks, hipStream_t st) {
   switch (cb) {
-    case 2: hipLaunchKernelGGL(plan_gemm_kernel<2>, dim3(blocks), dim3(512), 0, st, a); break;
-    case 4: hipLaunchKernelGGL(plan_gemm_kernel<4>, dim3(blocks), dim3(512), 0, st, a); break;
-    case 6: hipLaunchKernelGGL(plan_gemm_kernel<6>, dim3(blocks), dim3(512), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((plan_gemm_kernel<2, MAT5>), dim3(blocks), dim3(512), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((plan_gemm_kernel<4, MAT5>), dim3(blocks), dim3(512), 0, st, a); break;
+    case 6: hipLaunchKernelGGL((plan_gemm_kernel<6, MAT5>), dim3(blocks), dim3(512), 0, st, a); break;
     default: return FS_ERR_BAD_ARGUMENT;
   }
+  return FS_OK;
+}
+
+int launch_plan_gemm(const LaunchArgs& a, bool mat5, int cb, int blocks, hipStream_t st) {
+  const int rc = mat5 ? launch_cb<true>(a, cb, blocks, st) : launch_cb<false>(a, cb, blocks, st);
+  if (rc != FS_OK) return rc;
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

@@ -1,5 +1,5 @@
-// Plan-times-matrix products (gradient, apply_plan_mat) for large feature dimension (d > 128)
-// on fp16 planes: out_i = epilogue( sum_j exp2(logit_ij - M_i) V_j ).
+// Plan-times-matrix products (gradient, apply_plan_mat, mat5) for large feature dimension
+// (d > 128) on fp16 planes: out_i = epilogue( sum_j exp2(logit_ij - M_i) V_j ).
 //
 // A workgroup of 8 wavefronts owns 32 query rows and the output columns of one column group
 // (8 * CB blocks of 32 columns, the whole row for d <= 256 * CB) and walks its key chunk in
@@ -18,6 +18,11 @@
 // The fp32 sums of the probabilities stay exact (VALU); only the products run on fp16 planes,
 // whose two-plane split carries 22 bits per value.
 //
+// MAT5 (sum_j P_ij <A_i, y_j> y_j): the k-loop also accumulates T = A K^T from planes of A
+// staged next to the query rows, and the probabilities are multiplied by T before they go to
+// LDS.  |T| <= d * 2^30 in plane units, so a power-of-two factor 2^(-23 - ceil(log2 d))
+// keeps |p T| within 2^15 whatever the data; it is divided out with the plane scales at the end.
+//
 // Operand order of the key axis: accumulator register 8 s + e (s = 0, 1; e = 0..7) of lane
 // (li, h) of a 32 x 32 logits tile holds key 8 (2 s + e / 4) + 4 h + e % 4 of the block, so
 // the lane's own registers 8 s .. 8 s + 7 are its B operand of 16-key step s, and the V^T
@@ -31,7 +36,6 @@ namespace fs {
 
 constexpr int kPgKeys = 256;          // keys per tile
 constexpr int kPgRows = 32;           // query rows per workgroup
-constexpr int kPgStageRows = kPgRows + kPgKeys;
 constexpr float kPgLazyThresh = 8.0f; // probabilities stay below 2^8: safe in fp16
 
 // Largest |rowscale[r] * src[r, c]| (rowscale may be null): one partial maximum per block.
@@ -102,8 +106,11 @@ __global__ __launch_bounds__(256) void transpose_planes_f16_kernel(
   o[64] = u32x4{lo[0], lo[1], lo[2], lo[3]};
 }
 
-template <int CB>
+template <int CB, bool MAT5>
 __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args) {
+  // stage rows: 32 query rows, (MAT5) 32 rows of the second stationary operand, 256 key rows
+  constexpr int kKeyRow0 = MAT5 ? 2 * kPgRows : kPgRows;
+  constexpr int kPgStageRows = kKeyRow0 + kPgKeys;
   __shared__ __attribute__((aligned(16))) unsigned lds[2][kPgStageRows * 32];
   __shared__ __attribute__((aligned(16))) u32x4 lds_p[8 * 2 * 2 * 64];  // [key block][s][plane][lane]
   __shared__ float lds_x[8][32];                                        // per-wavefront row statistics
@@ -136,9 +143,12 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
 
   const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
   const float inv_lscale = 1.0f / lscale;
+  // MAT5: 2^(-23 - ceil(log2 d)) bounds |T| * t_unit by 2^7
+  const int lg_d = 32 - __clz(max(d, 2) - 1);
+  const float t_unit = __builtin_bit_cast(float, (unsigned)(127 - 23 - lg_d) << 23);
 
   // ---- loaders: wavefront w brings key rows [32 w, 32 w + 32) of the tile (4 instructions of
-  // 8 rows), wavefronts 0-3 also 8 query rows each ----
+  // 8 rows), wavefronts 0-3 also 8 query rows each, wavefronts 4-7 (MAT5) 8 rows of A ----
   int koff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -146,17 +156,17 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     koff[i] = lr * dp + (((lane & 7) ^ ((lr >> 1) & 7)) << 2);
   }
   const int qlr = (wave & 3) * 8 + (lane >> 3);
-  const unsigned* qsrc =
-      sd.qplanes + (size_t)(row0 + qlr) * (size_t)dp + (((lane & 7) ^ ((qlr >> 1) & 7)) << 2);
+  const unsigned* qsrc = ((MAT5 && wave >= 4) ? sd.q2planes : sd.qplanes) +
+                         (size_t)(row0 + qlr) * (size_t)dp + (((lane & 7) ^ ((qlr >> 1) & 7)) << 2);
   auto issue_loads = [&](int buf, int j0, int c) {
     const unsigned* kbase = sd.kplanes + (size_t)j0 * (size_t)dp + c * 32;
-    unsigned* kdst = &lds[buf][(kPgRows + wave * 32) * 32];
+    unsigned* kdst = &lds[buf][(kKeyRow0 + wave * 32) * 32];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       __builtin_amdgcn_global_load_lds(
           (const __attribute__((address_space(1))) void*)(kbase + koff[i]),
           (__attribute__((address_space(3))) void*)(kdst + i * 8 * 32), 16, 0, 0);
-    if (wave < 4)
+    if (MAT5 || wave < 4)  // rows 0-31 queries, 32-63 second operand: wavefront w fills 8 w ..
       __builtin_amdgcn_global_load_lds(
           (const __attribute__((address_space(1))) void*)(qsrc + c * 32),
           (__attribute__((address_space(3))) void*)(&lds[buf][(wave * 8) * 32]), 16, 0, 0);
@@ -199,11 +209,12 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   int buf = 0;
   for (int t = 0; t < ntiles; ++t) {
     const int j0 = j_begin + t * kPgKeys;
-    f32x16 acc, acc2;
+    f32x16 acc, acc2, tacc;  // one T accumulator: registers are short with CB = 6
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       acc[r] = 0.f;
       acc2[r] = 0.f;
+      tacc[r] = 0.f;
     }
     // ---- 1. logits of keys [32 wave, 32 wave + 32) x 32 queries ----
     for (int c = 0; c < nch; ++c) {
@@ -216,7 +227,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
           qr[p][kk] = lds_piece(stage, li, p * 4 + kk * 2 + h);
-          kr[p][kk] = lds_piece(stage, kPgRows + wave * 32 + li, p * 4 + kk * 2 + h);
+          kr[p][kk] = lds_piece(stage, kKeyRow0 + wave * 32 + li, p * 4 + kk * 2 + h);
         }
 #pragma unroll
       for (int prod = 0; prod < 3; ++prod) {
@@ -225,6 +236,21 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
                                                      __builtin_bit_cast(f16x8, qr[pq][0]), acc, 0, 0, 0);
         acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr[pk][1]),
                                                       __builtin_bit_cast(f16x8, qr[pq][1]), acc2, 0, 0, 0);
+      }
+      if constexpr (MAT5) {
+        u32x4 ar[2][2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) ar[p][kk] = lds_piece(stage, kPgRows + li, p * 4 + kk * 2 + h);
+#pragma unroll
+        for (int prod = 0; prod < 3; ++prod) {
+          const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
+          tacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr[pk][0]),
+                                                        __builtin_bit_cast(f16x8, ar[pq][0]), tacc, 0, 0, 0);
+          tacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr[pk][1]),
+                                                        __builtin_bit_cast(f16x8, ar[pq][1]), tacc, 0, 0, 0);
+        }
       }
       __builtin_amdgcn_s_waitcnt(0);  // this wavefront's direct loads have landed
       __syncthreads();
@@ -279,6 +305,10 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
       ps += p[r];
     }
     run_s += ps;
+    if constexpr (MAT5) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) p[r] *= tacc[r] * t_unit;
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       unsigned hi[4], lo[4];
@@ -337,7 +367,8 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
 #pragma unroll
   for (int w = 0; w < 8; ++w) s += lds_x[w][li];
   const float M = (ntiles > 0) ? run_m * lscale : kNegBig;
-  const float inv_vs = 1.0f / sd.vplane_scale[0];
+  float inv_vs = 1.0f / sd.vplane_scale[0];
+  if constexpr (MAT5) inv_vs /= t_unit * sd.q2plane_scale[0] * sd.kplane_scale[0];
   const bool live = row < sd.nq;
   const bool vec_ok = args.vec_ok != 0;
   if (sd.splits == 1) {
