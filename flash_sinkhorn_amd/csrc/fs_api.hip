@@ -3,6 +3,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 
 #include "flash_sinkhorn_hip.h"
@@ -164,6 +165,15 @@ int reduced_prec_default() {
   return v;
 }
 
+// Words per row of the chunked fp16 planes: the 32-column chunks (128 bytes) of a row, plus
+// one spare chunk when their count is even.  An odd count of 128-byte units per row spreads
+// the rows of a stage (same chunk of 256 consecutive rows) over all memory channels.
+int chunked_stride(int64_t d) {
+  static const int odd = env_int("FS_ODD_STRIDE", 1);
+  const int nch = ceil_div(d, 32);
+  return (odd ? (nch | 1) : nch) * 32;
+}
+
 LseConfig lse_config(int64_t d, uint32_t flags) {
   static const int use_gemm = env_int("FS_LSEGEMM", 1);
   LseConfig c;
@@ -174,7 +184,7 @@ LseConfig lse_config(int64_t d, uint32_t flags) {
   c.gemm = sliced && use_gemm && !(flags & (FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS));
   if (c.gemm) {
     c.prec = 3;
-    c.dp = ceil_div(d, 32) * 32;
+    c.dp = chunked_stride(d);
     c.np = 2;
   } else {
     c.dp = std::max(padded_d(d), 16);
@@ -320,6 +330,7 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
+  a.pstride = cfg.dp;
   int blocks[2] = {0, 0};
   for (int s = 0; s < nsides; ++s) {
     Side& sd = sides[s];
@@ -350,7 +361,7 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
 
 size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
   LseConfig c;
-  c.gemm = true; c.prec = 3; c.dp = ceil_div(d, 32) * 32; c.np = 2;
+  c.gemm = true; c.prec = 3; c.dp = chunked_stride(d); c.np = 2;
   size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
   auto part = [&](int64_t nq, int64_t nk, int total_ig) {
     const GemmPlan p = gemm_plan(nq, nk, total_ig);
@@ -379,11 +390,29 @@ void pg_columns(int64_t d, int& cb, int& ncg, int& dpo) {
   dpo = ncg * 8 * cb * 32;
 }
 
-PgPlan pg_plan(int64_t nq, int64_t nk, int ncg, int total_igroups) {
+// Planned per side, independent of what else shares the launch, so that the workspace a
+// caller sized with fs_workspace_bytes always fits.
+PgPlan pg_plan(int64_t nq, int64_t nk, int ncg) {
   PgPlan p;
   p.igroups = ceil_div(nq, kPgRowsApi);
-  int s = 1;
-  while ((int64_t)total_igroups * ncg * s < 512 && nk / (2 * s) >= kPgTile && s < 64) s *= 2;
+  // One workgroup per CU at a time: take the smallest power-of-two key split whose grid fills
+  // whole rounds of the 256 CUs to 85 % or better, else the best one.
+  const double base = (double)p.igroups * ncg / 256.0;
+  int s = 1, best = 1;
+  double best_eff = 0.0;
+  for (int c = 1; c <= 64 && (c == 1 || nk / c >= kPgTile); c *= 2) {
+    const double rounds = base * c;
+    const double eff = rounds / std::ceil(rounds);
+    if (eff > best_eff + 1e-9) {
+      best_eff = eff;
+      best = c;
+    }
+    if (eff >= 0.85) {
+      best = c;
+      break;
+    }
+  }
+  s = best;
   p.chunk = ceil_div(ceil_div(nk, s), kPgTile) * kPgTile;
   p.splits = ceil_div(nk, p.chunk);
   return p;
@@ -409,12 +438,10 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   int cb, ncg, dpo;
   pg_columns(d, cb, ncg, dpo);
   size_t need = ps.end;
-  int total_ig = 0;
-  for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kPgRowsApi);
   PgPlan plans[2];
   size_t vt_off[2], part_off[2], q2_off = 0;
   for (int s = 0; s < nsides; ++s) {
-    plans[s] = pg_plan(sides[s].nq, sides[s].nk, ncg, total_ig);
+    plans[s] = pg_plan(sides[s].nq, sides[s].nk, ncg);
     vt_off[s] = need;
     need += pg_vt_bytes(sides[s].nk, d) + kPgAuxBytes;
   }
@@ -432,6 +459,7 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
+  a.pstride = cfg.dp;
   a.nss = ncg;
   bool vec_ok = (d % 4 == 0);
   bool any_split = false;
@@ -508,14 +536,13 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
 
 size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bool mat5) {
   LseConfig c;
-  c.gemm = true; c.prec = 3; c.dp = ceil_div(d, 32) * 32; c.np = 2;
+  c.gemm = true; c.prec = 3; c.dp = chunked_stride(d); c.np = 2;
   size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
   if (mat5) planes += plane_bytes(n, c) + kPlaneAuxBytes;
   int cb, ncg, dpo;
   pg_columns(d, cb, ncg, dpo);
-  // planned alone a side gets the most key splits: an upper bound for shared launches
   auto side = [&](int64_t nq, int64_t nk) {
-    const PgPlan p = pg_plan(nq, nk, ncg, ceil_div(nq, kPgRowsApi));
+    const PgPlan p = pg_plan(nq, nk, ncg);
     return pg_vt_bytes(nk, d) + kPgAuxBytes + pg_partial_bytes(p, nq, dpo) + 16;
   };
   if (both) return planes + side(n, m) + side(m, n) + 64;

@@ -108,8 +108,29 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ a
   const long long cnt = second ? nb : na;
   const int blk = second ? blockIdx.x - kAbsmaxBlocks : blockIdx.x;
   float m = 0.f;
-  for (long long i = (long long)blk * 256 + threadIdx.x; i < cnt; i += 256LL * kAbsmaxBlocks)
-    m = fmaxf(m, fabsf(src[i]));
+  if ((reinterpret_cast<size_t>(src) & 15) == 0) {
+    // four float4 loads in flight per thread; the tail below takes what does not fill one
+    const long long n4 = cnt >> 2;
+    const float4* s4 = reinterpret_cast<const float4*>(src);
+    const long long stride = 256LL * kAbsmaxBlocks;
+    long long i = (long long)blk * 256 + threadIdx.x;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+      const float4 a0 = s4[i], a1 = s4[i + stride], a2 = s4[i + 2 * stride], a3 = s4[i + 3 * stride];
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a0.x), fabsf(a0.y)), fmaxf(fabsf(a0.z), fabsf(a0.w))));
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a1.x), fabsf(a1.y)), fmaxf(fabsf(a1.z), fabsf(a1.w))));
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a2.x), fabsf(a2.y)), fmaxf(fabsf(a2.z), fabsf(a2.w))));
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a3.x), fabsf(a3.y)), fmaxf(fabsf(a3.z), fabsf(a3.w))));
+    }
+    for (; i < n4; i += stride) {
+      const float4 a0 = s4[i];
+      m = fmaxf(m, fmaxf(fmaxf(fabsf(a0.x), fabsf(a0.y)), fmaxf(fabsf(a0.z), fabsf(a0.w))));
+    }
+    for (long long t = (n4 << 2) + (long long)blk * 256 + threadIdx.x; t < cnt; t += stride)
+      m = fmaxf(m, fabsf(src[t]));
+  } else {
+    for (long long i = (long long)blk * 256 + threadIdx.x; i < cnt; i += 256LL * kAbsmaxBlocks)
+      m = fmaxf(m, fabsf(src[i]));
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;

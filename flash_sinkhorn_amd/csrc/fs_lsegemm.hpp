@@ -38,8 +38,8 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   const bool second = bid >= args.blocks0;
   if (second) bid -= args.blocks0;
   const Side& sd = second ? args.side[1] : args.side[0];
-  const int dp = (args.d + kGemmCols - 1) / kGemmCols * kGemmCols;  // words per plane row pair
-  const int nch = dp / kGemmCols;
+  const int dp = args.pstride;  // words per plane row pair
+  const int nch = (args.d + kGemmCols - 1) / kGemmCols;
 
   const int bsplits = sd.splits >> 1;  // workgroup-level key splits
   const int split = bid % bsplits;

@@ -5,8 +5,9 @@
 // (8 * CB blocks of 32 columns, the whole row for d <= 256 * CB) and walks its key chunk in
 // tiles of 256 keys.  Per tile:
 //   1. logits: a k-loop over the feature axis in chunks of 32 columns, exactly the staging
-//      scheme of lse_gemm_kernel (direct global->LDS loads of the chunked hi/lo planes, double
-//      buffered, one barrier per k-step) with 32 query rows + 256 key rows per stage;
+//      scheme of lse_gemm_kernel (direct global->LDS loads of the chunked hi/lo planes, one
+//      barrier per k-step) with 32 query rows + 256 key rows per stage and three stages, two
+//      k-steps ahead: a k-step has only six MFMAs per wavefront to hide the loads behind;
 //      wavefront w multiplies keys [32 w, 32 w + 32) of the tile against the 32 queries;
 //   2. soft-max: the eight per-wavefront row maxima meet in LDS, every wavefront takes the
 //      same (lazy) decision on the running maximum, exponentiates its 32 x 32 tile once and
@@ -46,10 +47,23 @@ __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restric
   __shared__ float red[4];
   float m = 0.f;
   const long long cnt = rows * (long long)d;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < cnt; i += 256LL * gridDim.x) {
-    float v = src[i];
-    if (rowscale) v *= rowscale[i / d];
-    m = fmaxf(m, fabsf(v));
+  if ((d & 3) == 0 && (reinterpret_cast<size_t>(src) & 15) == 0) {
+    // rows are whole float4 runs: one row lookup per four values
+    const float4* s4 = reinterpret_cast<const float4*>(src);
+    const int d4 = d >> 2;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < (cnt >> 2);
+         i += 256LL * gridDim.x) {
+      const float4 a = s4[i];
+      float v = fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w)));
+      if (rowscale) v *= fabsf(rowscale[i / d4]);
+      m = fmaxf(m, v);
+    }
+  } else {
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < cnt; i += 256LL * gridDim.x) {
+      float v = src[i];
+      if (rowscale) v *= rowscale[i / d];
+      m = fmaxf(m, fabsf(v));
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
@@ -111,7 +125,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   // stage rows: 32 query rows, (MAT5) 32 rows of the second stationary operand, 256 key rows
   constexpr int kKeyRow0 = MAT5 ? 2 * kPgRows : kPgRows;
   constexpr int kPgStageRows = kKeyRow0 + kPgKeys;
-  __shared__ __attribute__((aligned(16))) unsigned lds[2][kPgStageRows * 32];
+  __shared__ __attribute__((aligned(16))) unsigned lds[3][kPgStageRows * 32];
   __shared__ __attribute__((aligned(16))) u32x4 lds_p[8 * 2 * 2 * 64];  // [key block][s][plane][lane]
   __shared__ float lds_x[8][32];                                        // per-wavefront row statistics
 
@@ -120,8 +134,8 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   if (second) bid -= args.blocks0;
   const Side& sd = second ? args.side[1] : args.side[0];
   const int d = args.d;
-  const int dp = (d + 31) / 32 * 32;  // words per row of the chunked planes
-  const int nch = dp / 32;
+  const int dp = args.pstride;  // words per row of the chunked planes
+  const int nch = (d + 31) / 32;
   const int ncb = nch;                // column blocks of the V^T planes
   const int ncg = args.nss;           // column groups
 
@@ -200,10 +214,36 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
   };
 
-  if (ntiles > 0) {
-    issue_loads(0, j_begin, 0);
-    __builtin_amdgcn_s_waitcnt(0);
-  }
+  // Three stage buffers: the loads of k-step g + 2 are issued at k-step g (their buffer was
+  // read at step g - 1, which every wavefront has left), so a stage has two steps to arrive.
+  // The sequence of steps runs across tiles; (lt, lc) is the next (tile, chunk) to load.
+  const int nsteps = ntiles * nch;
+  int lt = 0, lc = 0, lbuf = 0, issued = 0;
+  auto issue_next = [&]() {
+    if (issued < nsteps) {
+      issue_loads(lbuf, j_begin + lt * kPgKeys, lc);
+      lbuf = (lbuf == 2) ? 0 : lbuf + 1;
+      if (++lc == nch) {
+        lc = 0;
+        ++lt;
+      }
+    }
+    ++issued;
+  };
+  // at most the loads of the newest stage stay in flight (5 per wavefront, 4 for wavefronts
+  // 4-7 when there is no second stationary operand)
+  auto wait_stage = [&]() {
+    if (issued > nsteps) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    } else if (MAT5 || wave < 4) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 5);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+    }
+  };
+  issue_next();
+  issue_next();
+  wait_stage();
   __syncthreads();
 
   int buf = 0;
@@ -218,8 +258,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     }
     // ---- 1. logits of keys [32 wave, 32 wave + 32) x 32 queries ----
     for (int c = 0; c < nch; ++c) {
-      const bool wrap = (c + 1 == nch);
-      if (!wrap || t + 1 < ntiles) issue_loads(buf ^ 1, wrap ? j0 + kPgKeys : j0, wrap ? 0 : c + 1);
+      issue_next();
       const unsigned* stage = lds[buf];
       u32x4 qr[2][2], kr[2][2];  // [plane][16-column half]
 #pragma unroll
@@ -252,15 +291,16 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
                                                         __builtin_bit_cast(f16x8, ar[pq][1]), tacc, 0, 0, 0);
         }
       }
-      __builtin_amdgcn_s_waitcnt(0);  // this wavefront's direct loads have landed
+      wait_stage();  // this wavefront's direct loads of the next stage have landed
       __syncthreads();
-      buf ^= 1;
+      buf = (buf == 2) ? 0 : buf + 1;
     }
 
     // first V^T operands of the tile travel while the soft-max runs
     const int kb0 = j0 >> 5;
     u32x4 va[CB][2];
     load_vt(va, kb0, 0);
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- 2. bias - M fold, shared running maximum, probabilities into LDS ----
     {
@@ -329,6 +369,9 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     for (int st = 0; st < 16; ++st) {
       u32x4 vn[CB][2];
       if (st + 1 < 16) load_vt(vn, kb0 + ((st + 1) >> 1), (st + 1) & 1);
+      // the loads of the next step stay ahead of this step's MFMAs (the compiler would sink
+      // them to their first use to save registers, and every MFMA would wait for memory)
+      __builtin_amdgcn_sched_barrier(0);
       const u32x4 bh = lds_p[(st * 2 + 0) * 64 + lane];
       const u32x4 bl = lds_p[(st * 2 + 1) * 64 + lane];
 #pragma unroll
@@ -346,6 +389,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
         oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, va[i][0]),
                                                          __builtin_bit_cast(f16x8, bh), oacc[i], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
       if (st + 1 < 16) {
 #pragma unroll
         for (int i = 0; i < CB; ++i) {
