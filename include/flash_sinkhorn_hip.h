@@ -16,7 +16,7 @@
  *  - return value: FS_OK or a negative FS_ERR_* code (fs_error_string names it)
  *  - flags: FS_FLAG_EXP2 is accepted for interface parity (the kernels always
  *    work in base 2, which is the same function).  Operand precision of the
- *    log-sum-exp kernels for d <= 128 (everything accumulates in fp32):
+ *    log-sum-exp kernels (everything accumulates in fp32):
  *      default                    operands as two fp16 planes (22 significand bits) of
  *                                 the matrix scaled by a power of two, three MFMA
  *                                 products: error at or below that of fp32 MFMA operands
@@ -25,7 +25,10 @@
  *      FS_FLAG_FP32_MFMA          fp32 operands on v_mfma_f32_32x32x2_f32
  *      FS_FLAG_REDUCED_OPERANDS   two bf16 planes, three products (~2^-17 relative
  *                                 per product): the counterpart of allow_tf32=True
- *    The gradient / plan-product / large-d kernels always use fp32 MFMA operands.
+ *    For d > 128 every operation (log-sum-exp, gradient, plan products, mat5) runs on
+ *    the two-plane fp16 operands by default and with FS_FLAG_REDUCED_OPERANDS, and on fp32
+ *    MFMA operands with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS.  The gradient and
+ *    plan-product kernels for d <= 128 always use fp32 MFMA operands.
  */
 #ifndef FLASH_SINKHORN_HIP_H
 #define FLASH_SINKHORN_HIP_H

@@ -21,6 +21,8 @@ SHAPES = [  # (n, m, d): ragged tiles, d not a multiple of 4/8, every padded wid
     (600, 2000, 256),
     # wider than one workgroup's 1536 columns: super-slices
     (40, 50, 2048), (33, 70, 3100),
+    # GEMM-shaped large-d kernels: several key tiles, ragged key splits, column groups + splits
+    (64, 2048, 160), (100, 1100, 300), (40, 600, 2048),
 ]
 
 
@@ -182,3 +184,43 @@ def test_symmetric_step_is_scale_robust(scale, d):
     gf, gg = _symmetric_step_raw(X, Y, F, G, LA, LB, eps, cost_scale=1.0, alpha=0.5,
                                  damping_f=1.0, damping_g=1.0, allow_tf32=False)
     assert rel_err(gf, wf) < RTOL and rel_err(gg, wg) < RTOL
+
+
+@pytest.mark.parametrize("scale", [1e-4, 1.0, 3e4])
+def test_large_d_products_are_scale_robust(scale):
+    """The large-d product kernels multiply fp16 planes of x, y, the value matrix and (mat5) A,
+    each scaled by a power of two from its largest magnitude, and carry probabilities as fp16
+    planes: results must not depend on the units of any of the operands."""
+    from flash_sinkhorn_amd.kernels.apply_flash import (
+        apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
+    from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    n, m, d = 150, 700, 200
+    x, y, a, b = inputs(103, n, m, d, scale=2.0 / np.sqrt(d))
+    x = (x * scale).astype(np.float32)
+    y = (y * scale).astype(np.float32)
+    y[7, 3] *= 100.0      # one coordinate far above everything else
+    eps = 0.3 * scale * scale
+    rng = np.random.default_rng(9)
+    fh = (rng.standard_normal(n) * 0.3 * scale * scale).astype(np.float32)
+    gh = (rng.standard_normal(m) * 0.3 * scale * scale).astype(np.float32)
+    la, lb = np.log(a), np.log(b)
+    vscale = 1e3 / scale  # values in units unrelated to the clouds
+    V = (rng.standard_normal((m, d)) * vscale).astype(np.float32)
+    v = (rng.standard_normal(m) * vscale).astype(np.float32)
+    z = (rng.random(m) * 1e-3).astype(np.float32)
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, la, lb)
+    kw = dict(eps=eps, cost_scale=0.5)
+    got = apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, dev(V)[0], axis=1, scale=dev(z)[0], **kw)
+    assert rel_err(got, oracle.apply_plan_mat(x, y, fh, gh, la, lb, V, axis=1, scale=z, **kw)) < RTOL
+    got = apply_plan_vec_flashstyle(X, Y, F, G, LA, LB, dev(v)[0], axis=1, **kw)
+    assert rel_err(got, oracle.apply_plan_vec(x, y, fh, gh, la, lb, v, axis=1, **kw)) < RTOL
+    wx, wy = oracle.grad_barycentric(x, y, a, b, fh, gh, eps, cost_scale=0.5)
+    gx, gy = grad(X, Y, *dev(a, b), F, G, eps=eps, cost_scale=0.5, allow_tf32=False)
+    assert rel_err(gx, wx) < RTOL and rel_err(gy, wy) < RTOL
+    A = (rng.standard_normal((n, d)) * vscale).astype(np.float32)
+    f5 = fh - 2.0 * scale * scale
+    want = oracle.mat5(x, y, f5, gh, A, eps, 0.5)
+    got = mat5_sqeuclid(*dev(x, y, f5, gh, A), eps=eps, cost_scale=0.5)
+    assert rel_err(got, want) < RTOL
