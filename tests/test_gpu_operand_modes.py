@@ -1,0 +1,95 @@
+"""The non-default operand modes of the C ABI against the fp64 oracle.
+
+``FS_FLAG_FP32_MFMA`` and ``FS_FLAG_BF16X3_OPERANDS`` (Python: ``_lib.STRICT_OPERANDS``) route
+d <= 128 log-sum-exp launches to the fp32 / three-plane bf16 variants of the pipelined kernel
+and every d > 128 operation to the column-sliced fp32-MFMA kernels; ``allow_tf32=True``
+(``FS_FLAG_REDUCED_OPERANDS``) selects two bf16 planes for d <= 128.  Strict modes are held to
+the rel 1e-4 bar of the default mode; the reduced mode to 2e-3 (its products carry ~2^-17).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.golden.recipe import inputs
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-4
+
+# d <= 128 pipelined kernel, column-sliced kernels: (wavefronts, slice) families and super-slices
+SHAPES = [(300, 257, 64), (129, 1000, 3), (257, 300, 128), (100, 90, 200), (50, 140, 700),
+          (600, 2000, 256), (40, 33, 1536), (40, 50, 2048)]
+
+
+def dev(*arrs):
+    return [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in arrs]
+
+
+def rel_err(got, want):
+    got = got.detach().cpu().numpy().astype(np.float64)
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def problem(n, m, d, seed=0):
+    x, y, a, b = inputs(200 + seed, n, m, d, scale=1.0 / np.sqrt(max(d, 1)) * 2.0)
+    rng = np.random.default_rng(seed + 11)
+    f_hat = rng.standard_normal(n).astype(np.float32) * 0.3
+    g_hat = rng.standard_normal(m).astype(np.float32) * 0.3
+    return x, y, a, b, f_hat, g_hat
+
+
+@pytest.fixture(params=["fp32_mfma", "bf16x3"])
+def strict_mode(request, monkeypatch):
+    from flash_sinkhorn_amd import _lib
+    monkeypatch.setattr(_lib, "STRICT_OPERANDS", request.param)
+    return request.param
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_symmetric_step_in_strict_modes(strict_mode, n, m, d):
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    x, y, a, b, fh, gh = problem(n, m, d, seed=1)
+    la, lb = np.log(a), np.log(b)
+    wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, 0.3, 1.0, 0.5, 1.0, 1.0)
+    gf, gg = _symmetric_step_raw(*dev(x, y, fh, gh, la, lb), 0.3, cost_scale=1.0, alpha=0.5,
+                                 damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    assert rel_err(gf, wf) < RTOL and rel_err(gg, wg) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", [s for s in SHAPES if s[2] > 128])
+def test_large_d_products_on_fp32_mfma(strict_mode, n, m, d):
+    from flash_sinkhorn_amd.kernels.apply_flash import (
+        apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
+    from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    x, y, a, b, fh, gh = problem(n, m, d, seed=2)
+    la, lb = np.log(a), np.log(b)
+    rng = np.random.default_rng(12)
+    vm = rng.standard_normal(m).astype(np.float32)
+    Vm = rng.standard_normal((m, d)).astype(np.float32)
+    sc = rng.random(m).astype(np.float32)
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, la, lb)
+    kw = dict(eps=0.4, cost_scale=0.5)
+    got = apply_plan_vec_flashstyle(X, Y, F, G, LA, LB, dev(vm)[0], axis=1, **kw)
+    assert rel_err(got, oracle.apply_plan_vec(x, y, fh, gh, la, lb, vm, axis=1, **kw)) < RTOL
+    got = apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, dev(Vm)[0], axis=1, scale=dev(sc)[0], **kw)
+    assert rel_err(got, oracle.apply_plan_mat(x, y, fh, gh, la, lb, Vm, axis=1, scale=sc, **kw)) < RTOL
+    wx, wy = oracle.grad_barycentric(x, y, a, b, fh, gh, 0.3, cost_scale=0.5)
+    gx, gy = grad(X, Y, *dev(a, b), F, G, eps=0.3, cost_scale=0.5, allow_tf32=False)
+    assert rel_err(gx, wx) < RTOL and rel_err(gy, wy) < RTOL
+    A = rng.standard_normal((n, d)).astype(np.float32)
+    f5 = fh - 2.0
+    got = mat5_sqeuclid(*dev(x, y, f5, gh, A), eps=0.5, cost_scale=0.5)
+    assert rel_err(got, oracle.mat5(x, y, f5, gh, A, 0.5, 0.5)) < RTOL
+
+
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_symmetric_step_with_reduced_operands(n, m, d):
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    x, y, a, b, fh, gh = problem(n, m, d, seed=3)
+    la, lb = np.log(a), np.log(b)
+    wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, 0.3, 1.0, 0.5, 1.0, 1.0)
+    gf, gg = _symmetric_step_raw(*dev(x, y, fh, gh, la, lb), 0.3, cost_scale=1.0, alpha=0.5,
+                                 damping_f=1.0, damping_g=1.0, allow_tf32=True)
+    assert rel_err(gf, wf) < 2e-3 and rel_err(gg, wg) < 2e-3
