@@ -21,12 +21,16 @@ FS_FLAG_REDUCED_OPERANDS = 2
 FS_FLAG_FP32_MFMA = 4
 FS_FLAG_BF16X3_OPERANDS = 8
 FS_FLAG_OPERANDS_PREPARED = 16
+FS_FLAG_NO_TILE_SKIP = 32
 # allow_tf32=False normally runs the two-plane fp16 operands (fp32-grade accuracy).
 # STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" runs fp32 MFMA
 # operands, "bf16x3" the three-plane bf16 split instead.
 STRICT_OPERANDS = os.environ.get("FLASH_SINKHORN_STRICT_OPERANDS", "fp16x2")
 OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5 = range(6)
 
+# d <= 128 log-sum-exp kernel: leave out the exponentials of logits tiles that lie 2^40 below
+# the running row maxima (no effect on fp32 sums); False computes every exponential.
+TILE_SKIP = os.environ.get("FLASH_SINKHORN_TILE_SKIP", "1") != "0"
 _lib: Optional[ctypes.CDLL] = None
 
 _P = ctypes.c_void_p
@@ -105,6 +109,8 @@ def workspace(op: int, n: int, m: int, d: int, device) -> Optional[torch.Tensor]
 
 def flags(use_exp2: bool, allow_tf32: bool) -> int:
     f = FS_FLAG_EXP2 if use_exp2 else 0
+    if not TILE_SKIP:
+        f |= FS_FLAG_NO_TILE_SKIP
     if allow_tf32:
         return f | FS_FLAG_REDUCED_OPERANDS
     if STRICT_OPERANDS not in _STRICT_FLAGS:

@@ -647,6 +647,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
   } else if (lse2) {
     rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
+    a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
     if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, total, st);
   } else
   switch (mode) {

@@ -86,6 +86,8 @@ struct LaunchArgs {
   int vec_ok;    // rows are 16-byte aligned (d % 4 == 0 and aligned bases)
   int nss;       // column-sliced kernels: super-slices of 1536 columns (1 unless d > 1536)
   int pstride;   // GEMM-shaped kernels: words per row of the chunked fp16 planes
+  float skip_log2;  // lse2_kernel: tiles whose logits all lie this far (base 2, negative) below
+                    // the running maxima skip their exponentials; -inf-like to switch it off
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

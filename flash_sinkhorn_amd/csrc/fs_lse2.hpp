@@ -202,8 +202,9 @@ struct Geo2 {
 // place a piece after every few MFMAs of the NEXT tile: a wavefront issues in order, and only
 // VALU work that sits between the MFMAs in program order runs in their shadow.
 constexpr int kPieces = 12;
+constexpr int kMaxPieces = 3;  // pieces 0..2 find the largest logit of the unit
 struct SoftmaxStage {
-  float m[6], aa, bb, c, ps0, ps1;
+  float m[6], mx, aa, bb, c, ps0, ps1;
   float t[16], e[16];
 };
 
@@ -255,6 +256,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   float lscale = kBf ? sd.qscale : 1.0f;
   if constexpr (PREC == kH3) lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
   const float inv_lscale = kBf ? 1.0f / lscale : 1.0f;
+  const float skip_below = args.skip_log2 * inv_lscale;  // in accumulator units
 
   // ---- stationary query operands ----
   float xs[kBf ? 1 : RB][kBf ? 1 : DP / 2];
@@ -425,8 +427,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       s.m[5] = fmaxf(fmaxf(s.m[0], s.m[1]), a[15]);
     }
     if (p == 2) {
-      s.aa = fmaxf(s.m[5], fmaxf(fmaxf(s.m[2], s.m[3]), s.m[4]));
-      s.bb = s.aa;
+      s.mx = fmaxf(s.m[5], fmaxf(fmaxf(s.m[2], s.m[3]), s.m[4]));  // this lane's 16 keys
+      s.aa = s.mx;
+      s.bb = s.mx;
       swap_halves(s.aa, s.bb);
     }
     if (p == 3) {
@@ -612,8 +615,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         FS_SCHED_FENCE();
-#pragma unroll
-        for (int p = 0; p < kPieces; ++p) {
+        // MFMAs of piece p of this unit, the pipeline's memory traffic, and (soft) piece p
+        // of the previous unit's soft-max
+        auto step = [&](int p, auto soft) {
 #pragma unroll
           for (int k = (p * NMAIN) / kPieces; k < ((p + 1) * NMAIN) / kPieces; ++k)
             acc = mfma_k(k, acc, kr, rb);
@@ -628,10 +632,22 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             }
             if (rb == RB - 1 && js + 1 == NSUB && p == 2) load_keys(K[0], nxt, 0);
           }
-          softmax_piece(p, st, acc_prev, prev_rb);
+          if constexpr (decltype(soft)::value) softmax_piece(p, st, acc_prev, prev_rb);
           FS_SCHED_FENCE();
+        };
+#pragma unroll
+        for (int p = 0; p < kMaxPieces; ++p) step(p, std::true_type{});
+        // Every logit of the previous unit more than 2^40 (LaunchArgs::skip_log2) below its
+        // row's running maximum: its exponentials would not change the fp32 row sums, so
+        // they are not computed.
+        if (wave_any(st.mx > skip_below)) {
+#pragma unroll
+          for (int p = kMaxPieces; p < kPieces; ++p) step(p, std::true_type{});
+          softmax_tail(st, prev_rb);
+        } else {
+#pragma unroll
+          for (int p = kMaxPieces; p < kPieces; ++p) step(p, std::false_type{});
         }
-        softmax_tail(st, prev_rb);
         acc_prev = add_bias(acc, kr, rb);
         FS_SCHED_FENCE();
       }

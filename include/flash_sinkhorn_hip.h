@@ -25,6 +25,9 @@
  *      FS_FLAG_FP32_MFMA          fp32 operands on v_mfma_f32_32x32x2_f32
  *      FS_FLAG_REDUCED_OPERANDS   two bf16 planes, three products (~2^-17 relative
  *                                 per product): the counterpart of allow_tf32=True
+ *    The d <= 128 log-sum-exp kernel leaves out the exponentials of a 32 x 32 logits tile
+ *    whose every entry lies more than 2^40 below its row's running maximum (they cannot
+ *    change the fp32 row sums); FS_FLAG_NO_TILE_SKIP computes them all the same.
  *    For d > 128 every operation (log-sum-exp, gradient, plan products, mat5) runs on
  *    the two-plane fp16 operands by default and with FS_FLAG_REDUCED_OPERANDS, and on fp32
  *    MFMA operands with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS.  The gradient and
@@ -53,6 +56,7 @@ extern "C" {
 #define FS_FLAG_FP32_MFMA 4u
 #define FS_FLAG_BF16X3_OPERANDS 8u
 #define FS_FLAG_OPERANDS_PREPARED 16u
+#define FS_FLAG_NO_TILE_SKIP 32u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0

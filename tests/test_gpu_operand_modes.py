@@ -93,3 +93,33 @@ def test_symmetric_step_with_reduced_operands(n, m, d):
     gf, gg = _symmetric_step_raw(*dev(x, y, fh, gh, la, lb), 0.3, cost_scale=1.0, alpha=0.5,
                                  damping_f=1.0, damping_g=1.0, allow_tf32=True)
     assert rel_err(gf, wf) < 2e-3 and rel_err(gg, wg) < 2e-3
+
+
+def test_tile_skip_leaves_results_unchanged(monkeypatch):
+    """Peaked plan (small eps, clustered clouds): most 32 x 32 logits tiles lie far below the
+    running row maxima and the default launch leaves their exponentials out.  The result
+    must agree with the launch that computes every exponential to fp32 rounding, and with
+    the oracle."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    rng = np.random.default_rng(21)
+    n, m, d, eps = 3000, 4100, 64, 0.01
+    cx, cy = rng.standard_normal((8, d)) * 2.0, rng.standard_normal((8, d)) * 2.0
+    x = (cx[rng.integers(0, 8, n)] + rng.standard_normal((n, d))).astype(np.float32)
+    y = (cy[rng.integers(0, 8, m)] + rng.standard_normal((m, d))).astype(np.float32)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    fh = (-(x * x).sum(1)).astype(np.float32)
+    gh = (-(y * y).sum(1)).astype(np.float32)
+    la, lb = np.log(a), np.log(b)
+    args = dev(x, y, fh, gh, la, lb)
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    monkeypatch.setattr(_lib, "TILE_SKIP", True)
+    f1, g1 = _symmetric_step_raw(*args, eps, **kw)
+    monkeypatch.setattr(_lib, "TILE_SKIP", False)
+    f0, g0 = _symmetric_step_raw(*args, eps, **kw)
+    scale = float(f0.abs().max())
+    assert float((f1 - f0).abs().max()) <= 4e-7 * scale
+    assert float((g1 - g0).abs().max()) <= 4e-7 * scale
+    wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, eps, 1.0, 0.5, 1.0, 1.0)
+    assert rel_err(f1, wf) < RTOL and rel_err(g1, wg) < RTOL
