@@ -838,6 +838,33 @@ int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const 
   return run_stream(kLse, false, s, 2, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
+int fs_symmetric_steps(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                       const float* log_a, const float* log_b, float* f_a, float* g_a, float* f_b,
+                       float* g_b, const float* shift_x, const float* shift_y, int64_t n,
+                       int64_t m, int64_t d, const float* eps, const float* alpha,
+                       const float* damp_f, const float* damp_g, int n_steps, float coord_scale,
+                       uint32_t flags, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!f_a || !g_a || !f_b || !g_b || !eps || !alpha || !damp_f || !damp_g)
+    return FS_ERR_NULL_POINTER;
+  if (n_steps < 0) return FS_ERR_BAD_ARGUMENT;
+  if (f_a == f_b || g_a == g_b || f_a == g_b || f_b == g_a) return FS_ERR_BAD_ARGUMENT;
+  const float* f_in = f_hat;
+  const float* g_in = g_hat;
+  for (int s = 0; s < n_steps; ++s) {
+    float* f_out = (s & 1) ? f_b : f_a;
+    float* g_out = (s & 1) ? g_b : g_a;
+    const int rc = fs_symmetric_step(x, y, f_in, g_in, log_a, log_b, f_out, g_out,
+                                     damp_f[s] < 1.0f ? shift_x : nullptr,
+                                     damp_g[s] < 1.0f ? shift_y : nullptr, n, m, d, eps[s],
+                                     alpha[s], damp_f[s], damp_g[s], coord_scale, flags, workspace,
+                                     workspace_bytes, stream);
+    if (rc != FS_OK) return rc;
+    f_in = f_out;
+    g_in = g_out;
+  }
+  return FS_OK;
+}
+
 int fs_grad(const float* x, const float* y, const float* f, const float* g, const float* log_a,
             const float* log_b, const float* a, const float* b, const float* x2, const float* y2,
             const float* grad_scale, float* grad_x, float* grad_y, int64_t n, int64_t m,

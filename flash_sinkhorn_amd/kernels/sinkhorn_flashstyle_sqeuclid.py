@@ -137,6 +137,37 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
     return f_out, g_out
 
 
+def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale, shift_x=None,
+                         shift_y=None, allow_tf32=True, use_exp2=True, prepared=None):
+    """``steps`` = [(eps, alpha, damping_f, damping_g), ...] run back to back by one library call
+    (``fs_symmetric_steps``): the per-step host work is a kernel launch, not a Python round
+    trip.  Operands as for ``_symmetric_step_raw``; returns the potentials of the last step."""
+    import ctypes
+    k = len(steps)
+    if k == 0:
+        return f_hat, g_hat
+    n, d = x.shape
+    m = y.shape[0]
+    self_problem = (y is x and g_hat is f_hat and log_b is log_a and shift_y is shift_x
+                    and all(s[2] == s[3] for s in steps))
+    f_work = [torch.empty((n,), device=x.device, dtype=torch.float32) for _ in range(2)]
+    g_work = f_work if self_problem else [
+        torch.empty((m,), device=x.device, dtype=torch.float32) for _ in range(2)]
+    arr = ctypes.c_float * k
+    eps_a, alpha_a, df_a, dg_a = (arr(*[float(s[i]) for s in steps]) for i in range(4))
+    wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_SYMMETRIC_STEP, x, y,
+                                           _lib.flags(use_exp2, allow_tf32), prepared)
+    rc = _lib.lib().fs_symmetric_steps(
+        x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
+        log_b.data_ptr(), f_work[0].data_ptr(), g_work[0].data_ptr(), f_work[1].data_ptr(),
+        g_work[1].data_ptr(), _lib.ptr(shift_x), _lib.ptr(shift_y), n, m, d, eps_a, alpha_a, df_a,
+        dg_a, k, 2.0 * float(cost_scale), fl, wp, wn, _lib.stream_of(x))
+    _lib.check(rc, "fs_symmetric_steps")
+    last = (k - 1) & 1
+    f_out = f_work[last]
+    return f_out, (f_out if self_problem else g_work[last])
+
+
 def flashsinkhorn_symmetric_step(
     x: torch.Tensor, y: torch.Tensor, f_hat: torch.Tensor, g_hat: torch.Tensor,
     log_a: torch.Tensor, log_b: torch.Tensor, eps: float, *,

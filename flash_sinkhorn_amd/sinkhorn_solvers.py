@@ -137,7 +137,7 @@ def sinkhorn_flashstyle_symmetric(
     only returned when ``return_prelast and last_extrapolation``.
     """
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
-        _symmetric_step_raw, flashsinkhorn_lse,
+        _symmetric_step_raw, _symmetric_steps_raw, flashsinkhorn_lse,
     )
 
     use_labels = label_cost_active(label_x, label_y, label_cost_matrix, lambda_y)
@@ -203,14 +203,32 @@ def sinkhorn_flashstyle_symmetric(
             return f_c, g_c
         return (1.0 - w) * f_hat + w * f_c, (1.0 - w) * g_hat + w * g_c
 
+    def jacobi_run(f_hat, g_hat, run):
+        """Consecutive steps [(eps, weight), ...]: one library call when fused."""
+        if not fused:
+            for e, w in run:
+                f_hat, g_hat = jacobi(f_hat, g_hat, e, w)
+            return f_hat, g_hat
+        steps = [(e, w, dampening(e, rho_x), dampening(e, rho_y)) for e, w in run]
+        return _symmetric_steps_raw(
+            xf, yf, f_hat, g_hat, log_a, log_b, steps, cost_scale=cost_scale,
+            shift_x=alpha if rho_x is not None else None,
+            shift_y=beta if rho_y is not None else None,
+            allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared)
+
+    # the initial full step and the averaged steps, cut where a convergence check looks at
+    # the potentials
     used = 0
-    f_hat, g_hat = jacobi(f_hat, g_hat, eps_list[0], 1.0)
-    used += 1
     prev_f = prev_g = None
+    run = [(eps_list[0], 1.0)]
     for idx, e in enumerate(eps_list):
-        f_hat, g_hat = jacobi(f_hat, g_hat, e, 0.5)
-        used += 1
-        if threshold is not None and (idx + 1) % check_every == 0:
+        run.append((e, 0.5))
+        check = threshold is not None and (idx + 1) % check_every == 0
+        if check or idx + 1 == len(eps_list):
+            f_hat, g_hat = jacobi_run(f_hat, g_hat, run)
+            used += len(run)
+            run = []
+        if check:
             if prev_f is not None and _max_change(f_hat, g_hat, prev_f, prev_g) < threshold:
                 break
             prev_f, prev_g = f_hat.clone(), g_hat.clone()

@@ -126,6 +126,26 @@ int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const 
                       size_t workspace_bytes, void* stream);
 
 /*
+ * n_steps Jacobi steps of fs_symmetric_step back to back, enqueued by one call: step s runs
+ * with eps[s], alpha[s], damp_f[s], damp_g[s] (HOST arrays of n_steps floats) and reads the
+ * potentials step s-1 wrote (step 0 reads f_hat, g_hat).  Even steps write (f_a, g_a), odd
+ * steps (f_b, g_b); the result of the call is the pair of parity (n_steps - 1) & 1.  The four
+ * work vectors must not alias f_hat / g_hat or each other, except f_a == g_a and f_b == g_b
+ * for the self problem (see fs_symmetric_step).  shift_x / shift_y as there; they apply to
+ * every step whose damping is below 1.
+ * Replaces the iteration of sinkhorn_flashstyle_symmetric (sinkhorn_solvers.py:482-560: the
+ * initial step, the averaged steps over eps_list and the extrapolation step are each one
+ * flashsinkhorn_symmetric_step call there); the Python mirror batches the steps between two
+ * convergence checks into one call.
+ */
+int fs_symmetric_steps(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                       const float* log_a, const float* log_b, float* f_a, float* g_a, float* f_b,
+                       float* g_b, const float* shift_x, const float* shift_y, int64_t n,
+                       int64_t m, int64_t d, const float* eps, const float* alpha,
+                       const float* damp_f, const float* damp_g, int n_steps, float coord_scale,
+                       uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Analytic gradient: grad_x[i,:] = 2*cost_scale*gs*a_i*(x_i - sum_j w_ij y_j),
  * w_i. = softmax_j[(g_j - C_ij)/eps + log_b_j]; grad_y symmetric over i.
  * Standard (unshifted) potentials f, g; x2, y2 = row squared norms; gs is read

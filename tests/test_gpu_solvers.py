@@ -249,6 +249,38 @@ def test_prepared_operands_give_identical_results(n, m, d):
     want = oracle.lse_shifted_fused(x, y, gh, np.log(b), 0.2)
     assert rel_err(o2, want) < 1e-3
 
+@pytest.mark.parametrize("n,m,d", [(700, 500, 64), (300, 260, 200)])
+def test_multi_step_call_equals_single_steps(n, m, d):
+    """fs_symmetric_steps enqueues the same launches as a loop over fs_symmetric_step: the
+    potentials are bit-identical, for a schedule with changing eps, weights and dampings, for
+    odd and even step counts, and for the aliased self problem."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        _symmetric_step_raw, _symmetric_steps_raw)
+    x, y, a, b = inputs(43, n, m, d, scale=2.0 / np.sqrt(d))
+    X, Y, LA, LB = dev(x, y, np.log(a), np.log(b))
+    AL, BE = (X * X).sum(1).contiguous(), (Y * Y).sum(1).contiguous()
+    steps = [(0.8, 1.0, 1.0, 1.0), (0.5, 0.5, 0.9, 0.8), (0.3, 0.5, 0.9, 0.8),
+             (0.2, 0.5, 0.95, 0.85), (0.2, 1.0, 0.95, 0.85)]
+    for k in (1, 4, 5):
+        f, g = -AL, -BE
+        for e, w, df, dg in steps[:k]:
+            f, g = _symmetric_step_raw(X, Y, f, g, LA, LB, e, cost_scale=1.0, alpha=w,
+                                       damping_f=df, damping_g=dg, shift_x=AL, shift_y=BE,
+                                       allow_tf32=False)
+        f2, g2 = _symmetric_steps_raw(X, Y, -AL, -BE, LA, LB, steps[:k], cost_scale=1.0,
+                                      shift_x=AL, shift_y=BE, allow_tf32=False)
+        assert torch.equal(f, f2) and torch.equal(g, g2)
+    # self problem: one half-update per step, one tensor returned twice
+    f0 = -AL
+    sym = [(e, w, df, df) for e, w, df, _ in steps]
+    f, g = f0, f0
+    for e, w, df, _ in sym:
+        f, g = _symmetric_step_raw(X, X, f, g, LA, LA, e, cost_scale=1.0, alpha=w, damping_f=df,
+                                   damping_g=df, shift_x=AL, shift_y=AL, allow_tf32=False)
+    f2, g2 = _symmetric_steps_raw(X, X, f0, f0, LA, LA, sym, cost_scale=1.0, shift_x=AL,
+                                  shift_y=AL, allow_tf32=False)
+    assert f2 is g2 and torch.equal(f, f2)
+
 
 def test_inverse_hvp_against_dense_oracle():
     """Outer CG on the streaming HVP against a dense solve with the oracle's Hessian."""

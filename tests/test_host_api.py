@@ -43,6 +43,16 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
     # outputs may not alias inputs in the Jacobi step
     assert L.fs_symmetric_step(fake, fake, fake, fake, fake, fake, fake, fake, None, None, 8, 8,
                                4, 0.1, 0.5, 1.0, 1.0, 2.0, 0, None, 0, None) == -3
+    # the multi-step loop: host arrays missing, work vectors aliasing each other, nothing to do
+    import ctypes
+    one = (ctypes.c_float * 1)(0.1)
+    fk = [fake + 0x100 * i for i in range(12)]
+    assert L.fs_symmetric_steps(*fk[:10], None, None, 8, 8, 4, None, one, one, one, 1, 2.0, 0,
+                                None, 0, None) == -1
+    assert L.fs_symmetric_steps(*fk[:6], fk[6], fk[7], fk[6], fk[9], None, None, 8, 8, 4, one, one,
+                                one, one, 1, 2.0, 0, None, 0, None) == -3
+    assert L.fs_symmetric_steps(*fk[:10], None, None, 8, 8, 4, one, one, one, one, 0, 2.0, 0,
+                                None, 0, None) == 0
 
 
 def test_workspace_is_deterministic_and_zero_for_small_problems():
