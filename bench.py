@@ -41,10 +41,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2516.6
 EXP2_PER_S = 18.6e12  # v_exp_f32 lanes per second measured on the box (half rate)
 # Memory-side bytes per lse2_kernel launch of the default workload, per operand mode, from two
-# rocprofv3 --pmc runs (FETCH_SIZE 112,324 KiB x 2.0, WRITE_SIZE 12,511 KiB x 1.0; the factors
-# are what the same counters read for the 256 MiB copy of --copy-calibration: 131,094 and
-# 262,144 KiB).  Not measured for the other modes.
-MEASURED_TRAFFIC_BYTES = {"strict": int((112324 * 2.0 + 12511) * 1024)}
+# rocprofv3 --pmc runs (FETCH_SIZE 117,370 KiB x 2.0, WRITE_SIZE 12,508 KiB x 1.0; the factors
+# are what the same counters read for the 256 MiB copy of --copy-calibration: half the bytes
+# copied and all of them).  Not measured for the other modes.
+MEASURED_TRAFFIC_BYTES = {"strict": int((117370 * 2.0 + 12508) * 1024)}
 
 
 def gmm_cloud(rng, n, d, k=8):
