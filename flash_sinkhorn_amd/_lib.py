@@ -26,7 +26,7 @@ FS_FLAG_NO_TILE_SKIP = 32
 # STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" runs fp32 MFMA
 # operands, "bf16x3" the three-plane bf16 split instead.
 STRICT_OPERANDS = os.environ.get("FLASH_SINKHORN_STRICT_OPERANDS", "fp16x2")
-OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5 = range(6)
+OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5, OP_C_TRANSFORM = range(7)
 
 # d <= 128 log-sum-exp kernel: leave out the exponentials of logits tiles that lie 2^40 below
 # the running row maxima (no effect on fp32 sums); False computes every exponential.
@@ -53,6 +53,7 @@ _SIGNATURES = {
     "fs_apply_vec": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + [ctypes.c_int] + _TAIL),
     "fs_apply_mat": (ctypes.c_int, [_P] * 9 + [_I] * 4 + [_F] * 2 + [ctypes.c_int] + _TAIL),
     "fs_mat5": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + _TAIL),
+    "fs_c_transform": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] + _TAIL),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -351,9 +351,14 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
   if (total <= 0) return FS_OK;
 
   if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
-  if (rc == FS_OK) rc = launch_lse_gemm(a, vec, total, st);
+  if (rc == FS_OK) rc = launch_lse_gemm(a, mode, total, st);
   if (rc != FS_OK) return rc;
   const int items0 = a.side[0].nq, items1 = (nsides == 2) ? a.side[1].nq : 0;
+  if (mode == kArgmax) {  // one side; the partial values are already in output units
+    a.out_scale = 1.0f;
+    hipLaunchKernelGGL((finish_argmax_kernel<0>), dim3(ceil_div(items0, 256)), dim3(256), 0, st, a);
+    return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+  }
   hipLaunchKernelGGL((finish_kernel<false>), dim3(ceil_div(items0 + items1, 256)), dim3(256), 0, st,
                      a, cfg.dp, items0, items1);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
@@ -559,8 +564,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const int dp = fam.dp;
   const LseConfig cfg = lse_config(d, flags);
   const bool prepared = (flags & FS_FLAG_OPERANDS_PREPARED) != 0;
-  if ((mode == kLse || mode == kVec) && cfg.gemm)
+  if ((mode == kLse || mode == kVec || mode == kArgmax) && cfg.gemm)
     return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
+  if (mode == kArgmax && fam.sliced) return FS_ERR_UNSUPPORTED;  // d > 128 runs on fp16 planes only
   static const int use_plan_gemm = env_int("FS_PLANGEMM", 1);
   if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
@@ -658,10 +664,17 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
                 : launch_dp<kMat, false>(a, dp, rb, total, st);
       break;
     case kMat5: rc = launch_dp<kMat5, false>(a, dp, rb, total, st); break;
+    case kArgmax: rc = launch_dp<kArgmax, false>(a, dp, rb, total, st); break;
     default: rc = FS_ERR_BAD_ARGUMENT;
   }
   if (rc != FS_OK) return rc;
 
+  if (any_split && mode == kArgmax) {
+    a.out_scale = 1.0f;
+    hipLaunchKernelGGL((finish_argmax_kernel<0>), dim3(ceil_div(a.side[0].nq, 256)), dim3(256), 0, st,
+                       a);
+    return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+  }
   if (any_split) {
     // sides that were not split already wrote their output; give them no items
     const bool has_o = (mode == kMat || mode == kMat5);
@@ -748,6 +761,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     case FS_OP_APPLY_VEC: mode = kVec; either = true; break;
     case FS_OP_APPLY_MAT: mode = kMat; either = true; break;
     case FS_OP_MAT5: mode = kMat5; break;
+    case FS_OP_C_TRANSFORM: mode = kArgmax; break;
     default: return 0;
   }
   // rb may be lowered when two sides share a launch: size for the rb=1 plan too
@@ -761,7 +775,8 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   if (mode == kLse && !fam.sliced)
     planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
-  size_t gemm = ((mode == kLse || mode == kVec) && fam.sliced) ? gemm_ws_bytes(n, m, d, both, either) : 0;
+  size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)
+                    ? gemm_ws_bytes(n, m, d, both, either) : 0;
   if ((mode == kMat || mode == kMat5) && fam.sliced)
     gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
   if (both) return std::max(a + b - planes + 64, gemm);
@@ -937,6 +952,22 @@ int fs_apply_mat(const float* x, const float* y, const float* f_hat, const float
   s.ep.r0 = (axis == 1) ? f_hat : g_hat; s.ep.rc0 = kLog2e / eps;
   s.ep.r1 = (axis == 1) ? log_a : log_b; s.ep.rc1 = kLog2e;
   return run_stream(kMat, sepv, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
+}
+
+int fs_c_transform(const float* x, const float* y, const float* bias, float* min_out,
+                   int64_t* argmin_out, int64_t n, int64_t m, int64_t d, float coord_scale,
+                   uint32_t flags, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !y || !bias || !min_out || !argmin_out) return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  // min_j [-cs2 x.y + bias_j] = -max_j [cs2 x.y - bias_j]
+  Side s = lse_side(x, y, bias, -1.0f, nullptr, 0.f, n, m, coord_scale);
+  s.ep.kind = kEpiArgmax;
+  s.ep.out = min_out;
+  s.ep.idx_out = reinterpret_cast<long long*>(argmin_out);
+  // d > 128 runs on the fp16 planes whatever operand mode is asked for
+  if (d > kMaxStreamD) flags &= ~(uint32_t)(FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS);
+  return run_stream(kArgmax, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream,
+                    flags & ~(uint32_t)FS_FLAG_OPERANDS_PREPARED);
 }
 
 int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_ott,

@@ -28,8 +28,8 @@ constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kNegBig = -1.0e30f;   // finite stand-in for -inf on masked keys
 constexpr float kLazyThresh = 16.0f;  // rescale only when the tile max exceeds 2^16
 
-enum Mode : int { kLse = 0, kVec = 1, kMat = 2, kMat5 = 3 };
-enum EpiKind : int { kEpiLse = 0, kEpiApply = 1, kEpiGrad = 2 };
+enum Mode : int { kLse = 0, kVec = 1, kMat = 2, kMat5 = 3, kArgmax = 4 };
+enum EpiKind : int { kEpiLse = 0, kEpiApply = 1, kEpiGrad = 2, kEpiArgmax = 3 };
 
 // What to do with a finished row (M, s, O[.]) of base-2 soft-max statistics.
 struct Epilogue {
@@ -48,6 +48,8 @@ struct Epilogue {
   const float* w;
   const float* grad_scale;  // 1-element device array or null
   float gcoef;
+  // kEpiArgmax (c-transform): out = -max_j t_ij, idx_out = the smallest j attaining it
+  long long* idx_out;
 };
 
 // One half of a launch: which rows are stationary, which are streamed.
@@ -86,6 +88,7 @@ struct LaunchArgs {
   int vec_ok;    // rows are 16-byte aligned (d % 4 == 0 and aligned bases)
   int nss;       // column-sliced kernels: super-slices of 1536 columns (1 unless d > 1536)
   int pstride;   // GEMM-shaped kernels: words per row of the chunked fp16 planes
+  float out_scale;  // finish_argmax_kernel: units of the partial values (1, or the plane scale)
   float skip_log2;  // lse2_kernel: tiles whose logits all lie this far (base 2, negative) below
                     // the running maxima skip their exponentials; -inf-like to switch it off
 };

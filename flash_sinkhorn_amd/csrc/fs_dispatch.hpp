@@ -23,7 +23,7 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
                             int chunked, hipStream_t st);
 // GEMM-style LSE kernel for 128 < d <= 1536 on chunked fp16 planes; Side::splits counts
 // partial rows (twice the workgroup-level key splits).
-int launch_lse_gemm(const LaunchArgs& a, bool vec, int blocks, hipStream_t st);
+int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st);  // kLse, kVec, kArgmax
 // Plan-matrix products (mat5: with the second stationary operand) for d > 128 on fp16 planes: cb column blocks per wavefront (2, 4 or 6),
 // LaunchArgs::nss column groups.  The value matrix (times an optional per-row scale) is
 // brought into operand order by launch_transpose_planes; partial needs 256 floats.

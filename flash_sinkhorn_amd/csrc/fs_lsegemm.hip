@@ -5,11 +5,13 @@
 
 namespace fs {
 
-int launch_lse_gemm(const LaunchArgs& a, bool vec, int blocks, hipStream_t st) {
-  if (vec)
-    hipLaunchKernelGGL(lse_gemm_kernel<true>, dim3(blocks), dim3(512), 0, st, a);
+int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st) {
+  if (mode == kVec)
+    hipLaunchKernelGGL(lse_gemm_kernel<1>, dim3(blocks), dim3(512), 0, st, a);
+  else if (mode == kArgmax)
+    hipLaunchKernelGGL(lse_gemm_kernel<2>, dim3(blocks), dim3(512), 0, st, a);
   else
-    hipLaunchKernelGGL(lse_gemm_kernel<false>, dim3(blocks), dim3(512), 0, st, a);
+    hipLaunchKernelGGL(lse_gemm_kernel<0>, dim3(blocks), dim3(512), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

@@ -29,8 +29,11 @@ namespace fs {
 constexpr int kGemmRows = 256;   // query rows per workgroup = keys per tile
 constexpr int kGemmCols = 32;    // feature columns per k-step
 
-template <bool VEC>
+// GM: 0 log-sum-exp, 1 plan-vector (VEC), 2 running arg-max of the logits (c-transform).
+template <int GM>
 __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args) {
+  constexpr bool VEC = (GM == 1);
+  constexpr bool AMAX = (GM == 2);
   __shared__ __attribute__((aligned(16))) unsigned lds[2][2 * kGemmRows * 32];
   __shared__ __attribute__((aligned(16))) float lds_v[2][VEC ? kGemmRows : 4];  // v of a key tile
 
@@ -94,6 +97,8 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[qb][st][r] = 0.f;
   float run_m[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f}, run_o[2] = {0.f, 0.f};
+  int best_j[2] = {0, 0};  // AMAX: run_m holds the largest raw value so far, best_j its key
+  if constexpr (AMAX) run_m[0] = run_m[1] = -3.0e38f;
 
   auto swap_halves = [&](float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
@@ -163,6 +168,25 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
       ab[st] = h ? 1.0f : key_bias(sd, j0 + kg * 128 + st * 32 + li, j_end) * inv_lscale;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
+      if constexpr (AMAX) {
+        // keys ascend with st and r inside a lane, tiles ascend: a strict test keeps the
+        // smallest key among equal values
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+          acc[qb][st] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(ab[st], h ? 0.0f : 1.0f, acc[qb][st], 0, 0, 0);
+          const int jb = j0 + kg * 128 + st * 32 + 4 * h;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            if (acc[qb][st][r] > run_m[qb]) {
+              run_m[qb] = acc[qb][st][r];
+              best_j[qb] = jb + 8 * (r / 4) + (r % 4);
+            }
+            acc[qb][st][r] = 0.f;
+          }
+        }
+        continue;
+      }
       const float negm = h ? -run_m[qb] : 1.0f;
       float m = -3.0e38f;
 #pragma unroll
@@ -220,6 +244,23 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
     const int row = row0 + qg * 64 + qb * 32 + li;
+    if constexpr (AMAX) {
+      float best = run_m[qb];
+      int bj = best_j[qb];
+      const float ob = xor32(best);
+      const int oj = __shfl_xor(bj, 32, 64);
+      if (ob > best || (ob == best && oj < bj)) {
+        best = ob;
+        bj = oj;
+      }
+      if (row < sd.nq && h == 0) {
+        const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =
+            has_keys ? make_float2(best * lscale, __builtin_bit_cast(float, bj))
+                     : make_float2(-3.0e38f, __builtin_bit_cast(float, 0x7fffffff));
+      }
+      continue;
+    }
     const float s = run_s[qb] + xor32(run_s[qb]);
     if (row < sd.nq && h == 0) {
       const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;

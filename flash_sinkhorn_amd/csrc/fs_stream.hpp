@@ -174,10 +174,12 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
   }
 
   float run_m[RB], run_s[RB], run_o[RB];
+  int best_j[RB];  // kArgmax: run_m holds the largest value so far, best_j its key
   f32x16 oacc[kHasO ? RB : 1][kHasO ? G::NDB : 1];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    run_m[rb] = 0.f;
+    best_j[rb] = 0;
+    run_m[rb] = (MODE == kArgmax) ? -3.0e38f : 0.f;
     run_s[rb] = 0.f;
     run_o[rb] = 0.f;
     if constexpr (kHasO) {
@@ -297,6 +299,21 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
 #pragma unroll
         for (int kk = 0; kk < G::KK; ++kk)
           acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ya[kk], xs[rb][kk], acc, 0, 0, 0);
+        if constexpr (MODE == kArgmax) {
+          // value = scaled dot + key bias; register r of a lane holds key 8 (r / 4) + 4 h + r % 4
+          // of the sub-tile, ascending in r, and tiles ascend: a strict test keeps the
+          // smallest key among equal values
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
+          const int jb = j_begin + t * G::JT + js * 32 + 4 * h;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            if (acc[r] > run_m[rb]) {
+              run_m[rb] = acc[r];
+              best_j[rb] = jb + 8 * (r / 4) + (r % 4);
+            }
+          }
+          continue;
+        }
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
 
         f32x16 tacc;
@@ -379,10 +396,31 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = row0 + rb * 32 + li;
+    const bool live = row < sd.nq;
+    if constexpr (MODE == kArgmax) {
+      float best = run_m[rb];
+      int bj = best_j[rb];
+      const float ob = xor32(best);
+      const int oj = __shfl_xor(bj, 32, 64);
+      if (ob > best || (ob == best && oj < bj)) {
+        best = ob;
+        bj = oj;
+      }
+      if (live && h == 0) {
+        if (sd.splits == 1) {
+          sd.ep.out[row] = -best;
+          sd.ep.idx_out[row] = bj;
+        } else {
+          const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+          *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =
+              make_float2(best, __builtin_bit_cast(float, bj));
+        }
+      }
+      continue;
+    }
     const float M = run_m[rb];
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float o = run_o[rb] + xor32(run_o[rb]);
-    const bool live = row < sd.nq;
     if (sd.splits == 1) {
       if constexpr (!kHasO) {
         if (live && h == 0) epilogue_scalar(sd.ep, row, M, s, o);
@@ -457,6 +495,27 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
   } else {
     epilogue_scalar(sd.ep, row, M, s, o);
   }
+}
+
+// kArgmax: merge the partial (largest value, key) pairs of the key splits; equal values keep
+// the smaller key.  One thread per row; T only makes this a template (header-defined kernel).
+template <int T>
+__global__ __launch_bounds__(256) void finish_argmax_kernel(const LaunchArgs args) {
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  const Side& sd = args.side[0];
+  if (row >= sd.nq) return;
+  float best = -3.0e38f;
+  int bj = 0x7fffffff;
+  for (int sp = 0; sp < sd.splits; ++sp) {
+    const float2 v = *reinterpret_cast<const float2*>(&sd.part_ms[2 * ((size_t)sp * sd.nq + row)]);
+    const int j = __builtin_bit_cast(int, v.y);
+    if (v.x > best || (v.x == best && j < bj)) {
+      best = v.x;
+      bj = j;
+    }
+  }
+  sd.ep.out[row] = -best * args.out_scale;
+  sd.ep.idx_out[row] = bj;
 }
 
 }  // namespace fs

@@ -16,12 +16,13 @@ from flash_sinkhorn_amd.kernels.apply_flash import (
 from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
     sinkhorn_geomloss_online_grad_sqeuclid,
 )
+from flash_sinkhorn_amd.kernels.c_transform_sqeuclid import c_transform_kernel
 
 __all__ = [
     "epsilon_schedule", "max_diameter",
     "sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric",
     "apply_plan_vec_flashstyle", "apply_plan_mat_flashstyle",
-    "sinkhorn_geomloss_online_grad_sqeuclid",
+    "sinkhorn_geomloss_online_grad_sqeuclid", "c_transform_kernel",
 ]
 
 _BRIDGED = {

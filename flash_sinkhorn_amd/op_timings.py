@@ -3,7 +3,7 @@
 Prints one JSON line per shape with the average launch time (HIP events on the current
 stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop),
 one LSE half-update (2nmd), gradient of one side (4nmd), plan-vector (2nmd), plan-matrix
-(4nmd) and mat5 (6nmd), followed by end-to-end wall times of the five configurations
+(4nmd), mat5 (6nmd) and the hard c-transform (2nmd), followed by end-to-end wall times of the five configurations
 through the public API (solver loops, autograd, CG included).
 """
 from __future__ import annotations
@@ -14,7 +14,7 @@ import time
 
 import torch
 
-from flash_sinkhorn_amd import SamplesLoss
+from flash_sinkhorn_amd import SamplesLoss, c_transform_fwd
 from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating
 from flash_sinkhorn_amd.kernels.apply_flash import (apply_plan_mat_flashstyle,
                                                     apply_plan_vec_flashstyle)
@@ -81,6 +81,7 @@ def kernel_timings(name):
         "apply_mat": (4, lambda: apply_plan_mat_flashstyle(X, Y, fh, gh, la, lb, V, eps=eps,
                                                            axis=1)),
         "mat5": (6, lambda: mat5_sqeuclid(X, Y, fo, go, Am, eps=eps)),
+        "c_transform": (2, lambda: c_transform_fwd(X, Y, g, allow_tf32=False)),
     }
     out = {"shape": name, "n": n, "m": m, "d": d}
     for op, (k, fn) in ops.items():

@@ -65,6 +65,7 @@ extern "C" {
 #define FS_OP_APPLY_VEC 3
 #define FS_OP_APPLY_MAT 4
 #define FS_OP_MAT5 5
+#define FS_OP_C_TRANSFORM 6
 
 int fs_version(void);
 const char* fs_error_string(int code);
@@ -191,6 +192,18 @@ int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_o
             const float* A, const float* x2, const float* y2, float* out, int64_t n, int64_t m,
             int64_t d, float eps, float cost_scale, uint32_t flags, void* workspace,
             size_t workspace_bytes, void* stream);
+
+/*
+ * Hard c-transform, the eps -> 0 counterpart of fs_lse:
+ *   min_out[i] = min_j [-coord_scale x_i.y_j + bias_j],  argmin_out[i] = the smallest j
+ * attaining it (int64).  The caller passes bias_j = cost_scale |y_j|^2 - psi_j and adds
+ * cost_scale |x_i|^2 to min_out.  d <= 128 runs on fp32 MFMA operands, d > 128 on the
+ * two-plane fp16 operands (the operand flags are ignored there).
+ * Replaces c_transform_kernel (kernels/c_transform_sqeuclid.py:219-354, kernel 117-214).
+ */
+int fs_c_transform(const float* x, const float* y, const float* bias, float* min_out,
+                   int64_t* argmin_out, int64_t n, int64_t m, int64_t d, float coord_scale,
+                   uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

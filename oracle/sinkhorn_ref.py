@@ -28,6 +28,10 @@ Pin status (what each function is checked against in tests/test_oracle_*.py):
 * grad_barycentric / grad_plan ... golden vectors from
   FS/testing/reference_sinkhorn.py:195-233 and finite differences of the dual
 * apply_plan_vec / apply_plan_mat / mat5 ... brute-force python loops
+* c_transform / c_transform_cost_grads ... the defining inequalities (c_i + psi_j <= C_ij for
+  every j, equality at the returned j), the nearest-neighbour special case psi = 0, x = y,
+  the reference's own tie construction (FS/testing/test_c_transform.py:179-213) and finite
+  differences of the semi-dual objective
 * LabelCost (OTDD label-augmented cost) ... PARITY UNPINNED: no test or vector in the
   reference covers it; restated from the kernels as written and checked against a brute
   force evaluation of the same formulas
@@ -62,6 +66,8 @@ __all__ = [
     "apply_plan_vec",
     "apply_plan_mat",
     "mat5",
+    "c_transform",
+    "c_transform_cost_grads",
 ]
 
 
@@ -491,3 +497,41 @@ def mat5(x, y, f_ott, g_ott, A, eps, cost_scale=1.0, dtype=np.float64):
     c = sqeuclid_cost(x, y, cost_scale, dtype)
     p = np.exp((np.asarray(f_ott, dtype)[:, None] + np.asarray(g_ott, dtype)[None, :] - c) / eps)
     return (-4.0 * cost_scale / eps) * ((p * (A @ y.T)) @ y)
+
+
+# ---------------------------------------------------------------------------
+# hard c-transform  (FS/c_transform.py, FS/kernels/c_transform_sqeuclid.py)
+# ---------------------------------------------------------------------------
+
+def c_transform(x, y, psi, cost_scale=1.0, dtype=np.float64, chunk=2048):
+    """c_i = min_j [cost_scale*|x_i - y_j|^2 - psi_j] and the smallest j attaining it
+    (FS/c_transform.py:32-112; tie rule FS/kernels/c_transform_sqeuclid.py:150, 203).
+    Evaluated from the differences x_i - y_j, not from the factored form the kernels use."""
+    x = np.asarray(x, dtype)
+    y = np.asarray(y, dtype)
+    psi = np.asarray(psi, dtype)
+    n = x.shape[0]
+    vals = np.empty(n, dtype)
+    idx = np.empty(n, np.int64)
+    for i0 in range(0, n, chunk):
+        diff = x[i0:i0 + chunk, None, :] - y[None, :, :]
+        v = cost_scale * np.einsum("ijk,ijk->ij", diff, diff) - psi[None, :]
+        idx[i0:i0 + chunk] = np.argmin(v, axis=1)  # first occurrence = smallest j
+        vals[i0:i0 + chunk] = np.take_along_axis(v, idx[i0:i0 + chunk, None], axis=1)[:, 0]
+    return vals, idx
+
+
+def c_transform_cost_grads(x, y, psi, a, b, cost_scale=1.0, dtype=np.float64):
+    """Semi-dual objective L = sum_i a_i c_i + sum_j b_j psi_j and its Danskin gradients
+    dL/dx_i = 2 cs a_i (x_i - y_j*(i)),  dL/dpsi_j = b_j - sum_{i: j*(i) = j} a_i
+    (FS/c_transform.py:115-174).  Returns (L, grad_x, grad_psi, argmin)."""
+    x = np.asarray(x, dtype)
+    y = np.asarray(y, dtype)
+    psi = np.asarray(psi, dtype)
+    a = np.asarray(a, dtype)
+    b = np.asarray(b, dtype)
+    vals, idx = c_transform(x, y, psi, cost_scale, dtype)
+    loss = float((a * vals).sum() + (b * psi).sum())
+    grad_x = (2.0 * cost_scale * a)[:, None] * (x - y[idx])
+    grad_psi = b - np.bincount(idx, weights=a, minlength=y.shape[0])
+    return loss, grad_x, grad_psi, idx

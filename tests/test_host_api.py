@@ -43,6 +43,9 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
     # outputs may not alias inputs in the Jacobi step
     assert L.fs_symmetric_step(fake, fake, fake, fake, fake, fake, fake, fake, None, None, 8, 8,
                                4, 0.1, 0.5, 1.0, 1.0, 2.0, 0, None, 0, None) == -3
+    # c-transform: missing output, bad size
+    assert L.fs_c_transform(fake, fake, fake, fake, None, 8, 8, 4, 2.0, 0, None, 0, None) == -1
+    assert L.fs_c_transform(fake, fake, fake, fake, fake, 8, 0, 4, 2.0, 0, None, 0, None) == -2
     # the multi-step loop: host arrays missing, work vectors aliasing each other, nothing to do
     import ctypes
     one = (ctypes.c_float * 1)(0.1)

@@ -316,3 +316,47 @@ def test_inverse_hvp_inverts_the_hvp():
                                            cg_rtol=1e-13, cg_atol=1e-14)
     np.testing.assert_allclose(back, gr, rtol=1e-7, atol=1e-9)
     np.testing.assert_allclose(H, H.T, rtol=1e-6, atol=1e-9)  # a Hessian
+
+
+def test_c_transform_defining_properties():
+    """c_i + psi_j <= C_ij for every j with equality at the returned index; nearest neighbour
+    when psi = 0; the reference's tie construction resolves to the smaller index."""
+    rng = np.random.default_rng(31)
+    n, m, d, cs = 40, 57, 5, 0.5
+    x, y, psi = rng.standard_normal((n, d)), rng.standard_normal((m, d)), rng.standard_normal(m)
+    c, idx = oracle.c_transform(x, y, psi, cs)
+    C = cs * ((x[:, None, :] - y[None, :, :]) ** 2).sum(-1)
+    assert np.all(c[:, None] + psi[None, :] <= C + 1e-12)
+    np.testing.assert_allclose(c + psi[idx], C[np.arange(n), idx], rtol=0, atol=1e-12)
+    c0, i0 = oracle.c_transform(x, x, np.zeros(n), 1.0)
+    np.testing.assert_allclose(c0, 0.0, atol=1e-15)
+    assert np.array_equal(i0, np.arange(n))
+    # brute-force python loop
+    for i in range(0, n, 7):
+        best = min(range(m), key=lambda j: (cs * float(((x[i] - y[j]) ** 2).sum()) - psi[j], j))
+        assert idx[i] == best
+    # two equidistant targets: the smaller index wins (reference test_c_transform.py:179-213)
+    yt = np.zeros((96, 4)); yt[:, 0] = 100.0; yt[0, 0] = 1.0; yt[64, 0] = -1.0
+    _, it = oracle.c_transform(np.zeros((1, 4)), yt, np.zeros(96), 1.0)
+    assert it[0] == 0
+
+
+def test_c_transform_cost_gradients_by_finite_differences():
+    rng = np.random.default_rng(32)
+    n, m, d, cs = 12, 9, 3, 1.0
+    x, y, psi = rng.standard_normal((n, d)), rng.standard_normal((m, d)), rng.standard_normal(m)
+    a = rng.dirichlet(np.ones(n)); b = rng.dirichlet(np.ones(m))
+    L, gx, gp, idx = oracle.c_transform_cost_grads(x, y, psi, a, b, cs)
+    h = 1e-6  # far below the gap to the second-best target, so the minimiser does not move
+    for (i, k) in [(0, 0), (5, 2), (11, 1)]:
+        xp = x.copy(); xp[i, k] += h
+        xm = x.copy(); xm[i, k] -= h
+        fd = (oracle.c_transform_cost_grads(xp, y, psi, a, b, cs)[0]
+              - oracle.c_transform_cost_grads(xm, y, psi, a, b, cs)[0]) / (2 * h)
+        assert abs(fd - gx[i, k]) < 1e-6
+    for j in [0, 4, 8]:
+        pp = psi.copy(); pp[j] += h
+        pm = psi.copy(); pm[j] -= h
+        fd = (oracle.c_transform_cost_grads(x, y, pp, a, b, cs)[0]
+              - oracle.c_transform_cost_grads(x, y, pm, a, b, cs)[0]) / (2 * h)
+        assert abs(fd - gp[j]) < 1e-6
