@@ -450,9 +450,12 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     vt_off[s] = need;
     need += pg_vt_bytes(sides[s].nk, d) + kPgAuxBytes;
   }
-  if (mat5) {  // chunked planes of the second stationary operand and their aux block
+  size_t bounds_off = 0;
+  if (mat5) {  // chunked planes of the second stationary operand, their aux block, row bounds
     q2_off = need;
     need += plane_bytes(sides[0].nq, cfg) + kPlaneAuxBytes;
+    bounds_off = need;
+    need += (((size_t)sides[0].nq + 64) * sizeof(float) + 15) & ~(size_t)15;
   }
   for (int s = 0; s < nsides; ++s) {
     part_off[s] = need;
@@ -493,6 +496,8 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
       sd.q2plane_scale =
           reinterpret_cast<const float*>(base + q2_off + plane_bytes(sd.nq, cfg)) + 2 * 256;
       vec_ok = vec_ok && aligned16(sd.q2);
+      sd.kmax2 = reinterpret_cast<const float*>(base + bounds_off);
+      sd.q2norm2 = sd.kmax2 + 64;
     }
     vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.ep.out);
     blocks[s] = plans[s].igroups * plans[s].splits * ncg;
@@ -514,6 +519,9 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   }
   if (mat5 && rc == FS_OK) {
     const Side& sd = sides[0];
+    float* bounds = reinterpret_cast<float*>(base + bounds_off);
+    rc = launch_mat5_bounds(sd.q2, sd.nq, (int)d, sd.kb1, sd.nk, bounds + 64, bounds, st);
+    if (rc != FS_OK) return rc;
     float* partial = reinterpret_cast<float*>(base + q2_off + plane_bytes(sd.nq, cfg));
     rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
@@ -543,7 +551,7 @@ size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bool
   LseConfig c;
   c.gemm = true; c.prec = 3; c.dp = chunked_stride(d); c.np = 2;
   size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
-  if (mat5) planes += plane_bytes(n, c) + kPlaneAuxBytes;
+  if (mat5) planes += plane_bytes(n, c) + kPlaneAuxBytes + ((size_t)n + 64) * sizeof(float) + 16;
   int cb, ncg, dpo;
   pg_columns(d, cb, ncg, dpo);
   auto side = [&](int64_t nq, int64_t nk) {

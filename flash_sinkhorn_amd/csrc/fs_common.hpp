@@ -76,6 +76,8 @@ struct Side {
   const unsigned* q2planes; // plan_gemm_kernel, mat5: chunked fp16 planes of q2
   const float* q2plane_scale;  // scale of q2's planes [1]
   const float* kplane_scale;   // scale of the key matrix alone [1]
+  const float* q2norm2;        // mat5: |q2_i|^2 per row [nq]
+  const float* kmax2;          // mat5: 64 partial maxima of |k_j|^2
   float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;

@@ -28,6 +28,9 @@ int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st); 
 // LaunchArgs::nss column groups.  The value matrix (times an optional per-row scale) is
 // brought into operand order by launch_transpose_planes; partial needs 256 floats.
 int launch_plan_gemm(const LaunchArgs& a, bool mat5, int cb, int blocks, hipStream_t st);
+// mat5: squared row norms of q2 and the largest entry of k2 (= squared row norms of the keys).
+int launch_mat5_bounds(const float* q2, int nq, int d, const float* k2, long long nk, float* q2norm2,
+                       float* kmax2, hipStream_t st);
 int launch_transpose_planes(const float* src, const float* rowscale, unsigned* dst, int rows, int d,
                             int nkb, int ncb, float* partial, float* scale_out, hipStream_t st);
 int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, int blocks, hipStream_t st);

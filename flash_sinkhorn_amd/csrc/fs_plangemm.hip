@@ -22,6 +22,13 @@ int launch_plan_gemm(const LaunchArgs& a, bool mat5, int cb, int blocks, hipStre
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
+int launch_mat5_bounds(const float* q2, int nq, int d, const float* k2, long long nk, float* q2norm2,
+                       float* kmax2, hipStream_t st) {
+  hipLaunchKernelGGL(rownorm2_kernel, dim3((nq + 3) / 4), dim3(256), 0, st, q2, nq, d, q2norm2);
+  hipLaunchKernelGGL(vecmax_kernel, dim3(64), dim3(256), 0, st, k2, nk, kmax2);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
 int launch_transpose_planes(const float* src, const float* rowscale, unsigned* dst, int rows, int d,
                             int nkb, int ncb, float* partial, float* scale_out, hipStream_t st) {
   hipLaunchKernelGGL(absmax_rows_kernel, dim3(256), dim3(256), 0, st, src, (long long)rows, d,

@@ -21,8 +21,9 @@
 //
 // MAT5 (sum_j P_ij <A_i, y_j> y_j): the k-loop also accumulates T = A K^T from planes of A
 // staged next to the query rows, and the probabilities are multiplied by T before they go to
-// LDS.  |T| <= d * 2^30 in plane units, so a power-of-two factor 2^(-23 - ceil(log2 d))
-// keeps |p T| within 2^15 whatever the data; it is divided out with the plane scales at the end.
+// LDS.  |T_ij| <= |A_i| max_j |y_j| (Cauchy-Schwarz), so a per-row power of two taken from
+// that bound keeps |p T| within 2^15 whatever the data and as high in the fp16 range as a
+// safe bound allows; it is divided out with the plane scales at the end.
 //
 // Operand order of the key axis: accumulator register 8 s + e (s = 0, 1; e = 0..7) of lane
 // (li, h) of a 32 x 32 logits tile holds key 8 (2 s + e / 4) + 4 h + e % 4 of the block, so
@@ -120,6 +121,32 @@ __global__ __launch_bounds__(256) void transpose_planes_f16_kernel(
   o[64] = u32x4{lo[0], lo[1], lo[2], lo[3]};
 }
 
+// MAT5 helpers: out[r] = |src[r, :]|^2 (one wavefront per row), and 64 partial maxima of v.
+__global__ __launch_bounds__(256) void rownorm2_kernel(const float* __restrict__ src, int rows,
+                                                       int d, float* __restrict__ out) {
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const float* p = src + (size_t)r * (size_t)d;
+  float s = 0.f;
+  for (int c = threadIdx.x & 63; c < d; c += 64) s = __builtin_fmaf(p[c], p[c], s);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+  if ((threadIdx.x & 63) == 0) out[r] = s;
+}
+
+__global__ __launch_bounds__(256) void vecmax_kernel(const float* __restrict__ v, long long cnt,
+                                                     float* __restrict__ out) {  // out[gridDim.x]
+  __shared__ float red[4];
+  float m = 0.f;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < cnt; i += 256LL * gridDim.x)
+    m = fmaxf(m, v[i]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
 template <int CB, bool MAT5>
 __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args) {
   // stage rows: 32 query rows, (MAT5) 32 rows of the second stationary operand, 256 key rows
@@ -157,9 +184,18 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
 
   const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
   const float inv_lscale = 1.0f / lscale;
-  // MAT5: 2^(-23 - ceil(log2 d)) bounds |T| * t_unit by 2^7
-  const int lg_d = 32 - __clz(max(d, 2) - 1);
-  const float t_unit = __builtin_bit_cast(float, (unsigned)(127 - 23 - lg_d) << 23);
+  // MAT5: per-row power of two with |T_ij| * t_unit <= 2^7 from |T_ij| <= |A_i| max_j |y_j|
+  // (in plane units; sd.q2norm2 = |A_i|^2, sd.kmax2 = 64 partial maxima of |y_j|^2, fp32 rows)
+  float t_unit = 1.0f;
+  if constexpr (MAT5) {
+    const float a2 = (row < sd.nq) ? sd.q2norm2[row] : 0.f;
+    float km = sd.kmax2[lane];  // 64 partial maxima
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) km = fmaxf(km, __shfl_xor(km, o, 64));
+    const float bound = sqrtf(a2 * km) * sd.q2plane_scale[0] * sd.kplane_scale[0] * 1.0001f;
+    const int e = (int)((__builtin_bit_cast(unsigned, bound) >> 23) & 255u);  // bound < 2^(e-126)
+    if (e > 0 && e < 255) t_unit = __builtin_bit_cast(float, (unsigned)min(254, max(1, 127 + 7 - (e - 126))) << 23);
+  }
 
   // ---- loaders: wavefront w brings key rows [32 w, 32 w + 32) of the tile (4 instructions of
   // 8 rows), wavefronts 0-3 also 8 query rows each, wavefronts 4-7 (MAT5) 8 rows of A ----
