@@ -563,6 +563,129 @@ size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bool
   return planes + side(n, m) + 64;
 }
 
+// ---- d <= 64 plan-matrix / plan-vector products on fp16 planes (plan_tile_kernel) ----
+size_t pt_vt_bytes(int64_t nk, int dpk) {  // V^T operands: 32-key blocks x 32-column blocks x 4 KiB
+  return (size_t)ceil_div(nk, 64) * 2 * (size_t)((dpk + 31) / 32) * 4096;
+}
+
+// two row blocks per wavefront once the grid is large enough to fill the chip either way
+int pt_rows_per_wave(int64_t nq) { return nq >= 16384 ? 2 : 1; }
+
+// Workspace: plane region of x and y (the layout of lse2_kernel, so prepared planes serve),
+// then per side the V^T operands with their aux block (kMat), then per side the partial rows.
+int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig& cfg,
+                  const Family& fam, bool prepared, void* ws, size_t ws_bytes, hipStream_t st) {
+  PlaneSet ps;
+  int rc = side_plane_set(sides, nsides, cfg, ps);
+  if (rc != FS_OK) return rc;
+  const int dpk = cfg.dp;  // 16, 32 or 64
+  static const int rb_env = env_int("FS_PT_RB", 0);
+  int rb = 2;
+  for (int s = 0; s < nsides; ++s) rb = std::min(rb, pt_rows_per_wave(sides[s].nq));
+  if (rb_env > 0) rb = std::min(rb_env, 2);
+  size_t need = ps.end;
+  SidePlan plans[2];
+  size_t vt_off[2] = {0, 0}, part_off[2];
+  for (int s = 0; s < nsides; ++s) {
+    plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam, rb);
+    if (mode == kMat) {
+      vt_off[s] = need;
+      need += pt_vt_bytes(sides[s].nk, dpk) + kPgAuxBytes;
+    }
+  }
+  for (int s = 0; s < nsides; ++s) {
+    part_off[s] = need;
+    need += side_ws_floats(mode, plans[s], sides[s].nq, dpk) * sizeof(float);
+  }
+  if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
+  char* base = static_cast<char*>(ws);
+
+  LaunchArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.d = (int)d;
+  bool vec_ok = (d % 4 == 0);
+  bool any_split = false;
+  int blocks[2] = {0, 0};
+  for (int s = 0; s < nsides; ++s) {
+    Side& sd = sides[s];
+    const SidePlan& p = plans[s];
+    sd.splits = p.splits;
+    sd.chunk = p.chunk;
+    sd.igroups = p.igroups;
+    sd.part_ms = nullptr;
+    sd.part_o = nullptr;
+    if (p.splits > 1) {
+      any_split = true;
+      sd.part_ms = reinterpret_cast<float*>(base + part_off[s]);
+      sd.part_o = sd.part_ms + (((size_t)p.splits * (size_t)sd.nq * 2 + 3) & ~(size_t)3);
+    }
+    sd.plane_scale = plane_scales(ps, ws);
+    sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
+    sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
+    if (mode == kMat) {
+      sd.vplanes = reinterpret_cast<const unsigned*>(base + vt_off[s]);
+      sd.vplane_scale =
+          reinterpret_cast<const float*>(base + vt_off[s] + pt_vt_bytes(sd.nk, dpk)) + 256;
+      vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.ep.out);
+    }
+    blocks[s] = p.igroups * p.splits;
+    a.side[s] = sd;
+  }
+  if (nsides == 1) a.side[1] = a.side[0];
+  a.blocks0 = blocks[0];
+  a.vec_ok = vec_ok ? 1 : 0;
+  const int total = blocks[0] + blocks[1];
+  if (total <= 0) return FS_OK;
+
+  if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
+  for (int s = 0; s < nsides && rc == FS_OK && mode == kMat; ++s) {
+    const Side& sd = sides[s];
+    float* aux = reinterpret_cast<float*>(base + vt_off[s] + pt_vt_bytes(sd.nk, dpk));
+    rc = launch_transpose_planes(sd.v ? sd.v : sd.k, sd.vscale,
+                                 reinterpret_cast<unsigned*>(base + vt_off[s]), sd.nk, (int)d,
+                                 ceil_div(sd.nk, 64) * 2, (dpk + 31) / 32, aux, aux + 256, st);
+  }
+  if (rc == FS_OK) rc = launch_plan_tile(a, mode, dpk, rb, total, st);
+  if (rc != FS_OK) return rc;
+  if (any_split) {
+    const bool has_o = (mode == kMat);
+    const int per_row = has_o ? dpk / 4 : 1;
+    int items[2] = {0, 0};
+    for (int s = 0; s < nsides; ++s)
+      items[s] = (a.side[s].splits > 1) ? a.side[s].nq * per_row : 0;
+    LaunchArgs f = a;
+    if (items[0] == 0 && nsides == 2) {  // only the second side needs merging
+      f.side[0] = a.side[1];
+      items[0] = items[1];
+      items[1] = 0;
+    }
+    const int grid = ceil_div(items[0] + items[1], 256);
+    if (has_o)
+      hipLaunchKernelGGL((finish_kernel<true>), dim3(grid), dim3(256), 0, st, f, dpk, items[0], items[1]);
+    else
+      hipLaunchKernelGGL((finish_kernel<false>), dim3(grid), dim3(256), 0, st, f, dpk, items[0], items[1]);
+    if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
+  }
+  return FS_OK;
+}
+
+size_t pt_ws_bytes(int mode, int64_t n, int64_t m, int64_t d, bool both, bool either,
+                   const Family& fam) {
+  const int dpk = std::max(padded_d(d), 16);
+  const size_t planes =
+      (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (dpk / 2) * 4 + 64 + kPlaneAuxBytes;
+  auto side = [&](int64_t nq, int64_t nk) {
+    size_t b = 0;
+    for (int rb = 1; rb <= 2; ++rb)
+      b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dpk) * sizeof(float));
+    if (mode == kMat) b += pt_vt_bytes(nk, dpk) + kPgAuxBytes;
+    return b + 16;
+  };
+  if (both) return planes + side(n, m) + side(m, n) + 64;
+  if (either) return planes + std::max(side(n, m), side(m, n)) + 64;
+  return planes + side(n, m) + 64;
+}
+
 // Plans, carves the workspace, launches the streaming kernel over one or two
 // sides and, when keys were split, the merge kernel.
 int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws, size_t ws_bytes,
@@ -578,6 +701,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   static const int use_plan_gemm = env_int("FS_PLANGEMM", 1);
   if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
+  static const int use_plan_tile = env_int("FS_PLANTILE", 1);
+  if ((mode == kMat || mode == kVec) && !fam.sliced && cfg.prec == 3 && cfg.dp <= 64 && use_plan_tile)
+    return run_plan_tile(mode, sides, nsides, d, cfg, fam, prepared, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -787,6 +913,8 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
   if ((mode == kMat || mode == kMat5) && fam.sliced)
     gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
+  if ((mode == kMat || mode == kVec) && !fam.sliced && std::max(padded_d(d), 16) <= 64)
+    gemm = pt_ws_bytes(mode, n, m, d, both, either, fam);
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);
   return std::max(a + 64, gemm);

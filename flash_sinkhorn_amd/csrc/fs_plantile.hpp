@@ -1,0 +1,346 @@
+// Plan-times-matrix and plan-times-vector products for d <= 128 on fp16 planes
+// (gradient, apply_plan_mat, apply_plan_vec in the default operand mode).
+//
+// Same decomposition as lse2_kernel: a workgroup of 4 wavefronts shares key tiles of 64 keys,
+// brought into LDS by direct global->LDS loads of the two-plane fp16 rows (three buffers, the
+// tile two ahead in flight, XOR-swizzled 16-byte slots), and every wavefront owns RB blocks
+// of 32 query rows whose planes never leave its registers.  Per block and 32-key sub-tile:
+//   logits   3 fp16 MFMA products per 16 columns, then one fp32 MFMA that adds the key bias
+//            and subtracts the block's running maximum (both in units of the raw products);
+//   soft-max lane-private and lazy: the running maximum moves only when a tile exceeds it by
+//            2^8, so the probabilities stay below 2^8 and are fp16-safe;
+//   values   (kMat) the lane's own 16 probabilities are, as they stand, its B operands of the
+//            two 16-key steps; they are split into hi / lo fp16 and multiplied with the V^T
+//            operands that transpose_planes_f16_kernel laid out in MFMA order in global memory
+//            (one coalesced 1 KiB read per instruction, shared by the four wavefronts through
+//            L1): three products per column block and step.  (kVec) a weighted sum with the
+//            64 values of v of the tile, staged in LDS.
+// Row sums are exact fp32 VALU sums.  The key bias of the next tile travels in two registers
+// per lane; nothing in the loop needs a second barrier.
+#pragma once
+
+#include <type_traits>
+
+#include "fs_common.hpp"
+#include "fs_stream.hpp"
+
+namespace fs {
+
+constexpr int kPtKeys = 64;            // keys per tile
+constexpr float kPtLazyThresh = 8.0f;  // probabilities stay below 2^8
+
+template <int DP, int RB, int MODE>
+__global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args) {
+  static_assert(MODE == kMat || MODE == kVec, "plan_tile_kernel: kMat or kVec");
+  static_assert(DP == 16 || DP == 32 || DP == 64, "wider rows do not fit the register budget");
+  constexpr int KK16 = DP / 16;                 // 16-column steps of the logits
+  constexpr int NCB = (DP + 31) / 32;           // 32-column output blocks
+  constexpr int ROWW = DP;                      // words per two-plane row
+  constexpr int PPR = ROWW / 4;                 // 16-byte pieces per row
+  constexpr int PER_THREAD = kPtKeys * PPR / 256;
+  static_assert(kPtKeys * PPR % 256 == 0, "a tile is a whole number of load instructions");
+
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[3][kPtKeys * ROWW];
+  __shared__ __attribute__((aligned(16))) float lds_v[3][MODE == kVec ? kPtKeys : 4];
+
+  int bid = blockIdx.x;
+  const bool second = bid >= args.blocks0;
+  if (second) bid -= args.blocks0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const int d = args.d;
+  const bool vec_ok = args.vec_ok != 0;
+
+  const int split = bid % sd.splits;
+  const int ig = bid / sd.splits;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int h = lane >> 5;
+  const int row0 = (ig * 4 + wave) * (32 * RB);
+  const int j_begin = split * sd.chunk;
+  const int j_end = min(sd.nk, j_begin + sd.chunk);
+  const int ntiles = (j_end > j_begin) ? (j_end - j_begin + kPtKeys - 1) / kPtKeys : 0;
+
+  const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  const float inv_lscale = 1.0f / lscale;
+
+  // ---- stationary query planes: [block][plane][16-column step] ----
+  u32x4 xq[RB][2][KK16];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = min(row0 + rb * 32 + li, sd.nq - 1);
+    const unsigned* qrow = sd.qplanes + (size_t)row * (size_t)ROWW;
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk)
+        xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qrow + p * (DP / 2) + 8 * kk + 4 * h);
+  }
+
+  // ---- key tiles: lane idx of instruction c fills LDS slot idx and fetches the piece that
+  // belongs there (slot = piece ^ swz(row)) ----
+  auto swz = [&](int r) {
+    return PPR >= 16 ? (r & 15) : (PPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3));
+  };
+  const unsigned* kp[PER_THREAD];
+#pragma unroll
+  for (int c = 0; c < PER_THREAD; ++c) {
+    const int idx = tid + 256 * c;
+    const int r = idx / PPR;
+    const int piece = (idx % PPR) ^ swz(r);
+    kp[c] = sd.kplanes + (size_t)(j_begin + r) * (size_t)ROWW + piece * 4;
+  }
+  auto issue_tile = [&](int buf) {  // the next tile in sequence; the planes end in zero rows
+#pragma unroll
+    for (int c = 0; c < PER_THREAD; ++c) {
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)kp[c],
+          (__attribute__((address_space(3))) void*)(&lds_k[buf][(c * 256 + wave * 64) * 4]), 16, 0,
+          0);
+      kp[c] += kPtKeys * ROWW;
+    }
+  };
+  auto wait_newest_tile_only = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_THREAD & 15));
+  };
+  auto lds_piece = [&](const unsigned* tile, int r, int piece) {
+    return *reinterpret_cast<const u32x4*>(tile + r * ROWW + ((piece ^ swz(r)) << 2));
+  };
+  // bias of key j (lanes with h == 0 feed it to the fp32 MFMA), in units of the raw products
+  auto bias_of = [&](int j) {
+    return fmaxf(key_bias(sd, j, j_end) * inv_lscale, -3.0e38f);
+  };
+
+  // ---- V^T operands (kMat): unit (32-key block, column block, step) = 128 pieces ----
+  const u32x4* vt = reinterpret_cast<const u32x4*>(sd.vplanes);
+  auto load_vt = [&](u32x4 (&a)[NCB][2][2], int kb) {
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const u32x4* p = vt + (((size_t)kb * NCB + cb) * 2 + s) * 128 + lane;
+        a[cb][s][0] = p[0];
+        a[cb][s][1] = p[64];
+      }
+  };
+
+  f32x16 oacc[MODE == kMat ? RB : 1][MODE == kMat ? NCB : 1];
+  float run_m[RB], run_s[RB], run_o[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    run_m[rb] = 0.f;
+    run_s[rb] = 0.f;
+    run_o[rb] = 0.f;
+    if constexpr (MODE == kMat) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[rb][cb][r] = 0.f;
+    }
+  }
+
+  // ---- prologue: tiles 0 and 1 on their way, bias (and v) of tile 0 ----
+  float ab_next[2];
+  ab_next[0] = bias_of(j_begin + li);
+  ab_next[1] = bias_of(j_begin + 32 + li);
+  if constexpr (MODE == kVec) {
+    if (tid < kPtKeys) lds_v[0][tid] = (j_begin + tid < j_end) ? sd.v[j_begin + tid] : 0.f;
+  }
+  if (ntiles > 0) {
+    issue_tile(0);
+    issue_tile(1);
+    wait_newest_tile_only();
+  }
+  __syncthreads();
+
+  auto swap_halves = [&](float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  };
+
+  int buf = 0;
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = j_begin + t * kPtKeys;
+    const int nbuf = (buf == 2) ? 0 : buf + 1;
+    const int n2buf = (nbuf == 2) ? 0 : nbuf + 1;
+    const float ab_cur[2] = {ab_next[0], ab_next[1]};
+    // loads in program order: bias (and v) of tile t + 1, V^T of this tile, key tile t + 2;
+    // a wait for an older load never has to wait for a younger one
+    ab_next[0] = bias_of(j0 + kPtKeys + li);
+    ab_next[1] = bias_of(j0 + kPtKeys + 32 + li);
+    float v_next = 0.f;
+    if constexpr (MODE == kVec) {
+      if (tid < kPtKeys && j0 + kPtKeys + tid < j_end) v_next = sd.v[j0 + kPtKeys + tid];
+    }
+    const unsigned* tile = lds_k[buf];
+
+#pragma unroll
+    for (int js = 0; js < 2; ++js) {
+      u32x4 va[MODE == kMat ? NCB : 1][2][2];
+      if constexpr (MODE == kMat) load_vt(va, (j0 >> 5) + js);
+      if (js == 1) issue_tile(n2buf);  // tile t + 2, after the last register loads of tile t
+      __builtin_amdgcn_sched_barrier(0);
+
+      // A operands of the logits: key row js*32 + li, [plane][step]
+      u32x4 kq[2][KK16];
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int kk = 0; kk < KK16; ++kk)
+          kq[p][kk] = lds_piece(tile, js * 32 + li, p * (DP / 8) + 2 * kk + h);
+      const float ab = h ? 1.0f : ab_cur[js];
+      float vj[MODE == kVec ? 16 : 1];
+      if constexpr (MODE == kVec) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const float4 v = *reinterpret_cast<const float4*>(&lds_v[buf][js * 32 + 8 * g + 4 * h]);
+          vj[4 * g + 0] = v.x;
+          vj[4 * g + 1] = v.y;
+          vj[4 * g + 2] = v.z;
+          vj[4 * g + 3] = v.w;
+        }
+      }
+
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        // products lo*hi, hi*lo, hi*hi
+#pragma unroll
+        for (int prod = 0; prod < 3; ++prod) {
+          const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
+#pragma unroll
+          for (int kk = 0; kk < KK16; ++kk)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kq[pk][kk]),
+                                                         __builtin_bit_cast(f16x8, xq[rb][pq][kk]),
+                                                         acc, 0, 0, 0);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
+
+        // ---- lazy lane-private soft-max (the two half-waves of a query share run_m) ----
+        float tmax = fmaxf(acc[0], acc[1]);
+#pragma unroll
+        for (int r = 2; r < 16; ++r) tmax = fmaxf(tmax, acc[r]);
+        const bool first = (t == 0 && js == 0);
+        float cc = 0.f;
+        if (first || wave_any(tmax * lscale > kPtLazyThresh)) {
+          float a = tmax, b = tmax;
+          swap_halves(a, b);
+          const float tm = fmaxf(a, b);
+          const float delta = (first || tm * lscale > kPtLazyThresh) ? tm : 0.f;
+          cc = -delta * lscale;
+          const float resc = first ? 0.f : fast_exp2(cc);
+          run_m[rb] += delta;
+          run_s[rb] *= resc;
+          run_o[rb] *= resc;
+          if constexpr (MODE == kMat) {
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) oacc[rb][cb][r] *= resc;
+          }
+        }
+        float p[16];
+        float ps = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, cc));
+          ps += p[r];
+        }
+        run_s[rb] += ps;
+        if constexpr (MODE == kVec) {
+          float po = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) po = __builtin_fmaf(p[r], vj[r], po);
+          run_o[rb] += po;
+        }
+        if constexpr (MODE == kMat) {
+          // registers 8 s .. 8 s + 7 are this lane's B operand of 16-key step s
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            unsigned hi[4], lo[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float x0 = p[8 * s + 2 * e], x1 = p[8 * s + 2 * e + 1];
+              hi[e] = pack_f16(x0, x1);
+              const f16x2 hh = __builtin_bit_cast(f16x2, hi[e]);
+              lo[e] = pack_f16(x0 - (float)hh[0], x1 - (float)hh[1]);
+            }
+            const f16x8 bh = __builtin_bit_cast(f16x8, u32x4{hi[0], hi[1], hi[2], hi[3]});
+            const f16x8 bl = __builtin_bit_cast(f16x8, u32x4{lo[0], lo[1], lo[2], lo[3]});
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+              oacc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, va[cb][s][1]), bh, oacc[rb][cb], 0, 0, 0);
+              oacc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, va[cb][s][0]), bl, oacc[rb][cb], 0, 0, 0);
+              oacc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, va[cb][s][0]), bh, oacc[rb][cb], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+
+    if constexpr (MODE == kVec) {
+      if (tid < kPtKeys) lds_v[nbuf][tid] = v_next;
+    }
+    // tile t + 1 has landed (only the loads of tile t + 2 may still be in flight); after the
+    // barrier it is visible and every wavefront is done reading tile t
+    wait_newest_tile_only();
+    __syncthreads();
+    buf = nbuf;
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // tiles fetched past the chunk: let them land before exit
+
+  // ---- merge the two half-waves of each query, then finish or spill ----
+  const float inv_vs = (MODE == kMat) ? 1.0f / sd.vplane_scale[0] : 1.0f;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = row0 + rb * 32 + li;
+    const bool live = row < sd.nq;
+    const float M = (ntiles > 0) ? run_m[rb] * lscale : kNegBig;
+    const float s = run_s[rb] + xor32(run_s[rb]);
+    const float o = run_o[rb] + xor32(run_o[rb]);
+    if (sd.splits == 1) {
+      if constexpr (MODE == kVec) {
+        if (live && h == 0) epilogue_scalar(sd.ep, row, M, s, o);
+      } else {
+        if (live) {
+#pragma unroll
+          for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+              const int col = cb * 32 + 8 * q4 + 4 * h;
+              const float4 O =
+                  make_float4(oacc[rb][cb][4 * q4] * inv_vs, oacc[rb][cb][4 * q4 + 1] * inv_vs,
+                              oacc[rb][cb][4 * q4 + 2] * inv_vs, oacc[rb][cb][4 * q4 + 3] * inv_vs);
+              epilogue_vec4(sd.ep, sd.q, d, vec_ok, row, col, M, s, O);
+            }
+        }
+      }
+    } else if (live) {
+      const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+      if (h == 0) {
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M, s);
+        if constexpr (MODE == kVec) sd.part_o[pr] = o;
+      }
+      if constexpr (MODE == kMat) {
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const int col = cb * 32 + 8 * q4 + 4 * h;
+            if (DP % 32 == 0 || col < DP) {
+              *reinterpret_cast<float4*>(&sd.part_o[pr * DP + col]) =
+                  make_float4(oacc[rb][cb][4 * q4] * inv_vs, oacc[rb][cb][4 * q4 + 1] * inv_vs,
+                              oacc[rb][cb][4 * q4 + 2] * inv_vs, oacc[rb][cb][4 * q4 + 3] * inv_vs);
+            }
+          }
+      }
+    }
+  }
+}
+
+}  // namespace fs
