@@ -563,7 +563,7 @@ size_t pg_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bool
   return planes + side(n, m) + 64;
 }
 
-// ---- d <= 64 plan-matrix / plan-vector products on fp16 planes (plan_tile_kernel) ----
+// ---- d <= 128 plan-matrix / plan-vector products and c-transform on fp16 planes (plan_tile_kernel) ----
 size_t pt_vt_bytes(int64_t nk, int dpk) {  // V^T operands: 32-key blocks x 32-column blocks x 4 KiB
   return (size_t)ceil_div(nk, 64) * 2 * (size_t)((dpk + 31) / 32) * 4096;
 }
@@ -578,11 +578,12 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   PlaneSet ps;
   int rc = side_plane_set(sides, nsides, cfg, ps);
   if (rc != FS_OK) return rc;
-  const int dpk = cfg.dp;  // 16, 32 or 64
+  const int dpk = cfg.dp;  // 16, 32, 64 or 128
   static const int rb_env = env_int("FS_PT_RB", 0);
   int rb = 2;
   for (int s = 0; s < nsides; ++s) rb = std::min(rb, pt_rows_per_wave(sides[s].nq));
   if (rb_env > 0) rb = std::min(rb_env, 2);
+  if (dpk == 128) rb = 1;
   size_t need = ps.end;
   SidePlan plans[2];
   size_t vt_off[2] = {0, 0}, part_off[2];
@@ -647,6 +648,12 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   }
   if (rc == FS_OK) rc = launch_plan_tile(a, mode, dpk, rb, total, st);
   if (rc != FS_OK) return rc;
+  if (any_split && mode == kArgmax) {
+    a.out_scale = 1.0f;
+    hipLaunchKernelGGL((finish_argmax_kernel<0>), dim3(ceil_div(a.side[0].nq, 256)), dim3(256), 0, st,
+                       a);
+    return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+  }
   if (any_split) {
     const bool has_o = (mode == kMat);
     const int per_row = has_o ? dpk / 4 : 1;
@@ -702,8 +709,15 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   static const int use_plan_tile = env_int("FS_PLANTILE", 1);
-  if ((mode == kMat || mode == kVec) && !fam.sliced && cfg.prec == 3 && cfg.dp <= 64 && use_plan_tile)
-    return run_plan_tile(mode, sides, nsides, d, cfg, fam, prepared, ws, ws_bytes, st);
+  if ((mode == kMat || mode == kVec || mode == kArgmax) && !fam.sliced && use_plan_tile &&
+      (cfg.prec == 3 || cfg.prec == 1)) {
+    // the reduced mode runs on the fp16 planes too (same speed, smaller error); planes a caller
+    // prepared for it are bf16 and are not used here
+    const bool reduced = (cfg.prec == 1);
+    const LseConfig pcfg = reduced ? lse_config(d, flags & ~(uint32_t)FS_FLAG_REDUCED_OPERANDS) : cfg;
+    if (pcfg.prec == 3)
+      return run_plan_tile(mode, sides, nsides, d, pcfg, fam, prepared && !reduced, ws, ws_bytes, st);
+  }
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -913,7 +927,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
   if ((mode == kMat || mode == kMat5) && fam.sliced)
     gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
-  if ((mode == kMat || mode == kVec) && !fam.sliced && std::max(padded_d(d), 16) <= 64)
+  if ((mode == kMat || mode == kVec || mode == kArgmax) && !fam.sliced)
     gemm = pt_ws_bytes(mode, n, m, d, both, either, fam);
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);

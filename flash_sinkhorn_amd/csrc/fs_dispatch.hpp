@@ -33,8 +33,8 @@ int launch_mat5_bounds(const float* q2, int nq, int d, const float* k2, long lon
                        float* kmax2, hipStream_t st);
 int launch_transpose_planes(const float* src, const float* rowscale, unsigned* dst, int rows, int d,
                             int nkb, int ncb, float* partial, float* scale_out, hipStream_t st);
-// Plan-matrix (kMat) and plan-vector (kVec) products for d <= 64 on two-plane fp16 rows
-// (dp in {16, 32, 64}, rb row blocks per wavefront in {1, 2}).
+// Plan-matrix (kMat), plan-vector (kVec) products and running arg-max (kArgmax) for d <= 128 on
+// two-plane fp16 rows (dp in {16, 32, 64, 128}; rb row blocks per wavefront in {1, 2}, 1 at 128).
 int launch_plan_tile(const LaunchArgs& a, int mode, int dp, int rb, int blocks, hipStream_t st);
 int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, int blocks, hipStream_t st);
 

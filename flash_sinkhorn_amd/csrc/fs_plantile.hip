@@ -1,4 +1,4 @@
-// Launches of the d <= 64 plan-product kernel on fp16 planes.
+// Launches of the d <= 128 plan-product / c-transform kernel on fp16 planes.
 #include "fs_plantile.hpp"
 
 #include "fs_dispatch.hpp"
@@ -20,6 +20,9 @@ static int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_
     case 16: return launch_rb<16, MODE>(a, rb, blocks, st);
     case 32: return launch_rb<32, MODE>(a, rb, blocks, st);
     case 64: return launch_rb<64, MODE>(a, rb, blocks, st);
+    case 128:
+      hipLaunchKernelGGL((plan_tile_kernel<128, 1, MODE>), dim3(blocks), dim3(256), 0, st, a);
+      return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
   }
   return FS_ERR_UNSUPPORTED;
 }
@@ -27,6 +30,7 @@ static int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_
 int launch_plan_tile(const LaunchArgs& a, int mode, int dp, int rb, int blocks, hipStream_t st) {
   if (mode == kMat) return launch_dp<kMat>(a, dp, rb, blocks, st);
   if (mode == kVec) return launch_dp<kVec>(a, dp, rb, blocks, st);
+  if (mode == kArgmax) return launch_dp<kArgmax>(a, dp, rb, blocks, st);
   return FS_ERR_BAD_ARGUMENT;
 }
 

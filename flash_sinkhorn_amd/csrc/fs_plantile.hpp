@@ -1,7 +1,8 @@
-// Plan-times-matrix and plan-times-vector products for d <= 128 on fp16 planes
-// (gradient, apply_plan_mat, apply_plan_vec in the default operand mode).
+// Plan-times-matrix and plan-times-vector products and the hard c-transform for d <= 128 on
+// fp16 planes (gradient, apply_plan_mat, apply_plan_vec, c_transform in the default operand mode).
 //
-// Same decomposition as lse2_kernel: a workgroup of 4 wavefronts shares key tiles of 64 keys,
+// Same decomposition as lse2_kernel: a workgroup of 4 wavefronts shares key tiles of 64 keys
+// (32 for 128-column rows, which would not leave room for two workgroups per CU otherwise),
 // brought into LDS by direct global->LDS loads of the two-plane fp16 rows (three buffers, the
 // tile two ahead in flight, XOR-swizzled 16-byte slots), and every wavefront owns RB blocks
 // of 32 query rows whose planes never leave its registers.  Per block and 32-key sub-tile:
@@ -14,7 +15,8 @@
 //            operands that transpose_planes_f16_kernel laid out in MFMA order in global memory
 //            (one coalesced 1 KiB read per instruction, shared by the four wavefronts through
 //            L1): three products per column block and step.  (kVec) a weighted sum with the
-//            64 values of v of the tile, staged in LDS.
+//            values of v of the tile, staged in LDS.  (kArgmax) no soft-max at all: a running
+//            (largest value, key) pair per lane, ties to the smaller key.
 // Row sums are exact fp32 VALU sums.  The key bias of the next tile travels in two registers
 // per lane; nothing in the loop needs a second barrier.
 #pragma once
@@ -26,13 +28,16 @@
 
 namespace fs {
 
-constexpr int kPtKeys = 64;            // keys per tile
 constexpr float kPtLazyThresh = 8.0f;  // probabilities stay below 2^8
 
 template <int DP, int RB, int MODE>
 __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args) {
-  static_assert(MODE == kMat || MODE == kVec, "plan_tile_kernel: kMat or kVec");
-  static_assert(DP == 16 || DP == 32 || DP == 64, "wider rows do not fit the register budget");
+  static_assert(MODE == kMat || MODE == kVec || MODE == kArgmax, "plan_tile_kernel modes");
+  static_assert(DP == 16 || DP == 32 || DP == 64 || DP == 128, "padded row widths");
+  constexpr int kPtKeys = (DP == 128) ? 32 : 64;  // keys per tile
+  constexpr int NSUB = kPtKeys / 32;
+  // 128-column rows: key operands are read from LDS step by step instead of being held
+  constexpr bool kStreamK = (DP == 128);
   constexpr int KK16 = DP / 16;                 // 16-column steps of the logits
   constexpr int NCB = (DP + 31) / 32;           // 32-column output blocks
   constexpr int ROWW = DP;                      // words per two-plane row
@@ -127,9 +132,11 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
 
   f32x16 oacc[MODE == kMat ? RB : 1][MODE == kMat ? NCB : 1];
   float run_m[RB], run_s[RB], run_o[RB];
+  int best_j[RB];  // kArgmax: run_m is the largest raw value so far, best_j its key
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    run_m[rb] = 0.f;
+    best_j[rb] = 0;
+    run_m[rb] = (MODE == kArgmax) ? -3.0e38f : 0.f;
     run_s[rb] = 0.f;
     run_o[rb] = 0.f;
     if constexpr (MODE == kMat) {
@@ -141,9 +148,9 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
   }
 
   // ---- prologue: tiles 0 and 1 on their way, bias (and v) of tile 0 ----
-  float ab_next[2];
-  ab_next[0] = bias_of(j_begin + li);
-  ab_next[1] = bias_of(j_begin + 32 + li);
+  float ab_next[NSUB];
+#pragma unroll
+  for (int js = 0; js < NSUB; ++js) ab_next[js] = bias_of(j_begin + js * 32 + li);
   if constexpr (MODE == kVec) {
     if (tid < kPtKeys) lds_v[0][tid] = (j_begin + tid < j_end) ? sd.v[j_begin + tid] : 0.f;
   }
@@ -163,11 +170,14 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
     const int j0 = j_begin + t * kPtKeys;
     const int nbuf = (buf == 2) ? 0 : buf + 1;
     const int n2buf = (nbuf == 2) ? 0 : nbuf + 1;
-    const float ab_cur[2] = {ab_next[0], ab_next[1]};
+    float ab_cur[NSUB];
     // loads in program order: bias (and v) of tile t + 1, V^T of this tile, key tile t + 2;
     // a wait for an older load never has to wait for a younger one
-    ab_next[0] = bias_of(j0 + kPtKeys + li);
-    ab_next[1] = bias_of(j0 + kPtKeys + 32 + li);
+#pragma unroll
+    for (int js = 0; js < NSUB; ++js) {
+      ab_cur[js] = ab_next[js];
+      ab_next[js] = bias_of(j0 + kPtKeys + js * 32 + li);
+    }
     float v_next = 0.f;
     if constexpr (MODE == kVec) {
       if (tid < kPtKeys && j0 + kPtKeys + tid < j_end) v_next = sd.v[j0 + kPtKeys + tid];
@@ -175,19 +185,21 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
     const unsigned* tile = lds_k[buf];
 
 #pragma unroll
-    for (int js = 0; js < 2; ++js) {
+    for (int js = 0; js < NSUB; ++js) {
       u32x4 va[MODE == kMat ? NCB : 1][2][2];
       if constexpr (MODE == kMat) load_vt(va, (j0 >> 5) + js);
-      if (js == 1) issue_tile(n2buf);  // tile t + 2, after the last register loads of tile t
+      if (js == NSUB - 1) issue_tile(n2buf);  // tile t + 2, after the last register loads of tile t
       __builtin_amdgcn_sched_barrier(0);
 
       // A operands of the logits: key row js*32 + li, [plane][step]
-      u32x4 kq[2][KK16];
+      u32x4 kq[2][kStreamK ? 1 : KK16];
+      if constexpr (!kStreamK) {
 #pragma unroll
-      for (int p = 0; p < 2; ++p)
+        for (int p = 0; p < 2; ++p)
 #pragma unroll
-        for (int kk = 0; kk < KK16; ++kk)
-          kq[p][kk] = lds_piece(tile, js * 32 + li, p * (DP / 8) + 2 * kk + h);
+          for (int kk = 0; kk < KK16; ++kk)
+            kq[p][kk] = lds_piece(tile, js * 32 + li, p * (DP / 8) + 2 * kk + h);
+      }
       const float ab = h ? 1.0f : ab_cur[js];
       float vj[MODE == kVec ? 16 : 1];
       if constexpr (MODE == kVec) {
@@ -207,14 +219,45 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         // products lo*hi, hi*lo, hi*hi
+        if constexpr (kStreamK) {
 #pragma unroll
-        for (int prod = 0; prod < 3; ++prod) {
-          const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
-#pragma unroll
-          for (int kk = 0; kk < KK16; ++kk)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kq[pk][kk]),
-                                                         __builtin_bit_cast(f16x8, xq[rb][pq][kk]),
+          for (int kk = 0; kk < KK16; ++kk) {
+            const u32x4 k_hi = lds_piece(tile, js * 32 + li, 2 * kk + h);
+            const u32x4 k_lo = lds_piece(tile, js * 32 + li, (DP / 8) + 2 * kk + h);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, k_lo),
+                                                         __builtin_bit_cast(f16x8, xq[rb][0][kk]),
                                                          acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, k_hi),
+                                                         __builtin_bit_cast(f16x8, xq[rb][1][kk]),
+                                                         acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, k_hi),
+                                                         __builtin_bit_cast(f16x8, xq[rb][0][kk]),
+                                                         acc, 0, 0, 0);
+          }
+        } else {
+#pragma unroll
+          for (int prod = 0; prod < 3; ++prod) {
+            const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
+#pragma unroll
+            for (int kk = 0; kk < KK16; ++kk)
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, kq[pk][kk]), __builtin_bit_cast(f16x8, xq[rb][pq][kk]),
+                  acc, 0, 0, 0);
+          }
+        }
+        if constexpr (MODE == kArgmax) {
+          // value = raw product + key bias; register r holds key 8 (r / 4) + 4 h + r % 4 of the
+          // sub-tile, ascending in r, and tiles ascend: a strict test keeps the smallest key
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
+          const int jb = j0 + js * 32 + 4 * h;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            if (acc[r] > run_m[rb]) {
+              run_m[rb] = acc[r];
+              best_j[rb] = jb + 8 * (r / 4) + (r % 4);
+            }
+          }
+          continue;
         }
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
 
@@ -300,6 +343,28 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
   for (int rb = 0; rb < RB; ++rb) {
     const int row = row0 + rb * 32 + li;
     const bool live = row < sd.nq;
+    if constexpr (MODE == kArgmax) {
+      float best = run_m[rb];
+      int bj = best_j[rb];
+      const float ob = xor32(best);
+      const int oj = __shfl_xor(bj, 32, 64);
+      if (ob > best || (ob == best && oj < bj)) {
+        best = ob;
+        bj = oj;
+      }
+      if (live && h == 0) {
+        if (sd.splits == 1) {
+          sd.ep.out[row] = -best * lscale;
+          sd.ep.idx_out[row] = bj;
+        } else {
+          const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+          *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =
+              make_float2(ntiles > 0 ? best * lscale : -3.0e38f,
+                          __builtin_bit_cast(float, ntiles > 0 ? bj : 0x7fffffff));
+        }
+      }
+      continue;
+    }
     const float M = (ntiles > 0) ? run_m[rb] * lscale : kNegBig;
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float o = run_o[rb] + xor32(run_o[rb]);

@@ -30,8 +30,9 @@
  *    change the fp32 row sums); FS_FLAG_NO_TILE_SKIP computes them all the same.
  *    For d > 128 every operation (log-sum-exp, gradient, plan products, mat5) runs on
  *    the two-plane fp16 operands by default and with FS_FLAG_REDUCED_OPERANDS, and on fp32
- *    MFMA operands with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS.  The gradient and
- *    plan-product kernels for d <= 128 always use fp32 MFMA operands.
+ *    MFMA operands with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS.  For d <= 128 the
+ *    gradient, plan-vector / plan-matrix products and the c-transform do the same; mat5 uses
+ *    fp32 MFMA operands there.
  */
 #ifndef FLASH_SINKHORN_HIP_H
 #define FLASH_SINKHORN_HIP_H
@@ -197,8 +198,8 @@ int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_o
  * Hard c-transform, the eps -> 0 counterpart of fs_lse:
  *   min_out[i] = min_j [-coord_scale x_i.y_j + bias_j],  argmin_out[i] = the smallest j
  * attaining it (int64).  The caller passes bias_j = cost_scale |y_j|^2 - psi_j and adds
- * cost_scale |x_i|^2 to min_out.  d <= 128 runs on fp32 MFMA operands, d > 128 on the
- * two-plane fp16 operands (the operand flags are ignored there).
+ * cost_scale |x_i|^2 to min_out.  Runs on the two-plane fp16 operands (fp32 MFMA operands for
+ * d <= 128 with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS).
  * Replaces c_transform_kernel (kernels/c_transform_sqeuclid.py:219-354, kernel 117-214).
  */
 int fs_c_transform(const float* x, const float* y, const float* bias, float* min_out,
