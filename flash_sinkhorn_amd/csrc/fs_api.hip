@@ -583,16 +583,24 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   int rb = 2;
   for (int s = 0; s < nsides; ++s) rb = std::min(rb, pt_rows_per_wave(sides[s].nq));
   if (rb_env > 0) rb = std::min(rb_env, 2);
-  if (dpk == 128) rb = 1;
+  const bool mat5 = (mode == kMat5);
+  const bool has_o = (mode == kMat || mat5);
+  if (dpk == 128 || mat5) rb = 1;
   size_t need = ps.end;
   SidePlan plans[2];
-  size_t vt_off[2] = {0, 0}, part_off[2];
+  size_t vt_off[2] = {0, 0}, part_off[2], q2_off = 0, bounds_off = 0;
   for (int s = 0; s < nsides; ++s) {
     plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam, rb);
-    if (mode == kMat) {
+    if (has_o) {
       vt_off[s] = need;
       need += pt_vt_bytes(sides[s].nk, dpk) + kPgAuxBytes;
     }
+  }
+  if (mat5) {  // two-plane rows of the second stationary operand, their aux block, row bounds
+    q2_off = need;
+    need += plane_bytes(sides[0].nq, cfg) + kPlaneAuxBytes;
+    bounds_off = need;
+    need += (((size_t)sides[0].nq + 64) * sizeof(float) + 15) & ~(size_t)15;
   }
   for (int s = 0; s < nsides; ++s) {
     part_off[s] = need;
@@ -623,11 +631,19 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     sd.plane_scale = plane_scales(ps, ws);
     sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
     sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
-    if (mode == kMat) {
+    if (has_o) {
       sd.vplanes = reinterpret_cast<const unsigned*>(base + vt_off[s]);
       sd.vplane_scale =
           reinterpret_cast<const float*>(base + vt_off[s] + pt_vt_bytes(sd.nk, dpk)) + 256;
       vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.ep.out);
+    }
+    if (mat5) {
+      sd.kplane_scale = sd.plane_scale + plane_index(ps, sd.k, sd.nk);
+      sd.q2planes = reinterpret_cast<const unsigned*>(base + q2_off);
+      sd.q2plane_scale =
+          reinterpret_cast<const float*>(base + q2_off + plane_bytes(sd.nq, cfg)) + 2 * 256;
+      sd.kmax2 = reinterpret_cast<const float*>(base + bounds_off);
+      sd.q2norm2 = sd.kmax2 + 64;
     }
     blocks[s] = p.igroups * p.splits;
     a.side[s] = sd;
@@ -639,7 +655,17 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   if (total <= 0) return FS_OK;
 
   if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
-  for (int s = 0; s < nsides && rc == FS_OK && mode == kMat; ++s) {
+  if (mat5 && rc == FS_OK) {
+    const Side& sd = sides[0];
+    float* partial = reinterpret_cast<float*>(base + q2_off + plane_bytes(sd.nq, cfg));
+    float* bounds = reinterpret_cast<float*>(base + bounds_off);
+    rc = launch_mat5_bounds(sd.q2, sd.nq, (int)d, sd.kb1, sd.nk, bounds + 64, bounds, st);
+    if (rc == FS_OK) rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
+    if (rc == FS_OK)
+      rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, st);
+  }
+  for (int s = 0; s < nsides && rc == FS_OK && has_o; ++s) {
     const Side& sd = sides[s];
     float* aux = reinterpret_cast<float*>(base + vt_off[s] + pt_vt_bytes(sd.nk, dpk));
     rc = launch_transpose_planes(sd.v ? sd.v : sd.k, sd.vscale,
@@ -655,7 +681,6 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
   }
   if (any_split) {
-    const bool has_o = (mode == kMat);
     const int per_row = has_o ? dpk / 4 : 1;
     int items[2] = {0, 0};
     for (int s = 0; s < nsides; ++s)
@@ -685,7 +710,9 @@ size_t pt_ws_bytes(int mode, int64_t n, int64_t m, int64_t d, bool both, bool ei
     size_t b = 0;
     for (int rb = 1; rb <= 2; ++rb)
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dpk) * sizeof(float));
-    if (mode == kMat) b += pt_vt_bytes(nk, dpk) + kPgAuxBytes;
+    if (mode == kMat || mode == kMat5) b += pt_vt_bytes(nk, dpk) + kPgAuxBytes;
+    if (mode == kMat5)  // planes of the second operand (sized for three planes), aux, row bounds
+      b += (size_t)(nq + kPlanePadRowsApi) * 3 * (dpk / 2) * 4 + kPlaneAuxBytes + ((size_t)nq + 64) * 4 + 64;
     return b + 16;
   };
   if (both) return planes + side(n, m) + side(m, n) + 64;
@@ -709,8 +736,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   static const int use_plan_tile = env_int("FS_PLANTILE", 1);
-  if ((mode == kMat || mode == kVec || mode == kArgmax) && !fam.sliced && use_plan_tile &&
-      (cfg.prec == 3 || cfg.prec == 1)) {
+  const bool tile_mode = mode == kMat || mode == kVec || mode == kArgmax ||
+                         (mode == kMat5 && cfg.dp <= 64);
+  if (tile_mode && !fam.sliced && use_plan_tile && (cfg.prec == 3 || cfg.prec == 1)) {
     // the reduced mode runs on the fp16 planes too (same speed, smaller error); planes a caller
     // prepared for it are bf16 and are not used here
     const bool reduced = (cfg.prec == 1);
@@ -927,7 +955,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
   if ((mode == kMat || mode == kMat5) && fam.sliced)
     gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
-  if ((mode == kMat || mode == kVec || mode == kArgmax) && !fam.sliced)
+  if ((mode == kMat || mode == kVec || mode == kArgmax || (mode == kMat5 && d <= 64)) && !fam.sliced)
     gemm = pt_ws_bytes(mode, n, m, d, both, either, fam);
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);

@@ -15,7 +15,10 @@
 //            operands that transpose_planes_f16_kernel laid out in MFMA order in global memory
 //            (one coalesced 1 KiB read per instruction, shared by the four wavefronts through
 //            L1): three products per column block and step.  (kVec) a weighted sum with the
-//            values of v of the tile, staged in LDS.  (kArgmax) no soft-max at all: a running
+//            values of v of the tile, staged in LDS.  (kMat5) as kMat with the probabilities
+//            multiplied by T = <A_i, y_j>, a second contraction on planes of A held in
+//            registers, scaled per row by a power of two from |A_i| max|y_j| so that p T stays
+//            fp16-safe (see plan_gemm_kernel).  (kArgmax) no soft-max at all: a running
 //            (largest value, key) pair per lane, ties to the smaller key.
 // Row sums are exact fp32 VALU sums.  The key bias of the next tile travels in two registers
 // per lane; nothing in the loop needs a second barrier.
@@ -32,7 +35,10 @@ constexpr float kPtLazyThresh = 8.0f;  // probabilities stay below 2^8
 
 template <int DP, int RB, int MODE>
 __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args) {
-  static_assert(MODE == kMat || MODE == kVec || MODE == kArgmax, "plan_tile_kernel modes");
+  static_assert(MODE == kMat || MODE == kVec || MODE == kArgmax || MODE == kMat5,
+                "plan_tile_kernel modes");
+  static_assert(MODE != kMat5 || (DP <= 64 && RB == 1), "mat5: the second operand needs registers");
+  constexpr bool kHasO = (MODE == kMat || MODE == kMat5);
   static_assert(DP == 16 || DP == 32 || DP == 64 || DP == 128, "padded row widths");
   constexpr int kPtKeys = (DP == 128) ? 32 : 64;  // keys per tile
   constexpr int NSUB = kPtKeys / 32;
@@ -83,6 +89,27 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
         xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qrow + p * (DP / 2) + 8 * kk + 4 * h);
   }
 
+  u32x4 aq[MODE == kMat5 ? RB : 1][2][MODE == kMat5 ? KK16 : 1];
+  float t_unit = 1.0f;
+  if constexpr (MODE == kMat5) {
+    const int row = min(row0 + li, sd.nq - 1);
+    const unsigned* arow = sd.q2planes + (size_t)row * (size_t)ROWW;
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk)
+        aq[0][p][kk] = *reinterpret_cast<const u32x4*>(arow + p * (DP / 2) + 8 * kk + 4 * h);
+    // per-row power of two with |T_ij| * t_unit <= 2^7 from |T_ij| <= |A_i| max_j |y_j|
+    float km = sd.kmax2[lane];  // 64 partial maxima of |y_j|^2
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) km = fmaxf(km, __shfl_xor(km, o, 64));
+    const float bound =
+        sqrtf(sd.q2norm2[row] * km) * sd.q2plane_scale[0] * sd.kplane_scale[0] * 1.0001f;
+    const int e = (int)((__builtin_bit_cast(unsigned, bound) >> 23) & 255u);  // bound < 2^(e-126)
+    if (e > 0 && e < 255)
+      t_unit = __builtin_bit_cast(float, (unsigned)min(254, max(1, 127 + 7 - (e - 126))) << 23);
+  }
+
   // ---- key tiles: lane idx of instruction c fills LDS slot idx and fetches the piece that
   // belongs there (slot = piece ^ swz(row)) ----
   auto swz = [&](int r) {
@@ -130,7 +157,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
       }
   };
 
-  f32x16 oacc[MODE == kMat ? RB : 1][MODE == kMat ? NCB : 1];
+  f32x16 oacc[kHasO ? RB : 1][kHasO ? NCB : 1];
   float run_m[RB], run_s[RB], run_o[RB];
   int best_j[RB];  // kArgmax: run_m is the largest raw value so far, best_j its key
 #pragma unroll
@@ -139,7 +166,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
     run_m[rb] = (MODE == kArgmax) ? -3.0e38f : 0.f;
     run_s[rb] = 0.f;
     run_o[rb] = 0.f;
-    if constexpr (MODE == kMat) {
+    if constexpr (kHasO) {
 #pragma unroll
       for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
@@ -186,8 +213,8 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
 
 #pragma unroll
     for (int js = 0; js < NSUB; ++js) {
-      u32x4 va[MODE == kMat ? NCB : 1][2][2];
-      if constexpr (MODE == kMat) load_vt(va, (j0 >> 5) + js);
+      u32x4 va[kHasO ? NCB : 1][2][2];
+      if constexpr (kHasO) load_vt(va, (j0 >> 5) + js);
       if (js == NSUB - 1) issue_tile(n2buf);  // tile t + 2, after the last register loads of tile t
       __builtin_amdgcn_sched_barrier(0);
 
@@ -245,6 +272,20 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
                   acc, 0, 0, 0);
           }
         }
+        f32x16 tacc;
+        if constexpr (MODE == kMat5) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tacc[r] = 0.f;
+#pragma unroll
+          for (int prod = 0; prod < 3; ++prod) {
+            const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
+#pragma unroll
+            for (int kk = 0; kk < KK16; ++kk)
+              tacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, kq[pk][kk]), __builtin_bit_cast(f16x8, aq[rb][pq][kk]),
+                  tacc, 0, 0, 0);
+          }
+        }
         if constexpr (MODE == kArgmax) {
           // value = raw product + key bias; register r holds key 8 (r / 4) + 4 h + r % 4 of the
           // sub-tile, ascending in r, and tiles ascend: a strict test keeps the smallest key
@@ -277,7 +318,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
           run_m[rb] += delta;
           run_s[rb] *= resc;
           run_o[rb] *= resc;
-          if constexpr (MODE == kMat) {
+          if constexpr (kHasO) {
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
@@ -298,7 +339,11 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
           for (int r = 0; r < 16; ++r) po = __builtin_fmaf(p[r], vj[r], po);
           run_o[rb] += po;
         }
-        if constexpr (MODE == kMat) {
+        if constexpr (MODE == kMat5) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) p[r] *= tacc[r] * t_unit;
+        }
+        if constexpr (kHasO) {
           // registers 8 s .. 8 s + 7 are this lane's B operand of 16-key step s
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
@@ -338,7 +383,8 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
   __builtin_amdgcn_s_waitcnt(0x0F70);  // tiles fetched past the chunk: let them land before exit
 
   // ---- merge the two half-waves of each query, then finish or spill ----
-  const float inv_vs = (MODE == kMat) ? 1.0f / sd.vplane_scale[0] : 1.0f;
+  float inv_vs = kHasO ? 1.0f / sd.vplane_scale[0] : 1.0f;
+  if constexpr (MODE == kMat5) inv_vs /= t_unit * sd.q2plane_scale[0] * sd.kplane_scale[0];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = row0 + rb * 32 + li;
@@ -369,7 +415,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float o = run_o[rb] + xor32(run_o[rb]);
     if (sd.splits == 1) {
-      if constexpr (MODE == kVec) {
+      if constexpr (!kHasO) {
         if (live && h == 0) epilogue_scalar(sd.ep, row, M, s, o);
       } else {
         if (live) {
@@ -391,7 +437,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
         *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M, s);
         if constexpr (MODE == kVec) sd.part_o[pr] = o;
       }
-      if constexpr (MODE == kMat) {
+      if constexpr (kHasO) {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
