@@ -56,13 +56,16 @@ def test_symmetric_step_in_strict_modes(strict_mode, n, m, d):
     assert rel_err(gf, wf) < RTOL and rel_err(gg, wg) < RTOL
 
 
-@pytest.mark.parametrize("n,m,d", [s for s in SHAPES if s[2] > 128])
-def test_large_d_products_on_fp32_mfma(strict_mode, n, m, d):
+@pytest.mark.parametrize("n,m,d", SHAPES)
+def test_products_on_fp32_mfma(strict_mode, n, m, d):
+    """With either strict flag every product runs on fp32 MFMA operands: `stream_kernel` for
+    d <= 128, `sliced_kernel` beyond."""
     from flash_sinkhorn_amd.kernels.apply_flash import (
         apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
     from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
     from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
         sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    from flash_sinkhorn_amd import c_transform_fwd
     x, y, a, b, fh, gh = problem(n, m, d, seed=2)
     la, lb = np.log(a), np.log(b)
     rng = np.random.default_rng(12)
@@ -82,6 +85,14 @@ def test_large_d_products_on_fp32_mfma(strict_mode, n, m, d):
     f5 = fh - 2.0
     got = mat5_sqeuclid(*dev(x, y, f5, gh, A), eps=0.5, cost_scale=0.5)
     assert rel_err(got, oracle.mat5(x, y, f5, gh, A, 0.5, 0.5)) < RTOL
+    psi = rng.standard_normal(m).astype(np.float32)
+    c, idx = c_transform_fwd(X, Y, dev(psi)[0], cost_scale=0.5, allow_tf32=False)
+    wc, _ = oracle.c_transform(x, y, psi, 0.5)
+    scale = max(np.abs(wc).max(), 1.0)
+    assert np.abs(c.cpu().numpy() - wc).max() <= 1e-5 * scale
+    j = idx.cpu().numpy()
+    att = 0.5 * ((x.astype(np.float64) - y.astype(np.float64)[j]) ** 2).sum(1) - psi[j]
+    assert np.abs(att - wc).max() <= 2e-5 * scale
 
 
 @pytest.mark.parametrize("n,m,d", SHAPES)
