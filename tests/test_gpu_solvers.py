@@ -327,3 +327,42 @@ def test_implicit_gradient_against_oracle(cs):
     got2, _ = implicit_grad_x(X, Y, A, B, GF, GG, eps=eps, cost_scale=cs, n_iters=60,
                               max_cg_iter=300)
     assert rel_err(got2, want) < 2e-3
+
+
+def test_custom_operators_match_the_launchers():
+    """torch.ops.flash_sinkhorn_amd.* run the same library calls as the launchers they wrap."""
+    from flash_sinkhorn_amd import torch_ops  # noqa: F401  (registers the operators)
+    from flash_sinkhorn_amd.kernels.apply_flash import (
+        apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        flashsinkhorn_lse_fused, flashsinkhorn_symmetric_step)
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    ops = torch.ops.flash_sinkhorn_amd
+    n, m, d = 300, 260, 40
+    x, y, a, b = inputs(47, n, m, d, scale=2.0 / np.sqrt(d))
+    rng = np.random.default_rng(4)
+    fh = (rng.standard_normal(n) * 0.3).astype(np.float32)
+    gh = (rng.standard_normal(m) * 0.3).astype(np.float32)
+    X, Y, A, B, F, G, LA, LB = dev(x, y, a, b, fh, gh, np.log(a), np.log(b))
+    assert torch.equal(ops.lse_fused(X, Y, G, LB, 0.2),
+                       flashsinkhorn_lse_fused(X, Y, G, LB, 0.2, allow_tf32=False))
+    f1, g1 = ops.symmetric_step(X, Y, F, G, LA, LB, 0.2)
+    f2, g2 = flashsinkhorn_symmetric_step(X, Y, F, G, LA, LB, 0.2, allow_tf32=False)
+    assert torch.equal(f1, f2) and torch.equal(g1, g2)
+    gx1, gy1 = ops.grad(X, Y, A, B, F, G, 0.2, 0.5)
+    gx2, gy2 = grad(X, Y, A, B, F, G, eps=0.2, cost_scale=0.5, allow_tf32=False)
+    assert torch.equal(gx1, gx2) and torch.equal(gy1, gy2)
+    v = torch.randn(m, device="cuda")
+    V = torch.randn(m, d, device="cuda")
+    assert torch.equal(ops.apply_plan_vec(X, Y, F, G, LA, LB, v, 0.4, 1),
+                       apply_plan_vec_flashstyle(X, Y, F, G, LA, LB, v, eps=0.4, axis=1))
+    assert torch.equal(ops.apply_plan_mat(X, Y, F, G, LA, LB, V, 0.4, 1),
+                       apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, V, eps=0.4, axis=1))
+    c, idx = ops.c_transform(X, Y, (Y * Y).sum(1) - G)
+    want_c, want_idx = oracle.c_transform(x, y, gh, 1.0)
+    inner = want_c - (x.astype(np.float64) ** 2).sum(1)
+    assert np.abs(c.cpu().numpy() - inner).max() <= 1e-5 * np.abs(inner).max()
+    assert (idx.cpu().numpy() == want_idx).mean() > 0.99
+    torch.library.opcheck(ops.lse_fused.default, (X, Y, G, LB, 0.2),
+                          test_utils=("test_schema", "test_faketensor"))

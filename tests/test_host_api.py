@@ -217,3 +217,27 @@ def test_solver_argument_errors():
                                       use_epsilon_scaling=False)
     with pytest.raises(ValueError, match="non-empty"):
         sinkhorn_flashstyle_symmetric(x, x, torch.ones(4), torch.ones(4), eps_list=[])
+
+
+def test_custom_operators_are_registered_with_shape_inference():
+    """torch.ops.flash_sinkhorn_amd.*: every operator exists and its fake implementation gives
+    the output shapes and dtypes on meta tensors (no GPU, no library call)."""
+    from flash_sinkhorn_amd import torch_ops
+    ops = torch.ops.flash_sinkhorn_amd
+    for name in torch_ops.OPERATORS:
+        assert hasattr(ops, name)
+    n, m, d = 7, 5, 3
+    mt = lambda *s: torch.empty(*s, device="meta")  # noqa: E731
+    x, y = mt(n, d), mt(m, d)
+    assert ops.lse(x, y, mt(m), 0.1).shape == (n,)
+    assert ops.lse_fused(x, y, mt(m), mt(m), 0.1).shape == (n,)
+    f, g = ops.symmetric_step(x, y, mt(n), mt(m), mt(n), mt(m), 0.1)
+    assert f.shape == (n,) and g.shape == (m,)
+    gx, gy = ops.grad(x, y, mt(n), mt(m), mt(n), mt(m), 0.1)
+    assert gx.shape == (n, d) and gy.shape == (m, d)
+    assert ops.apply_plan_vec(x, y, mt(n), mt(m), mt(n), mt(m), mt(m), 0.1, 1).shape == (n,)
+    assert ops.apply_plan_vec(x, y, mt(n), mt(m), mt(n), mt(m), mt(n), 0.1, 0).shape == (m,)
+    assert ops.apply_plan_mat(x, y, mt(n), mt(m), mt(n), mt(m), mt(m, d), 0.1, 1).shape == (n, d)
+    assert ops.mat5(x, y, mt(n), mt(m), mt(n, d), 0.1).shape == (n, d)
+    c, idx = ops.c_transform(x, y, mt(m))
+    assert c.shape == (n,) and idx.dtype == torch.int64 and c.dtype == torch.float32
