@@ -147,9 +147,9 @@ class PreparedOperands:
               "fs_prepare_operands")
 
     def serves(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int) -> bool:
+        # the workspace layout depends on the set of matrices, so the call must name the same set
         return (flag_bits == self.flag_bits and x.shape[1] == self.d
-                and (x.data_ptr(), x.shape[0]) in self.keys
-                and (y.data_ptr(), y.shape[0]) in self.keys)
+                and {(x.data_ptr(), x.shape[0]), (y.data_ptr(), y.shape[0])} == self.keys)
 
 
 def lse_workspace(op: int, x: torch.Tensor, y: torch.Tensor, flag_bits: int,

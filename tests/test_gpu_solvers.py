@@ -249,6 +249,34 @@ def test_prepared_operands_give_identical_results(n, m, d):
     want = oracle.lse_shifted_fused(x, y, gh, np.log(b), 0.2)
     assert rel_err(o2, want) < 1e-3
 
+@pytest.mark.parametrize("n,m,d", [(3000, 4100, 64), (129, 1000, 3), (5000, 300, 128), (260, 260, 32)])
+def test_launches_are_repeatable_on_one_workspace(n, m, d):
+    """Split keys leave partial rows in the workspace between the streaming kernel and the merge:
+    every launch on one prepared workspace must give the bits of the first, and of a call with
+    a fresh workspace (nothing carried over, no dependence on workgroup arrival order)."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    x, y, a, b = inputs(47, n, m, d, scale=2.0 / np.sqrt(d))
+    rng = np.random.default_rng(5)
+    fh = (rng.standard_normal(n) * 0.3).astype(np.float32)
+    gh = (rng.standard_normal(m) * 0.3).astype(np.float32)
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, np.log(a), np.log(b))
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    f0, g0 = _symmetric_step_raw(X, Y, F, G, LA, LB, 0.2, **kw)
+    wf, wg = oracle.symmetric_step(x, y, fh, gh, np.log(a), np.log(b), 0.2, 1.0, 0.5, 1.0, 1.0)
+    assert rel_err(f0, wf) < RTOL and rel_err(g0, wg) < RTOL
+    prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+    for _ in range(25):
+        f1, g1 = _symmetric_step_raw(X, Y, F, G, LA, LB, 0.2, prepared=prep, **kw)
+        assert torch.equal(f0, f1) and torch.equal(g0, g1)
+    if n == m:  # the aliased self problem on its own prepared workspace
+        s0, _ = _symmetric_step_raw(X, X, F, F, LA, LA, 0.2, **kw)
+        prep = _lib.PreparedOperands(X, X, _lib.flags(True, False))
+        for _ in range(10):
+            s1, _ = _symmetric_step_raw(X, X, F, F, LA, LA, 0.2, prepared=prep, **kw)
+            assert torch.equal(s0, s1)
+
+
 @pytest.mark.parametrize("n,m,d", [(700, 500, 64), (300, 260, 200)])
 def test_multi_step_call_equals_single_steps(n, m, d):
     """fs_symmetric_steps enqueues the same launches as a loop over fs_symmetric_step: the
