@@ -766,13 +766,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = cfg.dp;
   if (lse2 && prec == 2 && dp >= 64) rb = 1;  // three planes of 64 columns x two row blocks spill
-  if (lse2 && prec == 3 && dp == 64) {
-    // three row blocks per wavefront amortise key reads and staging a little further
-    bool big = true;
-    for (int s = 0; s < nsides; ++s) big = big && sides[s].nq >= 8192;
-    if (big) rb = 3;
-  }
-  if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, (dp == 64 && prec == 3) ? 3 : 2);
+  if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
   PlaneSet ps;
   ps.n = 0;
   ps.end = 0;

@@ -13,9 +13,6 @@ static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
 
 template <int DP, int PREC>
 static int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
-  if constexpr (DP == 64 && PREC == kH3) {
-    if (rb == 3) return launch_cfg<DP, 3, PREC>(a, blocks, st);
-  }
   if constexpr (DP <= 64 && !(PREC == kBf6 && DP == 64)) {
     if (rb >= 2) return launch_cfg<DP, 2, PREC>(a, blocks, st);
   }

@@ -1,27 +1,32 @@
 // Software-pipelined log-sum-exp kernel (d <= 128).
 //
 // Same decomposition as stream_kernel<kLse> (stationary query blocks in VGPRs,
-// key tiles through LDS, transposed logits, lane-private online soft-max, bias
-// and running max folded into one extra MFMA), with these changes that matter for
-// speed:
+// key tiles through LDS, transposed logits, lane-private online soft-max), with these changes
+// that matter for speed:
 //   * the soft-max of logits tile u-1 is cut into pieces that sit in program order BETWEEN
 //     the MFMAs of tile u, fenced with sched_barrier so the compiler keeps them there.  A
 //     wavefront issues in order and a chain of dependent MFMAs blocks its issue slot, so
-//     only VALU work interleaved this way runs in the MFMA shadow.  The loop body is one
-//     basic block: a branch would let the compiler sink the pieces past the MFMAs;
-//   * the online soft-max is branch free (per-lane max, rescale by exp2(-delta) every
+//     only VALU work interleaved this way runs in the MFMA shadow;
+//   * the online soft-max is branch free per lane (per-lane max, rescale by exp2(-delta) every
 //     tile).  With the keys split into chunks every chunk is short, new running
 //     maxima are frequent, and a wave-wide "does any lane need a rescale" branch
-//     would be taken on almost every tile.  Only the first tile of a block is handled apart;
+//     would be taken on almost every tile.  Only the first tile of a block is handled apart.
+//     The one wave-uniform decision is whether a tile's exponentials can matter at all
+//     (LaunchArgs::skip_log2); if not, the tile runs its MFMAs only;
 //   * the A operands of the next 32-key sub-tile are read from LDS while the current one is
 //     multiplied, and key tiles are fetched two tiles ahead (direct global->LDS loads in the
-//     two-plane modes, through registers otherwise), with one barrier per 64 keys.
+//     two-plane modes, through registers otherwise), with one barrier per 64 keys;
+//   * key bias and running max.  Two-plane modes at d <= 64: the MFMA chain of a tile starts
+//     from the key bias (16 floats per lane, read from LDS into the registers the previous
+//     tile's soft-max has just let go of; two accumulator tiles swap roles from tile to tile
+//     and nothing is copied), and the running max enters through the addend of the exp2
+//     argument's FMA.  Other modes: one extra fp32 MFMA per tile adds bias - max.
 //
 // Operand precision (PREC):
 //   kF32   v_mfma_f32_32x32x2_f32 on fp32 operands (needs d % 4 == 0 and aligned rows).
 //          (The 16-bit modes read operands that the split kernels have already cut into
-//          packed planes; the logit scale is applied in the exp2 argument's FMA and the
-//          bias / running-max fold uses one fp32 MFMA, so no per-tile conversion work.)
+//          packed planes and apply the logit scale in the exp2 argument's FMA, so there is no
+//          per-tile conversion work.)
 //   kBf3   operands split into two bf16 planes (hi, lo); hi*hi + hi*lo + lo*hi on
 //          v_mfma_f32_32x32x16_bf16, fp32 accumulate: ~2^-17 relative per product,
 //          the counterpart of the reference's allow_tf32=True.
@@ -203,8 +208,9 @@ struct Geo2 {
 // VALU work that sits between the MFMAs in program order runs in their shadow.
 constexpr int kPieces = 12;
 constexpr int kMaxPieces = 3;  // pieces 0..2 find the largest logit of the unit
+constexpr int kBiasPiece = 4;  // pieces 4..7 read the next unit's bias from LDS, 16 bytes each
 struct SoftmaxStage {
-  float m[6], mx, aa, bb, c, ps0, ps1;
+  float m[6], mx, aa, bb, c, cx, ps0, ps1;  // c: exponent of the rescale, cx: offset of the logits
   float t[16], e[16];
 };
 
@@ -219,6 +225,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // Key-register prefetch (A operands of the next 32-key sub-tile are read from LDS while the
   // current one is multiplied) and the early LDS store it needs; off where registers are short.
   constexpr bool KPF = (NSUB == 2) && !(PREC == kBf6 && RB == 2);
+  // Two-plane modes with the key-register prefetch: the key bias is the initial value of the MFMA
+  // chain's accumulator (16 floats per lane read from LDS while the previous unit finishes)
+  // and the running max is subtracted inside the exp2 argument's FMA, which takes the fp32
+  // bias MFMA (64 of 448 MFMA cycles per unit at d = 64) out of the loop.
+  constexpr bool BIASC = (PREC == kH3 || PREC == kBf3) && KPF;
   // Two-plane modes bring key tiles into LDS with direct global->LDS loads (no staging
   // registers, no ds_write): rows are unpadded and 16-byte piece p of row r sits in slot
   // p ^ swz(r), which keeps the b128 reads of 16 consecutive rows conflict free.  With the
@@ -286,11 +297,15 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     }
   }
 
-  float run_m[RB], run_s[RB];
+  // run_m: running max in accumulator units; run_c (BIASC): -run_m * lscale as rounded once,
+  // the offset every exponent of the row uses, so that rescaling by differences of run_c is
+  // consistent with the exponents already summed
+  float run_m[RB], run_s[RB], run_c[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     run_m[rb] = 0.f;
     run_s[rb] = 0.f;
+    run_c[rb] = 0.f;
   }
 
   // ---- staging (global -> registers -> LDS), branch free: rows are clamped, masked by bias ----
@@ -303,6 +318,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   const int krow_words = kBf ? ROWW : d;
   const float* kb1p = sd.kb1 ? sd.kb1 : sd.kb0;  // always loadable; unused terms are dropped
   const float* kb2p = sd.kb2 ? sd.kb2 : sd.kb0;
+  // read once: inside the loop the launch arguments would be fetched again for every tile
+  const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
+  const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
   // Plane buffers end with kPlanePadRows zero rows, so the 16-bit modes walk them with plain
   // running pointers (tiles up to two past the chunk are fetched and masked by the bias);
   // the fp32 mode reads the caller's matrix and clamps the row instead.
@@ -318,8 +336,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     if constexpr (DIRECT) piece ^= swz(r);  // lane idx fills LDS slot idx; it fetches this piece
     kp[c] = krows + (size_t)(j_begin + r) * (size_t)krow_words + piece * 4;
   }
-  // No branches anywhere in the main loop: a branch would split the basic block and let the
-  // compiler sink the soft-max pieces out from between the MFMAs.
+  // The staging code is branch free (clamped rows, additive masks): the only branches of the
+  // main loop are the wave-uniform ones around soft-max pieces.
   auto stage_load = [&](int j0, int dbuf) {  // dbuf: LDS buffer of the direct loads
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
@@ -365,8 +383,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       }
     }
     // masked rows get a penalty ADDED (not selected), so the loads stay unconditional
-    float b = sd.kc0 * st_b0 + (sd.kb1 ? sd.kc1 * st_b1 : 0.f);
-    b += (sd.kb2 ? sd.kc2 * st_b2 : 0.f);
+    float b = kc0 * st_b0 + (has_kb1 ? kc1 * st_b1 : 0.f);
+    b += (has_kb2 ? kc2 * st_b2 : 0.f);
     lds_b[buf][tid] = (fmaxf(b, kNegBig) + st_pen) * inv_lscale;
   };
 
@@ -391,6 +409,20 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   };
   // classic online soft-max step; acc holds (logit - M)/lscale for the current M = run_m[rb]
   auto softmax = [&](const f32x16& acc, int rb) {
+    if constexpr (BIASC) {  // acc holds logit/lscale itself
+      const float m_new = fmaxf(column_max(acc), run_m[rb]);
+      const float c_new = -m_new * lscale;
+      float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        ps0 += fast_exp2(__builtin_fmaf(acc[r], lscale, c_new));
+        ps1 += fast_exp2(__builtin_fmaf(acc[r + 1], lscale, c_new));
+      }
+      run_s[rb] = run_s[rb] * fast_exp2(c_new - run_c[rb]) + (ps0 + ps1);
+      run_m[rb] = m_new;
+      run_c[rb] = c_new;
+      return;
+    }
     const float delta = fmaxf(column_max(acc), 0.f);
     // the max actually applied is what fp32 can represent next to the old one
     const float m_new = run_m[rb] + delta;
@@ -412,6 +444,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     for (int r = 0; r < 16; ++r) ps += fast_exp2(__builtin_fmaf(acc[r], lscale, c));
     run_s[rb] = ps;
     run_m[rb] = delta;
+    run_c[rb] = c;
   };
   // The same step as `softmax`, piece p of kPieces; fma / exp2 / add of a value sit in
   // consecutive pieces so that no piece waits on its own results.
@@ -433,17 +466,33 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       swap_halves(s.aa, s.bb);
     }
     if (p == 3) {
-      const float delta = fmaxf(fmaxf(s.aa, s.bb), 0.f);
-      const float m_new = run_m[rb] + delta;
-      s.c = -(m_new - run_m[rb]) * lscale;
-      run_m[rb] = m_new;
+      if constexpr (BIASC) {
+        const float m_new = fmaxf(fmaxf(s.aa, s.bb), run_m[rb]);
+        s.cx = -m_new * lscale;
+        s.c = s.cx - run_c[rb];
+        run_m[rb] = m_new;
+        run_c[rb] = s.cx;
+      } else {
+        const float delta = fmaxf(fmaxf(s.aa, s.bb), 0.f);
+        const float m_new = run_m[rb] + delta;
+        s.c = -(m_new - run_m[rb]) * lscale;
+        s.cx = s.c;
+        run_m[rb] = m_new;
+      }
       s.ps0 = 0.f;
       s.ps1 = 0.f;
     }
     const int q = p - 3;  // two values per piece: fma at q, exp2 at q + 1, add at q + 2
-    if (q >= 0 && q < 8) {
-      s.t[2 * q] = __builtin_fmaf(a[2 * q], lscale, s.c);
-      s.t[2 * q + 1] = __builtin_fmaf(a[2 * q + 1], lscale, s.c);
+    if constexpr (BIASC) {
+      // four fmas per piece: the logits registers are free again after piece 6 and take the
+      // next unit's bias while the exponentials go on
+      if (q >= 0 && q < 4) {
+#pragma unroll
+        for (int r = 4 * q; r < 4 * q + 4; ++r) s.t[r] = __builtin_fmaf(a[r], lscale, s.cx);
+      }
+    } else if (q >= 0 && q < 8) {
+      s.t[2 * q] = __builtin_fmaf(a[2 * q], lscale, s.cx);
+      s.t[2 * q + 1] = __builtin_fmaf(a[2 * q + 1], lscale, s.cx);
     }
     if (q >= 1 && q < 9) {
       s.e[2 * q - 2] = fast_exp2(s.t[2 * q - 2]);
@@ -517,16 +566,36 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
                                                        acc, 0, 0, 0);
     }
   };
-  auto chain = [&](const KeyRegs& kr, int rb) {
-    f32x16 acc;
+  // BIASC: the key bias of sub-tile js as the accumulator layout holds it (register r of lane
+  // (li, h) is key 8(r/4) + 4h + r%4): four 16-byte reads, the same address in each half-wave
+  auto load_bias4 = [&](f32x16& b, int c, int buf, int js) {
+    const float4 v = *reinterpret_cast<const float4*>(&lds_b[buf][js * 32 + 8 * c + 4 * h]);
+    b[4 * c + 0] = v.x;
+    b[4 * c + 1] = v.y;
+    b[4 * c + 2] = v.z;
+    b[4 * c + 3] = v.w;
+  };
+  auto load_bias16 = [&](int buf, int js) {
+    f32x16 b;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int c = 0; c < 4; ++c) load_bias4(b, c, buf, js);
+    return b;
+  };
+  auto chain = [&](const KeyRegs& kr, int rb, int buf, int js) {
+    f32x16 acc;
+    if constexpr (BIASC) {
+      acc = load_bias16(buf, js);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    }
 #pragma unroll
     for (int k = 0; k < NMAIN; ++k) acc = mfma_k(k, acc, kr, rb);
     return acc;
   };
   // The bias MFMA (fp32 operands in every mode): adds kbias_j - M_i with the freshest M.
-  auto add_bias = [&](f32x16 acc, const KeyRegs& kr, int rb) {
+  auto add_bias = [&](f32x16 acc, const KeyRegs& kr, int rb) -> f32x16 {
+    if constexpr (BIASC) return acc;  // the chain started from the bias
     return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
   };
 
@@ -584,7 +653,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             load_keys(K[0], nxt, 0);
           }
         }
-        const f32x16 acc = add_bias(chain(kr, rb), kr, rb);
+        const f32x16 acc = add_bias(chain(kr, rb, cur, js), kr, rb);
         if (js == 0) softmax_first(acc, rb); else softmax(acc, rb);
       }
     }
@@ -596,9 +665,15 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     rotate();
   }
 
-  f32x16 acc_prev;
+  // R1: logits of the previous unit.  BIASC: R0 and R1 swap roles from unit to unit (one holds
+  // the running MFMA chain, the other the previous logits, whose registers take the next
+  // unit's bias as the soft-max lets go of them); a tile has an even number of units, so the
+  // roles are fixed in the unrolled code and nothing is ever copied.
+  f32x16 R0, R1;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc_prev[r] = kNegBig;
+  for (int r = 0; r < 16; ++r) R1[r] = kNegBig;
+  if constexpr (BIASC) R0 = load_bias16(cur, 0);
+  static_assert(!BIASC || (NSUB * RB) % 2 == 0, "units per tile must be even");
 
   // ---- steady state: the soft-max of the previous logits tile rides between the MFMAs ----
   for (int t = 1; t < ntiles; ++t) {
@@ -611,13 +686,18 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       for (int rb = 0; rb < RB; ++rb) {
         const int prev_rb = (rb + RB - 1) % RB;
         SoftmaxStage st;
-        f32x16 acc;
+        const bool odd = ((js * RB + rb) & 1) != 0;
+        f32x16 acc_zero;
+        f32x16& acc = BIASC ? (odd ? R1 : R0) : acc_zero;
+        f32x16& acc_prev = BIASC ? (odd ? R0 : R1) : R1;
+        if constexpr (!BIASC) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+          for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        }
         FS_SCHED_FENCE();
         // MFMAs of piece p of this unit, the pipeline's memory traffic, and (soft) piece p
         // of the previous unit's soft-max
-        auto step = [&](int p, auto soft) {
+        auto step = [&](int p, bool soft) {
 #pragma unroll
           for (int k = (p * NMAIN) / kPieces; k < ((p + 1) * NMAIN) / kPieces; ++k)
             acc = mfma_k(k, acc, kr, rb);
@@ -632,23 +712,43 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             }
             if (rb == RB - 1 && js + 1 == NSUB && p == 2) load_keys(K[0], nxt, 0);
           }
-          if constexpr (decltype(soft)::value) softmax_piece(p, st, acc_prev, prev_rb);
+          if constexpr (BIASC) {
+            // piece p - 1 was the last to read logits 4(p - 4) .. 4(p - 4) + 3 of the previous
+            // unit: their registers take the next unit's bias
+            if (p >= kBiasPiece && p < kBiasPiece + 4) {
+              const bool same_js = rb + 1 < RB;
+              const bool same_tile = same_js || js + 1 < NSUB;
+              load_bias4(acc_prev, p - kBiasPiece, same_tile ? cur : nxt,
+                         same_js ? js : (js + 1) % NSUB);
+            }
+          }
+          // a wave-uniform branch around VALU work only: the MFMA chain itself stays one
+          // straight line, accumulating in place
+          if (soft) softmax_piece(p, st, acc_prev, prev_rb);
           FS_SCHED_FENCE();
         };
 #pragma unroll
-        for (int p = 0; p < kMaxPieces; ++p) step(p, std::true_type{});
+        for (int p = 0; p < kMaxPieces; ++p) step(p, true);
         // Every logit of the previous unit more than 2^40 (LaunchArgs::skip_log2) below its
         // row's running maximum: its exponentials would not change the fp32 row sums, so
         // they are not computed.
-        if (wave_any(st.mx > skip_below)) {
+        const float mx_rel = BIASC ? st.mx - run_m[prev_rb] : st.mx;
+        const bool soft = wave_any(mx_rel > skip_below);
+        if constexpr (BIASC) {
+          // one branch per piece: a two-sided branch with the MFMAs on both sides makes the
+          // compiler move the accumulator tile at the join
 #pragma unroll
-          for (int p = kMaxPieces; p < kPieces; ++p) step(p, std::true_type{});
+          for (int p = kMaxPieces; p < kPieces; ++p) step(p, soft);
+          if (soft) softmax_tail(st, prev_rb);
+        } else if (soft) {
+#pragma unroll
+          for (int p = kMaxPieces; p < kPieces; ++p) step(p, true);
           softmax_tail(st, prev_rb);
         } else {
 #pragma unroll
-          for (int p = kMaxPieces; p < kPieces; ++p) step(p, std::false_type{});
+          for (int p = kMaxPieces; p < kPieces; ++p) step(p, false);
         }
-        acc_prev = add_bias(acc, kr, rb);
+        if constexpr (!BIASC) R1 = add_bias(acc, kr, rb);
         FS_SCHED_FENCE();
       }
     }
@@ -659,13 +759,13 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     }
     rotate();
   }
-  softmax(acc_prev, RB - 1);
+  softmax(R1, RB - 1);  // BIASC: the last unit of a tile is an odd one, its chain ran in R1
 
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = row0 + rb * 32 + li;
     const float s = run_s[rb] + xor32(run_s[rb]);
-    const float M2 = run_m[rb] * lscale;
+    const float M2 = BIASC ? -run_c[rb] : run_m[rb] * lscale;
     if (row < sd.nq && h == 0) {
       if (sd.splits == 1) {
         epilogue_scalar(sd.ep, row, M2, s, 0.f);
