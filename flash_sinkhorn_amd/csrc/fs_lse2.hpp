@@ -339,6 +339,16 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // The staging code is branch free (clamped rows, additive masks): the only branches of the
   // main loop are the wave-uniform ones around soft-max pieces.
   auto stage_load = [&](int j0, int dbuf) {  // dbuf: LDS buffer of the direct loads
+    {  // raw key-bias terms of row j0 + tid; combined at store time so that nothing here
+       // waits for the loads (threads beyond the tile fetch a clamped, unused row).  Issued
+       // before the tile itself: loads complete in order, and whoever waits for these three
+       // values should not have to wait for the tile as well
+      const int j = max(0, min(j0 + tid, j_end - 1));
+      st_b0 = sd.kb0[j];
+      st_b1 = kb1p[j];
+      st_b2 = kb2p[j];
+      st_pen = (j0 + tid < j_end) ? 0.f : 2.0f * kNegBig;
+    }
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
       if constexpr (DIRECT) {
@@ -360,14 +370,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         if (c4 >= d) v = u32x4{0u, 0u, 0u, 0u};
         st_k[c] = v;
       }
-    }
-    {  // raw key-bias terms of row j0 + tid; combined at store time so that nothing here
-       // waits for the loads (threads beyond the tile fetch a clamped, unused row)
-      const int j = max(0, min(j0 + tid, j_end - 1));
-      st_b0 = sd.kb0[j];
-      st_b1 = kb1p[j];
-      st_b2 = kb2p[j];
-      st_pen = (j0 + tid < j_end) ? 0.f : 2.0f * kNegBig;
     }
   };
   auto stage_store = [&](int buf) {
@@ -515,6 +517,26 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     u32x4 yq[kBf ? NP : 1][kBf ? G::KK16 : 1];
     float ab;
   };
+  // Direct mode: the key operands are read with ds_read_b128 written out by hand.  The compiler
+  // cannot tell a read of one ring buffer from the global->LDS loads still filling another, and
+  // would make every key read wait for ALL of them (vmcnt(0)), which cuts the two-tile
+  // prefetch down to a fraction of a tile; the waits this kernel needs are the explicit ones
+  // before the barrier.  The price: the compiler does not see these reads either, so every
+  // consumer sits behind wait_lds().
+  auto lds_read16 = [&](const unsigned* p) -> u32x4 {
+    if constexpr (DIRECT) {
+      u32x4 v;
+      const unsigned addr =
+          (unsigned)(size_t)(const __attribute__((address_space(3))) unsigned*)p;
+      asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+      return v;
+    } else {
+      return *reinterpret_cast<const u32x4*>(p);
+    }
+  };
+  auto wait_lds = [&]() {  // lgkmcnt(0): every LDS read issued so far has returned
+    if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0xC07F);
+  };
   auto load_keys = [&](KeyRegs& kr, int buf, int js) {
     const unsigned* yrow = lds_k[buf] + (js * 32 + li) * LDWK;
     if constexpr (!kBf) {
@@ -533,7 +555,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         for (int kk = 0; kk < G::KK16; ++kk) {
           const int piece = p * (DP / 8) + 2 * kk + h;
           const int slot = DIRECT ? (piece ^ swz(li)) : piece;  // swz(js*32 + li) == swz(li)
-          kr.yq[p][kk] = *reinterpret_cast<const u32x4*>(yrow + slot * 4);
+          kr.yq[p][kk] = lds_read16(yrow + slot * 4);
         }
     }
     const float b = lds_b[buf][js * 32 + li];
@@ -610,6 +632,10 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int kLoadsPerTile = (DIRECT ? PER_THREAD : 0) + 3;  // direct loads + bias terms
   auto wait_all_vm = [&]() { wait_vm(std::integral_constant<int, 0>{}); };
   auto wait_older_tiles = [&]() { wait_vm(std::integral_constant<int, kLoadsPerTile>{}); };
+  auto wait_older_tiles_and_lds = [&]() {  // the same, and lgkmcnt(0)
+    constexpr int n = kLoadsPerTile;
+    __builtin_amdgcn_s_waitcnt(0x0070 | (n & 15) | ((n >> 4) << 14));
+  };
 
   // LDS buffers rotate: cur holds the tile being multiplied, nxt the next one, nx2 (direct
   // mode with three buffers) the one after that; with two buffers nx2 is cur.
@@ -653,6 +679,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             load_keys(K[0], nxt, 0);
           }
         }
+        wait_lds();
+        FS_SCHED_FENCE();
         const f32x16 acc = add_bias(chain(kr, rb, cur, js), kr, rb);
         if (js == 0) softmax_first(acc, rb); else softmax(acc, rb);
       }
@@ -694,6 +722,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         }
+        wait_lds();  // this unit's key operands (read one unit ago) are in their registers
         FS_SCHED_FENCE();
         // MFMAs of piece p of this unit, the pipeline's memory traffic, and (soft) piece p
         // of the previous unit's soft-max
@@ -707,8 +736,16 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             if (js == 0 && rb == 0 && p == 1) stage_load(j_begin + (t + 2) * G::JT, nx2);
             if (rb == RB - 1 && js + 1 < NSUB && p == 1) load_keys(K[(js + 1) & 1], cur, js + 1);
             if (rb == RB - 1 && js + 1 == NSUB && p == 1) {
-              if constexpr (DIRECT) wait_older_tiles();  // tile t+1 has landed
-              __syncthreads();
+              if constexpr (DIRECT) {
+                // tile t+1 has landed and this wave's bias store has been performed; tile
+                // t+2 stays in flight across the barrier.  A bare s_barrier: __syncthreads()
+                // carries a release fence, for which the compiler waits for every
+                // outstanding global->LDS load, the ones of tile t+2 included.
+                wait_older_tiles_and_lds();
+                __builtin_amdgcn_s_barrier();
+              } else {
+                __syncthreads();
+              }
             }
             if (rb == RB - 1 && js + 1 == NSUB && p == 2) load_keys(K[0], nxt, 0);
           }

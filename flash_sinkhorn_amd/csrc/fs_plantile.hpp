@@ -139,9 +139,27 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
   auto lds_piece = [&](const unsigned* tile, int r, int piece) {
     return *reinterpret_cast<const u32x4*>(tile + r * ROWW + ((piece ^ swz(r)) << 2));
   };
-  // bias of key j (lanes with h == 0 feed it to the fp32 MFMA), in units of the raw products
-  auto bias_of = [&](int j) {
-    return fmaxf(key_bias(sd, j, j_end) * inv_lscale, -3.0e38f);
+  // Bias of key j (lanes with h == 0 feed it to the fp32 MFMA), in units of the raw products.
+  // Its up to three terms are fetched raw, one tile ahead and without branches (absent terms
+  // re-read the first vector and are dropped when the terms are combined a tile later), so
+  // that no wavefront ever sits on a load it has just issued; coefficients are read once.
+  const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
+  const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
+  const float* kb0p = sd.kb0;
+  const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
+  const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
+  struct RawBias {
+    float b0, b1, b2;
+  };
+  auto load_raw_bias = [&](int j) {
+    const int jj = max(0, min(j, j_end - 1));
+    return RawBias{kb0p[jj], kb1p[jj], kb2p[jj]};
+  };
+  auto combine_bias = [&](const RawBias& r, int j) {
+    float b = kc0 * r.b0 + (has_kb1 ? kc1 * r.b1 : 0.f);
+    b += (has_kb2 ? kc2 * r.b2 : 0.f);
+    b = (j < j_end) ? fmaxf(b, kNegBig) : kNegBig;
+    return fmaxf(b * inv_lscale, -3.0e38f);
   };
 
   // ---- V^T operands (kMat): unit (32-key block, column block, step) = 128 pieces ----
@@ -175,9 +193,9 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
   }
 
   // ---- prologue: tiles 0 and 1 on their way, bias (and v) of tile 0 ----
-  float ab_next[NSUB];
+  RawBias raw_next[NSUB];
 #pragma unroll
-  for (int js = 0; js < NSUB; ++js) ab_next[js] = bias_of(j_begin + js * 32 + li);
+  for (int js = 0; js < NSUB; ++js) raw_next[js] = load_raw_bias(j_begin + js * 32 + li);
   if constexpr (MODE == kVec) {
     if (tid < kPtKeys) lds_v[0][tid] = (j_begin + tid < j_end) ? sd.v[j_begin + tid] : 0.f;
   }
@@ -198,12 +216,16 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
     const int nbuf = (buf == 2) ? 0 : buf + 1;
     const int n2buf = (nbuf == 2) ? 0 : nbuf + 1;
     float ab_cur[NSUB];
-    // loads in program order: bias (and v) of tile t + 1, V^T of this tile, key tile t + 2;
-    // a wait for an older load never has to wait for a younger one
+    // Key tile t + 2 first (its buffer was read during tile t - 1, which every wavefront has
+    // left).  While global->LDS loads are in flight the compiler turns each of its own waits
+    // for a register load into a wait for everything, so the tile load goes out as far ahead
+    // of the first such wait (the V^T operands, after the first logits and soft-max) as it can.
+    issue_tile(n2buf);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int js = 0; js < NSUB; ++js) {
-      ab_cur[js] = ab_next[js];
-      ab_next[js] = bias_of(j0 + kPtKeys + js * 32 + li);
+      ab_cur[js] = combine_bias(raw_next[js], j0 + js * 32 + li);
+      raw_next[js] = load_raw_bias(j0 + kPtKeys + js * 32 + li);
     }
     float v_next = 0.f;
     if constexpr (MODE == kVec) {
@@ -215,7 +237,6 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
     for (int js = 0; js < NSUB; ++js) {
       u32x4 va[kHasO ? NCB : 1][2][2];
       if constexpr (kHasO) load_vt(va, (j0 >> 5) + js);
-      if (js == NSUB - 1) issue_tile(n2buf);  // tile t + 2, after the last register loads of tile t
       __builtin_amdgcn_sched_barrier(0);
 
       // A operands of the logits: key row js*32 + li, [plane][step]
