@@ -113,9 +113,19 @@ class _SinkhornCostFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, y, a, b, eps_list: Tuple[float, ...], config: _SinkhornConfig,
-                label_x, label_y, label_cost_matrix):
+                label_x, label_y, label_cost_matrix, presolved=None):
+        """``presolved``: the tuple ``sinkhorn_flashstyle_symmetric`` would return for this
+        problem (with ``return_prelast=config.last_extrapolation``), when the caller has already
+        run the solve (the two self terms of a debiased loss are solved together)."""
         eps_last = float(eps_list[-1])
-        if config.backend == "alternating":
+        if presolved is not None:
+            if config.last_extrapolation:
+                f_cost, g_cost, f_grad, g_grad = presolved
+            else:
+                f_cost, g_cost = presolved
+                f_grad, g_grad = f_cost, g_cost
+            balanced_formula = config.rho_x is None or config.rho_y is None
+        elif config.backend == "alternating":
             f_cost, g_cost = sinkhorn_flashstyle_alternating(
                 x, y, a, b, eps=eps_last, n_iters=len(eps_list), cost_scale=config.cost_scale,
                 rho_x=config.rho_x, rho_y=config.rho_y, allow_tf32=config.allow_tf32,
@@ -167,4 +177,4 @@ class _SinkhornCostFn(torch.autograd.Function):
             grad_a = grad_out * f_cost
         if b.requires_grad:
             grad_b = grad_out * g_cost
-        return grad_x, grad_y, grad_a, grad_b, None, None, None, None, None
+        return grad_x, grad_y, grad_a, grad_b, None, None, None, None, None, None

@@ -49,6 +49,7 @@ _SIGNATURES = {
     "fs_lse_fused": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_symmetric_step": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + _TAIL),
     "fs_symmetric_steps": (ctypes.c_int, [_P] * 12 + [_I] * 3 + [_P] * 4 + [ctypes.c_int, _F] + _TAIL),
+    "fs_self_pair_steps": (ctypes.c_int, [_P] * 12 + [_I] * 3 + [_P] * 5 + [ctypes.c_int, _F] + _TAIL),
     "fs_grad": (ctypes.c_int, [_P] * 13 + [_I] * 3 + [_F] * 2 + _TAIL),
     "fs_apply_vec": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + [ctypes.c_int] + _TAIL),
     "fs_apply_mat": (ctypes.c_int, [_P] * 9 + [_I] * 4 + [_F] * 2 + [ctypes.c_int] + _TAIL),
@@ -131,12 +132,15 @@ class PreparedOperands:
     run on the stream current at construction.
     """
 
-    def __init__(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int):
+    def __init__(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int, self_pair: bool = False):
         n, d = x.shape
         m = y.shape[0]
         L = lib()
         nbytes = max(int(L.fs_workspace_bytes(op, n, m, d))
                      for op in (OP_LSE, OP_SYMMETRIC_STEP))
+        if self_pair:  # the two self problems of fs_self_pair_steps share the workspace
+            nbytes = max(nbytes, int(L.fs_workspace_bytes(OP_SYMMETRIC_STEP, n, n, d))
+                         + int(L.fs_workspace_bytes(OP_SYMMETRIC_STEP, m, m, d)))
         self.ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
         self.nbytes = nbytes
         self.flag_bits = flag_bits

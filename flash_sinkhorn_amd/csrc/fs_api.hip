@@ -340,6 +340,8 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
     sd.part_ms = reinterpret_cast<float*>(base + part_off[s]);
     sd.part_o = vec ? reinterpret_cast<float*>(base + part_o_off[s]) : nullptr;
     sd.plane_scale = plane_scales(ps, ws);
+    sd.ps_q = plane_index(ps, sd.q, sd.nq);
+    sd.ps_k = plane_index(ps, sd.k, sd.nk);
     sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
     sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
     blocks[s] = plans[s].igroups * plans[s].bsplits;
@@ -485,6 +487,8 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
       sd.part_o = sd.part_ms + (((size_t)sd.splits * (size_t)sd.nq * 2 + 3) & ~(size_t)3);
     }
     sd.plane_scale = plane_scales(ps, ws);
+    sd.ps_q = plane_index(ps, sd.q, sd.nq);
+    sd.ps_k = plane_index(ps, sd.k, sd.nk);
     sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
     sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
     sd.vplanes = reinterpret_cast<const unsigned*>(base + vt_off[s]);
@@ -630,6 +634,8 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
       sd.part_o = sd.part_ms + (((size_t)p.splits * (size_t)sd.nq * 2 + 3) & ~(size_t)3);
     }
     sd.plane_scale = plane_scales(ps, ws);
+    sd.ps_q = plane_index(ps, sd.q, sd.nq);
+    sd.ps_k = plane_index(ps, sd.k, sd.nk);
     sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
     sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
     if (has_o) {
@@ -809,6 +815,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       sd.qplanes = plane_of(ps, ws, sd.q, sd.nq);
       sd.kplanes = plane_of(ps, ws, sd.k, sd.nk);
       sd.plane_scale = plane_scales(ps, ws);
+      sd.ps_q = plane_index(ps, sd.q, sd.nq);
+      sd.ps_k = plane_index(ps, sd.k, sd.nk);
     }
     a.side[s] = sd;
   }
@@ -1049,6 +1057,43 @@ int fs_symmetric_steps(const float* x, const float* y, const float* f_hat, const
     if (rc != FS_OK) return rc;
     f_in = f_out;
     g_in = g_out;
+  }
+  return FS_OK;
+}
+
+int fs_self_pair_steps(const float* x, const float* y, const float* fx_hat, const float* fy_hat,
+                       const float* log_a, const float* log_b, float* fx_a, float* fy_a,
+                       float* fx_b, float* fy_b, const float* shift_x, const float* shift_y,
+                       int64_t n, int64_t m, int64_t d, const float* eps_x, const float* eps_y,
+                       const float* alpha, const float* damp_x, const float* damp_y, int n_steps,
+                       float coord_scale, uint32_t flags, void* workspace, size_t workspace_bytes,
+                       void* stream) {
+  if (!x || !y || !fx_hat || !fy_hat || !log_a || !log_b || !fx_a || !fy_a || !fx_b || !fy_b ||
+      !eps_x || !eps_y || !alpha || !damp_x || !damp_y)
+    return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (n_steps < 0) return FS_ERR_BAD_ARGUMENT;
+  if (fx_a == fx_b || fy_a == fy_b || fx_a == fx_hat || fx_b == fx_hat || fy_a == fy_hat ||
+      fy_b == fy_hat || fx_a == fy_a || fx_a == fy_b || fx_b == fy_a || fx_b == fy_b)
+    return FS_ERR_BAD_ARGUMENT;
+  const float* fx_in = fx_hat;
+  const float* fy_in = fy_hat;
+  for (int s = 0; s < n_steps; ++s) {
+    if (!(eps_x[s] > 0.f) || !(eps_y[s] > 0.f)) return FS_ERR_BAD_ARGUMENT;
+    float* fx_out = (s & 1) ? fx_b : fx_a;
+    float* fy_out = (s & 1) ? fy_b : fy_a;
+    Side sd[2];
+    sd[0] = lse_side(x, x, fx_in, kLog2e / eps_x[s], log_a, kLog2e, n, n,
+                     coord_scale / eps_x[s] * kLog2e);
+    lse_epilogue(sd[0], fx_out, fx_in, alpha[s], eps_x[s], damp_x[s], shift_x);
+    sd[1] = lse_side(y, y, fy_in, kLog2e / eps_y[s], log_b, kLog2e, m, m,
+                     coord_scale / eps_y[s] * kLog2e);
+    lse_epilogue(sd[1], fy_out, fy_in, alpha[s], eps_y[s], damp_y[s], shift_y);
+    const int rc = run_stream(kLse, false, sd, 2, d, workspace, workspace_bytes,
+                              (hipStream_t)stream, flags);
+    if (rc != FS_OK) return rc;
+    fx_in = fx_out;
+    fy_in = fy_out;
   }
   return FS_OK;
 }

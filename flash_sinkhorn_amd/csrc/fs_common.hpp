@@ -71,6 +71,8 @@ struct Side {
   const unsigned* qplanes;  // split-bf16 kernels: query rows as packed bf16 planes [nq][NP][DP/2]
   const unsigned* kplanes;  // same for the key rows [nk][NP][DP/2]
   const float* plane_scale; // fp16 planes: power-of-two scales of the two operand matrices [2]
+  int ps_q, ps_k;           // which of the two scales belongs to the query / key matrix (a side
+                            // may pair a matrix with itself while another matrix is present)
   const unsigned* vplanes;  // plan_gemm_kernel: fp16 planes of the value matrix in operand order
   const float* vplane_scale;  // their power-of-two scale [1]
   const unsigned* q2planes; // plan_gemm_kernel, mat5: chunked fp16 planes of q2

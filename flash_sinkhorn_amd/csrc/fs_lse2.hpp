@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // inside the exp2 argument, and the bias / running max are kept in dot-product units.
   // fp16 planes carry a power-of-two scale per matrix, which lscale takes out again.
   float lscale = kBf ? sd.qscale : 1.0f;
-  if constexpr (PREC == kH3) lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  if constexpr (PREC == kH3) lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = kBf ? 1.0f / lscale : 1.0f;
   const float skip_below = args.skip_log2 * inv_lscale;  // in accumulator units
 

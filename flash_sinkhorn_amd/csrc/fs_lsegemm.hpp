@@ -59,7 +59,7 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   const int j_end = min(sd.nk, j_begin + sd.chunk);
   const int ntiles = (j_end - j_begin + kGemmRows - 1) / kGemmRows;
 
-  const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = 1.0f / lscale;
 
   // ---- loader role: wavefronts 0-3 bring query rows, 4-7 key rows (64 rows each) ----

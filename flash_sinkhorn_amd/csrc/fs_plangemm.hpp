@@ -182,7 +182,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   const int ntiles = (j_end > j_begin) ? (j_end - j_begin + kPgKeys - 1) / kPgKeys : 0;
   const int cb0 = (cg * 8 + wave) * CB;  // first column block of this wavefront
 
-  const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = 1.0f / lscale;
   // MAT5: per-row power of two with |T_ij| * t_unit <= 2^7 from |T_ij| <= |A_i| max_j |y_j|
   // (in plane units; sd.q2norm2 = |A_i|^2, sd.kmax2 = 64 partial maxima of |y_j|^2, fp32 rows)

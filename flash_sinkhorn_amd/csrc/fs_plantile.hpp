@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
   const int j_end = min(sd.nk, j_begin + sd.chunk);
   const int ntiles = (j_end > j_begin) ? (j_end - j_begin + kPtKeys - 1) / kPtKeys : 0;
 
-  const float lscale = sd.qscale / (sd.plane_scale[0] * sd.plane_scale[1]);
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = 1.0f / lscale;
 
   // ---- stationary query planes: [block][plane][16-column step] ----

@@ -168,6 +168,41 @@ def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale,
     return f_out, (f_out if self_problem else g_work[last])
 
 
+def _self_pair_steps_raw(x, y, fx_hat, fy_hat, log_a, log_b, steps, *, cost_scale, shift_x=None,
+                         shift_y=None, allow_tf32=True, use_exp2=True, prepared=None):
+    """The self problems OT(x, x; a) and OT(y, y; b) advanced together (``fs_self_pair_steps``):
+    ``steps`` = [(eps_x, eps_y, alpha, damping_x, damping_y), ...], one launch per step for both.
+    ``prepared`` must have been built with ``self_pair=True``.  Returns (fx_hat, fy_hat)."""
+    import ctypes
+    k = len(steps)
+    if k == 0:
+        return fx_hat, fy_hat
+    n, d = x.shape
+    m = y.shape[0]
+    fx_work = [torch.empty((n,), device=x.device, dtype=torch.float32) for _ in range(2)]
+    fy_work = [torch.empty((m,), device=x.device, dtype=torch.float32) for _ in range(2)]
+    arr = ctypes.c_float * k
+    ex, ey, al, dx, dy = (arr(*[float(s[i]) for s in steps]) for i in range(5))
+    flag_bits = _lib.flags(use_exp2, allow_tf32)
+    if prepared is not None and prepared.serves(x, y, flag_bits):
+        wp, wn, fl, _keep = (prepared.ws.data_ptr(), prepared.nbytes,
+                             flag_bits | _lib.FS_FLAG_OPERANDS_PREPARED, prepared.ws)
+    else:
+        L = _lib.lib()
+        nbytes = (int(L.fs_workspace_bytes(_lib.OP_SYMMETRIC_STEP, n, n, d))
+                  + int(L.fs_workspace_bytes(_lib.OP_SYMMETRIC_STEP, m, m, d)))
+        _keep = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+        wp, wn, fl = _keep.data_ptr(), nbytes, flag_bits
+    rc = _lib.lib().fs_self_pair_steps(
+        x.data_ptr(), y.data_ptr(), fx_hat.data_ptr(), fy_hat.data_ptr(), log_a.data_ptr(),
+        log_b.data_ptr(), fx_work[0].data_ptr(), fy_work[0].data_ptr(), fx_work[1].data_ptr(),
+        fy_work[1].data_ptr(), _lib.ptr(shift_x), _lib.ptr(shift_y), n, m, d, ex, ey, al, dx, dy,
+        k, 2.0 * float(cost_scale), fl, wp, wn, _lib.stream_of(x))
+    _lib.check(rc, "fs_self_pair_steps")
+    last = (k - 1) & 1
+    return fx_work[last], fy_work[last]
+
+
 def flashsinkhorn_symmetric_step(
     x: torch.Tensor, y: torch.Tensor, f_hat: torch.Tensor, g_hat: torch.Tensor,
     log_a: torch.Tensor, log_b: torch.Tensor, eps: float, *,

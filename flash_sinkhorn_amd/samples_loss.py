@@ -17,6 +17,7 @@ from flash_sinkhorn_amd._autograd import _SinkhornConfig, _SinkhornCostFn
 from flash_sinkhorn_amd.kernels._common import epsilon_schedule, max_diameter
 from flash_sinkhorn_amd.sinkhorn_solvers import (
     sinkhorn_flashstyle_alternating, sinkhorn_flashstyle_symmetric,
+    sinkhorn_flashstyle_symmetric_self_pair,
 )
 
 __all__ = ["SamplesLoss"]
@@ -232,17 +233,33 @@ class SamplesLoss(torch.nn.Module):
             raise ValueError("flash_sinkhorn.SamplesLoss requires CUDA tensors.")
         config = self._make_config()
 
-        def ot(xb, yb, ab, bb, lx, ly):
+        def ot(xb, yb, ab, bb, lx, ly, presolved=None):
             sched = tuple(self._eps_list_for_inputs(xb, yb))
             return _SinkhornCostFn.apply(xb, yb, ab, bb, sched, config, lx, ly,
-                                         self.label_cost_matrix)
+                                         self.label_cost_matrix, presolved)
+
+        # The self terms are independent solves; without early stopping, labels or an
+        # asymmetric relaxation they advance together, one launch per step for both.
+        labelled = (self.label_cost_matrix is not None and label_x is not None
+                    and label_y is not None and self.lambda_y != 0.0)
+        pair_ok = (self.backend == "symmetric" and self.threshold is None and not labelled
+                   and self.rho_x == self.rho_y)
 
         def cost(xb, yb, ab, bb):
-            # debias: OT(a,b) - OT(a,a)/2 - OT(b,b)/2, each an independent solve
+            # debias: OT(a,b) - OT(a,a)/2 - OT(b,b)/2
             c = ot(xb, yb, ab, bb, label_x, label_y)
             if self.debias:
-                c = c - 0.5 * ot(xb, xb, ab, ab, label_x, label_x) \
-                      - 0.5 * ot(yb, yb, bb, bb, label_y, label_y)
+                pre_x = pre_y = None
+                if pair_ok:
+                    pre_x, pre_y = sinkhorn_flashstyle_symmetric_self_pair(
+                        xb, ab, yb, bb, blur=self.blur, scaling=self.scaling,
+                        use_epsilon_scaling=self.use_epsilon_scaling, eps=self.eps,
+                        n_iters=self.n_iters, allow_tf32=self.allow_tf32,
+                        use_exp2=self.use_exp2, cost_scale=self.cost_scale, rho=self.rho_x,
+                        last_extrapolation=self.last_extrapolation,
+                        return_prelast=self.last_extrapolation)
+                c = c - 0.5 * ot(xb, xb, ab, ab, label_x, label_x, pre_x) \
+                      - 0.5 * ot(yb, yb, bb, bb, label_y, label_y, pre_y)
             return c
 
         if parsed.batched:

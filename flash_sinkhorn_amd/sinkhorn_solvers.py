@@ -245,3 +245,80 @@ def sinkhorn_flashstyle_symmetric(
     if return_n_iters:
         out = out + (used,)
     return out
+
+
+def sinkhorn_flashstyle_symmetric_self_pair(
+    x: torch.Tensor, a: torch.Tensor, y: torch.Tensor, b: torch.Tensor, *,
+    blur: float = 0.05, scaling: float = 0.5, use_epsilon_scaling: bool = True,
+    last_extrapolation: bool = True, cost_scale: float = 1.0,
+    eps: Optional[float] = None, n_iters: Optional[int] = None,
+    rho: Optional[float] = None, allow_tf32: bool = True, use_exp2: bool = True,
+    return_prelast: bool = False,
+):
+    """The two self problems of a debiased divergence solved together.
+
+    Returns ``(out_x, out_y)`` where ``out_x`` is what
+    ``sinkhorn_flashstyle_symmetric(x, x, a, a, ...)`` returns with the same keyword
+    arguments (``rho`` standing for ``rho_x = rho_y``) and ``out_y`` likewise for
+    ``(y, y, b, b)``: in a self problem both potentials stay equal, a step is one half-update,
+    and the half-updates of the two problems share a launch (``fs_self_pair_steps``).  Each
+    problem follows its own eps schedule (its own diameter under eps-scaling); where one
+    schedule is longer, its remaining steps run alone.  No early stopping, warm start or
+    label cost: callers use the single-problem solver for those.
+    """
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
+        _self_pair_steps_raw, _symmetric_steps_raw,
+    )
+
+    def schedule(pts):
+        if use_epsilon_scaling:
+            lst = list(epsilon_schedule(max_diameter(pts, pts), blur, scaling, p=2.0))
+        else:
+            if eps is None or n_iters is None:
+                raise ValueError("When use_epsilon_scaling=False, provide eps and n_iters")
+            lst = [float(eps)] * int(n_iters)
+        if n_iters is not None:
+            lst = lst[: int(n_iters)]
+        if len(lst) == 0:
+            raise ValueError("eps_list must be non-empty")
+        return lst
+
+    xf, yf = x.detach().float().contiguous(), y.detach().float().contiguous()
+    ex, ey = schedule(xf), schedule(yf)
+    alpha_x = (cost_scale * (xf * xf).sum(dim=1)).contiguous()
+    alpha_y = (cost_scale * (yf * yf).sum(dim=1)).contiguous()
+    log_a, log_b = _f32c(log_weights(a.detach())), _f32c(log_weights(b.detach()))
+    fx, fy = -alpha_x, -alpha_y
+    shift_x = alpha_x if rho is not None else None
+    shift_y = alpha_y if rho is not None else None
+    prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32), self_pair=True)
+    kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
+
+    def pair(fx, fy, steps):  # steps: [(eps_x, eps_y, weight)]
+        full = [(e1, e2, w, dampening(e1, rho), dampening(e2, rho)) for e1, e2, w in steps]
+        return _self_pair_steps_raw(xf, yf, fx, fy, log_a, log_b, full, shift_x=shift_x,
+                                    shift_y=shift_y, prepared=prepared, **kw)
+
+    def alone(pts, f, log_w, shift, steps):  # steps: [(eps, weight)]
+        full = [(e, w, dampening(e, rho), dampening(e, rho)) for e, w in steps]
+        return _symmetric_steps_raw(pts, pts, f, f, log_w, log_w, full, shift_x=shift,
+                                    shift_y=shift, **kw)[0]
+
+    sx = [(ex[0], 1.0)] + [(e, 0.5) for e in ex]
+    sy = [(ey[0], 1.0)] + [(e, 0.5) for e in ey]
+    k = min(len(sx), len(sy))
+    fx, fy = pair(fx, fy, [(sx[i][0], sy[i][0], sx[i][1]) for i in range(k)])
+    if len(sx) > k:
+        fx = alone(xf, fx, log_a, shift_x, sx[k:])
+    if len(sy) > k:
+        fy = alone(yf, fy, log_b, shift_y, sy[k:])
+
+    pre_x = pre_y = None
+    if last_extrapolation:
+        pre_x, pre_y = fx + alpha_x, fy + alpha_y
+        fx, fy = pair(fx, fy, [(ex[-1], ey[-1], 1.0)])
+    out_x = (fx + alpha_x,) * 2
+    out_y = (fy + alpha_y,) * 2
+    if return_prelast and last_extrapolation:
+        out_x, out_y = out_x + (pre_x, pre_x), out_y + (pre_y, pre_y)
+    return out_x, out_y

@@ -148,6 +148,28 @@ int fs_symmetric_steps(const float* x, const float* y, const float* f_hat, const
                        uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The two self problems OT(x, x; a) and OT(y, y; b) of a debiased divergence, n_steps Jacobi
+ * steps each, one launch per step for both: in a self problem both potentials stay equal, so a
+ * step is one half-update per problem, fx' = (1-alpha) fx + alpha*(-eps_x*damp_x*LSE_j[...]) over
+ * the rows of x against x itself, and likewise fy' over y.  eps_x, eps_y, alpha, damp_x, damp_y
+ * are HOST arrays of n_steps floats (the two problems may follow different eps schedules; the
+ * averaging weight is shared).  Step s reads what step s-1 wrote (step 0 reads fx_hat, fy_hat);
+ * even steps write (fx_a, fy_a), odd steps (fx_b, fy_b).  shift_x / shift_y as in
+ * fs_symmetric_step.  Workspace: fs_workspace_bytes(FS_OP_SYMMETRIC_STEP, n, n, d) +
+ * fs_workspace_bytes(FS_OP_SYMMETRIC_STEP, m, m, d) bytes suffice; with
+ * FS_FLAG_OPERANDS_PREPARED the planes are those fs_prepare_operands(x, y, ...) wrote.
+ * Replaces the two independent solves sinkhorn_flashstyle_symmetric(x, x, a, a, ...) and
+ * (y, y, b, b, ...) that SamplesLoss(debias=True) runs (samples_loss.py:494-512).
+ */
+int fs_self_pair_steps(const float* x, const float* y, const float* fx_hat, const float* fy_hat,
+                       const float* log_a, const float* log_b, float* fx_a, float* fy_a,
+                       float* fx_b, float* fy_b, const float* shift_x, const float* shift_y,
+                       int64_t n, int64_t m, int64_t d, const float* eps_x, const float* eps_y,
+                       const float* alpha, const float* damp_x, const float* damp_y, int n_steps,
+                       float coord_scale, uint32_t flags, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
+/*
  * Analytic gradient: grad_x[i,:] = 2*cost_scale*gs*a_i*(x_i - sum_j w_ij y_j),
  * w_i. = softmax_j[(g_j - C_ij)/eps + log_b_j]; grad_y symmetric over i.
  * Standard (unshifted) potentials f, g; x2, y2 = row squared norms; gs is read

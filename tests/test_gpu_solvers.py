@@ -394,3 +394,58 @@ def test_custom_operators_match_the_launchers():
     assert (idx.cpu().numpy() == want_idx).mean() > 0.99
     torch.library.opcheck(ops.lse_fused.default, (X, Y, G, LB, 0.2),
                           test_utils=("test_schema", "test_faketensor"))
+
+
+@pytest.mark.parametrize("n,m,d", [(700, 500, 64), (300, 260, 200), (2000, 2000, 3)])
+@pytest.mark.parametrize("kw", [
+    dict(use_epsilon_scaling=False, eps=0.1, n_iters=12),
+    dict(use_epsilon_scaling=False, eps=0.1, n_iters=7, last_extrapolation=False),
+    dict(use_epsilon_scaling=True, blur=0.3, scaling=0.7),
+    dict(use_epsilon_scaling=True, blur=0.3, scaling=0.7, rho=2.0),
+])
+def test_self_pair_equals_separate_self_solves(n, m, d, kw):
+    """The two debiasing self problems advanced in shared launches (fs_self_pair_steps) give
+    the potentials of the two independent self solves; under eps-scaling the clouds have
+    different diameters, hence schedules of different lengths."""
+    from flash_sinkhorn_amd.sinkhorn_solvers import (
+        sinkhorn_flashstyle_symmetric, sinkhorn_flashstyle_symmetric_self_pair)
+    x, y, a, b = inputs(61, n, m, d, scale=1.0 / np.sqrt(d))
+    y = (y * 2.5).astype(np.float32)          # a wider cloud: a longer eps schedule
+    X, Y, A, B = dev(x, y, a, b)
+    solo = dict(kw)
+    rho = solo.pop("rho", None)
+    last = kw.get("last_extrapolation", True)
+    out_x, out_y = sinkhorn_flashstyle_symmetric_self_pair(
+        X, A, Y, B, allow_tf32=False, return_prelast=True, **kw)
+    for pts, w, got in ((X, A, out_x), (Y, B, out_y)):
+        want = sinkhorn_flashstyle_symmetric(pts, pts, w, w, allow_tf32=False, rho_x=rho,
+                                             rho_y=rho, return_prelast=True, **solo)
+        assert len(got) == len(want) == (4 if last else 2)
+        for g, wv in zip(got, want):
+            scale = float(wv.abs().max())
+            assert float((g - wv).abs().max()) <= 2e-6 * scale
+
+
+def test_debiased_loss_with_paired_self_terms_equals_separate(monkeypatch):
+    """SamplesLoss(debias=True) solves its two self terms together; loss and gradients equal
+    those of the three independent solves."""
+    import flash_sinkhorn_amd.samples_loss as sl
+    from flash_sinkhorn_amd import SamplesLoss
+    x, y, a, b = inputs(63, 900, 700, 8, scale=0.5)
+    for cfg in (dict(blur=0.1, use_epsilon_scaling=False, eps=0.01, n_iters=20),
+                dict(blur=0.2, scaling=0.6), dict(blur=0.2, scaling=0.6, reach=1.5)):
+        results = []
+        for paired in (True, False):
+            X, Y, A, B = dev(x, y, a, b)
+            X.requires_grad_(True)
+            Y.requires_grad_(True)
+            loss_fn = SamplesLoss("sinkhorn", debias=True, allow_tf32=False, **cfg)
+            if not paired:
+                loss_fn.threshold = 1e-30      # never met: switches the pairing off only
+            val = loss_fn(A, X, B, Y)
+            gx, gy = torch.autograd.grad(val, [X, Y])
+            results.append((val.detach(), gx, gy))
+        (v1, gx1, gy1), (v0, gx0, gy0) = results
+        assert abs(float(v1 - v0)) <= 1e-5 * max(abs(float(v0)), 1e-3)
+        assert float((gx1 - gx0).abs().max()) <= 1e-5 * float(gx0.abs().max())
+        assert float((gy1 - gy0).abs().max()) <= 1e-5 * float(gy0.abs().max())

@@ -56,6 +56,16 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
                                 one, one, 1, 2.0, 0, None, 0, None) == -3
     assert L.fs_symmetric_steps(*fk[:10], None, None, 8, 8, 4, one, one, one, one, 0, 2.0, 0,
                                 None, 0, None) == 0
+    # the paired self problems: null schedule, aliased work vectors, bad eps, zero steps
+    assert L.fs_self_pair_steps(*fk[:10], None, None, 8, 8, 4, one, None, one, one, one, 1, 2.0, 0,
+                                None, 0, None) == -1
+    assert L.fs_self_pair_steps(*fk[:6], fk[6], fk[6], fk[8], fk[9], None, None, 8, 8, 4, one, one,
+                                one, one, one, 1, 2.0, 0, None, 0, None) == -3
+    zero = (ctypes.c_float * 1)(0.0)
+    assert L.fs_self_pair_steps(*fk[:10], None, None, 8, 8, 4, one, zero, one, one, one, 1, 2.0, 0,
+                                None, 0, None) == -3
+    assert L.fs_self_pair_steps(*fk[:10], None, None, 8, 8, 4, one, one, one, one, one, 0, 2.0, 0,
+                                None, 0, None) == 0
 
 
 def test_workspace_is_deterministic_and_zero_for_small_problems():
