@@ -743,8 +743,9 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   static const int use_plan_tile = env_int("FS_PLANTILE", 1);
+  static const int mat5_128 = env_int("FS_MAT5_128", 1);
   const bool tile_mode = mode == kMat || mode == kVec || mode == kArgmax ||
-                         (mode == kMat5 && cfg.dp <= 64);
+                         (mode == kMat5 && (cfg.dp <= 64 || mat5_128));
   if (tile_mode && !fam.sliced && use_plan_tile && (cfg.prec == 3 || cfg.prec == 1)) {
     // the reduced mode runs on the fp16 planes too (same speed, smaller error); planes a caller
     // prepared for it are bf16 and are not used here
@@ -958,7 +959,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
   if ((mode == kMat || mode == kMat5) && fam.sliced)
     gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
-  if ((mode == kMat || mode == kVec || mode == kArgmax || (mode == kMat5 && d <= 64)) && !fam.sliced)
+  if ((mode == kMat || mode == kVec || mode == kArgmax || mode == kMat5) && !fam.sliced)
     gemm = pt_ws_bytes(mode, n, m, d, both, either, fam);
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);

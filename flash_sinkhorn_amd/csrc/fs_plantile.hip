@@ -31,11 +31,12 @@ int launch_plan_tile(const LaunchArgs& a, int mode, int dp, int rb, int blocks, 
   if (mode == kMat) return launch_dp<kMat>(a, dp, rb, blocks, st);
   if (mode == kVec) return launch_dp<kVec>(a, dp, rb, blocks, st);
   if (mode == kArgmax) return launch_dp<kArgmax>(a, dp, rb, blocks, st);
-  if (mode == kMat5) {  // one row block per wavefront, rows of at most 64 columns
+  if (mode == kMat5) {  // one row block per wavefront
     switch (dp) {
       case 16: hipLaunchKernelGGL((plan_tile_kernel<16, 1, kMat5>), dim3(blocks), dim3(256), 0, st, a); break;
       case 32: hipLaunchKernelGGL((plan_tile_kernel<32, 1, kMat5>), dim3(blocks), dim3(256), 0, st, a); break;
       case 64: hipLaunchKernelGGL((plan_tile_kernel<64, 1, kMat5>), dim3(blocks), dim3(256), 0, st, a); break;
+      case 128: hipLaunchKernelGGL((plan_tile_kernel<128, 1, kMat5>), dim3(blocks), dim3(256), 0, st, a); break;
       default: return FS_ERR_UNSUPPORTED;
     }
     return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;

@@ -34,10 +34,10 @@ namespace fs {
 constexpr float kPtLazyThresh = 8.0f;  // probabilities stay below 2^8
 
 template <int DP, int RB, int MODE>
-__global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args) {
+__global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void plan_tile_kernel(const LaunchArgs args) {
   static_assert(MODE == kMat || MODE == kVec || MODE == kArgmax || MODE == kMat5,
                 "plan_tile_kernel modes");
-  static_assert(MODE != kMat5 || (DP <= 64 && RB == 1), "mat5: the second operand needs registers");
+  static_assert(MODE != kMat5 || RB == 1, "mat5: the second operand needs registers");
   constexpr bool kHasO = (MODE == kMat || MODE == kMat5);
   static_assert(DP == 16 || DP == 32 || DP == 64 || DP == 128, "padded row widths");
   constexpr int kPtKeys = (DP == 128) ? 32 : 64;  // keys per tile
@@ -263,9 +263,12 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
 
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        f32x16 acc;
+        f32x16 acc, tacc;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        for (int r = 0; r < 16; ++r) {
+          acc[r] = 0.f;
+          tacc[r] = 0.f;
+        }
         // products lo*hi, hi*lo, hi*hi
         if constexpr (kStreamK) {
 #pragma unroll
@@ -281,6 +284,17 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, k_hi),
                                                          __builtin_bit_cast(f16x8, xq[rb][0][kk]),
                                                          acc, 0, 0, 0);
+            if constexpr (MODE == kMat5) {  // second contraction on the same key operands
+              tacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, k_lo), __builtin_bit_cast(f16x8, aq[rb][0][kk]), tacc,
+                  0, 0, 0);
+              tacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, k_hi), __builtin_bit_cast(f16x8, aq[rb][1][kk]), tacc,
+                  0, 0, 0);
+              tacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, k_hi), __builtin_bit_cast(f16x8, aq[rb][0][kk]), tacc,
+                  0, 0, 0);
+            }
           }
         } else {
 #pragma unroll
@@ -293,10 +307,7 @@ __global__ __launch_bounds__(256, 2) void plan_tile_kernel(const LaunchArgs args
                   acc, 0, 0, 0);
           }
         }
-        f32x16 tacc;
-        if constexpr (MODE == kMat5) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) tacc[r] = 0.f;
+        if constexpr (MODE == kMat5 && !kStreamK) {
 #pragma unroll
           for (int prod = 0; prod < 3; ++prod) {
             const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;

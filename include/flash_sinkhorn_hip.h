@@ -28,11 +28,10 @@
  *    The d <= 128 log-sum-exp kernel leaves out the exponentials of a 32 x 32 logits tile
  *    whose every entry lies more than 2^40 below its row's running maximum (they cannot
  *    change the fp32 row sums); FS_FLAG_NO_TILE_SKIP computes them all the same.
- *    For d > 128 every operation (log-sum-exp, gradient, plan products, mat5) runs on
- *    the two-plane fp16 operands by default and with FS_FLAG_REDUCED_OPERANDS, and on fp32
- *    MFMA operands with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS.  For d <= 128 the
- *    gradient, plan-vector / plan-matrix products and the c-transform do the same; mat5 uses
- *    fp32 MFMA operands there.
+ *    The gradient, the plan-vector / plan-matrix products, mat5 and the c-transform, and for
+ *    d > 128 the log-sum-exp as well, run on the two-plane fp16 operands by default and with
+ *    FS_FLAG_REDUCED_OPERANDS, and on fp32 MFMA operands with FS_FLAG_FP32_MFMA or
+ *    FS_FLAG_BF16X3_OPERANDS.
  */
 #ifndef FLASH_SINKHORN_HIP_H
 #define FLASH_SINKHORN_HIP_H

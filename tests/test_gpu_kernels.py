@@ -161,6 +161,24 @@ def test_mat5(n, m, d):
     assert rel_err(got, want) < RTOL
 
 
+@pytest.mark.parametrize("n,m,d,scale", [(300, 5000, 96, 1.0), (1500, 2100, 128, 1.0),
+                                         (260, 1300, 128, 3e3), (260, 1300, 72, 1e-3)])
+def test_mat5_wide_rows_on_planes(n, m, d, scale):
+    """64 < d <= 128: mat5 runs on fp16 planes with the key operands streamed from LDS step by
+    step and both stationary operands in registers (one wavefront per SIMD); several key tiles,
+    split keys, and clouds / A in unrelated units."""
+    from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
+    x, y, a, b, f, g = problem(n, m, d, seed=7)
+    x, y = (x * scale).astype(np.float32), (y * scale).astype(np.float32)
+    eps = 0.5 * scale * scale
+    f = ((f - 2.0) * scale * scale).astype(np.float32)
+    g = (g * scale * scale).astype(np.float32)
+    A = (np.random.default_rng(8).standard_normal((n, d)) * 50.0 / scale).astype(np.float32)
+    want = oracle.mat5(x, y, f, g, A, eps, 0.5)
+    got = mat5_sqeuclid(*dev(x, y, f, g, A), eps=eps, cost_scale=0.5)
+    assert rel_err(got, want) < RTOL
+
+
 @pytest.mark.parametrize("scale", [1e-4, 1.0, 3e4])
 @pytest.mark.parametrize("d", [64, 200])
 def test_symmetric_step_is_scale_robust(scale, d):
