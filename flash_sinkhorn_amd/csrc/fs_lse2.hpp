@@ -742,7 +742,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
                 // carries a release fence, for which the compiler waits for every
                 // outstanding global->LDS load, the ones of tile t+2 included.
                 wait_older_tiles_and_lds();
+                // the empty asm statements keep the compiler from moving LDS accesses across
+                // the barrier (the barrier builtin itself is not a memory operation to it)
+                asm volatile("" ::: "memory");
                 __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
               } else {
                 __syncthreads();
               }
