@@ -221,8 +221,20 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
           (const __attribute__((address_space(1))) void*)(qsrc + c * 32),
           (__attribute__((address_space(3))) void*)(&lds[buf][(wave * 8) * 32]), 16, 0, 0);
   };
+  // Stage reads are ds_read_b128 written out by hand: the compiler cannot tell a read of one
+  // stage buffer from the global->LDS loads filling the others and would make every read wait
+  // for all of them, which leaves the three-stage ring no load in flight across a k-step.  It
+  // does not see these reads either: their consumers sit behind wait_lds().
   auto lds_piece = [&](const unsigned* stage, int r, int p) {
-    return *reinterpret_cast<const u32x4*>(stage + r * 32 + ((p ^ ((r >> 1) & 7)) << 2));
+    u32x4 v;
+    const unsigned addr = (unsigned)(size_t)(const __attribute__((address_space(3))) unsigned*)(
+        stage + r * 32 + ((p ^ ((r >> 1) & 7)) << 2));
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+  };
+  auto wait_lds = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- V^T operands: unit (key block, column block, s) = 128 pieces of 16 bytes ----
@@ -304,6 +316,14 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
           qr[p][kk] = lds_piece(stage, li, p * 4 + kk * 2 + h);
           kr[p][kk] = lds_piece(stage, kKeyRow0 + wave * 32 + li, p * 4 + kk * 2 + h);
         }
+      u32x4 ar[MAT5 ? 2 : 1][2];
+      if constexpr (MAT5) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) ar[p][kk] = lds_piece(stage, kPgRows + li, p * 4 + kk * 2 + h);
+      }
+      wait_lds();
 #pragma unroll
       for (int prod = 0; prod < 3; ++prod) {
         const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
@@ -313,11 +333,6 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
                                                       __builtin_bit_cast(f16x8, qr[pq][1]), acc2, 0, 0, 0);
       }
       if constexpr (MAT5) {
-        u32x4 ar[2][2];
-#pragma unroll
-        for (int p = 0; p < 2; ++p)
-#pragma unroll
-          for (int kk = 0; kk < 2; ++kk) ar[p][kk] = lds_piece(stage, kPgRows + li, p * 4 + kk * 2 + h);
 #pragma unroll
         for (int prod = 0; prod < 3; ++prod) {
           const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
@@ -327,8 +342,13 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
                                                         __builtin_bit_cast(f16x8, ar[pq][1]), tacc, 0, 0, 0);
         }
       }
-      wait_stage();  // this wavefront's direct loads of the next stage have landed
-      __syncthreads();
+      // this wavefront's direct loads of the next stage have landed; the stage after it stays
+      // in flight across the barrier (a bare s_barrier: __syncthreads() carries a release
+      // fence, for which the compiler waits for every outstanding global->LDS load)
+      wait_stage();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
       buf = (buf == 2) ? 0 : buf + 1;
     }
 
