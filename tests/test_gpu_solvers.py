@@ -449,3 +449,30 @@ def test_debiased_loss_with_paired_self_terms_equals_separate(monkeypatch):
         assert abs(float(v1 - v0)) <= 1e-5 * max(abs(float(v0)), 1e-3)
         assert float((gx1 - gx0).abs().max()) <= 1e-5 * float(gx0.abs().max())
         assert float((gy1 - gy0).abs().max()) <= 1e-5 * float(gy0.abs().max())
+
+
+def test_debiased_loss_side_stream_matches_single_stream(monkeypatch):
+    """The self terms of a debiased loss run on a second stream; loss and gradient are those of
+    the single-stream path bit for bit, also when the loss is called repeatedly (the allocator
+    must not hand the side stream's results out again while they are in use)."""
+    import flash_sinkhorn_amd.samples_loss as sl
+    from flash_sinkhorn_amd import SamplesLoss
+    x, y, a, b = inputs(67, 1500, 1300, 16, scale=0.4)
+    loss_fn = SamplesLoss("sinkhorn", debias=True, allow_tf32=False, blur=0.1,
+                          use_epsilon_scaling=False, eps=0.01, n_iters=30)
+
+    def run():
+        X, Y, A, B = dev(x, y, a, b)
+        X.requires_grad_(True)
+        v = loss_fn(A, X, B, Y)
+        g, = torch.autograd.grad(v, [X])
+        return v.detach().clone(), g.clone()
+
+    monkeypatch.setattr(sl, "DEBIAS_SIDE_STREAM", False)
+    v0, g0 = run()
+    monkeypatch.setattr(sl, "DEBIAS_SIDE_STREAM", True)
+    for _ in range(6):
+        v1, g1 = run()
+        junk = [torch.randn(1500, 16, device="cuda") for _ in range(4)]  # allocator churn
+        assert torch.equal(v0, v1) and torch.equal(g0, g1)
+        del junk
