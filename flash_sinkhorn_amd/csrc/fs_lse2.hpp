@@ -413,7 +413,12 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   auto softmax = [&](const f32x16& acc, int rb) {
     if constexpr (BIASC) {  // acc holds logit/lscale itself
       const float m_new = fmaxf(column_max(acc), run_m[rb]);
-      const float c_new = -m_new * lscale;
+      // rounded once, on purpose: the exponents below, the rescale and the value handed to the
+      // merge must all see the same number.  The empty asm hides the product from the
+      // compiler: fused into the subtraction below (fp contraction) it would rescale by
+      // 2^(rounding residual) on every tile, which adds up over a long key chunk.
+      float c_new = -m_new * lscale;
+      asm volatile("" : "+v"(c_new));
       float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
@@ -440,7 +445,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   };
   auto softmax_first = [&](const f32x16& acc, int rb) {
     const float delta = column_max(acc);
-    const float c = -delta * lscale;
+    float c = -delta * lscale;
+    if constexpr (BIASC) asm volatile("" : "+v"(c));
     float ps = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) ps += fast_exp2(__builtin_fmaf(acc[r], lscale, c));
@@ -471,6 +477,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       if constexpr (BIASC) {
         const float m_new = fmaxf(fmaxf(s.aa, s.bb), run_m[rb]);
         s.cx = -m_new * lscale;
+        asm volatile("" : "+v"(s.cx));  // see softmax(): the rounded product, nothing fused
         s.c = s.cx - run_c[rb];
         run_m[rb] = m_new;
         run_c[rb] = s.cx;

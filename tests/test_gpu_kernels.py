@@ -161,6 +161,24 @@ def test_mat5(n, m, d):
     assert rel_err(got, want) < RTOL
 
 
+@pytest.mark.parametrize("n,m,d,eps", [(40000, 200000, 4, 0.5), (30000, 120000, 16, 0.05)])
+def test_long_key_chunks_keep_fp32_accuracy(n, m, d, eps):
+    """Hundreds of key tiles per workgroup: whatever is applied once per tile (the rescale of
+    the running sum, the offset of the exponents) must not carry a rounding residual, or the
+    residuals add up.  Sampled rows against the fp64 oracle, 3e-6 of the largest potential
+    (a residual of half an ulp of the running maximum per tile gives 2e-5 here)."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import flashsinkhorn_lse_fused
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    y = (rng.standard_normal((m, d)) + 0.3).astype(np.float32)
+    gh = (-(y * y).sum(1) + rng.standard_normal(m) * 0.1).astype(np.float32)
+    lb = np.full(m, -np.log(m), np.float32)
+    got = flashsinkhorn_lse_fused(*dev(x, y, gh, lb), eps, allow_tf32=False).cpu().numpy()
+    rows = np.concatenate([rng.choice(n, 96, replace=False), [0, n - 1]])
+    want = oracle.lse_shifted_fused(x[rows], y, gh, lb, eps)
+    assert np.abs(got[rows] - want).max() <= 3e-6 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("n,m,d,scale", [(300, 5000, 96, 1.0), (1500, 2100, 128, 1.0),
                                          (260, 1300, 128, 3e3), (260, 1300, 72, 1e-3)])
 def test_mat5_wide_rows_on_planes(n, m, d, scale):
