@@ -192,7 +192,8 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
 template <int DP, int PREC>
 struct Geo2 {
   static constexpr int NP = (PREC == kF32) ? 1 : (PREC == kBf6 ? 3 : 2);
-  static constexpr int JT = (DP >= 128) ? 32 : 64;
+  // keys per tile: 64, except 128-column rows outside the two-plane modes (LDS)
+  static constexpr int JT = (DP >= 128 && (PREC == kF32 || PREC == kBf6)) ? 32 : 64;
   static constexpr int NSUB = JT / 32;
   // LDS row stride in 32-bit words: fp32 row + 4, or NP 16-bit planes + 4
   static constexpr int LDW = (PREC == kF32) ? (DP + 4) : (NP * DP / 2 + 4);
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int ROWW = kBf ? NP * DP / 2 : DP;  // 32-bit words per operand row in global memory
   // Key-register prefetch (A operands of the next 32-key sub-tile are read from LDS while the
   // current one is multiplied) and the early LDS store it needs; off where registers are short.
-  constexpr bool KPF = (NSUB == 2) && !(PREC == kBf6 && RB == 2);
+  constexpr bool KPF = (NSUB == 2) && DP < 128 && !(PREC == kBf6 && RB == 2);
   // Two-plane modes with the key-register prefetch: the key bias is the initial value of the MFMA
   // chain's accumulator (16 floats per lane read from LDS while the previous unit finishes)
   // and the running max is subtracted inside the exp2 argument's FMA, which takes the fp32
