@@ -589,8 +589,8 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   if (rb_env > 0) rb = std::min(rb_env, 2);
   const bool mat5 = (mode == kMat5);
   const bool has_o = (mode == kMat || mat5);
-  // one row block where two would spill: 128-column rows, mat5, and the matrix product at 64
-  if (dpk == 128 || mat5 || (mode == kMat && dpk == 64 && rb_env == 0)) rb = 1;
+  // one row block where two would spill: 128-column rows and mat5
+  if (dpk == 128 || mat5) rb = 1;
   size_t need = ps.end;
   SidePlan plans[2];
   size_t vt_off[2] = {0, 0}, part_off[2], q2_off = 0, bounds_off = 0;

@@ -42,8 +42,9 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
   static_assert(DP == 16 || DP == 32 || DP == 64 || DP == 128, "padded row widths");
   constexpr int kPtKeys = (DP == 128) ? 32 : 64;  // keys per tile
   constexpr int NSUB = kPtKeys / 32;
-  // 128-column rows: key operands are read from LDS step by step instead of being held
-  constexpr bool kStreamK = (DP == 128);
+  // 128-column rows, and the matrix product with two row blocks at 64 columns (which spills
+  // otherwise): key operands are read from LDS step by step instead of being held
+  constexpr bool kStreamK = (DP == 128) || (DP == 64 && RB == 2 && MODE == kMat);
   constexpr int KK16 = DP / 16;                 // 16-column steps of the logits
   constexpr int NCB = (DP + 31) / 32;           // 32-column output blocks
   constexpr int ROWW = DP;                      // words per two-plane row

@@ -161,6 +161,40 @@ def test_mat5(n, m, d):
     assert rel_err(got, want) < RTOL
 
 
+@pytest.mark.parametrize("n,m,d", [(17000, 3000, 64), (16500, 2500, 40), (16400, 700, 20)])
+def test_products_with_two_row_blocks_per_wave(n, m, d):
+    """From 16384 query rows on, the d <= 64 product kernels give every wavefront two blocks of
+    32 rows (at 64 columns the matrix product then streams its key operands from LDS): sampled
+    rows of plan*matrix, plan*vector, the gradient and the c-transform against the oracle."""
+    from flash_sinkhorn_amd.kernels.apply_flash import (
+        apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    from flash_sinkhorn_amd import c_transform_fwd
+    x, y, a, b, fh, gh = problem(n, m, d, seed=9)
+    la, lb = np.log(a), np.log(b)
+    rng = np.random.default_rng(10)
+    V = rng.standard_normal((m, d)).astype(np.float32)
+    v = rng.standard_normal(m).astype(np.float32)
+    rows = np.concatenate([rng.choice(n, 120, replace=False), [0, 31, 32, 63, 64, n - 1]])
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, la, lb)
+    kw = dict(eps=0.4, cost_scale=0.5)
+    got = apply_plan_mat_flashstyle(X, Y, F, G, LA, LB, dev(V)[0], axis=1, allow_tf32=False, **kw)
+    want = oracle.apply_plan_mat(x[rows], y, fh[rows], gh, la[rows], lb, V, axis=1, **kw)
+    assert rel_err(got[torch.from_numpy(rows).cuda()], want) < RTOL
+    got = apply_plan_vec_flashstyle(X, Y, F, G, LA, LB, dev(v)[0], axis=1, allow_tf32=False, **kw)
+    want = oracle.apply_plan_vec(x[rows], y, fh[rows], gh, la[rows], lb, v, axis=1, **kw)
+    assert rel_err(got[torch.from_numpy(rows).cuda()], want) < RTOL
+    gx, _ = grad(X, Y, *dev(a, b), F, G, eps=0.3, cost_scale=0.5, allow_tf32=False,
+                 compute_grad_y=False)
+    wx, _ = oracle.grad_barycentric(x[rows], y, a[rows], b, fh[rows], gh, 0.3, cost_scale=0.5)
+    assert rel_err(gx[torch.from_numpy(rows).cuda()], wx) < RTOL
+    psi = rng.standard_normal(m).astype(np.float32)
+    c, _ = c_transform_fwd(X, Y, dev(psi)[0], cost_scale=0.5, allow_tf32=False)
+    wc, _ = oracle.c_transform(x[rows], y, psi, 0.5)
+    assert np.abs(c.cpu().numpy()[rows] - wc).max() <= 1e-5 * max(np.abs(wc).max(), 1.0)
+
+
 @pytest.mark.parametrize("n,m,d,eps", [(40000, 200000, 4, 0.5), (30000, 120000, 16, 0.05)])
 def test_long_key_chunks_keep_fp32_accuracy(n, m, d, eps):
     """Hundreds of key tiles per workgroup: whatever is applied once per tile (the rescale of
