@@ -16,6 +16,8 @@ RTOL = 1e-4
 SHAPES = [  # (n, m, d): ragged tiles, d not a multiple of 4/8, every padded width
     (64, 48, 32), (300, 257, 64), (129, 1000, 3), (1000, 130, 20), (257, 300, 128),
     (70, 65, 100), (4500, 3000, 64), (33, 5, 8), (1, 1, 1),
+    # two row blocks per wavefront at the narrow widths (2048 rows and more)
+    (2100, 2300, 20), (2050, 300, 3),
     # column-sliced kernels (d > 128): every (wavefronts, slice) configuration, ragged d
     (100, 90, 200), (64, 70, 512), (50, 140, 700), (40, 33, 1536), (33, 20, 1030), (70, 300, 130),
     (600, 2000, 256),
