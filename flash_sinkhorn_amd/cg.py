@@ -13,7 +13,7 @@ from typing import Callable, Optional, Tuple
 
 import torch
 
-__all__ = ["CGInfo", "conjugate_gradient"]
+__all__ = ["CGInfo", "conjugate_gradient", "conjugate_gradient_device"]
 
 
 @dataclass(frozen=True)
@@ -80,3 +80,55 @@ def conjugate_gradient(
         rz = rz_next
 
     return sol, CGInfo(False, int(max_iter), _norm(res), r0)
+
+
+def conjugate_gradient_device(
+    matvec: Callable[[torch.Tensor], torch.Tensor],
+    b: torch.Tensor,
+    *,
+    max_iter: int = 300,
+    rtol: float = 1e-6,
+    atol: float = 1e-6,
+    check_every: int = 1,
+) -> Tuple[torch.Tensor, CGInfo]:
+    """``conjugate_gradient`` without preconditioner or warm start, with the vector updates,
+    dot products and the stopping decision of an iteration in one device launch
+    (``fs_cg_update``) instead of a dozen PyTorch launches and two host read-backs.
+
+    The host looks at the device state every ``check_every`` iterations.  Iterations enqueued
+    after the one that met the tolerance leave the iterate alone, so the solution and the
+    reported iteration count are those of a loop that stopped at once; only their
+    matrix-vector products are wasted, which is why large problems use ``check_every=1``.
+    Same tolerance rule and ``CGInfo`` conventions as ``conjugate_gradient``.
+    """
+    from flash_sinkhorn_amd import _lib
+    L = _lib.lib()
+    rhs = b.detach().float().contiguous()
+    m = rhs.numel()
+    sol, res, direction = (torch.empty_like(rhs) for _ in range(3))
+    state = torch.empty(8, device=rhs.device, dtype=torch.float32)
+    stream = _lib.stream_of(rhs)
+    _lib.check(L.fs_cg_init(rhs.data_ptr(), sol.data_ptr(), res.data_ptr(), direction.data_ptr(),
+                            state.data_ptr(), m, float(rtol), float(atol), stream), "fs_cg_init")
+    every = max(1, int(check_every))
+    enqueued = 0
+    host = None
+    while enqueued < int(max_iter):
+        for _ in range(min(every, int(max_iter) - enqueued)):
+            a_dir = matvec(direction).float().contiguous()
+            _lib.check(L.fs_cg_update(a_dir.data_ptr(), sol.data_ptr(), res.data_ptr(),
+                                      direction.data_ptr(), state.data_ptr(), m, stream),
+                       "fs_cg_update")
+            enqueued += 1
+        host = state.cpu()
+        if float(host[4]) != 0.0:
+            break
+    if host is None:
+        host = state.cpu()
+    converged = float(host[5]) != 0.0
+    iters = int(host[6]) if converged else int(max_iter)
+    if converged:
+        rnorm = float(host[3])
+    else:
+        rnorm = float(torch.linalg.norm(res).cpu())
+    return sol, CGInfo(converged, iters, rnorm, float(host[1]))

@@ -1149,6 +1149,36 @@ int fs_apply_vec(const float* x, const float* y, const float* f_hat, const float
   return run_stream(kVec, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
 }
 
+int fs_schur_matvec(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                    const float* log_a, const float* log_b, const float* z, const float* inv_diag_x,
+                    const float* denom, float* piz, float* out, int64_t n, int64_t m, int64_t d,
+                    float eps, float coord_scale, uint32_t flags, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  if (!x || !y || !f_hat || !g_hat || !log_a || !log_b || !z || !inv_diag_x || !denom || !piz ||
+      !out)
+    return FS_ERR_NULL_POINTER;
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (!(eps > 0.f) || out == z || piz == inv_diag_x) return FS_ERR_BAD_ARGUMENT;
+  const float qs = coord_scale / eps * kLog2e;
+  // piz = (P z) / diag_x
+  Side s1 = lse_side(x, y, g_hat, kLog2e / eps, log_b, kLog2e, n, m, qs);
+  s1.v = z;
+  s1.ep.kind = kEpiApply; s1.ep.out = piz; s1.ep.post = 1.0f;
+  s1.ep.r0 = f_hat; s1.ep.rc0 = kLog2e / eps;
+  s1.ep.r1 = log_a; s1.ep.rc1 = kLog2e;
+  s1.ep.mul = inv_diag_x;
+  int rc = run_stream(kVec, false, &s1, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
+  if (rc != FS_OK) return rc;
+  // out = denom * z - P^T piz
+  Side s2 = lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
+  s2.v = piz;
+  s2.ep.kind = kEpiApply; s2.ep.out = out; s2.ep.post = 1.0f;
+  s2.ep.r0 = g_hat; s2.ep.rc0 = kLog2e / eps;
+  s2.ep.r1 = log_b; s2.ep.rc1 = kLog2e;
+  s2.ep.add_a = denom; s2.ep.add_b = z; s2.ep.res_coef = -1.0f;
+  return run_stream(kVec, false, &s2, 1, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
+}
+
 int fs_apply_mat(const float* x, const float* y, const float* f_hat, const float* g_hat,
                  const float* log_a, const float* log_b, const float* mat, const float* scale,
                  float* out, int64_t n, int64_t m, int64_t d, int64_t dv, float eps,

@@ -44,6 +44,12 @@ struct Epilogue {
   const float* r1;
   const float* r2;
   float rc0, rc1, rc2, post;
+  // kEpiApply, scalar outputs only: then out *= mul[i] (if given) and, with add_a,
+  // out = add_a[i]*add_b[i] + res_coef*out (the two halves of a Schur-complement product)
+  const float* mul;
+  const float* add_a;
+  const float* add_b;
+  float res_coef;
   // kEpiGrad: out = gcoef * gs * w[i] * (q[i,:] - O/s)
   const float* w;
   const float* grad_scale;  // 1-element device array or null

@@ -87,7 +87,10 @@ __device__ __forceinline__ void epilogue_scalar(const Epilogue& ep, int row, flo
     if (ep.shift) r -= ep.shift_coef * ep.shift[row];
     ep.out[row] = r;
   } else {
-    ep.out[row] = apply_row_factor(ep, row, M) * o;
+    float r = apply_row_factor(ep, row, M) * o;
+    if (ep.mul) r *= ep.mul[row];
+    if (ep.add_a) r = ep.add_a[row] * ep.add_b[row] + ep.res_coef * r;
+    ep.out[row] = r;
   }
 }
 

@@ -21,7 +21,8 @@ from typing import Optional, Sequence, Tuple
 
 import torch
 
-from flash_sinkhorn_amd.cg import conjugate_gradient
+from flash_sinkhorn_amd import _lib
+from flash_sinkhorn_amd.cg import conjugate_gradient, conjugate_gradient_device
 from flash_sinkhorn_amd.kernels._common import log_weights
 from flash_sinkhorn_amd.kernels.sinkhorn_triton_apply_sqeuclid import (
     apply_plan_mat_flashstyle, apply_plan_vec_flashstyle, mat5_sqeuclid,
@@ -151,7 +152,26 @@ def hvp_x_sqeuclid_from_potentials(
     def B(v):
         return PT(P(v) / diag_x) / denom
 
-    if mode == "none":
+    if mode == "none" and cg_x0 is None and not cg_stabilise_every:
+        # CG bookkeeping on the device; small problems look at the state every few iterations
+        # (their iterations are launch bound), large ones after each (a wasted matvec costs more
+        # than a read-back)
+        from flash_sinkhorn_amd.kernels.sinkhorn_triton_apply_fused_sqeuclid import (
+            _schur_matvec_raw)
+        inv_diag_x = (1.0 / diag_x).contiguous()
+        denom_c = denom.contiguous()
+        piz_buf = torch.empty((n,), device=x.device, dtype=torch.float32)
+        schur_ws = _lib.workspace(_lib.OP_APPLY_VEC, n, m, d, x.device)
+
+        def schur(v):  # denom * v - P^T((P v) / diag_x): two launches, factors in the epilogues
+            return _schur_matvec_raw(xf, yf, f_sh, g_sh, log_a, log_b, v, inv_diag_x, denom_c,
+                                     eps=e, cost_scale=cs, allow_tf32=allow_tf32,
+                                     use_exp2=use_exp2, piz=piz_buf, workspace=schur_ws)[0]
+
+        z, cg = conjugate_gradient_device(
+            schur, rhs, max_iter=max_cg_iter, rtol=cg_rtol, atol=cg_atol,
+            check_every=4 if float(n) * float(m) * float(d) < 2.0e9 else 1)
+    elif mode == "none":
         z, cg = conjugate_gradient(
             lambda v: denom * v - PT(P(v) / diag_x), rhs, x0=cg_x0, max_iter=max_cg_iter,
             rtol=cg_rtol, atol=cg_atol, preconditioner=None, stabilise_every=cg_stabilise_every)

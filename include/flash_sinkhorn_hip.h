@@ -147,6 +147,42 @@ int fs_symmetric_steps(const float* x, const float* y, const float* f_hat, const
                        uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Schur-complement product of the Hessian-vector path: piz = (P z) / diag_x (n values), then
+ * out = denom * z - P^T piz (m values), P as in fs_apply_vec.  Two stream-ordered launches with
+ * the element-wise factors folded into their epilogues; inv_diag_x holds 1 / diag_x.  out must
+ * not alias z.  Workspace: fs_workspace_bytes(FS_OP_APPLY_VEC, n, m, d).
+ * Replaces fused_schur_matvec_sqeuclid (kernels/sinkhorn_triton_apply_fused_sqeuclid.py:283-470;
+ * the reference's single launch joins its two phases with a spin-wait grid barrier and falls
+ * back to two launches when the grid does not fit the device; here the two launches are the
+ * design: a kernel that waits for other workgroups must not exist on this machine).
+ */
+int fs_schur_matvec(const float* x, const float* y, const float* f_hat, const float* g_hat,
+                    const float* log_a, const float* log_b, const float* z, const float* inv_diag_x,
+                    const float* denom, float* piz, float* out, int64_t n, int64_t m, int64_t d,
+                    float eps, float coord_scale, uint32_t flags, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/*
+ * Conjugate gradients with the bookkeeping on the device (no counterpart kernel in the
+ * reference: its conjugate_gradient, cg.py:27-121, runs these vector operations as separate
+ * PyTorch launches and reads the residual norm back every iteration).
+ * fs_cg_init: sol = 0, res = dir = b, state = {r.r, |r0|, tol = max(atol, rtol*|r0|), |r|,
+ * done = 0, converged = 0, iterations = 0, -} (8 floats on the device).
+ * fs_cg_update, after the caller has computed a_dir = A dir: the curvature dir.a_dir, the step,
+ * sol += step*dir, res -= step*a_dir, |res|; stops (done = converged = 1) when |res| <= tol,
+ * stops without convergence when the curvature is exactly zero, otherwise
+ * dir = res + (|res|^2 / r.r) dir.  Once done is set further updates change nothing, so a
+ * caller may enqueue several iterations between two looks at the state and still get the
+ * iterate and the iteration count of the step that met the tolerance.  Sums are accumulated in
+ * double precision.  One workgroup per launch: meant for the n- and m-vectors of the Schur
+ * system, not for large unknowns.
+ */
+int fs_cg_init(const float* b, float* sol, float* res, float* dir, float* state, int64_t m,
+               float rtol, float atol, void* stream);
+int fs_cg_update(const float* a_dir, float* sol, float* res, float* dir, float* state, int64_t m,
+                 void* stream);
+
+/*
  * The two self problems OT(x, x; a) and OT(y, y; b) of a debiased divergence, n_steps Jacobi
  * steps each, one launch per step for both: in a self problem both potentials stay equal, so a
  * step is one half-update per problem, fx' = (1-alpha) fx + alpha*(-eps_x*damp_x*LSE_j[...]) over

@@ -476,3 +476,74 @@ def test_debiased_loss_side_stream_matches_single_stream(monkeypatch):
         junk = [torch.randn(1500, 16, device="cuda") for _ in range(4)]  # allocator churn
         assert torch.equal(v0, v1) and torch.equal(g0, g1)
         del junk
+
+
+@pytest.mark.parametrize("m,every", [(300, 1), (300, 4), (5000, 3), (70000, 2)])
+def test_device_cg_matches_host_cg(m, every):
+    """fs_cg_init / fs_cg_update against the PyTorch-op CG on a dense SPD system: same
+    solution, same convergence flag and iteration count, also when several iterations are
+    enqueued between two looks at the state; non-convergence and zero right-hand sides follow
+    the same conventions."""
+    from flash_sinkhorn_amd.cg import conjugate_gradient, conjugate_gradient_device
+    g = torch.Generator(device="cpu").manual_seed(m)
+    k = 40
+    U = torch.randn(m, k, generator=g).cuda() / np.sqrt(k)
+    dvec = (1.0 + torch.rand(m, generator=g)).cuda()
+    b = torch.randn(m, generator=g).cuda()
+
+    def matvec(v):
+        return dvec * v + U @ (U.t() @ v)
+
+    want, wi = conjugate_gradient(matvec, b, max_iter=200, rtol=1e-6, atol=1e-10)
+    got, gi = conjugate_gradient_device(matvec, b, max_iter=200, rtol=1e-6, atol=1e-10,
+                                        check_every=every)
+    assert wi.cg_converged and gi.cg_converged
+    assert abs(gi.cg_iters - wi.cg_iters) <= 1
+    assert float((got - want).abs().max()) <= 1e-5 * float(want.abs().max())
+    assert abs(gi.cg_initial_residual - wi.cg_initial_residual) <= 1e-5 * wi.cg_initial_residual
+    assert gi.cg_residual <= max(1e-10, 1e-6 * gi.cg_initial_residual)
+    # too few iterations: not converged, the count is the limit
+    _, g2 = conjugate_gradient_device(matvec, b, max_iter=2, rtol=1e-12, atol=0.0,
+                                      check_every=every)
+    _, w2 = conjugate_gradient(matvec, b, max_iter=2, rtol=1e-12, atol=0.0)
+    assert (g2.cg_converged, g2.cg_iters) == (w2.cg_converged, w2.cg_iters) == (False, 2)
+    assert abs(g2.cg_residual - w2.cg_residual) <= 1e-4 * w2.cg_residual
+    # zero right-hand side: zero curvature ends the loop, solution zero
+    z, g3 = conjugate_gradient_device(matvec, torch.zeros_like(b), max_iter=5, check_every=every)
+    assert float(z.abs().max()) == 0.0 and not g3.cg_converged and g3.cg_iters == 5
+
+
+@pytest.mark.parametrize("n,m,d", [(300, 257, 64), (129, 1000, 3), (100, 1100, 300),
+                                   (2100, 2300, 20), (257, 300, 128)])
+@pytest.mark.parametrize("cs", [1.0, 0.5])
+def test_fused_schur_matvec_against_dense_oracle(n, m, d, cs):
+    """out = denom*z - P^T((P z)/diag_x) with OTT potentials, P = exp((f+g-C)/eps): the two
+    launches with their element-wise factors in the epilogues against the dense fp64 product;
+    the returned buffer holds (P z)/diag_x and is reused when passed back."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_apply_fused_sqeuclid import (
+        fused_schur_matvec_sqeuclid)
+    x, y, a, b = inputs(71, n, m, d, scale=2.0 / np.sqrt(d))
+    rng = np.random.default_rng(13)
+    eps = 0.4
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    C = cs * ((x64[:, None, :] - y64[None, :, :]) ** 2).sum(-1)
+    f = (rng.standard_normal(n) * 0.2 + eps * np.log(a) - 1.0).astype(np.float32)
+    g = (rng.standard_normal(m) * 0.2 + eps * np.log(b)).astype(np.float32)
+    P = np.exp((f.astype(np.float64)[:, None] + g.astype(np.float64)[None, :] - C) / eps)
+    z = rng.standard_normal(m).astype(np.float32)
+    diag_x = (P.sum(1) * (1.0 + rng.random(n))).astype(np.float32)
+    denom = (P.sum(0) * (1.0 + rng.random(m)) + 1e-3).astype(np.float32)
+    piz_want = (P @ z.astype(np.float64)) / diag_x.astype(np.float64)
+    want = denom.astype(np.float64) * z - P.T @ piz_want
+    X, Y, F, G, Z, DX, DN = dev(x, y, f, g, z, diag_x, denom)
+    out, piz = fused_schur_matvec_sqeuclid(X, Y, F, G, Z, DX, DN, eps=eps, cost_scale=cs)
+    assert rel_err(piz, piz_want) < RTOL
+    assert float(np.abs(out.cpu().numpy() - want).max()) <= RTOL * max(
+        np.abs(denom * z).max(), np.abs(P.T @ piz_want).max())
+    out2, piz2 = fused_schur_matvec_sqeuclid(X, Y, F, G, Z, DX, DN, eps=eps, cost_scale=cs,
+                                             piz_buffer=piz)
+    assert piz2 is piz and torch.equal(out, out2)
+    with pytest.raises(ValueError):
+        fused_schur_matvec_sqeuclid(X, Y, F, G, Z[:-1], DX, DN, eps=eps)
+    with pytest.raises(ValueError):
+        fused_schur_matvec_sqeuclid(X, Y, F, G, Z, DX[:-1], DN, eps=eps)
