@@ -18,6 +18,7 @@ operator                   launcher it wraps                                    
 ``apply_plan_mat``         ``kernels.apply_flash.apply_plan_mat_flashstyle``       ``fs_apply_mat``
 ``mat5``                   ``kernels.apply_ott.mat5_sqeuclid``                     ``fs_mat5``
 ``c_transform``            ``kernels.c_transform_sqeuclid.c_transform_kernel``     ``fs_c_transform``
+``schur_matvec``           ``kernels.sinkhorn_triton_apply_fused_sqeuclid``        ``fs_schur_matvec``
 =========================  =====================================================  ==================
 """
 from __future__ import annotations
@@ -31,7 +32,7 @@ __all__ = ["NAMESPACE", "OPERATORS"]
 
 NAMESPACE = "flash_sinkhorn_amd"
 OPERATORS = ("lse", "lse_fused", "symmetric_step", "grad", "apply_plan_vec", "apply_plan_mat",
-             "mat5", "c_transform")
+             "mat5", "c_transform", "schur_matvec")
 
 
 def _f32(shape, like: Tensor) -> Tensor:
@@ -156,3 +157,19 @@ def c_transform(x: Tensor, y: Tensor, bias: Tensor, cost_scale: float = 1.0,
 @c_transform.register_fake
 def _(x, y, bias, cost_scale=1.0, allow_tf32=False):
     return _f32((x.shape[0],), x), torch.empty((x.shape[0],), dtype=torch.int64, device=x.device)
+
+
+@torch.library.custom_op(f"{NAMESPACE}::schur_matvec", mutates_args=())
+def schur_matvec(x: Tensor, y: Tensor, f: Tensor, g: Tensor, z: Tensor, diag_x: Tensor,
+                 denom: Tensor, eps: float, cost_scale: float = 1.0,
+                 allow_tf32: bool = False) -> Tuple[Tensor, Tensor]:
+    """(denom*z - P^T((P z)/diag_x), (P z)/diag_x) with OTT-style potentials f, g."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_apply_fused_sqeuclid import (
+        fused_schur_matvec_sqeuclid)
+    return fused_schur_matvec_sqeuclid(x, y, f, g, z, diag_x, denom, eps=eps,
+                                       cost_scale=cost_scale, allow_tf32=allow_tf32)
+
+
+@schur_matvec.register_fake
+def _(x, y, f, g, z, diag_x, denom, eps, cost_scale=1.0, allow_tf32=False):
+    return _f32((y.shape[0],), x), _f32((x.shape[0],), x)

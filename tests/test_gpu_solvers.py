@@ -392,6 +392,12 @@ def test_custom_operators_match_the_launchers():
     inner = want_c - (x.astype(np.float64) ** 2).sum(1)
     assert np.abs(c.cpu().numpy() - inner).max() <= 1e-5 * np.abs(inner).max()
     assert (idx.cpu().numpy() == want_idx).mean() > 0.99
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_apply_fused_sqeuclid import (
+        fused_schur_matvec_sqeuclid)
+    dx, dn = torch.rand(n, device="cuda") + 0.5, torch.rand(m, device="cuda") + 0.5
+    o1, p1 = ops.schur_matvec(X, Y, F, G, v, dx, dn, 0.4)
+    o2, p2 = fused_schur_matvec_sqeuclid(X, Y, F, G, v, dx, dn, eps=0.4)
+    assert torch.equal(o1, o2) and torch.equal(p1, p2)
     torch.library.opcheck(ops.lse_fused.default, (X, Y, G, LB, 0.2),
                           test_utils=("test_schema", "test_faketensor"))
 

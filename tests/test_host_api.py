@@ -251,3 +251,5 @@ def test_custom_operators_are_registered_with_shape_inference():
     assert ops.mat5(x, y, mt(n), mt(m), mt(n, d), 0.1).shape == (n, d)
     c, idx = ops.c_transform(x, y, mt(m))
     assert c.shape == (n,) and idx.dtype == torch.int64 and c.dtype == torch.float32
+    out, piz = ops.schur_matvec(x, y, mt(n), mt(m), mt(m), mt(n), mt(m), 0.1)
+    assert out.shape == (m,) and piz.shape == (n,)
