@@ -633,6 +633,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 
   // Wait until at most `newer` of this wavefront's vector-memory operations are outstanding
   // (the direct loads write LDS behind the compiler's back, so their waits are explicit).
+  // Loads complete in issue order, register loads and global->LDS loads alike, which is what
+  // lets a count stand for "everything older than the newest tile has landed".  gfx9 encoding
+  // of s_waitcnt: vmcnt in bits 3:0 and 15:14, expcnt 6:4 (7 = no wait), lgkmcnt 11:8.
   auto wait_vm = [&](auto newer) {
     constexpr int n = decltype(newer)::value;
     __builtin_amdgcn_s_waitcnt(0x0F70 | (n & 15) | ((n >> 4) << 14));
