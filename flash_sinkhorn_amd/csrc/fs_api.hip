@@ -744,7 +744,10 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   static const int use_plan_tile = env_int("FS_PLANTILE", 1);
   static const int mat5_128 = env_int("FS_MAT5_128", 1);
-  const bool tile_mode = mode == kMat || mode == kVec || mode == kArgmax ||
+  // the plan-vector product at <= 64 columns rides on the pipelined log-sum-exp kernel
+  static const int vec_on_lse2 = env_int("FS_VEC_LSE2", 1);
+  const bool vec_lse2 = mode == kVec && vec_on_lse2 && cfg.prec == 3 && cfg.dp <= 64 && !fam.sliced;
+  const bool tile_mode = mode == kMat || (mode == kVec && !vec_lse2) || mode == kArgmax ||
                          (mode == kMat5 && (cfg.dp <= 64 || mat5_128));
   if (tile_mode && !fam.sliced && use_plan_tile && (cfg.prec == 3 || cfg.prec == 1)) {
     // the reduced mode runs on the fp16 planes too (same speed, smaller error); planes a caller
@@ -771,7 +774,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   for (int s = 0; s < nsides; ++s) aligned = aligned && aligned16(sides[s].q) && aligned16(sides[s].k);
   const int prec = cfg.prec;
   // pipelined LSE kernel: the 16-bit plane modes take any d <= 128, the fp32 mode needs aligned rows
-  const bool lse2 = (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
+  const bool lse2 = vec_lse2 ||
+                    (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = cfg.dp;
   if (lse2 && prec == 2 && dp >= 64) rb = 1;  // three planes of 64 columns x two row blocks spill
   if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
@@ -834,7 +838,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   } else if (lse2) {
     rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
     a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
-    if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, total, st);
+    if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, mode == kVec, total, st);
   } else
   switch (mode) {
     case kLse: rc = launch_dp<kLse, false>(a, dp, rb, total, st); break;

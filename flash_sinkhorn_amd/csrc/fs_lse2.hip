@@ -5,27 +5,28 @@
 
 namespace fs {
 
-template <int DP, int RB, int PREC>
+template <int DP, int RB, int PREC, bool VEC>
 static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
-  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC>), dim3(blocks), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC, VEC>), dim3(blocks), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
-template <int DP, int PREC>
+template <int DP, int PREC, bool VEC>
 static int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
   if constexpr (DP <= 64 && !(PREC == kBf6 && DP == 64)) {
-    if (rb >= 2) return launch_cfg<DP, 2, PREC>(a, blocks, st);
+    if (rb >= 2) return launch_cfg<DP, 2, PREC, VEC>(a, blocks, st);
   }
-  return launch_cfg<DP, 1, PREC>(a, blocks, st);
+  return launch_cfg<DP, 1, PREC, VEC>(a, blocks, st);
 }
 
-template <int PREC>
+template <int PREC, bool VEC>
 static int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
   switch (dp) {
-    case 16: return launch_rb<16, PREC>(a, rb, blocks, st);
-    case 32: return launch_rb<32, PREC>(a, rb, blocks, st);
-    case 64: return launch_rb<64, PREC>(a, rb, blocks, st);
-    case 128: return launch_rb<128, PREC>(a, rb, blocks, st);
+    case 16: return launch_rb<16, PREC, VEC>(a, rb, blocks, st);
+    case 32: return launch_rb<32, PREC, VEC>(a, rb, blocks, st);
+    case 64: return launch_rb<64, PREC, VEC>(a, rb, blocks, st);
+    case 128:
+      if constexpr (!VEC) return launch_rb<128, PREC, false>(a, rb, blocks, st);
   }
   return FS_ERR_UNSUPPORTED;
 }
@@ -57,12 +58,16 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
-int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, int blocks, hipStream_t st) {
+int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, int blocks,
+                hipStream_t st) {
+  if (vec) {  // plan-vector product: fp16 planes, rows of at most 64 columns
+    return prec == kH3 ? launch_dp<kH3, true>(a, dp, rb, blocks, st) : FS_ERR_UNSUPPORTED;
+  }
   switch (prec) {
-    case kF32: return launch_dp<kF32>(a, dp, rb, blocks, st);
-    case kBf3: return launch_dp<kBf3>(a, dp, rb, blocks, st);
-    case kBf6: return launch_dp<kBf6>(a, dp, rb, blocks, st);
-    case kH3: return launch_dp<kH3>(a, dp, rb, blocks, st);
+    case kF32: return launch_dp<kF32, false>(a, dp, rb, blocks, st);
+    case kBf3: return launch_dp<kBf3, false>(a, dp, rb, blocks, st);
+    case kBf6: return launch_dp<kBf6, false>(a, dp, rb, blocks, st);
+    case kH3: return launch_dp<kH3, false>(a, dp, rb, blocks, st);
   }
   return FS_ERR_BAD_ARGUMENT;
 }

@@ -211,11 +211,15 @@ constexpr int kPieces = 12;
 constexpr int kMaxPieces = 3;  // pieces 0..2 find the largest logit of the unit
 constexpr int kBiasPiece = 4;  // pieces 4..7 read the next unit's bias from LDS, 16 bytes each
 struct SoftmaxStage {
-  float m[6], mx, aa, bb, c, cx, ps0, ps1;  // c: exponent of the rescale, cx: offset of the logits
+  float m[6], mx, aa, bb, c, cx, ps0, ps1, po;  // c: exponent of the rescale, cx: offset of the logits
   float t[16], e[16];
+  float v[2][4];  // VEC: two groups of four v values in flight
 };
 
-template <int DP, int RB, int PREC>
+// VEC: the plan-vector product (kVec) on the same pipeline: next to the row sums the kernel
+// keeps o_i = sum_j p_ij v_j, with v staged through LDS beside the key bias.  Two-plane modes
+// at d <= 64 only (the bias-as-accumulator-start variants).
+template <int DP, int RB, int PREC, bool VEC = false>
 __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   using G = Geo2<DP, PREC>;
   constexpr int NP = G::NP;
@@ -231,6 +235,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // and the running max is subtracted inside the exp2 argument's FMA, which takes the fp32
   // bias MFMA (64 of 448 MFMA cycles per unit at d = 64) out of the loop.
   constexpr bool BIASC = (PREC == kH3 || PREC == kBf3) && KPF;
+  static_assert(!VEC || BIASC, "the vector mode rides on the bias-as-accumulator-start pipeline");
   // Two-plane modes bring key tiles into LDS with direct global->LDS loads (no staging
   // registers, no ds_write): rows are unpadded and 16-byte piece p of row r sits in slot
   // p ^ swz(r), which keeps the b128 reads of 16 consecutive rows conflict free.  With the
@@ -242,6 +247,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 
   __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][G::JT * LDWK];
   __shared__ __attribute__((aligned(16))) float lds_b[NBUF][256];  // [buf][thread]; first JT used
+  __shared__ __attribute__((aligned(16))) float lds_v[VEC ? NBUF : 1][VEC ? 256 : 4];  // VEC: v_j
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;
@@ -301,12 +307,13 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // run_m: running max in accumulator units; run_c (BIASC): -run_m * lscale as rounded once,
   // the offset every exponent of the row uses, so that rescaling by differences of run_c is
   // consistent with the exponents already summed
-  float run_m[RB], run_s[RB], run_c[RB];
+  float run_m[RB], run_s[RB], run_c[RB], run_o[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     run_m[rb] = 0.f;
     run_s[rb] = 0.f;
     run_c[rb] = 0.f;
+    run_o[rb] = 0.f;
   }
 
   // ---- staging (global -> registers -> LDS), branch free: rows are clamped, masked by bias ----
@@ -314,7 +321,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int C16_TOTAL = G::JT * C16_PER_ROW;
   constexpr int PER_THREAD = (C16_TOTAL + 255) / 256;
   u32x4 st_k[DIRECT ? 1 : PER_THREAD];
-  float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f, st_pen = 0.f;
+  float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f, st_pen = 0.f, st_v = 0.f;
   const unsigned* krows = kBf ? sd.kplanes : reinterpret_cast<const unsigned*>(sd.k);
   const int krow_words = kBf ? ROWW : d;
   const float* kb1p = sd.kb1 ? sd.kb1 : sd.kb0;  // always loadable; unused terms are dropped
@@ -349,6 +356,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       st_b1 = kb1p[j];
       st_b2 = kb2p[j];
       st_pen = (j0 + tid < j_end) ? 0.f : 2.0f * kNegBig;
+      if constexpr (VEC) st_v = sd.v[j];  // masked keys carry probability zero
     }
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
@@ -389,6 +397,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     float b = kc0 * st_b0 + (has_kb1 ? kc1 * st_b1 : 0.f);
     b += (has_kb2 ? kc2 * st_b2 : 0.f);
     lds_b[buf][tid] = (fmaxf(b, kNegBig) + st_pen) * inv_lscale;
+    if constexpr (VEC) lds_v[buf][tid] = st_v;
   };
 
   // v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its
@@ -411,7 +420,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     return fmaxf(a, b);
   };
   // classic online soft-max step; acc holds (logit - M)/lscale for the current M = run_m[rb]
-  auto softmax = [&](const f32x16& acc, int rb) {
+  auto softmax = [&](const f32x16& acc, int rb, const f32x16& v16) {
     if constexpr (BIASC) {  // acc holds logit/lscale itself
       const float m_new = fmaxf(column_max(acc), run_m[rb]);
       // rounded once, on purpose: the exponents below, the rescale and the value handed to the
@@ -420,13 +429,18 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       // 2^(rounding residual) on every tile, which adds up over a long key chunk.
       float c_new = -m_new * lscale;
       asm volatile("" : "+v"(c_new));
-      float ps0 = 0.f, ps1 = 0.f;
+      float ps0 = 0.f, ps1 = 0.f, po = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        ps0 += fast_exp2(__builtin_fmaf(acc[r], lscale, c_new));
-        ps1 += fast_exp2(__builtin_fmaf(acc[r + 1], lscale, c_new));
+        const float e0 = fast_exp2(__builtin_fmaf(acc[r], lscale, c_new));
+        const float e1 = fast_exp2(__builtin_fmaf(acc[r + 1], lscale, c_new));
+        ps0 += e0;
+        ps1 += e1;
+        if constexpr (VEC) po = __builtin_fmaf(e0, v16[r], __builtin_fmaf(e1, v16[r + 1], po));
       }
-      run_s[rb] = run_s[rb] * fast_exp2(c_new - run_c[rb]) + (ps0 + ps1);
+      const float resc = fast_exp2(c_new - run_c[rb]);
+      run_s[rb] = run_s[rb] * resc + (ps0 + ps1);
+      if constexpr (VEC) run_o[rb] = run_o[rb] * resc + po;
       run_m[rb] = m_new;
       run_c[rb] = c_new;
       return;
@@ -444,20 +458,25 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     run_s[rb] = run_s[rb] * fast_exp2(c) + (ps0 + ps1);
     run_m[rb] = m_new;
   };
-  auto softmax_first = [&](const f32x16& acc, int rb) {
+  auto softmax_first = [&](const f32x16& acc, int rb, const f32x16& v16) {
     const float delta = column_max(acc);
     float c = -delta * lscale;
     if constexpr (BIASC) asm volatile("" : "+v"(c));
-    float ps = 0.f;
+    float ps = 0.f, po = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ps += fast_exp2(__builtin_fmaf(acc[r], lscale, c));
+    for (int r = 0; r < 16; ++r) {
+      const float e = fast_exp2(__builtin_fmaf(acc[r], lscale, c));
+      ps += e;
+      if constexpr (VEC) po = __builtin_fmaf(e, v16[r], po);
+    }
+    if constexpr (VEC) run_o[rb] = po;
     run_s[rb] = ps;
     run_m[rb] = delta;
     run_c[rb] = c;
   };
   // The same step as `softmax`, piece p of kPieces; fma / exp2 / add of a value sit in
   // consecutive pieces so that no piece waits on its own results.
-  auto softmax_piece = [&](int p, SoftmaxStage& s, const f32x16& a, int rb) {
+  auto softmax_piece = [&](int p, SoftmaxStage& s, const f32x16& a, int rb, const float* vsrc) {
     if (p == 0) {
       s.m[0] = fmaxf(fmaxf(a[0], a[1]), a[2]);
       s.m[1] = fmaxf(fmaxf(a[3], a[4]), a[5]);
@@ -491,6 +510,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       }
       s.ps0 = 0.f;
       s.ps1 = 0.f;
+      s.po = 0.f;
     }
     const int q = p - 3;  // two values per piece: fma at q, exp2 at q + 1, add at q + 2
     if constexpr (BIASC) {
@@ -508,15 +528,36 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       s.e[2 * q - 2] = fast_exp2(s.t[2 * q - 2]);
       s.e[2 * q - 1] = fast_exp2(s.t[2 * q - 1]);
     }
+    if constexpr (VEC) {
+      // v of values 4g .. 4g+3 (used by the adds of q = 2g+2, 2g+3) is read at q = 2g: four
+      // to eight of the sixteen values are in registers at any time
+      if (q >= 0 && q < 8 && q % 2 == 0) {
+        const float4 t = *reinterpret_cast<const float4*>(vsrc + 8 * (q / 2));
+        s.v[(q / 2) & 1][0] = t.x;
+        s.v[(q / 2) & 1][1] = t.y;
+        s.v[(q / 2) & 1][2] = t.z;
+        s.v[(q / 2) & 1][3] = t.w;
+      }
+    }
     if (q >= 2 && q < 10) {
       s.ps0 += s.e[2 * q - 4];
       s.ps1 += s.e[2 * q - 3];
+      if constexpr (VEC) {
+        const int r = 2 * q - 4;  // values r, r + 1 of group r / 4
+        s.po = __builtin_fmaf(s.e[r], s.v[(r / 4) & 1][r % 4],
+                              __builtin_fmaf(s.e[r + 1], s.v[(r / 4) & 1][r % 4 + 1], s.po));
+      }
     }
   };
   auto softmax_tail = [&](SoftmaxStage& s, int rb) {  // what pieces 0..11 left undone
     s.ps0 += s.e[14];
     s.ps1 += s.e[15];
-    run_s[rb] = run_s[rb] * fast_exp2(s.c) + (s.ps0 + s.ps1);
+    const float resc = fast_exp2(s.c);
+    run_s[rb] = run_s[rb] * resc + (s.ps0 + s.ps1);
+    if constexpr (VEC) {
+      s.po = __builtin_fmaf(s.e[14], s.v[1][2], __builtin_fmaf(s.e[15], s.v[1][3], s.po));
+      run_o[rb] = run_o[rb] * resc + s.po;
+    }
   };
 
   // A operands (one 32-key sub-tile) from LDS
@@ -604,6 +645,18 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     b[4 * c + 1] = v.y;
     b[4 * c + 2] = v.z;
     b[4 * c + 3] = v.w;
+  };
+  auto load_v16 = [&](int buf, int js) {  // VEC: v_j in the accumulator layout, like the bias
+    f32x16 v;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float4 t = *reinterpret_cast<const float4*>(&lds_v[VEC ? buf : 0][js * 32 + 8 * c + 4 * h]);
+      v[4 * c + 0] = t.x;
+      v[4 * c + 1] = t.y;
+      v[4 * c + 2] = t.z;
+      v[4 * c + 3] = t.w;
+    }
+    return v;
   };
   auto load_bias16 = [&](int buf, int js) {
     f32x16 b;
@@ -693,7 +746,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         wait_lds();
         FS_SCHED_FENCE();
         const f32x16 acc = add_bias(chain(kr, rb, cur, js), kr, rb);
-        if (js == 0) softmax_first(acc, rb); else softmax(acc, rb);
+        f32x16 v16;
+        if constexpr (VEC) v16 = load_v16(cur, js);
+        if (js == 0) softmax_first(acc, rb, v16); else softmax(acc, rb, v16);
       }
     }
     if constexpr (!KPF) {
@@ -732,6 +787,15 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         if constexpr (!BIASC) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        }
+        // VEC: v of the previous unit's keys (its soft-max runs during this unit).  The previous
+        // unit sits on the same sub-tile, on the one before, or on the last one of the previous
+        // tile, whose buffer is the third of the ring until the next tile's staging reuses it.
+        const float* vsrc = nullptr;
+        if constexpr (VEC) {
+          const bool same_js = rb > 0;
+          const bool same_tile = same_js || js > 0;
+          vsrc = &lds_v[same_tile ? cur : nx2][(same_js ? js : (js + NSUB - 1) % NSUB) * 32 + 4 * h];
         }
         wait_lds();  // this unit's key operands (read one unit ago) are in their registers
         FS_SCHED_FENCE();
@@ -776,7 +840,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
           }
           // a wave-uniform branch around VALU work only: the MFMA chain itself stays one
           // straight line, accumulating in place
-          if (soft) softmax_piece(p, st, acc_prev, prev_rb);
+          if (soft) softmax_piece(p, st, acc_prev, prev_rb, vsrc);
           FS_SCHED_FENCE();
         };
 #pragma unroll
@@ -811,19 +875,25 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     }
     rotate();
   }
-  softmax(R1, RB - 1);  // BIASC: the last unit of a tile is an odd one, its chain ran in R1
+  {  // BIASC: the last unit of a tile is an odd one, its chain ran in R1
+    f32x16 v16;
+    if constexpr (VEC) v16 = load_v16(nx2, NSUB - 1);  // after rotate(): the tile just finished
+    softmax(R1, RB - 1, v16);
+  }
 
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = row0 + rb * 32 + li;
     const float s = run_s[rb] + xor32(run_s[rb]);
+    const float o = VEC ? run_o[rb] + xor32(run_o[rb]) : 0.f;
     const float M2 = BIASC ? -run_c[rb] : run_m[rb] * lscale;
     if (row < sd.nq && h == 0) {
       if (sd.splits == 1) {
-        epilogue_scalar(sd.ep, row, M2, s, 0.f);
+        epilogue_scalar(sd.ep, row, M2, s, o);
       } else {
         const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
         *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
+        if constexpr (VEC) sd.part_o[pr] = o;
       }
     }
   }
