@@ -22,6 +22,7 @@ FS_FLAG_FP32_MFMA = 4
 FS_FLAG_BF16X3_OPERANDS = 8
 FS_FLAG_OPERANDS_PREPARED = 16
 FS_FLAG_NO_TILE_SKIP = 32
+FS_FLAG_COARSE_TEST = 64
 # allow_tf32=False normally runs the two-plane fp16 operands (fp32-grade accuracy).
 # STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" runs fp32 MFMA
 # operands, "bf16x3" the three-plane bf16 split instead.

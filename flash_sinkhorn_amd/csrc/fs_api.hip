@@ -838,7 +838,10 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   } else if (lse2) {
     rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
     a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
-    if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, mode == kVec, total, st);
+    static const int coarse_env = env_int("FS_COARSE", 0);
+    const bool coarse = (coarse_env || (flags & FS_FLAG_COARSE_TEST)) && mode == kLse &&
+                        !(flags & FS_FLAG_NO_TILE_SKIP);
+    if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, mode == kVec, coarse, total, st);
   } else
   switch (mode) {
     case kLse: rc = launch_dp<kLse, false>(a, dp, rb, total, st); break;

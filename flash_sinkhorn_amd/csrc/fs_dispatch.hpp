@@ -36,7 +36,7 @@ int launch_transpose_planes(const float* src, const float* rowscale, unsigned* d
 // Plan-matrix (kMat), plan-vector (kVec) products and running arg-max (kArgmax) for d <= 128 on
 // two-plane fp16 rows (dp in {16, 32, 64, 128}; rb row blocks per wavefront in {1, 2}, 1 at 128).
 int launch_plan_tile(const LaunchArgs& a, int mode, int dp, int rb, int blocks, hipStream_t st);
-int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, int blocks,
+int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, bool coarse, int blocks,
                 hipStream_t st);
 
 }  // namespace fs

@@ -5,9 +5,9 @@
 
 namespace fs {
 
-template <int DP, int RB, int PREC, bool VEC>
+template <int DP, int RB, int PREC, bool VEC, bool COARSE = false>
 static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
-  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC, VEC>), dim3(blocks), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC, VEC, COARSE>), dim3(blocks), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
@@ -58,8 +58,25 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
-int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, int blocks,
+// fp16 planes, log-sum-exp, rows of at most 64 columns: the variants with the coarse test
+static int launch_coarse(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
+  switch (dp) {
+    case 16:
+      return rb >= 2 ? launch_cfg<16, 2, kH3, false, true>(a, blocks, st)
+                     : launch_cfg<16, 1, kH3, false, true>(a, blocks, st);
+    case 32:
+      return rb >= 2 ? launch_cfg<32, 2, kH3, false, true>(a, blocks, st)
+                     : launch_cfg<32, 1, kH3, false, true>(a, blocks, st);
+    case 64:
+      return rb >= 2 ? launch_cfg<64, 2, kH3, false, true>(a, blocks, st)
+                     : launch_cfg<64, 1, kH3, false, true>(a, blocks, st);
+  }
+  return FS_ERR_UNSUPPORTED;
+}
+
+int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, bool coarse, int blocks,
                 hipStream_t st) {
+  if (coarse && !vec && prec == kH3 && dp <= 64) return launch_coarse(a, dp, rb, blocks, st);
   if (vec) {  // plan-vector product: fp16 planes, rows of at most 64 columns
     return prec == kH3 ? launch_dp<kH3, true>(a, dp, rb, blocks, st) : FS_ERR_UNSUPPORTED;
   }

@@ -115,11 +115,12 @@ def flashsinkhorn_lse_fused(
 
 def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, alpha, damping_f,
                         damping_g, shift_x=None, shift_y=None, allow_tf32=True, use_exp2=True,
-                        prepared=None):
+                        prepared=None, coarse=False):
     """One launch on already contiguous fp32 operands.  With shift_x/shift_y the
     unbalanced shift correction is applied inside the epilogue.  When every paired argument
     is the same tensor (the self problem OT(x, x)) the library computes the one distinct
-    half-update and the same tensor is returned twice."""
+    half-update and the same tensor is returned twice.  ``coarse`` sets
+    ``FS_FLAG_COARSE_TEST`` (tiles tested after their hi*hi plane product)."""
     n, d = x.shape
     m = y.shape[0]
     f_out = torch.empty((n,), device=x.device, dtype=torch.float32)
@@ -128,6 +129,8 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
     g_out = f_out if self_problem else torch.empty((m,), device=x.device, dtype=torch.float32)
     wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_SYMMETRIC_STEP, x, y,
                                            _lib.flags(use_exp2, allow_tf32), prepared)
+    if coarse:
+        fl |= _lib.FS_FLAG_COARSE_TEST
     rc = _lib.lib().fs_symmetric_step(
         x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), f_out.data_ptr(), g_out.data_ptr(), _lib.ptr(shift_x),
@@ -138,7 +141,8 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
 
 
 def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale, shift_x=None,
-                         shift_y=None, allow_tf32=True, use_exp2=True, prepared=None):
+                         shift_y=None, allow_tf32=True, use_exp2=True, prepared=None,
+                         coarse=False):
     """``steps`` = [(eps, alpha, damping_f, damping_g), ...] run back to back by one library call
     (``fs_symmetric_steps``): the per-step host work is a kernel launch, not a Python round
     trip.  Operands as for ``_symmetric_step_raw``; returns the potentials of the last step."""
@@ -157,6 +161,8 @@ def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale,
     eps_a, alpha_a, df_a, dg_a = (arr(*[float(s[i]) for s in steps]) for i in range(4))
     wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_SYMMETRIC_STEP, x, y,
                                            _lib.flags(use_exp2, allow_tf32), prepared)
+    if coarse:
+        fl |= _lib.FS_FLAG_COARSE_TEST
     rc = _lib.lib().fs_symmetric_steps(
         x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), f_work[0].data_ptr(), g_work[0].data_ptr(), f_work[1].data_ptr(),

@@ -8,6 +8,7 @@ correction live in the kernel epilogue.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -19,6 +20,37 @@ from flash_sinkhorn_amd.kernels._common import (
 )
 
 __all__ = ["sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric"]
+
+# Long fixed-eps solves on large clouds run on rows and keys grouped by k-means cluster, and
+# time a few steps with and without FS_FLAG_COARSE_TEST to pick the faster kernel variant: with
+# neighbouring rows next to each other, whole key tiles fall below the 2^-40 criterion for all
+# rows of a workgroup at once, which the coarse test turns into fewer MFMAs.  The potentials
+# come back in the caller's order; values agree with the unordered solve to fp32 rounding.
+CLUSTER_ORDER = os.environ.get("FLASH_SINKHORN_CLUSTER_ORDER", "1") != "0"
+# None: time both variants in the first steps of such a solve; True / False: no timing
+COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_TEST", ""))
+_CLUSTER_MIN_ROWS = 16384
+_CLUSTER_MIN_STEPS = 24
+_TUNE_STEPS = 3  # steps timed per variant
+_RETUNE_AFTER = 24  # steps between the first choice and the second one of a long run
+
+
+def _cluster_order(pts: torch.Tensor, k: int = 16, iters: int = 4) -> torch.Tensor:
+    """Permutation that groups the rows of ``pts`` by k-means cluster (Lloyd iterations from
+    evenly spaced rows; GEMM-shaped updates, no host synchronisation)."""
+    n = pts.shape[0]
+    centres = pts[torch.arange(k, device=pts.device) * (n // k)].clone()
+    labels = None
+    for it in range(iters + 1):
+        score = (centres * centres).sum(dim=1)[None, :] - 2.0 * (pts @ centres.T)
+        labels = score.argmin(dim=1)
+        if it == iters:
+            break
+        onehot = torch.nn.functional.one_hot(labels, k).to(pts.dtype)
+        count = onehot.sum(dim=0)
+        mean = (onehot.T @ pts) / count.clamp_min(1.0)[:, None]
+        centres = torch.where(count[:, None] > 0, mean, centres)
+    return torch.argsort(labels, stable=True)
 
 # Reference switches from the one-launch step to two launches at this n
 # (sinkhorn_solvers.py:463-468).  Both give the same numbers; here the one-launch
@@ -179,6 +211,31 @@ def sinkhorn_flashstyle_symmetric(
             and (a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape))):
         yf, beta, log_b, g_hat = xf, alpha, log_a, f_hat
 
+    # cluster order (see CLUSTER_ORDER): every per-row array is permuted, the results are
+    # put back in the caller's order at the end
+    inv_x = inv_y = None
+    coarse = [False, False]  # [variant in use, still to be tuned]
+    if (CLUSTER_ORDER and fused and not use_labels and not allow_tf32 and _lib.TILE_SKIP
+            and _lib.STRICT_OPERANDS == "fp16x2" and xf.shape[1] <= 64
+            and min(xf.shape[0], yf.shape[0]) >= _CLUSTER_MIN_ROWS
+            and len(eps_list) >= _CLUSTER_MIN_STEPS
+            and all(e == eps_list[0] for e in eps_list)):
+        self_problem = yf is xf
+        perm_x = _cluster_order(xf)
+        inv_x = torch.empty_like(perm_x)
+        inv_x[perm_x] = torch.arange(perm_x.numel(), device=perm_x.device)
+        xf, alpha, log_a, f_hat = (xf[perm_x].contiguous(), alpha[perm_x], log_a[perm_x],
+                                   f_hat[perm_x])
+        if self_problem:
+            yf, beta, log_b, g_hat, inv_y = xf, alpha, log_a, f_hat, inv_x
+        else:
+            perm_y = _cluster_order(yf)
+            inv_y = torch.empty_like(perm_y)
+            inv_y[perm_y] = torch.arange(perm_y.numel(), device=perm_y.device)
+            yf, beta, log_b, g_hat = (yf[perm_y].contiguous(), beta[perm_y], log_b[perm_y],
+                                      g_hat[perm_y])
+        coarse[0], coarse[1] = bool(COARSE_TEST), COARSE_TEST is None
+
     # operand planes are converted once for the whole loop
     prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32))
 
@@ -189,7 +246,7 @@ def sinkhorn_flashstyle_symmetric(
                 xf, yf, f_hat, g_hat, log_a, log_b, e, cost_scale=cost_scale, alpha=w,
                 damping_f=damp_f, damping_g=damp_g,
                 shift_x=alpha if damp_f < 1.0 else None, shift_y=beta if damp_g < 1.0 else None,
-                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared)
+                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=coarse[0])
         # two launches, raw-bias kernel, averaging and shift correction on the host
         kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
                   _prepared=prepared)
@@ -210,11 +267,41 @@ def sinkhorn_flashstyle_symmetric(
                 f_hat, g_hat = jacobi(f_hat, g_hat, e, w)
             return f_hat, g_hat
         steps = [(e, w, dampening(e, rho_x), dampening(e, rho_y)) for e, w in run]
-        return _symmetric_steps_raw(
-            xf, yf, f_hat, g_hat, log_a, log_b, steps, cost_scale=cost_scale,
-            shift_x=alpha if rho_x is not None else None,
-            shift_y=beta if rho_y is not None else None,
-            allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared)
+
+        def launch(f_hat, g_hat, part, variant):
+            return _symmetric_steps_raw(
+                xf, yf, f_hat, g_hat, log_a, log_b, part, cost_scale=cost_scale,
+                shift_x=alpha if rho_x is not None else None,
+                shift_y=beta if rho_y is not None else None,
+                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=variant)
+
+        def tune(f_hat, g_hat, window):
+            # the steps of `window` alternate between the two variants (all of them steps of
+            # the solve), each timed on the stream; the coarse variant takes the earlier step
+            # of each pair (early steps get faster as the plan sharpens)
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(window) + 1)]
+            ev[0].record()
+            for i in range(len(window)):
+                f_hat, g_hat = launch(f_hat, g_hat, window[i:i + 1], i % 2 == 0)
+                ev[i + 1].record()
+            ev[-1].synchronize()
+            took = [ev[i].elapsed_time(ev[i + 1]) for i in range(len(window))]
+            return f_hat, g_hat, sum(took[0::2]) < 0.98 * sum(took[1::2])
+
+        if coarse[1] and len(steps) >= 2 * _TUNE_STEPS + 2:
+            # first choice after the very first step (it starts from flat potentials); a long
+            # run chooses again some thirty steps in: a device that was idle before the solve
+            # takes that long to settle, and the first choice may have seen it cold
+            w = 2 * _TUNE_STEPS
+            f_hat, g_hat = launch(f_hat, g_hat, steps[:1], False)
+            f_hat, g_hat, coarse[0] = tune(f_hat, g_hat, steps[1:1 + w])
+            steps = steps[1 + w:]
+            if len(steps) >= _RETUNE_AFTER + 2 * w:
+                f_hat, g_hat = launch(f_hat, g_hat, steps[:_RETUNE_AFTER], coarse[0])
+                f_hat, g_hat, coarse[0] = tune(f_hat, g_hat, steps[_RETUNE_AFTER:_RETUNE_AFTER + w])
+                steps = steps[_RETUNE_AFTER + w:]
+            coarse[1] = False
+        return launch(f_hat, g_hat, steps, coarse[0])
 
     # the initial full step and the averaged steps, cut where a convergence check looks at
     # the potentials
@@ -242,6 +329,8 @@ def sinkhorn_flashstyle_symmetric(
     out = (f_hat + alpha, g_hat + beta)
     if return_prelast and last_extrapolation:
         out = out + (f_prelast, g_prelast)
+    if inv_x is not None:  # back to the caller's row order
+        out = tuple(t[inv_x if i % 2 == 0 else inv_y] for i, t in enumerate(out))
     if return_n_iters:
         out = out + (used,)
     return out

@@ -28,6 +28,14 @@
  *    The d <= 128 log-sum-exp kernel leaves out the exponentials of a 32 x 32 logits tile
  *    whose every entry lies more than 2^40 below its row's running maximum (they cannot
  *    change the fp32 row sums); FS_FLAG_NO_TILE_SKIP computes them all the same.
+ *    FS_FLAG_COARSE_TEST (log-sum-exp entry points, default operand mode, d <= 64) applies the
+ *    same 2^40 criterion one stage earlier: the hi*hi plane product of a tile is tested
+ *    against the running maximum, lowered by a per-row bound on the two cross products, and a
+ *    tile that fails ends there (4 of its 12 MFMAs); a workgroup first takes the largest
+ *    logit of 64 keys sampled from the whole key set as its running maximum.  Results stay
+ *    within fp32 rounding of the full computation.  It pays when rows and keys are ordered so
+ *    that neighbouring rows have neighbouring keys (e.g. sorted by cluster) and the plan is
+ *    peaked; on other inputs the test costs about 10 %.  Ignored where it does not apply.
  *    The gradient, the plan-vector / plan-matrix products, mat5 and the c-transform, and for
  *    d > 128 the log-sum-exp as well, run on the two-plane fp16 operands by default and with
  *    FS_FLAG_REDUCED_OPERANDS, and on fp32 MFMA operands with FS_FLAG_FP32_MFMA or
@@ -57,6 +65,7 @@ extern "C" {
 #define FS_FLAG_BF16X3_OPERANDS 8u
 #define FS_FLAG_OPERANDS_PREPARED 16u
 #define FS_FLAG_NO_TILE_SKIP 32u
+#define FS_FLAG_COARSE_TEST 64u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0

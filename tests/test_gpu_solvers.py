@@ -553,3 +553,70 @@ def test_fused_schur_matvec_against_dense_oracle(n, m, d, cs):
         fused_schur_matvec_sqeuclid(X, Y, F, G, Z[:-1], DX, DN, eps=eps)
     with pytest.raises(ValueError):
         fused_schur_matvec_sqeuclid(X, Y, F, G, Z, DX[:-1], DN, eps=eps)
+
+
+def _clustered(rng, n, d, k=8, spread=2.0):
+    centres = rng.standard_normal((k, d)) * spread
+    lab = rng.integers(0, k, n)
+    return (centres[lab] + rng.standard_normal((n, d))).astype(np.float32), lab
+
+
+@pytest.mark.parametrize("n,m,d,eps,sort", [(3000, 4100, 64, 0.01, True), (3000, 4100, 64, 0.01, False),
+                                            (2100, 2300, 20, 0.3, False), (129, 1000, 3, 0.05, True),
+                                            (40, 33, 16, 0.5, False)])
+def test_coarse_tile_test_leaves_results_unchanged(n, m, d, eps, sort):
+    """FS_FLAG_COARSE_TEST (tiles tested after their hi*hi plane product, running maximum started
+    from 64 sampled keys) against the oracle and against the launch without the flag, on peaked
+    plans over rows sorted by cluster (most tiles end at the test) and on generic inputs."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    rng = np.random.default_rng(31)
+    x, lx = _clustered(rng, n, d)
+    y, ly = _clustered(rng, m, d)
+    if sort:
+        x, y = x[np.argsort(lx, kind="stable")], y[np.argsort(ly, kind="stable")]
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    fh = (-(x * x).sum(1) + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    gh = (-(y * y).sum(1) + 0.1 * rng.standard_normal(m)).astype(np.float32)
+    la, lb = np.log(a), np.log(b)
+    args = dev(x, y, fh, gh, la, lb)
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    f1, g1 = _symmetric_step_raw(*args, eps, coarse=True, **kw)
+    f0, g0 = _symmetric_step_raw(*args, eps, coarse=False, **kw)
+    wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, eps, 1.0, 0.5, 1.0, 1.0)
+    assert rel_err(f1, wf) < RTOL and rel_err(g1, wg) < RTOL
+    # the two launches differ by the order of the plane products only
+    assert rel_err(f1, f0.cpu().numpy()) < 2e-6 and rel_err(g1, g0.cpu().numpy()) < 2e-6
+
+
+@pytest.mark.parametrize("variant", [True, False, None])
+def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
+    """Long fixed-eps solves on large clouds run on rows grouped by k-means cluster and hand the
+    potentials back in the caller's order; with the coarse tile test forced on, off, or chosen by
+    timing, the result is the unordered solve's to rounding."""
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    rng = np.random.default_rng(32)
+    n, m, d = 16500, 16400, 8
+    x, _ = _clustered(rng, n, d)
+    y, _ = _clustered(rng, m, d)
+    a = rng.random(n).astype(np.float32) + 0.5
+    b = rng.random(m).astype(np.float32) + 0.5
+    X, Y, A, B = dev(x, y, a / a.sum(), b / b.sum())
+    kw = dict(use_epsilon_scaling=False, eps=0.05, n_iters=26, allow_tf32=False,
+              return_prelast=True)
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
+    want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", True)
+    monkeypatch.setattr(solvers, "COARSE_TEST", variant)
+    got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+    for u, v in zip(got, want):
+        assert rel_err(u, v.cpu().numpy()) < 2e-5
+    # the self problem keeps its single half-update per step under the ordering
+    ws = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, **kw)
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
+    wu = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, **kw)
+    # these potentials are small differences of shifted potentials of size |x|^2
+    scale = float((X * X).sum(dim=1).max())
+    for u, v in zip(ws, wu):
+        assert float((u - v).abs().max()) < 2e-6 * scale
+    assert float((ws[0] - ws[1]).abs().max()) == 0.0
