@@ -20,6 +20,9 @@ products per algorithmic product, so the algorithmic rate is priced against the 
 2516.6 TFLOP/s fp16/bf16 peak divided by that factor (838.9 or 419.4 TFLOP/s; 157.3 for fp32
 MFMA operands); the ratio to the fp32 MFMA peak and the serial / overlapped MFMA+exp roofline
 times of the whole 102-step solve are reported next to it.
+The solver groups rows by k-means cluster and picks, by timing a few steps, between the plain
+kernel and the one that tests a tile after its hi*hi plane product; the roofline launch is
+timed on the same row order and variant (reported under roofline.tile_skip).
 cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores on a
 bounded sample and scaled to the metric's unit.
 """
@@ -123,6 +126,7 @@ def main():
     import torch
 
     from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd import sinkhorn_solvers as solvers
     from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric
     from flash_sinkhorn_amd.kernels._common import log_weights
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
@@ -157,15 +161,28 @@ def main():
     la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
     fh, gh = (f - alpha).contiguous(), (g - beta).contiguous()
 
-    def launch_ms(mode, reps=20):
+    # the launch as the solve runs it: rows in the solver's cluster order and the kernel variant
+    # it chose (main mode only; the other modes have neither)
+    solve_info = dict(solvers.LAST_SOLVE)
+    ordered = None
+    if solve_info["cluster_order"]:
+        px, py = solvers._cluster_order(X), solvers._cluster_order(Y)
+        ordered = (X[px].contiguous(), Y[py].contiguous(), fh[px].contiguous(),
+                   gh[py].contiguous(), la[px].contiguous(), lb[py].contiguous())
+
+    def launch_ms(mode, reps=20, as_solved=False, coarse=False):
         tf32 = set_mode(mode)
         kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=tf32)
-        _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, **kw)
+        ops = (X, Y, fh, gh, la, lb)
+        if as_solved and ordered is not None:
+            ops = ordered
+            kw["coarse"] = coarse
+        _symmetric_step_raw(*ops, EPS, **kw)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
-            _symmetric_step_raw(X, Y, fh, gh, la, lb, EPS, **kw)
+            _symmetric_step_raw(*ops, EPS, **kw)
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / reps
@@ -196,7 +213,7 @@ def main():
                                      "overlapped": max(t_mfma, t_exp)}
         return r
 
-    main_ms = launch_ms(args.mode)
+    main_ms = launch_ms(args.mode, as_solved=True, coarse=solve_info["coarse_test"])
     line = {
         "metric": "ms per 100 symmetric Sinkhorn iterations (n=m=50k, d=64, fp32)",
         "value": ms_per_step, "unit": "ms", "n_gpus": 1, "steps": args.steps,
@@ -220,8 +237,14 @@ def main():
     _lib.TILE_SKIP = True
     line["roofline"]["tile_skip"] = {
         "enabled": True, "launch_ms_with_every_exp": ms_noskip,
+        "rows_in_cluster_order": solve_info["cluster_order"],
+        "coarse_test": solve_info["coarse_test"],
+        "launch_ms_caller_order_no_coarse_test": launch_ms(args.mode, reps=10),
         "note": "tiles whose logits all lie more than 2^40 below the running row maxima skip "
-                "their exp2 (no change to fp32 sums); MFMA work is never skipped"}
+                "their exp2 (no change to fp32 sums); with coarse_test such a tile is recognised "
+                "after its hi*hi plane product (bound on the cross products) and skips the other "
+                "8 of its 12 MFMAs too, so the executed MFMA flop are fewer than the algorithmic "
+                "flop `achieved` counts; launch_ms_with_every_exp computes everything"}
     if not args.no_other_modes:
         others = {}
         for mode in MODES:

@@ -644,8 +644,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     kr.ab = h ? 1.0f : b;
   };
   // MFMA number k (0 <= k < NMAIN) of one logits tile (32 keys x 32 queries) of query block
-  // rb.  Plane products run from the lowest weight to hi*hi; those below 2^-16 (2^-24 with
-  // three planes) are skipped.
+  // rb.  Plane products run from the lowest weight to hi*hi (COARSE: hi*hi first, it is what
+  // the early test looks at); those below 2^-16 (2^-24 with three planes) are skipped.
   auto mfma_k = [&](int k, f32x16 acc, const KeyRegs& kr, int rb) {
     if constexpr (!kBf) {
       return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ya[k], xs[rb][k], acc, 0, 0, 0);

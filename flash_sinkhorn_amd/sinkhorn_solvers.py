@@ -31,6 +31,8 @@ CLUSTER_ORDER = os.environ.get("FLASH_SINKHORN_CLUSTER_ORDER", "1") != "0"
 COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_TEST", ""))
 _CLUSTER_MIN_ROWS = 16384
 _CLUSTER_MIN_STEPS = 24
+# what the last symmetric solve did: {"cluster_order": bool, "coarse_test": bool}
+LAST_SOLVE = {"cluster_order": False, "coarse_test": False}
 _TUNE_STEPS = 3  # steps timed per variant
 _RETUNE_AFTER = 24  # steps between the first choice and the second one of a long run
 
@@ -329,6 +331,7 @@ def sinkhorn_flashstyle_symmetric(
     out = (f_hat + alpha, g_hat + beta)
     if return_prelast and last_extrapolation:
         out = out + (f_prelast, g_prelast)
+    LAST_SOLVE["cluster_order"], LAST_SOLVE["coarse_test"] = inv_x is not None, coarse[0]
     if inv_x is not None:  # back to the caller's row order
         out = tuple(t[inv_x if i % 2 == 0 else inv_y] for i, t in enumerate(out))
     if return_n_iters:
