@@ -44,10 +44,11 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2516.6
 EXP2_PER_S = 18.6e12  # v_exp_f32 lanes per second measured on the box (half rate)
 # Memory-side bytes per lse2_kernel launch of the default workload, per operand mode, from two
-# rocprofv3 --pmc runs (FETCH_SIZE 117,370 KiB x 2.0, WRITE_SIZE 12,508 KiB x 1.0; the factors
+# rocprofv3 --pmc runs (FETCH_SIZE 113,782 KiB x 2.0, WRITE_SIZE 12,510 KiB x 1.0 for the kernel
+# variant with the coarse tile test, 112,309 / 12,509 for the plain one; the factors
 # are what the same counters read for the 256 MiB copy of --copy-calibration: half the bytes
 # copied and all of them).  Not measured for the other modes.
-MEASURED_TRAFFIC_BYTES = {"strict": int((112406 * 2.0 + 12510) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"strict": int((113782 * 2.0 + 12510) * 1024)}
 
 
 def gmm_cloud(rng, n, d, k=8):
