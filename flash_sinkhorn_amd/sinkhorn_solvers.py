@@ -29,7 +29,9 @@ __all__ = ["sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric"]
 CLUSTER_ORDER = os.environ.get("FLASH_SINKHORN_CLUSTER_ORDER", "1") != "0"
 # None: time both variants in the first steps of such a solve; True / False: no timing
 COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_TEST", ""))
-_CLUSTER_MIN_ROWS = 16384
+# measured on the benchmark's mixtures at d = 64: below about 40,000 rows per cloud the ordering
+# and the timed steps cost more than the coarse variant returns (25,000: +4 %; 32,768: even)
+_CLUSTER_MIN_ROWS = 40000
 _CLUSTER_MIN_STEPS = 24
 # what the last symmetric solve did: {"cluster_order": bool, "coarse_test": bool}
 LAST_SOLVE = {"cluster_order": False, "coarse_test": False}

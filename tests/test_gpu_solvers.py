@@ -606,9 +606,14 @@ def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
               return_prelast=True)
     monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
     want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+    assert not solvers.LAST_SOLVE["cluster_order"]
     monkeypatch.setattr(solvers, "CLUSTER_ORDER", True)
+    monkeypatch.setattr(solvers, "_CLUSTER_MIN_ROWS", 16384)  # the default only orders larger clouds
     monkeypatch.setattr(solvers, "COARSE_TEST", variant)
     got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+    assert solvers.LAST_SOLVE["cluster_order"]
+    if variant is not None:
+        assert solvers.LAST_SOLVE["coarse_test"] == variant
     for u, v in zip(got, want):
         assert rel_err(u, v.cpu().numpy()) < 2e-5
     # the self problem keeps its single half-update per step under the ordering
