@@ -1,4 +1,4 @@
-"""Per-operation timings at the BASELINE shapes: ``python -m flash_sinkhorn_amd.op_timings [c1 c2 c3 c4 c5]``.
+"""Per-operation timings at the benchmark shapes: ``python -m flash_sinkhorn_amd.op_timings [c1 c2 c3 c4 c5]``.
 
 Prints one JSON line per shape with the average launch time (HIP events on the current
 stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop),

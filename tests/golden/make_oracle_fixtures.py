@@ -1,7 +1,7 @@
 """Cache slow fp64 ORACLE results (not reference output) so GPU tests need not recompute them.
 
 ``python tests/golden/make_oracle_fixtures.py [config1 config2 config4 config5]`` writes one
-``oracle_<config>.npz`` per BASELINE configuration named (all of them by default).  Each
+``oracle_<config>.npz`` per benchmark configuration named (all of them by default).  Each
 takes minutes of CPU time; inputs are regenerated from the seed by the ``*_inputs``
 functions below, which the tests import.  Large outputs are stored for a seeded sample of
 rows only (the row indices are stored with them).

@@ -1,4 +1,4 @@
-"""BASELINE-size checks through size-independent properties and sampled-row oracle parity."""
+"""Full-size checks through size-independent properties and sampled-row oracle parity."""
 import numpy as np
 import pytest
 import torch
@@ -81,7 +81,7 @@ def test_config3_solve_and_gradient_properties(c3):
 
 
 def test_config2_loss_and_potentials():
-    """BASELINE config 2 (n=m=10,000, d=64, eps=0.01, 100 iterations) against the fp64
+    """Benchmark configuration 2 (n=m=10,000, d=64, eps=0.01, 100 iterations) against the fp64
     oracle on all rows; the oracle side is cached in tests/golden/oracle_config2.npz."""
     import os
     from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric
@@ -109,7 +109,7 @@ def _fixture(name):
 
 
 def test_config1_debiased_loss_and_gradient():
-    """BASELINE config 1 at full size (n=m=2000, d=3, half cost, debiased, eps=0.01, 100
+    """Benchmark configuration 1 at full size (n=m=2000, d=3, half cost, debiased, eps=0.01, 100
     iterations) against the fp64 oracle cached in tests/golden/oracle_config1.npz."""
     from flash_sinkhorn_amd import SamplesLoss
     from tests.golden.make_oracle_fixtures import config1_inputs
@@ -130,7 +130,7 @@ def test_config1_debiased_loss_and_gradient():
 @pytest.mark.parametrize("tag,kw", [("reach", dict(reach=1.0)),
                                     ("semi", dict(reach_x=1.0, reach_y=None))])
 def test_config4_unbalanced_alternating(tag, kw):
-    """BASELINE config 4 (n=20,000, m=30,000, d=128, eps=0.05^2, Dirichlet weights of mass
+    """Benchmark configuration 4 (n=20,000, m=30,000, d=128, eps=0.05^2, Dirichlet weights of mass
     1.0 / 1.3, 10 alternating iterations with the early-stop check at 10) against the fp64
     oracle cached in tests/golden/oracle_config4.npz, all rows."""
     from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating
@@ -147,7 +147,7 @@ def test_config4_unbalanced_alternating(tag, kw):
 
 
 def test_config5_large_d_loss_gradient_and_hvp():
-    """BASELINE config 5 (n=m=8192, d=1536, eps=0.25, 50 iterations): debiased loss and
+    """Benchmark configuration 5 (n=m=8192, d=1536, eps=0.25, 50 iterations): debiased loss and
     grad_x through the column-sliced kernels, then the Hessian-vector product of the xy term
     by double backward (streaming CG, at most 20 iterations), against the fp64 oracle cached
     in tests/golden/oracle_config5.npz (48 sampled rows plus Frobenius norms)."""

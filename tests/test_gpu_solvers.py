@@ -115,7 +115,7 @@ def _loss_oracle(x, y, a, b, *, eps, n_iters, cost_scale, debias):
 
 
 def test_samples_loss_value_and_gradient_config1_shape():
-    # BASELINE config 1 at reduced n: debiased, half cost, eps=0.01, d=3, uniform weights
+    # benchmark configuration 1 at reduced n: debiased, half cost, eps=0.01, d=3, uniform weights
     from flash_sinkhorn_amd import SamplesLoss
     rng = np.random.default_rng(1)
     n = m = 400
