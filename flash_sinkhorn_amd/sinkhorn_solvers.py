@@ -284,10 +284,11 @@ def sinkhorn_flashstyle_symmetric(
             # the solve), each timed on the stream; the coarse variant takes the earlier step
             # of each pair (early steps get faster as the plan sharpens)
             ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(window) + 1)]
-            ev[0].record()
+            stream = torch.cuda.current_stream(xf.device)  # the stream the launches go to
+            ev[0].record(stream)
             for i in range(len(window)):
                 f_hat, g_hat = launch(f_hat, g_hat, window[i:i + 1], i % 2 == 0)
-                ev[i + 1].record()
+                ev[i + 1].record(stream)
             ev[-1].synchronize()
             took = [ev[i].elapsed_time(ev[i + 1]) for i in range(len(window))]
             return f_hat, g_hat, sum(took[0::2]) < 0.98 * sum(took[1::2])
