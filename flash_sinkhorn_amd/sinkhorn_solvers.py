@@ -224,7 +224,8 @@ def sinkhorn_flashstyle_symmetric(
             and min(xf.shape[0], yf.shape[0]) >= _CLUSTER_MIN_ROWS
             and len(eps_list) >= _CLUSTER_MIN_STEPS
             and all(e == eps_list[0] for e in eps_list)):
-        self_problem = yf is xf
+        # the aliased form set up above; x passed twice with two weight vectors is not it
+        self_problem = yf is xf and log_b is log_a and g_hat is f_hat and beta is alpha
         perm_x = _cluster_order(xf)
         inv_x = torch.empty_like(perm_x)
         inv_x[perm_x] = torch.arange(perm_x.numel(), device=perm_x.device)

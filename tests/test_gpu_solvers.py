@@ -625,3 +625,12 @@ def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
     for u, v in zip(ws, wu):
         assert float((u - v).abs().max()) < 2e-6 * scale
     assert float((ws[0] - ws[1]).abs().max()) == 0.0
+    # one cloud passed twice with two weight vectors is an ordinary two-sided problem
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", True)
+    monkeypatch.setattr(solvers, "_CLUSTER_MIN_ROWS", 16384)
+    A2 = torch.flip(A, dims=[0]).contiguous()
+    got2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
+    want2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
+    for u, v in zip(got2, want2):
+        assert float((u - v).abs().max()) < 2e-6 * scale
