@@ -84,6 +84,13 @@ def _resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y):
     return rho_x, rho_y
 
 
+def _require_cuda(x, y) -> None:
+    # the same complaint the kernel launchers make (sinkhorn_flashstyle_sqeuclid.py:1000-1001),
+    # raised before any host-side preparation touches the tensors
+    if not x.is_cuda or not y.is_cuda:
+        raise ValueError("x and y must be CUDA tensors")
+
+
 def _max_change(f, g, prev_f, prev_g) -> float:
     return max((f - prev_f).abs().max().item(), (g - prev_g).abs().max().item())
 
@@ -114,6 +121,7 @@ def sinkhorn_flashstyle_alternating(
 
     rho_x, rho_y = _resolve_rho(rho, reach, rho_x, rho_y, reach_x, reach_y)
     damp_f, damp_g = dampening(eps, rho_x), dampening(eps, rho_y)
+    _require_cuda(x, y)
     xf, yf = x.float().contiguous(), y.float().contiguous()
     alpha = cost_scale * (xf * xf).sum(dim=1)
     beta = cost_scale * (yf * yf).sum(dim=1)
@@ -196,6 +204,7 @@ def sinkhorn_flashstyle_symmetric(
     if n_iters is not None:
         eps_list = list(eps_list)[: int(n_iters)]
 
+    _require_cuda(x, y)
     xf, yf = x.float().contiguous(), y.float().contiguous()
     alpha = (cost_scale * (xf * xf).sum(dim=1)).contiguous()
     beta = (cost_scale * (yf * yf).sum(dim=1)).contiguous()

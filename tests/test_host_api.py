@@ -272,3 +272,15 @@ def test_cluster_order_is_a_permutation_that_groups_clusters():
     assert runs <= 16  # at most one run per k-means centre
     same = torch.zeros(40, 3)
     assert _cluster_order(same, k=4).tolist() == list(range(40))  # ties keep the caller's order
+
+
+def test_solvers_refuse_cpu_tensors_before_touching_them():
+    import torch
+    from flash_sinkhorn_amd.sinkhorn_solvers import (
+        sinkhorn_flashstyle_alternating, sinkhorn_flashstyle_symmetric)
+    x = torch.randn(10, 3)
+    w = torch.full((10,), 0.1)
+    with pytest.raises(ValueError, match="CUDA tensors"):
+        sinkhorn_flashstyle_symmetric(x, x, w, w, use_epsilon_scaling=False, eps=0.1, n_iters=3)
+    with pytest.raises(ValueError, match="CUDA tensors"):
+        sinkhorn_flashstyle_alternating(x, x, w, w, eps=0.1, n_iters=3)
