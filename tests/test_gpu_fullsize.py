@@ -80,6 +80,26 @@ def test_config3_solve_and_gradient_properties(c3):
     assert torch.isfinite(gy).all()
 
 
+@pytest.mark.parametrize("order,coarse", [(True, True), (True, False), (False, None)])
+def test_config3_solve_variants_match_oracle_rows(c3, monkeypatch, order, coarse):
+    """The same solve on rows grouped by cluster with the coarse tile test forced on, forced off,
+    and in the caller's order on the plain kernel: sampled rows of the final extrapolation step
+    (f = softmin of the pre-extrapolation g, g likewise) against the dense fp64 oracle."""
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    x, y, a, b, (X, Y, A, B) = c3
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", order)
+    monkeypatch.setattr(solvers, "COARSE_TEST", coarse)
+    f, g, fp, gp = solvers.sinkhorn_flashstyle_symmetric(
+        X, Y, A, B, use_epsilon_scaling=False, eps=EPS, n_iters=100, allow_tf32=False,
+        return_prelast=True)
+    assert solvers.LAST_SOLVE == {"cluster_order": order, "coarse_test": bool(order and coarse)}
+    rows = np.random.default_rng(2).choice(50_000, 96, replace=False)
+    want_f = oracle.softmin(x[rows], y, gp.cpu().numpy(), np.log(b), EPS)
+    want_g = oracle.softmin(y[rows], x, fp.cpu().numpy(), np.log(a), EPS)
+    assert rel_err(f.cpu().numpy()[rows], want_f) < 1e-4
+    assert rel_err(g.cpu().numpy()[rows], want_g) < 1e-4
+
+
 def test_config2_loss_and_potentials():
     """Benchmark configuration 2 (n=m=10,000, d=64, eps=0.01, 100 iterations) against the fp64
     oracle on all rows; the oracle side is cached in tests/golden/oracle_config2.npz."""
