@@ -21,10 +21,17 @@ Pin status (what each function is checked against in tests/test_oracle_*.py):
   FS/testing/reference_sinkhorn.py:65-82
 * sinkhorn_alternating, GeomLoss convention (balanced) ... relation to the OTT
   convention f_ott = f + eps*log a, fixed point marginals
-* unbalanced / semi-unbalanced (symmetric and alternating) ... PARITY UNPINNED
-  by any reference-held artefact (the reference checks these against GeomLoss,
-  which is not installed); pinned only by the limits rho->inf == balanced,
-  reach_x == reach_y == reach, and the unbalanced fixed-point equation
+* unbalanced / semi-unbalanced symmetric solver ... no reference-held artefact exists (the
+  reference checks these against GeomLoss, which is not installed); pinned by the mathematics:
+  at the fixed point the plan is stationary for the primal problem
+  <C,P> + eps KL(P|ab) + rho_x KL(P1|a) + rho_y KL(P^T1|b) with rho_x != rho_y and with one side
+  balanced (a swapped rho or a wrong damping fails), the marginals obey
+  P1 = a exp(-f/rho_x), P^T1 = b exp(-g/rho_y), strong duality ties sinkhorn_cost to the primal
+  objective, plus the limits rho->inf == balanced and reach_x == reach_y == reach
+* unbalanced alternating solver ... restates FS/sinkhorn_solvers.py:240-259 AS WRITTEN (the
+  damping quirk is the reference's, no mathematical problem fixes it); pinned by one step
+  written out with python loops for rho_x != rho_y (which rho damps which side, Gauss-Seidel
+  order); values beyond that reading are PARITY UNPINNED by any reference-held artefact
 * grad_barycentric / grad_plan ... golden vectors from
   FS/testing/reference_sinkhorn.py:195-233 and finite differences of the dual
 * apply_plan_vec / apply_plan_mat / mat5 ... brute-force python loops

@@ -1,9 +1,10 @@
 """Cache slow fp64 ORACLE results (not reference output) so GPU tests need not recompute them.
 
-``python tests/golden/make_oracle_fixtures.py [config1 config2 config4 config5]`` writes one
-``oracle_<config>.npz`` per benchmark configuration named (all of them by default).  Each
-takes minutes of CPU time; inputs are regenerated from the seed by the ``*_inputs``
-functions below, which the tests import.  Large outputs are stored for a seeded sample of
+``python tests/golden/make_oracle_fixtures.py [config1 config2 config3 config4 config5]`` writes
+one ``oracle_<config>.npz`` per benchmark configuration named (all but config3 by default).  Each
+takes minutes of CPU time (config3: about an hour and a half on 8 cores with
+ORACLE_THREADS=8); inputs are regenerated from the seed by the ``*_inputs`` functions below,
+which the tests import.  Large outputs are stored for a seeded sample of
 rows only (the row indices are stored with them).
 """
 import os
@@ -91,6 +92,34 @@ def make_config2():
     print("config2 loss", c_xy, "debiased", loss)
 
 
+def config3_inputs():
+    """n=m=50,000, d=64; each cloud a seeded mixture of 8 unit Gaussians with means ~ N(0, 4I);
+    uniform weights (seed 3).  The generator is the benchmark's own."""
+    from bench import make_inputs
+    return make_inputs(50_000, 50_000, 64)
+
+
+def make_config3():
+    """The headline solve in fp64: 100 iterations at eps = 0.01 (102 Jacobi steps), its loss, all
+    four potential vectors, and 256 sampled rows of the analytic grad_x."""
+    x, y, a, b = config3_inputs()
+    eps = 0.01
+    f, g, fp, gp = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=eps,
+                                             n_iters=100, return_prelast=True)
+    loss = oracle.sinkhorn_cost(a, b, f, g, eps)
+    rows = np.sort(np.random.default_rng(33).choice(x.shape[0], 256, replace=False))
+    # grad_x needs only the sampled query rows against every key
+    c = oracle.sqeuclid_cost(x[rows], y)
+    lg = (gp[None, :] - c) / eps + np.log(b.astype(np.float64))[None, :]
+    w = np.exp(lg - lg.max(axis=1, keepdims=True))
+    w /= w.sum(axis=1, keepdims=True)
+    gx_rows = 2.0 * a[rows, None].astype(np.float64) * (x[rows].astype(np.float64)
+                                                       - w @ y.astype(np.float64))
+    np.savez_compressed(os.path.join(HERE, "oracle_config3.npz"), loss=np.array(loss), f=f, g=g,
+                        f_prelast=fp, g_prelast=gp, rows=rows, grad_x_rows=gx_rows)
+    print("config3 loss", loss)
+
+
 def make_config4():
     x, y, a, b = config4_inputs()
     out = {}
@@ -124,5 +153,5 @@ def make_config5():
 if __name__ == "__main__":
     todo = sys.argv[1:] or ["config1", "config2", "config4", "config5"]
     for name in todo:
-        {"config1": make_config1, "config2": make_config2, "config4": make_config4,
-         "config5": make_config5}[name]()
+        {"config1": make_config1, "config2": make_config2, "config3": make_config3,
+         "config4": make_config4, "config5": make_config5}[name]()

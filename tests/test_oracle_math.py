@@ -119,6 +119,115 @@ def test_unbalanced_limits_and_fixed_point():
     np.testing.assert_allclose(fq, want, rtol=1e-10)
 
 
+def _primal_kkt_residual(x, y, a, b, f, g, eps, rho_x, rho_y):
+    """Stationarity of  <C,P> + eps KL(P | a b^T) + rho_x KL(P 1 | a) + rho_y KL(P^T 1 | b)  in P at
+    P = a b^T exp((f + g - C)/eps), written from the primal problem (no dual update formula):
+    C_ij + eps log(P_ij / a_i b_j) + rho_x log((P 1)_i / a_i) + rho_y log((P^T 1)_j / b_j) = 0;
+    a balanced side (rho None) is the hard constraint P 1 = a with f_i its free multiplier."""
+    a = a.astype(np.float64); b = b.astype(np.float64)
+    C = np.empty((len(a), len(b)))
+    for i in range(len(a)):
+        for j in range(len(b)):
+            C[i, j] = float(((x[i].astype(np.float64) - y[j].astype(np.float64)) ** 2).sum())
+    P = a[:, None] * b[None, :] * np.exp((f[:, None] + g[None, :] - C) / eps)
+    r, c = P.sum(1), P.sum(0)
+    res = C + eps * np.log(P / (a[:, None] * b[None, :]))
+    feas = 0.0
+    if rho_x is None:
+        res = res - f[:, None]
+        feas = max(feas, np.abs(r / a - 1).max())
+    else:
+        res = res + rho_x * np.log(r / a)[:, None]
+    if rho_y is None:
+        res = res - g[None, :]
+        feas = max(feas, np.abs(c / b - 1).max())
+    else:
+        res = res + rho_y * np.log(c / b)[None, :]
+    return np.abs(res).max(), feas, r, c
+
+
+@pytest.mark.parametrize("rho_x,rho_y", [(2.0, 0.7), (0.7, 2.0), (1.5, None), (None, 0.9)])
+def test_unbalanced_symmetric_fixed_point_solves_the_primal_problem(rho_x, rho_y):
+    """Pins the unbalanced / semi-unbalanced symmetric solver: at its fixed point the plan is
+    stationary for the primal unbalanced problem with THESE rho_x, rho_y (a swapped rho, a
+    wrong damping or a damping applied to the wrong side leaves a residual of order rho_x - rho_y),
+    and the marginals obey P 1 = a exp(-f/rho_x), P^T 1 = b exp(-g/rho_y)."""
+    x, y, a, b = inputs(31, 11, 9, 3)
+    eps = 0.3
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, rho_x=rho_x, rho_y=rho_y,
+                                     use_epsilon_scaling=False, eps=eps, n_iters=3000,
+                                     last_extrapolation=False)
+    res, feas, r, c = _primal_kkt_residual(x, y, a, b, f, g, eps, rho_x, rho_y)
+    assert res < 1e-9 and feas < 1e-9
+    if rho_x is not None:
+        np.testing.assert_allclose(r, a * np.exp(-f / rho_x), rtol=1e-9)
+    if rho_y is not None:
+        np.testing.assert_allclose(c, b * np.exp(-g / rho_y), rtol=1e-9)
+    # the check has teeth: the potentials of the problem with the two rho swapped fail it
+    if rho_x != rho_y:
+        fs_, gs_ = oracle.sinkhorn_symmetric(x, y, a, b, rho_x=rho_y, rho_y=rho_x,
+                                             use_epsilon_scaling=False, eps=eps, n_iters=3000,
+                                             last_extrapolation=False)
+        bad, bad_feas, _, _ = _primal_kkt_residual(x, y, a, b, fs_, gs_, eps, rho_x, rho_y)
+        assert max(bad, bad_feas) > 1e-3
+    # the extrapolation step leaves a fixed point where it is
+    f2, g2 = oracle.sinkhorn_symmetric(x, y, a, b, rho_x=rho_x, rho_y=rho_y,
+                                       use_epsilon_scaling=False, eps=eps, n_iters=3000)
+    np.testing.assert_allclose(f2, f, atol=1e-9)
+    np.testing.assert_allclose(g2, g, atol=1e-9)
+
+
+def test_unbalanced_symmetric_cost_is_the_primal_objective():
+    """sinkhorn_cost with both marginals relaxed (FS/_autograd.py:436-455, GeomLoss's formula
+    (rho+eps/2) <a, 1-exp(-f/rho)> per side) against the primal unbalanced objective evaluated
+    at the fixed-point plan, through strong duality written out from the problem itself."""
+    x, y, a, b = inputs(32, 10, 12, 2)
+    eps, rx, ry = 0.4, 1.7, 0.6
+    f, g = oracle.sinkhorn_symmetric(x, y, a, b, rho_x=rx, rho_y=ry, use_epsilon_scaling=False,
+                                     eps=eps, n_iters=3000, last_extrapolation=False)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    C = oracle.sqeuclid_cost(x, y)
+    ab = a64[:, None] * b64[None, :]
+    P = ab * np.exp((f[:, None] + g[None, :] - C) / eps)
+
+    def kl(p, q):  # generalised KL between positive measures
+        return float((p * np.log(p / q) - p + q).sum())
+
+    primal = float((P * C).sum()) + eps * kl(P, ab) + rx * kl(P.sum(1), a64) + ry * kl(P.sum(0), b64)
+    dual = (rx * (a64 * (1 - np.exp(-f / rx))).sum() + ry * (b64 * (1 - np.exp(-g / ry))).sum()
+            - eps * (P.sum() - ab.sum()))
+    assert primal == pytest.approx(dual, rel=1e-9)  # strong duality at the fixed point
+    # the reference's cost formula is that dual value with eps*(m(a)m(b) - m(P)) rewritten through
+    # the marginal conditions: m(P) = <a, e^{-f/rho_x}> = <b, e^{-g/rho_y}>, half to each side
+    # (exact for unit masses, which `inputs` produces)
+    got = oracle.sinkhorn_cost(a, b, f, g, eps, rx, ry)
+    assert got == pytest.approx(dual, rel=1e-6)
+
+
+def test_unbalanced_alternating_one_step_as_written_with_two_rhos():
+    """The reference's alternating loop damps the whole shifted value and applies no shift
+    correction (FS/sinkhorn_solvers.py:240-259; damp_f from rho_x, damp_g from rho_y, :135-136):
+    f1 = damp_f softmin(g0) + (1-damp_f) |x|^2 with g0 = 0, then g1 from the NEW f1.  Written out
+    with python loops for rho_x != rho_y, so that a swapped pair or a Jacobi-style g1 fails."""
+    x, y, a, b = inputs(33, 6, 5, 2)
+    eps, rx, ry = 0.3, 2.0, 0.5
+    f1, g1 = oracle.sinkhorn_alternating(x, y, a, b, eps=eps, n_iters=1, rho_x=rx, rho_y=ry)
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    df, dg = 1 / (1 + eps / rx), 1 / (1 + eps / ry)
+
+    def smin(p, q, pot, w, i):
+        t = [(pot[j] - float(((p[i] - q[j]) ** 2).sum())) / eps + math.log(w[j]) for j in range(len(q))]
+        mx = max(t)
+        return -eps * (mx + math.log(sum(math.exp(v - mx) for v in t)))
+
+    want_f = np.array([df * smin(x64, y64, np.zeros(5), b, i) + (1 - df) * float((x64[i] ** 2).sum())
+                       for i in range(6)])
+    want_g = np.array([dg * smin(y64, x64, want_f, a, j) + (1 - dg) * float((y64[j] ** 2).sum())
+                       for j in range(5)])
+    np.testing.assert_allclose(f1, want_f, rtol=1e-10)
+    np.testing.assert_allclose(g1, want_g, rtol=1e-10)
+
+
 def test_early_stop_bookkeeping():
     x, y, a, b = inputs(25, 20, 20, 2)
     # first check only snapshots => earliest stop after 2*check_every averaged steps
