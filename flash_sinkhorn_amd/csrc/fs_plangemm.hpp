@@ -38,7 +38,10 @@ namespace fs {
 
 constexpr int kPgKeys = 256;          // keys per tile
 constexpr int kPgRows = 32;           // query rows per workgroup
-constexpr float kPgLazyThresh = 8.0f; // probabilities stay below 2^8: safe in fp16
+constexpr float kPgLazyThresh = 8.0f; // exponentials stay below 2^8 relative to the running maximum
+// exponentials are taken 2^7 up before the fp16 split and the reported maximum 7 down, as in
+// plan_tile_kernel: a probability keeps a nonzero fp16 image down to 2^-31 of the row's largest
+constexpr float kPgUp = 7.0f;
 
 // Largest |rowscale[r] * src[r, c]| (rowscale may be null): one partial maximum per block.
 __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ src,
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
 
   const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = 1.0f / lscale;
-  // MAT5: per-row power of two with |T_ij| * t_unit <= 2^7 from |T_ij| <= |A_i| max_j |y_j|
+  // MAT5: per-row power of two with |T_ij| * t_unit <= 1 from |T_ij| <= |A_i| max_j |y_j|
   // (in plane units; sd.q2norm2 = |A_i|^2, sd.kmax2 = 64 partial maxima of |y_j|^2, fp32 rows)
   float t_unit = 1.0f;
   if constexpr (MAT5) {
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     for (int o = 32; o > 0; o >>= 1) km = fmaxf(km, __shfl_xor(km, o, 64));
     const float bound = sqrtf(a2 * km) * sd.q2plane_scale[0] * sd.kplane_scale[0] * 1.0001f;
     const int e = (int)((__builtin_bit_cast(unsigned, bound) >> 23) & 255u);  // bound < 2^(e-126)
-    if (e > 0 && e < 255) t_unit = __builtin_bit_cast(float, (unsigned)min(254, max(1, 127 + 7 - (e - 126))) << 23);
+    if (e > 0 && e < 255) t_unit = __builtin_bit_cast(float, (unsigned)min(254, max(1, 127 - (e - 126))) << 23);
   }
 
   // ---- loaders: wavefront w brings key rows [32 w, 32 w + 32) of the tile (4 instructions of
@@ -395,9 +398,10 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     }
     float p[16];
     float ps = 0.f;
+    const float ccu = cc + kPgUp;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, cc));
+      p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, ccu));
       ps += p[r];
     }
     run_s += ps;
@@ -466,7 +470,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   float s = 0.f;
 #pragma unroll
   for (int w = 0; w < 8; ++w) s += lds_x[w][li];
-  const float M = (ntiles > 0) ? run_m * lscale : kNegBig;
+  const float M = (ntiles > 0) ? run_m * lscale - kPgUp : kNegBig;
   float inv_vs = 1.0f / sd.vplane_scale[0];
   if constexpr (MAT5) inv_vs /= t_unit * sd.q2plane_scale[0] * sd.kplane_scale[0];
   const bool live = row < sd.nq;

@@ -31,7 +31,12 @@
 
 namespace fs {
 
-constexpr float kPtLazyThresh = 8.0f;  // probabilities stay below 2^8
+constexpr float kPtLazyThresh = 8.0f;  // exponentials stay below 2^8 relative to the running maximum
+// The exponentials are taken 2^7 up before they are cut into fp16 planes (values up to 2^15), and
+// the maximum a row reports is lowered by the same 7: the pair (maximum, sums) means the same
+// thing, while a probability keeps a nonzero fp16 image down to 2^-31 of the row's largest one
+// instead of 2^-24 (a tail of many far keys would otherwise be rounded away one-sidedly).
+constexpr float kPtUp = 7.0f;
 
 template <int DP, int RB, int MODE>
 __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void plan_tile_kernel(const LaunchArgs args) {
@@ -100,7 +105,7 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
 #pragma unroll
       for (int kk = 0; kk < KK16; ++kk)
         aq[0][p][kk] = *reinterpret_cast<const u32x4*>(arow + p * (DP / 2) + 8 * kk + 4 * h);
-    // per-row power of two with |T_ij| * t_unit <= 2^7 from |T_ij| <= |A_i| max_j |y_j|
+    // per-row power of two with |T_ij| * t_unit <= 1 from |T_ij| <= |A_i| max_j |y_j|
     float km = sd.kmax2[lane];  // 64 partial maxima of |y_j|^2
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) km = fmaxf(km, __shfl_xor(km, o, 64));
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
         sqrtf(sd.q2norm2[row] * km) * sd.q2plane_scale[0] * sd.kplane_scale[0] * 1.0001f;
     const int e = (int)((__builtin_bit_cast(unsigned, bound) >> 23) & 255u);  // bound < 2^(e-126)
     if (e > 0 && e < 255)
-      t_unit = __builtin_bit_cast(float, (unsigned)min(254, max(1, 127 + 7 - (e - 126))) << 23);
+      t_unit = __builtin_bit_cast(float, (unsigned)min(254, max(1, 127 - (e - 126))) << 23);
   }
 
   // ---- key tiles: lane idx of instruction c fills LDS slot idx and fetches the piece that
@@ -360,9 +365,10 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
         }
         float p[16];
         float ps = 0.f;
+        const float ccu = cc + kPtUp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, cc));
+          p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, ccu));
           ps += p[r];
         }
         run_s[rb] += ps;
@@ -444,7 +450,7 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
       }
       continue;
     }
-    const float M = (ntiles > 0) ? run_m[rb] * lscale : kNegBig;
+    const float M = (ntiles > 0) ? run_m[rb] * lscale - kPtUp : kNegBig;
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float o = run_o[rb] + xor32(run_o[rb]);
     if (sd.splits == 1) {

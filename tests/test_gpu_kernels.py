@@ -296,3 +296,41 @@ def test_large_d_products_are_scale_robust(scale):
     want = oracle.mat5(x, y, f5, gh, A, eps, 0.5)
     got = mat5_sqeuclid(*dev(x, y, f5, gh, A), eps=eps, cost_scale=0.5)
     assert rel_err(got, want) < RTOL
+
+
+@pytest.mark.parametrize("m,d", [(40_000, 64), (36_000, 160)])
+def test_far_tail_of_the_plan_survives_the_fp16_probability_split(m, d):
+    """One dominant key and a bulk of m - 1 keys at 2^-26 of its weight each (6e-4 of the row
+    mass together, sitting somewhere else): the products that cut the probabilities into fp16
+    planes (gradient, plan-matrix; d <= 128 and the large-d kernel) must keep that tail.  The
+    dominant key comes first, so it is the running maximum from the first tile on and the tail
+    sits 26 binades below the largest probability of its row."""
+    from flash_sinkhorn_amd.kernels.apply_flash import apply_plan_mat_flashstyle
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    rng = np.random.default_rng(11)
+    n, eps = 96, 1.0
+    x = (0.01 * rng.standard_normal((n, d))).astype(np.float32)
+    y = (0.01 * rng.standard_normal((m, d))).astype(np.float32)
+    y[1:] += np.float32(1.0 / np.sqrt(d))
+    y[0] -= np.float32(1.0 / np.sqrt(d))
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    g = np.full(m, -26.0 * np.log(2.0) * eps, np.float32)
+    g[0] = 0.0
+    g += ((y.astype(np.float64) ** 2).sum(1) - (y[0].astype(np.float64) ** 2).sum()).astype(np.float32)
+    f = np.zeros(n, np.float32)
+    wx, _ = oracle.grad_barycentric(x, y, a, b, f, g, eps)
+    # the tail carries a visible share of the answer: without it the result is off by > 3e-4
+    w0, _ = oracle.grad_barycentric(x, y[:1], a, b[:1], f, g[:1], eps)
+    assert np.abs(w0 - wx).max() / np.abs(wx).max() > 3e-4
+    X, Y, A, B, F, G = dev(x, y, a, b, f, g)
+    gx, _ = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False, compute_grad_y=False)
+    assert rel_err(gx, wx) < RTOL
+    # plan-matrix product with the same plan: P V, V = key rows
+    la, lb = np.log(a), np.log(b)
+    f_hat = (f - (x.astype(np.float64) ** 2).sum(1)).astype(np.float32)
+    g_hat = (g - (y.astype(np.float64) ** 2).sum(1)).astype(np.float32)
+    want = oracle.apply_plan_mat(x, y, f_hat, g_hat, la, lb, y, eps, axis=1)
+    got = apply_plan_mat_flashstyle(X, Y, *dev(f_hat, g_hat, la, lb), Y, eps=eps, axis=1)
+    assert rel_err(got, want) < RTOL
