@@ -5,24 +5,27 @@ eps=0.01, n_iters=100, last_extrapolation=True, allow_tf32=False)`` = 102 double
 log-sum-exp launches, on a seeded 8-component Gaussian mixture per cloud with
 uniform weights, inputs already resident in HBM.  Prints ONE JSON line.
 
-Operand modes of the log-sum-exp kernel (results are fp32 in all of them):
-  strict (default, allow_tf32=False)  two fp16 planes per operand (22 significand bits) of the
-                                      power-of-two scaled matrix, three MFMA products, fp32
-                                      accumulate: error <= that of fp32 MFMA operands
-  bf16x3 (--mode bf16x3)              three bf16 planes, six products: same accuracy class
-  fp32_mfma (--mode fp32_mfma)        fp32 operands on v_mfma_f32_32x32x2_f32
-  reduced (--mode reduced)            two bf16 planes, three products (allow_tf32=True)
+Operand modes (results are fp32 in both):
+  strict (default)          two fp16 planes per operand (22 significand bits) of the power-of-two
+                            scaled matrix, three MFMA products, fp32 accumulate: error <= that
+                            of fp32 MFMA operands; allow_tf32=True runs the same kernels
+  fp32_mfma (--mode ...)    fp32 operands on v_mfma_f32_32x32x2_f32
 
-roofline: one symmetric-step launch does 4*n*m*d algorithmic matrix flop (both
-half-updates) plus 2*n*m exp2; its duration is measured here with HIP events on the
-launch stream.  The split modes execute 3 (fp16x2, reduced) or 6 (bf16x3) 16-bit MFMA
-products per algorithmic product, so the algorithmic rate is priced against the published
-2516.6 TFLOP/s fp16/bf16 peak divided by that factor (838.9 or 419.4 TFLOP/s; 157.3 for fp32
-MFMA operands); the ratio to the fp32 MFMA peak and the serial / overlapped MFMA+exp roofline
-times of the whole 102-step solve are reported next to it.
-The solver groups rows by k-means cluster and picks, by timing a few steps, between the plain
-kernel and the one that tests a tile after its hi*hi plane product; the roofline launch is
-timed on the same row order and variant (reported under roofline.tile_skip).
+roofline (dominant kernel: lse2_kernel, one launch = both half-updates of a symmetric step, with
+its small merge kernel): the launch is timed with HIP events on the launch stream, on the
+operand planes, row order and kernel variant the solve used.
+  algorithmic work of a launch   4*n*m*d matrix flop (2*n*m*d per half-update) + 2*n*m exp2
+  executed work                  the fp16 two-plane mode runs three 16-bit MFMA products per
+                                 algorithmic product; the variant with the coarse tile test ends
+                                 a 32x32 tile after its hi*hi product (1 of 3) when no logit of
+                                 it can matter, and counts such tiles on the device
+  roofline.achieved              EXECUTED 16-bit MFMA flop / launch time, against the published
+                                 dense fp16 peak (2516.6 TFLOP/s); roofline.frac = their ratio.
+                                 roofline.algorithmic_tflops = 4*n*m*d / launch time is what a
+                                 user gets (it counts flop the coarse test never ran).
+The solver groups rows by k-means cluster and lets the device decide, from the share of tiles that
+end at the coarse test in the first steps, which kernel variant runs; value_data_independent_ms
+is the same solve with that switched off (caller's row order, plain kernel on every tile).
 cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores on a
 bounded sample and scaled to the metric's unit.
 """
@@ -39,15 +42,14 @@ if ROOT not in sys.path:
 N, M, D = 50_000, 50_000, 64
 EPS = 0.01
 ITERS = 100
-MODES = ["strict", "bf16x3", "fp32_mfma", "reduced"]
+MODES = ["strict", "fp32_mfma"]
 FP32_MFMA_PEAK_TFLOPS = 157.3
-BF16_MFMA_PEAK_TFLOPS = 2516.6
+F16_MFMA_PEAK_TFLOPS = 2516.6
 EXP2_PER_S = 18.6e12  # v_exp_f32 lanes per second measured on the box (half rate)
-# Memory-side bytes per lse2_kernel launch of the default workload, per operand mode, from two
-# rocprofv3 --pmc runs (FETCH_SIZE 113,782 KiB x 2.0, WRITE_SIZE 12,510 KiB x 1.0 for the kernel
-# variant with the coarse tile test, 112,309 / 12,509 for the plain one; the factors
-# are what the same counters read for the 256 MiB copy of --copy-calibration: half the bytes
-# copied and all of them).  Not measured for the other modes.
+# Memory-side bytes per lse2_kernel launch of the default workload (rows in cluster order, coarse
+# tile test), from two rocprofv3 --pmc runs: FETCH_SIZE 113,782 KiB x 2.0 and WRITE_SIZE
+# 12,510 KiB x 1.0; the factors are what the same counters read for the 256 MiB device copy of
+# --copy-calibration (half the bytes copied, and all of them).
 MEASURED_TRAFFIC_BYTES = {"strict": int((113782 * 2.0 + 12510) * 1024)}
 
 
@@ -68,6 +70,17 @@ def make_inputs(n, m, d, seed=3):
     a = np.full(n, 1.0 / n, np.float32)
     b = np.full(m, 1.0 / m, np.float32)
     return x, y, a, b
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def cpu_baseline(x, y, a, b, budget_s=20.0):
@@ -96,7 +109,7 @@ def cpu_baseline(x, y, a, b, budget_s=20.0):
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
     return {
         "value": ms_per_100, "unit": "ms per 100 symmetric iterations", "cores": cores,
-        "kind": "port",
+        "cpu_model": cpu_model(), "kind": "port",
         "sample": f"{done} of {n} query rows of each half-update against all {m} keys "
                   f"({el:.1f} s of the numpy fp32 oracle, BLAS threads = host default), scaled "
                   "to 102 steps",
@@ -113,8 +126,9 @@ def main():
     ap.add_argument("--d", type=int, default=D)
     ap.add_argument("--mode", choices=MODES, default="strict")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-other-modes", action="store_true",
-                    help="skip the one-launch timings of the other operand modes")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the comparison timings (other operand mode, data-independent "
+                         "solve, every-exponential launch, 101-step solve)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device copy: under rocprofv3 --pmc its "
                          "FETCH_SIZE / WRITE_SIZE give the counters' scale factors")
@@ -130,7 +144,7 @@ def main():
     from flash_sinkhorn_amd import sinkhorn_solvers as solvers
     from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric
     from flash_sinkhorn_amd.kernels._common import log_weights
-    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_steps_raw
 
     n, m, d = args.n, args.m, args.d
     x, y, a, b = make_inputs(n, m, d)
@@ -138,123 +152,168 @@ def main():
     X, Y, A, B = (torch.from_numpy(t).to(dev) for t in (x, y, a, b))
 
     def set_mode(mode):
-        _lib.STRICT_OPERANDS = {"fp32_mfma": "fp32_mfma", "bf16x3": "bf16x3"}.get(mode, "fp16x2")
-        return mode == "reduced"  # allow_tf32
+        _lib.STRICT_OPERANDS = "fp32_mfma" if mode == "fp32_mfma" else "fp16x2"
 
-    def solve(mode):
-        tf32 = set_mode(mode)
-        return sinkhorn_flashstyle_symmetric(
-            X, Y, A, B, use_epsilon_scaling=False, eps=EPS, n_iters=ITERS,
-            last_extrapolation=True, allow_tf32=tf32)
+    def solve(mode, info=None, **kw):
+        set_mode(mode)
+        opts = dict(use_epsilon_scaling=False, eps=EPS, n_iters=ITERS, last_extrapolation=True,
+                    allow_tf32=False, solve_info=info)
+        opts.update(kw)
+        return sinkhorn_flashstyle_symmetric(X, Y, A, B, **opts)
 
+    def timed_solves(reps, warm, **kw):
+        for _ in range(warm):
+            solve(args.mode, **kw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            out = solve(args.mode, **kw)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / reps, out
+
+    solve_info = {}
     for _ in range(args.warmup):
         solve(args.mode)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        f, g = solve(args.mode)
+        f, g = solve(args.mode, solve_info)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    chosen = solve_info["prepared"].variant_state() if solve_info["coarse"] == "auto" else None
+    coarse_ran = (solve_info["coarse"] is True
+                  or (chosen is not None and not chosen["plain_selected"]))
 
-    # dominant kernel: one symmetric-step launch, timed with events on the launch stream
+    # dominant kernel: symmetric-step launches on prepared operand planes, in the row order and
+    # with the kernel variant of the solve, timed with events on the launch stream
     alpha = (X * X).sum(1).contiguous()
     beta = (Y * Y).sum(1).contiguous()
     la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
     fh, gh = (f - alpha).contiguous(), (g - beta).contiguous()
-
-    # the launch as the solve runs it: rows in the solver's cluster order and the kernel variant
-    # it chose (main mode only; the other modes have neither)
-    solve_info = dict(solvers.LAST_SOLVE)
-    ordered = None
+    plain_ops = (X, Y, fh, gh, la, lb)
+    ordered_ops = plain_ops
     if solve_info["cluster_order"]:
         px, py = solvers._cluster_order(X), solvers._cluster_order(Y)
-        ordered = (X[px].contiguous(), Y[py].contiguous(), fh[px].contiguous(),
-                   gh[py].contiguous(), la[px].contiguous(), lb[py].contiguous())
+        ordered_ops = (X[px].contiguous(), Y[py].contiguous(), fh[px].contiguous(),
+                       gh[py].contiguous(), la[px].contiguous(), lb[py].contiguous())
 
-    def launch_ms(mode, reps=20, as_solved=False, coarse=False):
-        tf32 = set_mode(mode)
-        kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=tf32)
-        ops = (X, Y, fh, gh, la, lb)
-        if as_solved and ordered is not None:
-            ops = ordered
-            kw["coarse"] = coarse
-        _symmetric_step_raw(*ops, EPS, **kw)
+    def launch_ms(mode, ops, coarse=False, reps=20):
+        """(ms per launch, device counters of the coarse variant over the timed launches)"""
+        set_mode(mode)
+        prep = _lib.PreparedOperands(ops[0], ops[1], _lib.flags(True, False))
+        kw = dict(cost_scale=1.0, allow_tf32=False, prepared=prep, coarse=coarse)
+        steps = [(EPS, 0.5, 1.0, 1.0)] * reps
+        _symmetric_steps_raw(*ops, steps[:4], **kw)  # also the launches that take the decision
         torch.cuda.synchronize()
+        before = prep.variant_state()
+        stream = torch.cuda.current_stream(dev)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            _symmetric_step_raw(*ops, EPS, **kw)
-        e1.record()
+        e0.record(stream)
+        _symmetric_steps_raw(*ops, steps, **kw)
+        e1.record(stream)
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps
+        after = prep.variant_state()
+        counts = {k: (after[k] - before[k]) / reps for k in ("tiles_ended", "tiles_tested")}
+        counts["plain_selected"] = after["plain_selected"]
+        return e0.elapsed_time(e1) / reps, counts
 
     flop = 4.0 * n * m * d
-    products = {"strict": 3, "bf16x3": 6, "reduced": 3, "fp32_mfma": 0}
-    dtypes = {"strict": "fp16x2-planes/fp32-accumulate (fp32-grade)",
-              "bf16x3": "bf16x3-planes/fp32-accumulate (fp32-grade)", "fp32_mfma": "f32",
-              "reduced": "bf16x2-planes/fp32-accumulate"}
+    dp = 16 if d <= 16 else (32 if d <= 32 else (64 if d <= 64 else 128))
+    tiles_all = 2.0 * -(-n // 32) * -(-m // 32)  # 32 x 32 logits tiles of a launch, both sides
+    flop_per_tile_product = 2.0 * 32 * 32 * dp   # one plane product of one tile
 
-    def roofline_for(mode, ms):
-        achieved = flop / (ms * 1e-3) / 1e12
-        peak = BF16_MFMA_PEAK_TFLOPS / products[mode] if products[mode] else FP32_MFMA_PEAK_TFLOPS
-        r = {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-             "frac": achieved / peak,
-             "traffic": MEASURED_TRAFFIC_BYTES.get(mode) if (n, m, d) == (N, M, D) else None,
-             "kernel": "one symmetric step (both half-updates) = absmax + split_planes + "
-                       "lse2_kernel + finish_kernel; 4*n*m*d algorithmic flop",
-             "launch_ms": ms, "exp_per_s": 2.0 * n * m / (ms * 1e-3),
-             "frac_of_fp32_mfma_peak": achieved / FP32_MFMA_PEAK_TFLOPS}
-        if products[mode]:
-            r["peak_note"] = (f"published 16-bit MFMA peak {BF16_MFMA_PEAK_TFLOPS} TFLOP/s / "
-                              f"{products[mode]} products per fp32-grade product")
-        # MFMA + exp roofline of the whole solve (102 steps), exp2 at the measured 18.6e12 /s
-        t_mfma = (ITERS + 2) * flop / (peak * 1e12) * 1e3
-        t_exp = (ITERS + 2) * 2.0 * n * m / EXP2_PER_S * 1e3
-        r["mfma_exp_roofline_ms"] = {"mfma": t_mfma, "exp": t_exp, "serial": t_mfma + t_exp,
-                                     "overlapped": max(t_mfma, t_exp)}
+    def roofline_for(mode, ms, counts):
+        r = {"bound": "mfma", "unit": "TFLOP/s",
+             "kernel": "lse2_kernel (+ its merge kernel): one launch = both half-updates of a "
+                       "symmetric step on prepared operand planes; algorithmic work 4*n*m*d flop "
+                       "+ 2*n*m exp2",
+             "launch_ms": ms, "algorithmic_tflops": flop / (ms * 1e-3) / 1e12,
+             "exp_per_s": 2.0 * n * m / (ms * 1e-3)}
+        if mode == "fp32_mfma":
+            r.update(achieved=r["algorithmic_tflops"], peak=FP32_MFMA_PEAK_TFLOPS,
+                     peak_note="published dense fp32 MFMA peak; executed = algorithmic flop")
+        else:
+            # three plane products per tile; a tile that ends at the coarse test ran one, and a
+            # workgroup of that variant first runs the hi*hi product of one sampled tile per
+            # row block (as many tiles as it has first tiles, which the test does not see)
+            products = 3.0 * tiles_all
+            if counts is not None and counts["tiles_tested"] > 0 and not counts["plain_selected"]:
+                products += -2.0 * counts["tiles_ended"] + (tiles_all - counts["tiles_tested"])
+                r["coarse_test"] = {
+                    "share_of_tested_tiles_ended": counts["tiles_ended"] / counts["tiles_tested"],
+                    "mfma_products_per_tile": products / tiles_all}
+            executed = products * flop_per_tile_product
+            r.update(achieved=executed / (ms * 1e-3) / 1e12, peak=F16_MFMA_PEAK_TFLOPS,
+                     executed_flop_per_launch=executed,
+                     peak_note="published dense fp16 MFMA peak; achieved counts the 16-bit MFMA "
+                               "flop the launch executed (three plane products per algorithmic "
+                               "product, one for tiles that end at the coarse test, padding of "
+                               "d to the MFMA width included)")
+        r["frac"] = r["achieved"] / r["peak"]
+        r["traffic"] = MEASURED_TRAFFIC_BYTES.get(mode) if (n, m, d) == (N, M, D) else None
         return r
 
-    main_ms = launch_ms(args.mode, as_solved=True, coarse=solve_info["coarse_test"])
+    as_solved = "auto" if solve_info["coarse"] == "auto" else bool(solve_info["coarse"])
+    main_ms, main_counts = launch_ms(args.mode, ordered_ops, coarse=as_solved)
     line = {
         "metric": "ms per 100 symmetric Sinkhorn iterations (n=m=50k, d=64, fp32)",
         "value": ms_per_step, "unit": "ms", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": dtypes[args.mode],
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if args.mode == "fp32_mfma" else
+                 "fp16x2-planes/fp32-accumulate (fp32-grade)",
         "data": "synthetic",
         "config": {"workload": f"balanced symmetric FlashSinkhorn, n={n}, m={m}, d={d}, seeded "
                                "8-component Gaussian mixtures, uniform weights, eps=0.01, "
                                "100 iterations + init + extrapolation = 102 steps",
                    "operand_mode": args.mode,
+                   "rows_in_cluster_order": solve_info["cluster_order"],
+                   "kernel_variant": "coarse tile test" if coarse_ran else "plain",
+                   "variant_chosen_by": ("device counters" if solve_info["coarse"] == "auto"
+                                         else "caller"),
                    "loss": float((A * f).sum() + (B * g).sum())},
-        "roofline": roofline_for(args.mode, main_ms),
+        "roofline": roofline_for(args.mode, main_ms, main_counts),
     }
-    line["roofline"]["frac_of_serial_mfma_exp_roofline"] = (
-        line["roofline"]["mfma_exp_roofline_ms"]["serial"] / ms_per_step)
-    # The kernel leaves out the exponentials of 32x32 logits tiles that lie 2^40 below their
-    # rows' running maxima (exact in fp32; how many there are depends on the data: about 60 %
-    # on this workload).  The same launch with every exponential computed, for comparison:
-    _lib.TILE_SKIP = False
-    ms_noskip = launch_ms(args.mode, reps=10)
-    _lib.TILE_SKIP = True
-    line["roofline"]["tile_skip"] = {
-        "enabled": True, "launch_ms_with_every_exp": ms_noskip,
-        "rows_in_cluster_order": solve_info["cluster_order"],
-        "coarse_test": solve_info["coarse_test"],
-        "launch_ms_caller_order_no_coarse_test": launch_ms(args.mode, reps=10),
-        "note": "tiles whose logits all lie more than 2^40 below the running row maxima skip "
-                "their exp2 (no change to fp32 sums); with coarse_test such a tile is recognised "
-                "after its hi*hi plane product (bound on the cross products) and skips the other "
-                "8 of its 12 MFMAs too, so the executed MFMA flop are fewer than the algorithmic "
-                "flop `achieved` counts; launch_ms_with_every_exp computes everything"}
-    if not args.no_other_modes:
-        others = {}
-        for mode in MODES:
-            if mode != args.mode:
-                ms = launch_ms(mode, reps=10)
-                rf = roofline_for(mode, ms)
-                others[mode] = {"launch_ms": ms, "ms_per_100_iters_est": ms * (ITERS + 2),
-                                "achieved": rf["achieved"], "peak": rf["peak"], "frac": rf["frac"]}
-        line["other_operand_modes"] = others
+    rf = line["roofline"]
+    # MFMA + exp roofline of the whole solve for the work executed (exp2 at the measured rate)
+    t_mfma = (ITERS + 2) * rf["achieved"] * main_ms / rf["peak"]
+    t_exp = (ITERS + 2) * 2.0 * n * m / EXP2_PER_S * 1e3
+    rf["mfma_exp_roofline_ms"] = {"mfma": t_mfma, "exp_every_logit": t_exp,
+                                  "serial": t_mfma + t_exp, "overlapped": max(t_mfma, t_exp)}
+    rf["frac_of_serial_mfma_exp_roofline"] = (t_mfma + t_exp) / ms_per_step
+
+    if not args.no_extras:
+        solvers_order = solvers.CLUSTER_ORDER
+        # the data-independent figure: caller's row order, plain kernel on every tile
+        solvers.CLUSTER_ORDER = False
+        line["value_data_independent_ms"], _ = timed_solves(max(2, args.steps // 2), 1)
+        solvers.CLUSTER_ORDER = solvers_order
+        # the 101-step variant (no extrapolation step) that the reference's README times
+        line["value_without_last_extrapolation_ms"], _ = timed_solves(
+            max(2, args.steps // 2), 1, last_extrapolation=False)
+        plain_ms, _ = launch_ms(args.mode, plain_ops)
+        _lib.TILE_SKIP = False
+        every_exp_ms, _ = launch_ms(args.mode, plain_ops, reps=10)
+        _lib.TILE_SKIP = True
+        rf["other_launches"] = {
+            "caller_order_plain_kernel": {
+                "launch_ms": plain_ms, **{k: v for k, v in roofline_for(
+                    args.mode, plain_ms, None).items() if k in ("achieved", "frac",
+                                                                "algorithmic_tflops")}},
+            "caller_order_plain_kernel_every_exp": {
+                "launch_ms": every_exp_ms, **{k: v for k, v in roofline_for(
+                    args.mode, every_exp_ms, None).items() if k in ("achieved", "frac",
+                                                                    "algorithmic_tflops")}},
+            "note": "the plain kernel runs every MFMA and leaves out only the exp2 of tiles "
+                    "whose logits all lie 2^40 below their rows' running maxima (exact in "
+                    "fp32); every_exp computes those too"}
+        other = "fp32_mfma" if args.mode == "strict" else "strict"
+        o_ms, _ = launch_ms(other, plain_ops, reps=5)
+        orf = roofline_for(other, o_ms, None)
+        line["other_operand_mode"] = {"mode": other, "launch_ms": o_ms,
+                                      "ms_per_100_iters_est": o_ms * (ITERS + 2),
+                                      "achieved": orf["achieved"], "peak": orf["peak"],
+                                      "frac": orf["frac"]}
         set_mode(args.mode)
     if args.copy_calibration:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)

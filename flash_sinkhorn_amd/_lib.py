@@ -19,13 +19,14 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 FS_FLAG_EXP2 = 1
 FS_FLAG_REDUCED_OPERANDS = 2
 FS_FLAG_FP32_MFMA = 4
-FS_FLAG_BF16X3_OPERANDS = 8
 FS_FLAG_OPERANDS_PREPARED = 16
 FS_FLAG_NO_TILE_SKIP = 32
 FS_FLAG_COARSE_TEST = 64
-# allow_tf32=False normally runs the two-plane fp16 operands (fp32-grade accuracy).
-# STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" runs fp32 MFMA
-# operands, "bf16x3" the three-plane bf16 split instead.
+FS_FLAG_COARSE_AUTO = 128
+# Every call runs on the two-plane fp16 operands (fp32-grade accuracy, the fastest mode here),
+# whatever allow_tf32 says: permission to reduce precision is not an obligation.
+# STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" makes allow_tf32=False
+# mean fp32 operands on the fp32 MFMA instruction instead.
 STRICT_OPERANDS = os.environ.get("FLASH_SINKHORN_STRICT_OPERANDS", "fp16x2")
 OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5, OP_C_TRANSFORM = range(7)
 
@@ -46,6 +47,7 @@ _SIGNATURES = {
     "fs_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "fs_workspace_bytes": (_Z, [ctypes.c_int, _I, _I, _I]),
     "fs_prepare_operands": (ctypes.c_int, [_P] * 2 + [_I] * 3 + _TAIL),
+    "fs_variant_state_offset": (_Z, [_P] * 2 + [_I] * 3 + [_U]),
     "fs_lse": (ctypes.c_int, [_P] * 4 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_lse_fused": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_symmetric_step": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + _TAIL),
@@ -118,14 +120,14 @@ def flags(use_exp2: bool, allow_tf32: bool) -> int:
     f = FS_FLAG_EXP2 if use_exp2 else 0
     if not TILE_SKIP:
         f |= FS_FLAG_NO_TILE_SKIP
-    if allow_tf32:
-        return f | FS_FLAG_REDUCED_OPERANDS
     if STRICT_OPERANDS not in _STRICT_FLAGS:
         raise ValueError(f"STRICT_OPERANDS must be one of {sorted(_STRICT_FLAGS)}")
+    if allow_tf32:
+        return f | FS_FLAG_REDUCED_OPERANDS  # accepted by the library, same kernels as the default
     return f | _STRICT_FLAGS[STRICT_OPERANDS]
 
 
-_STRICT_FLAGS = {"fp16x2": 0, "fp32_mfma": FS_FLAG_FP32_MFMA, "bf16x3": FS_FLAG_BF16X3_OPERANDS}
+_STRICT_FLAGS = {"fp16x2": 0, "fp32_mfma": FS_FLAG_FP32_MFMA}
 
 
 class PreparedOperands:
@@ -150,14 +152,35 @@ class PreparedOperands:
         self.flag_bits = flag_bits
         self.keys = {(x.data_ptr(), n), (y.data_ptr(), m)}
         self.d = d
+        self.state_offset = int(L.fs_variant_state_offset(x.data_ptr(), y.data_ptr(), n, m, d,
+                                                          flag_bits))
         check(L.fs_prepare_operands(x.data_ptr(), y.data_ptr(), n, m, d, flag_bits,
                                     self.ws.data_ptr(), nbytes, stream_of(x)),
               "fs_prepare_operands")
 
+    def variant_state(self) -> dict:
+        """What ``FS_FLAG_COARSE_AUTO`` has done on these planes so far (reads the device: a
+        diagnostic, not part of any solve): which variant the steps now run, and how many
+        32 x 32 logits tiles of the coarse variant ended at its test."""
+        if self.state_offset == 0:
+            return {"plain_selected": True, "decisions": 0, "tiles_ended": 0, "tiles_tested": 0}
+        w = self.ws[self.state_offset:self.state_offset + 24].cpu().view(torch.int32).tolist()
+        u = [v & 0xFFFFFFFF for v in w]
+        return {"plain_selected": u[0] != 0, "decisions": u[1],
+                "tiles_ended": u[2] | (u[3] << 32), "tiles_tested": u[4] | (u[5] << 32)}
+
     def serves(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int) -> bool:
         # the workspace layout depends on the set of matrices, so the call must name the same set
-        return (flag_bits == self.flag_bits and x.shape[1] == self.d
+        same = ~FS_FLAG_REDUCED_OPERANDS  # the permission bit does not change the planes
+        return ((flag_bits & same) == (self.flag_bits & same) and x.shape[1] == self.d
                 and {(x.data_ptr(), x.shape[0]), (y.data_ptr(), y.shape[0])} == self.keys)
+
+
+def coarse_flag(coarse) -> int:
+    """Flag bits for the ``coarse`` argument of the step launchers: False, True or "auto"."""
+    if coarse == "auto":
+        return FS_FLAG_COARSE_AUTO
+    return FS_FLAG_COARSE_TEST if coarse else 0
 
 
 def lse_workspace(op: int, x: torch.Tensor, y: torch.Tensor, flag_bits: int,

@@ -2,7 +2,6 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-#include <cstdlib>
 #include <cmath>
 #include <cstring>
 
@@ -18,7 +17,9 @@ constexpr int kMaxStreamD = 128;    // register-stationary streaming kernels
 constexpr int kMaxSlicedD = 16384;  // widest supported rows
 constexpr int kSlicedSpan = 1536;   // columns one workgroup of the column-sliced kernels spans
 constexpr int kPlanePadRowsApi = 256;  // must match kPlanePadRows of the plane-splitting kernels
-constexpr size_t kPlaneAuxBytes = (2 * 256 + 4) * sizeof(float);  // absmax partials + plane scales
+// after the planes: absmax partials [2][256], plane scales [4] (+4 spare), variant-choice state
+constexpr size_t kPlaneAuxBytes = (2 * 256 + 8 + kSelWords) * sizeof(float);
+static_assert(kSelWords <= 256, "the state is cleared by one workgroup");
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
@@ -30,17 +31,8 @@ inline int padded_d(int64_t d) {
   return 128;
 }
 
-int env_int(const char* name, int dflt) {
-  const char* v = std::getenv(name);
-  return (v && *v) ? std::atoi(v) : dflt;
-}
-
-// Tunables (read once): blocks a launch should reach before key splitting stops.
-int target_blocks(bool has_o) {
-  static const int t_lse = env_int("FS_TARGET_BLOCKS", 2048);
-  static const int t_mat = env_int("FS_TARGET_BLOCKS_MAT", 1024);
-  return has_o ? t_mat : t_lse;
-}
+// Blocks a launch should reach before key splitting stops (8 and 4 per CU).
+int target_blocks(bool has_o) { return has_o ? 1024 : 2048; }
 
 struct SidePlan {
   int rb, igroups, splits, chunk;
@@ -151,46 +143,22 @@ int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
 // planes written once by fs_prepare_operands serve every later step on the same operands.
 struct LseConfig {
   bool gemm;    // lse_gemm_kernel (128 < d <= 1536, fp16 planes)
-  int prec;     // Prec of lse2_kernel: 0 fp32, 1 two bf16, 2 three bf16, 3 two fp16 planes
+  int prec;     // Prec of lse2_kernel: kF32 (0) fp32 operands, kH3 (3) two fp16 planes
   int dp;       // padded columns of a plane row
   int np;       // planes per operand
 };
 
-int strict_prec_default() {
-  static const int v = env_int("FS_STRICT_PREC", 3);  // 3: two fp16 planes, 2: three bf16 planes, 0: fp32 MFMA
-  return v;
-}
-int reduced_prec_default() {
-  static const int v = env_int("FS_REDUCED_PREC", 1);  // 1: two bf16 planes, 0: fp32 MFMA
-  return v;
-}
-
 // Words per row of the chunked fp16 planes: the 32-column chunks (128 bytes) of a row, plus
 // one spare chunk when their count is even.  An odd count of 128-byte units per row spreads
 // the rows of a stage (same chunk of 256 consecutive rows) over all memory channels.
-int chunked_stride(int64_t d) {
-  static const int odd = env_int("FS_ODD_STRIDE", 1);
-  const int nch = ceil_div(d, 32);
-  return (odd ? (nch | 1) : nch) * 32;
-}
+int chunked_stride(int64_t d) { return (ceil_div(d, 32) | 1) * 32; }
 
 LseConfig lse_config(int64_t d, uint32_t flags) {
-  static const int use_gemm = env_int("FS_LSEGEMM", 1);
   LseConfig c;
-  c.prec = (flags & FS_FLAG_REDUCED_OPERANDS) ? reduced_prec_default()
-           : ((flags & FS_FLAG_FP32_MFMA) ? 0
-              : ((flags & FS_FLAG_BF16X3_OPERANDS) ? 2 : strict_prec_default()));
-  const bool sliced = d > kMaxStreamD;
-  c.gemm = sliced && use_gemm && !(flags & (FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS));
-  if (c.gemm) {
-    c.prec = 3;
-    c.dp = chunked_stride(d);
-    c.np = 2;
-  } else {
-    c.dp = std::max(padded_d(d), 16);
-    c.np = (c.prec == 2) ? 3 : 2;
-    if (sliced) c.prec = 0;  // column-sliced fp32 kernels: no planes
-  }
+  c.prec = (flags & FS_FLAG_FP32_MFMA) ? 0 : 3;
+  c.gemm = d > kMaxStreamD && c.prec == 3;
+  c.dp = c.gemm ? chunked_stride(d) : std::max(padded_d(d), 16);
+  c.np = 2;
   return c;
 }
 
@@ -245,6 +213,10 @@ const float* plane_scales(const PlaneSet& ps, void* ws) {
   return reinterpret_cast<const float*>(static_cast<char*>(ws) + ps.aux_off) + 2 * 256;
 }
 
+unsigned* select_state(const PlaneSet& ps, void* ws) {
+  return reinterpret_cast<unsigned*>(static_cast<char*>(ws) + ps.aux_off) + 2 * 256 + 8;
+}
+
 const unsigned* plane_of(const PlaneSet& ps, void* ws, const float* src, int rows) {
   for (int i = 0; i < ps.n; ++i)
     if (ps.src[i] == src && ps.rows[i] == rows)
@@ -257,7 +229,7 @@ int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws
   if (ps.n == 0) return FS_OK;
   char* base = static_cast<char*>(ws);
   int rc = FS_OK;
-  if (c.prec == 3) {
+  {
     float* partial = reinterpret_cast<float*>(base + ps.aux_off);
     float* scales = partial + 2 * 256;
     const bool two = ps.n > 1;
@@ -266,11 +238,8 @@ int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws
     for (int i = 0; i < ps.n && rc == FS_OK; ++i)
       rc = launch_split_planes_f16(ps.src[i], reinterpret_cast<unsigned*>(base + ps.off[i]),
                                    ps.rows[i], (int)d, c.dp, partial + 256 * i, scales + i,
-                                   two ? nullptr : scales + 1, c.gemm ? 1 : 0, st);
-  } else {
-    for (int i = 0; i < ps.n && rc == FS_OK; ++i)
-      rc = launch_split_planes(ps.src[i], reinterpret_cast<unsigned*>(base + ps.off[i]),
-                               ps.rows[i], (int)d, c.dp, c.np, st);
+                                   two ? nullptr : scales + 1, c.gemm ? 1 : 0,
+                                   i == 0 ? select_state(ps, ws) : nullptr, st);
   }
   return rc;
 }
@@ -530,7 +499,7 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
       rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
-                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, st);
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, nullptr, st);
   }
   if (rc == FS_OK) rc = launch_plan_gemm(a, mat5, cb, total, st);
   if (rc != FS_OK) return rc;
@@ -583,10 +552,8 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   int rc = side_plane_set(sides, nsides, cfg, ps);
   if (rc != FS_OK) return rc;
   const int dpk = cfg.dp;  // 16, 32, 64 or 128
-  static const int rb_env = env_int("FS_PT_RB", 0);
   int rb = 2;
   for (int s = 0; s < nsides; ++s) rb = std::min(rb, pt_rows_per_wave(sides[s].nq));
-  if (rb_env > 0) rb = std::min(rb_env, 2);
   const bool mat5 = (mode == kMat5);
   const bool has_o = (mode == kMat || mat5);
   // one row block where two would spill: 128-column rows and mat5
@@ -670,7 +637,7 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     if (rc == FS_OK) rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
       rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
-                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, st);
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, nullptr, st);
   }
   for (int s = 0; s < nsides && rc == FS_OK && has_o; ++s) {
     const Side& sd = sides[s];
@@ -712,14 +679,14 @@ size_t pt_ws_bytes(int mode, int64_t n, int64_t m, int64_t d, bool both, bool ei
                    const Family& fam) {
   const int dpk = std::max(padded_d(d), 16);
   const size_t planes =
-      (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (dpk / 2) * 4 + 64 + kPlaneAuxBytes;
+      (size_t)(n + m + 2 * kPlanePadRowsApi) * 2 * (dpk / 2) * 4 + 64 + kPlaneAuxBytes;
   auto side = [&](int64_t nq, int64_t nk) {
     size_t b = 0;
     for (int rb = 1; rb <= 2; ++rb)
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dpk) * sizeof(float));
     if (mode == kMat || mode == kMat5) b += pt_vt_bytes(nk, dpk) + kPgAuxBytes;
-    if (mode == kMat5)  // planes of the second operand (sized for three planes), aux, row bounds
-      b += (size_t)(nq + kPlanePadRowsApi) * 3 * (dpk / 2) * 4 + kPlaneAuxBytes + ((size_t)nq + 64) * 4 + 64;
+    if (mode == kMat5)  // planes of the second operand, aux, row bounds
+      b += (size_t)(nq + kPlanePadRowsApi) * 2 * (dpk / 2) * 4 + kPlaneAuxBytes + ((size_t)nq + 64) * 4 + 64;
     return b + 16;
   };
   if (both) return planes + side(n, m) + side(m, n) + 64;
@@ -739,24 +706,12 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if ((mode == kLse || mode == kVec || mode == kArgmax) && cfg.gemm)
     return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
   if (mode == kArgmax && fam.sliced) return FS_ERR_UNSUPPORTED;  // d > 128 runs on fp16 planes only
-  static const int use_plan_gemm = env_int("FS_PLANGEMM", 1);
-  if ((mode == kMat || mode == kMat5) && cfg.gemm && use_plan_gemm)
+  if ((mode == kMat || mode == kMat5) && cfg.gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
-  static const int use_plan_tile = env_int("FS_PLANTILE", 1);
-  static const int mat5_128 = env_int("FS_MAT5_128", 1);
   // the plan-vector product at <= 64 columns rides on the pipelined log-sum-exp kernel
-  static const int vec_on_lse2 = env_int("FS_VEC_LSE2", 1);
-  const bool vec_lse2 = mode == kVec && vec_on_lse2 && cfg.prec == 3 && cfg.dp <= 64 && !fam.sliced;
-  const bool tile_mode = mode == kMat || (mode == kVec && !vec_lse2) || mode == kArgmax ||
-                         (mode == kMat5 && (cfg.dp <= 64 || mat5_128));
-  if (tile_mode && !fam.sliced && use_plan_tile && (cfg.prec == 3 || cfg.prec == 1)) {
-    // the reduced mode runs on the fp16 planes too (same speed, smaller error); planes a caller
-    // prepared for it are bf16 and are not used here
-    const bool reduced = (cfg.prec == 1);
-    const LseConfig pcfg = reduced ? lse_config(d, flags & ~(uint32_t)FS_FLAG_REDUCED_OPERANDS) : cfg;
-    if (pcfg.prec == 3)
-      return run_plan_tile(mode, sides, nsides, d, pcfg, fam, prepared && !reduced, ws, ws_bytes, st);
-  }
+  const bool vec_lse2 = mode == kVec && cfg.prec == 3 && cfg.dp <= 64 && !fam.sliced;
+  if (mode != kLse && !vec_lse2 && !fam.sliced && cfg.prec == 3)
+    return run_plan_tile(mode, sides, nsides, d, cfg, fam, prepared, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
@@ -768,17 +723,12 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam);
     rb = std::min(rb, plans[s].rb);
   }
-  static const int use_v2 = env_int("FS_LSE2", 1);
-  static const int rb_override = env_int("FS_RB", 0);
   bool aligned = (d % 4 == 0);
   for (int s = 0; s < nsides; ++s) aligned = aligned && aligned16(sides[s].q) && aligned16(sides[s].k);
   const int prec = cfg.prec;
   // pipelined LSE kernel: the 16-bit plane modes take any d <= 128, the fp32 mode needs aligned rows
-  const bool lse2 = vec_lse2 ||
-                    (mode == kLse && !fam.sliced && use_v2 && (prec != 0 || (aligned && dp >= 16)));
+  const bool lse2 = vec_lse2 || (mode == kLse && !fam.sliced && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = cfg.dp;
-  if (lse2 && prec == 2 && dp >= 64) rb = 1;  // three planes of 64 columns x two row blocks spill
-  if (lse2 && rb_override > 0 && dp <= 64) rb = std::min(rb_override, 2);
   PlaneSet ps;
   ps.n = 0;
   ps.end = 0;
@@ -833,15 +783,26 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (total <= 0) return FS_OK;
 
   int rc;
+  bool auto_sel = false;
   if (fam.sliced) {
     rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
   } else if (lse2) {
     rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
     a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
-    static const int coarse_env = env_int("FS_COARSE", 0);
-    const bool coarse = (coarse_env || (flags & FS_FLAG_COARSE_TEST)) && mode == kLse &&
-                        !(flags & FS_FLAG_NO_TILE_SKIP);
-    if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, mode == kVec, coarse, total, st);
+    const bool can_coarse = mode == kLse && prec == 3 && dp2 <= 64 && !(flags & FS_FLAG_NO_TILE_SKIP);
+    const bool coarse = (flags & FS_FLAG_COARSE_TEST) && can_coarse;
+    // device-chosen variant: both are enqueued, the one the state word names runs; the state
+    // belongs to prepared planes (a call that writes its own planes would start it afresh)
+    auto_sel = (flags & FS_FLAG_COARSE_AUTO) && can_coarse && !coarse && prepared;
+    if (auto_sel) {
+      a.sel = select_state(ps, ws);
+      a.sel_want = 1u;
+      if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, false, false, total, st);
+      a.sel_want = 0u;
+      if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, false, true, total, st);
+    } else if (rc == FS_OK) {
+      rc = launch_lse2(a, dp2, rb, prec, mode == kVec, coarse, total, st);
+    }
   } else
   switch (mode) {
     case kLse: rc = launch_dp<kLse, false>(a, dp, rb, total, st); break;
@@ -861,6 +822,10 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     hipLaunchKernelGGL((finish_argmax_kernel<0>), dim3(ceil_div(a.side[0].nq, 256)), dim3(256), 0, st,
                        a);
     return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+  }
+  if (auto_sel && !any_split) {  // no merge launch to carry the decision
+    hipLaunchKernelGGL((coarse_decide_kernel<0>), dim3(1), dim3(64), 0, st, a.sel);
+    if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
   }
   if (any_split) {
     // sides that were not split already wrote their output; give them no items
@@ -958,9 +923,9 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dp));
     return b * sizeof(float);
   };
-  size_t planes = 0;  // bf16 planes of x and y for the pipelined LSE kernel (three planes at most)
+  size_t planes = 0;  // two fp16 planes of x and y for the pipelined LSE kernel
   if (mode == kLse && !fam.sliced)
-    planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 3 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
+    planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 2 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
@@ -986,6 +951,17 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
   if (rc != FS_OK || ps.n == 0) return rc;
   if (ps.end > workspace_bytes || workspace == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
   return launch_plane_set(ps, cfg, d, workspace, (hipStream_t)stream);
+}
+
+size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
+                               uint32_t flags) {
+  if (!x || !y || bad_sizes(n, m, d) || d > kMaxSlicedD) return 0;
+  const LseConfig cfg = lse_config(d, flags);
+  const float* ptrs[2] = {x, y};
+  const int rows[2] = {(int)n, (int)m};
+  PlaneSet ps;
+  if (make_plane_set(ptrs, rows, 2, cfg, ps) != FS_OK || ps.n == 0) return 0;
+  return ps.aux_off + (2 * 256 + 8) * sizeof(float);
 }
 
 int fs_lse(const float* x, const float* y, const float* bias, float* out, int64_t n, int64_t m,
@@ -1221,7 +1197,7 @@ int fs_c_transform(const float* x, const float* y, const float* bias, float* min
   s.ep.out = min_out;
   s.ep.idx_out = reinterpret_cast<long long*>(argmin_out);
   // d > 128 runs on the fp16 planes whatever operand mode is asked for
-  if (d > kMaxStreamD) flags &= ~(uint32_t)(FS_FLAG_FP32_MFMA | FS_FLAG_BF16X3_OPERANDS);
+  if (d > kMaxStreamD) flags &= ~(uint32_t)FS_FLAG_FP32_MFMA;
   return run_stream(kArgmax, false, &s, 1, d, workspace, workspace_bytes, (hipStream_t)stream,
                     flags & ~(uint32_t)FS_FLAG_OPERANDS_PREPARED);
 }

@@ -101,7 +101,44 @@ struct LaunchArgs {
   float out_scale;  // finish_argmax_kernel: units of the partial values (1, or the plane scale)
   float skip_log2;  // lse2_kernel: tiles whose logits all lie this far (base 2, negative) below
                     // the running maxima skip their exponentials; -inf-like to switch it off
+  // lse2_kernel, variant chosen on the device: a launch with `sel` set runs only when
+  // sel[kSelWord] == sel_want (its workgroups return at once otherwise).  The variant with the
+  // coarse tile test counts its units into the slots of the same state block.
+  unsigned* sel;
+  unsigned sel_want;
 };
+
+// Device state of the variant choice (unsigned words), zeroed when the operand planes are
+// written: which variant runs (0: coarse tile test, 1: plain), how many decisions were taken,
+// running totals, and per-launch counters spread over kSelSlots slots (slot = workgroup % slots).
+constexpr int kSelWord = 0, kSelDecisions = 1, kSelCumEnded = 2, kSelCumUnits = 4;  // totals: u64
+constexpr int kSelSlots = 64, kSelEnded = 8, kSelUnits = kSelEnded + kSelSlots;
+constexpr int kSelWords = kSelUnits + kSelSlots;
+constexpr unsigned kSelDecideSteps = 3;  // the first launches of the coarse variant decide
+constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
+
+// One wavefront: add the launch's counters to the totals, clear them, and while decisions are
+// still open leave the coarse variant when too few units ended at its test.
+__device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
+  unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane];
+  st[kSelEnded + lane] = 0u;
+  st[kSelUnits + lane] = 0u;
+  unsigned long long es = e, us = u;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    es += __shfl_xor(es, o, 64);
+    us += __shfl_xor(us, o, 64);
+  }
+  if (lane == 0 && us > 0) {
+    unsigned long long* cum = reinterpret_cast<unsigned long long*>(st + kSelCumEnded);
+    cum[0] += es;
+    cum[1] += us;
+    if (st[kSelDecisions] < kSelDecideSteps) {
+      st[kSelDecisions] += 1u;
+      if (es * 100ull < us * (unsigned long long)kSelMinPercent) st[kSelWord] = 1u;
+    }
+  }
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

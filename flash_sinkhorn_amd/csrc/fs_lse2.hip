@@ -13,7 +13,7 @@ static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
 
 template <int DP, int PREC, bool VEC>
 static int launch_rb(const LaunchArgs& a, int rb, int blocks, hipStream_t st) {
-  if constexpr (DP <= 64 && !(PREC == kBf6 && DP == 64)) {
+  if constexpr (DP <= 64) {
     if (rb >= 2) return launch_cfg<DP, 2, PREC, VEC>(a, blocks, st);
   }
   return launch_cfg<DP, 1, PREC, VEC>(a, blocks, st);
@@ -31,17 +31,6 @@ static int launch_dp(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_
   return FS_ERR_UNSUPPORTED;
 }
 
-int launch_split_planes(const float* src, unsigned* dst, int rows, int d, int dp, int np,
-                        hipStream_t st) {
-  const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
-  const int grid = (int)((items + 255) / 256);
-  if (np == 2)
-    hipLaunchKernelGGL((split_planes_kernel<2>), dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp);
-  else
-    hipLaunchKernelGGL((split_planes_kernel<3>), dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp);
-  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
-}
-
 int launch_absmax(const float* a, long long na, const float* b, long long nb, float* partial,
                   hipStream_t st) {
   hipLaunchKernelGGL(absmax_kernel, dim3(2 * kAbsmaxBlocks), dim3(256), 0, st, a, na, b, nb, partial);
@@ -50,11 +39,11 @@ int launch_absmax(const float* a, long long na, const float* b, long long nb, fl
 
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
-                            int chunked, hipStream_t st) {
+                            int chunked, unsigned* clear_state, hipStream_t st) {
   const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
   const int grid = (int)((items + 255) / 256);
   hipLaunchKernelGGL(split_planes_f16_kernel, dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp,
-                     partial_max, scale_out, scale_out2, chunked);
+                     partial_max, scale_out, scale_out2, chunked, clear_state);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
@@ -82,8 +71,6 @@ int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, bool co
   }
   switch (prec) {
     case kF32: return launch_dp<kF32, false>(a, dp, rb, blocks, st);
-    case kBf3: return launch_dp<kBf3, false>(a, dp, rb, blocks, st);
-    case kBf6: return launch_dp<kBf6, false>(a, dp, rb, blocks, st);
     case kH3: return launch_dp<kH3, false>(a, dp, rb, blocks, st);
   }
   return FS_ERR_BAD_ARGUMENT;

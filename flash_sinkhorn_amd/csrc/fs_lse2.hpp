@@ -24,20 +24,14 @@
 //
 // Operand precision (PREC):
 //   kF32   v_mfma_f32_32x32x2_f32 on fp32 operands (needs d % 4 == 0 and aligned rows).
-//          (The 16-bit modes read operands that the split kernels have already cut into
-//          packed planes and apply the logit scale in the exp2 argument's FMA, so there is no
+//          (The plane mode reads operands that the split kernel has already cut into
+//          packed planes and applies the logit scale in the exp2 argument's FMA, so there is no
 //          per-tile conversion work.)
-//   kBf3   operands split into two bf16 planes (hi, lo); hi*hi + hi*lo + lo*hi on
-//          v_mfma_f32_32x32x16_bf16, fp32 accumulate: ~2^-17 relative per product,
-//          the counterpart of the reference's allow_tf32=True.
-//   kBf6   three bf16 planes, the six products whose weight is >= 2^-16: same
-//          accuracy class as fp32 operands (the planes sum to the fp32 value exactly)
-//          at 6/16 of the fp32 MFMA time.
 //   kH3    two fp16 planes (hi, lo) of the operand times a power of two that brings the
 //          matrix's largest magnitude to [2^14, 2^15); hi*hi + hi*lo + lo*hi on
 //          v_mfma_f32_32x32x16_f16.  The planes carry 22 significand bits and the dropped
 //          lo*lo term weighs 2^-22, so a dot product is as accurate as one accumulated in
-//          fp32 from exact products, at the MFMA cost of kBf3.
+//          fp32 from exact products, at 3/16 of the fp32 MFMA time.
 #pragma once
 
 #include <type_traits>
@@ -47,60 +41,11 @@
 
 namespace fs {
 
-enum Prec : int { kF32 = 0, kBf3 = 1, kBf6 = 2, kH3 = 3 };
+enum Prec : int { kF32 = 0, kH3 = 3 };
 
 constexpr int kPlanePadRows = 256;  // zero rows after the last row of a plane buffer
 constexpr int kAbsmaxBlocks = 256;  // partial maxima per matrix written by absmax_kernel
 
-
-__device__ __forceinline__ unsigned pack_bf16(float a, float b) {
-  f32x2 v = {a, b};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
-}
-__device__ __forceinline__ float bf16_lo_as_f32(unsigned p) {
-  return __builtin_bit_cast(float, p << 16);
-}
-__device__ __forceinline__ float bf16_hi_as_f32(unsigned p) {
-  return __builtin_bit_cast(float, p & 0xffff0000u);
-}
-
-// Split the pair (a, b) into NP packed bf16 planes with round-to-nearest pieces.
-template <int NP>
-__device__ __forceinline__ void split_pair(float a, float b, unsigned (&out)[NP]) {
-#pragma unroll
-  for (int p = 0; p < NP; ++p) {
-    out[p] = pack_bf16(a, b);
-    if (p + 1 < NP) {
-      a -= bf16_lo_as_f32(out[p]);
-      b -= bf16_hi_as_f32(out[p]);
-    }
-  }
-}
-
-// x[rows, d] (fp32) -> packed bf16 planes [rows + kPlanePadRows][NP][DP/2] (32-bit words), zero
-// padded to DP columns and in the trailing rows; plane p holds the p-th round-to-nearest bf16
-// piece, so the planes sum to x.
-template <int NP>
-__global__ __launch_bounds__(256) void split_planes_kernel(const float* __restrict__ src,
-                                                           unsigned* __restrict__ dst, int rows,
-                                                           int d, int dp) {
-  const int per_row = dp / 4;
-  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (long long)(rows + kPlanePadRows) * per_row) return;
-  const int r = (int)(idx / per_row);
-  const int c4 = (int)(idx % per_row) * 4;
-  const float* p = src + (size_t)min(r, rows - 1) * (size_t)d;
-  float v[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) v[t] = (c4 + t < d && r < rows) ? p[c4 + t] : 0.f;
-  unsigned p01[NP], p23[NP];
-  split_pair<NP>(v[0], v[1], p01);
-  split_pair<NP>(v[2], v[3], p23);
-  unsigned* o = dst + (size_t)r * (size_t)(NP * dp / 2);
-#pragma unroll
-  for (int pl = 0; pl < NP; ++pl)
-    *reinterpret_cast<uint2*>(o + pl * (dp / 2) + c4 / 2) = make_uint2(p01[pl], p23[pl]);
-}
 
 // Largest |value| of two matrices: blocks [0, kAbsmaxBlocks) scan a, the rest scan b; one
 // partial maximum per block goes to partial[2][kAbsmaxBlocks].
@@ -146,12 +91,13 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ a
 
 // x[rows, d] (fp32) -> two packed fp16 planes [rows + kPlanePadRows][2][DP/2] of scale*x, zero
 // padded to DP columns and in the trailing rows.  scale is derived from the partial maxima of
-// absmax_kernel; block 0 also publishes it in *scale_out for the consuming kernel.  With
-// `chunked` the two planes are interleaved per 32 columns (layout of lse_gemm_kernel).
+// absmax_kernel; block 0 also publishes it in *scale_out for the consuming kernel and clears
+// the kSelWords words at `clear_state` (the variant-choice state that belongs to the planes).
+// With `chunked` the two planes are interleaved per 32 columns (layout of lse_gemm_kernel).
 __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     const float* __restrict__ src, unsigned* __restrict__ dst, int rows, int d, int dp,
     const float* __restrict__ partial_max, float* __restrict__ scale_out,
-    float* __restrict__ scale_out2, int chunked) {
+    float* __restrict__ scale_out2, int chunked, unsigned* __restrict__ clear_state) {
   __shared__ float red[4];
   float m = partial_max[threadIdx.x];  // kAbsmaxBlocks == blockDim.x
 #pragma unroll
@@ -163,6 +109,7 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     *scale_out = sc;
     if (scale_out2) *scale_out2 = sc;  // the same matrix plays both roles
   }
+  if (blockIdx.x == 0 && clear_state != nullptr && threadIdx.x < kSelWords) clear_state[threadIdx.x] = 0u;
 
   const int per_row = dp / 4;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -191,15 +138,15 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
 
 template <int DP, int PREC>
 struct Geo2 {
-  static constexpr int NP = (PREC == kF32) ? 1 : (PREC == kBf6 ? 3 : 2);
-  // keys per tile: 64, except 128-column rows outside the two-plane modes (LDS)
-  static constexpr int JT = (DP >= 128 && (PREC == kF32 || PREC == kBf6)) ? 32 : 64;
+  static constexpr int NP = (PREC == kF32) ? 1 : 2;
+  // keys per tile: 64, except 128-column fp32 rows (LDS)
+  static constexpr int JT = (DP >= 128 && PREC == kF32) ? 32 : 64;
   static constexpr int NSUB = JT / 32;
   // LDS row stride in 32-bit words: fp32 row + 4, or NP 16-bit planes + 4
   static constexpr int LDW = (PREC == kF32) ? (DP + 4) : (NP * DP / 2 + 4);
   static constexpr int KK16 = DP / 16;  // 16-bit MFMAs per plane pair
   // MFMAs of one logits tile, the bias one excluded
-  static constexpr int NMAIN = (PREC == kF32) ? DP / 2 : (NP == 2 ? 3 : 6) * KK16;
+  static constexpr int NMAIN = (PREC == kF32) ? DP / 2 : 3 * KK16;
 };
 
 #define FS_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -225,16 +172,16 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int NP = G::NP;
   constexpr int NSUB = G::NSUB;
   constexpr int NMAIN = G::NMAIN;
-  constexpr bool kBf = (PREC != kF32);
-  constexpr int ROWW = kBf ? NP * DP / 2 : DP;  // 32-bit words per operand row in global memory
+  constexpr bool kPlanes = (PREC != kF32);
+  constexpr int ROWW = kPlanes ? NP * DP / 2 : DP;  // 32-bit words per operand row in global memory
   // Key-register prefetch (A operands of the next 32-key sub-tile are read from LDS while the
   // current one is multiplied) and the early LDS store it needs; off where registers are short.
-  constexpr bool KPF = (NSUB == 2) && DP < 128 && !(PREC == kBf6 && RB == 2);
+  constexpr bool KPF = (NSUB == 2) && DP < 128;
   // Two-plane modes with the key-register prefetch: the key bias is the initial value of the MFMA
   // chain's accumulator (16 floats per lane read from LDS while the previous unit finishes)
   // and the running max is subtracted inside the exp2 argument's FMA, which takes the fp32
   // bias MFMA (64 of 448 MFMA cycles per unit at d = 64) out of the loop.
-  constexpr bool BIASC = (PREC == kH3 || PREC == kBf3) && KPF;
+  constexpr bool BIASC = (PREC == kH3) && KPF;
   static_assert(!VEC || BIASC, "the vector mode rides on the bias-as-accumulator-start pipeline");
   // fp16 planes, log-sum-exp: the hi*hi product of a unit runs first and is tested before the two
   // cross products.  |x_hi.y_lo + x_lo.y_hi| has a bound per query row that needs no look at the
@@ -250,7 +197,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // registers, no ds_write): rows are unpadded and 16-byte piece p of row r sits in slot
   // p ^ swz(r), which keeps the b128 reads of 16 consecutive rows conflict free.  With the
   // key-register prefetch the tile two ahead is in flight, hence three buffers.
-  constexpr bool DIRECT = kBf && NP == 2;
+  constexpr bool DIRECT = kPlanes;
   constexpr int NBUF = (DIRECT && KPF) ? 3 : 2;
   constexpr int LDWK = DIRECT ? ROWW : G::LDW;  // LDS row stride in words
   constexpr int PPR = ROWW / 4;                 // 16-byte pieces per row
@@ -258,6 +205,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][G::JT * LDWK];
   __shared__ __attribute__((aligned(16))) float lds_b[NBUF][256];  // [buf][thread]; first JT used
   __shared__ __attribute__((aligned(16))) float lds_v[VEC ? NBUF : 1][VEC ? 256 : 4];  // VEC: v_j
+
+  // variant chosen on the device: the launch of the variant that was not chosen ends here
+  if (args.sel != nullptr && args.sel[kSelWord] != args.sel_want) return;
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;
@@ -281,18 +231,18 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // 16-bit plane modes: MFMAs produce raw dot products; lscale turns them into base-2 logits
   // inside the exp2 argument, and the bias / running max are kept in dot-product units.
   // fp16 planes carry a power-of-two scale per matrix, which lscale takes out again.
-  float lscale = kBf ? sd.qscale : 1.0f;
+  float lscale = kPlanes ? sd.qscale : 1.0f;
   if constexpr (PREC == kH3) lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
-  const float inv_lscale = kBf ? 1.0f / lscale : 1.0f;
+  const float inv_lscale = kPlanes ? 1.0f / lscale : 1.0f;
   const float skip_below = args.skip_log2 * inv_lscale;  // in accumulator units
 
   // ---- stationary query operands ----
-  float xs[kBf ? 1 : RB][kBf ? 1 : DP / 2];
-  u32x4 xq[kBf ? RB : 1][kBf ? NP : 1][kBf ? G::KK16 : 1];
+  float xs[kPlanes ? 1 : RB][kPlanes ? 1 : DP / 2];
+  u32x4 xq[kPlanes ? RB : 1][kPlanes ? NP : 1][kPlanes ? G::KK16 : 1];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = min(row0 + rb * 32 + li, sd.nq - 1);
-    if constexpr (!kBf) {
+    if constexpr (!kPlanes) {
       const float* qrow = sd.q + (size_t)row * (size_t)d;
 #pragma unroll
       for (int q = 0; q < DP / 8; ++q) {
@@ -355,8 +305,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   constexpr int PER_THREAD = (C16_TOTAL + 255) / 256;
   u32x4 st_k[DIRECT ? 1 : PER_THREAD];
   float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f, st_pen = 0.f, st_v = 0.f;
-  const unsigned* krows = kBf ? sd.kplanes : reinterpret_cast<const unsigned*>(sd.k);
-  const int krow_words = kBf ? ROWW : d;
+  const unsigned* krows = kPlanes ? sd.kplanes : reinterpret_cast<const unsigned*>(sd.k);
+  const int krow_words = kPlanes ? ROWW : d;
   const float* kb1p = sd.kb1 ? sd.kb1 : sd.kb0;  // always loadable; unused terms are dropped
   const float* kb2p = sd.kb2 ? sd.kb2 : sd.kb0;
   // read once: inside the loop the launch arguments would be fetched again for every tile
@@ -398,9 +348,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
             (const __attribute__((address_space(1))) void*)kp[c],
             (__attribute__((address_space(3))) void*)(&lds_k[dbuf][(c * 256 + wave * 64) * 4]),
             16, 0, 0);
-        kp[c] += G::JT * ROWW;
-      } else if constexpr (kBf) {
-        st_k[c] = *reinterpret_cast<const u32x4*>(kp[c]);
         kp[c] += G::JT * ROWW;
       } else {
         const int idx = tid + 256 * c;
@@ -595,8 +542,8 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 
   // A operands (one 32-key sub-tile) from LDS
   struct KeyRegs {
-    float ya[kBf ? 1 : DP / 2];
-    u32x4 yq[kBf ? NP : 1][kBf ? G::KK16 : 1];
+    float ya[kPlanes ? 1 : DP / 2];
+    u32x4 yq[kPlanes ? NP : 1][kPlanes ? G::KK16 : 1];
     float ab;
   };
   // Direct mode: the key operands are read with ds_read_b128 written out by hand.  The compiler
@@ -621,7 +568,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   };
   auto load_keys = [&](KeyRegs& kr, int buf, int js) {
     const unsigned* yrow = lds_k[buf] + (js * 32 + li) * LDWK;
-    if constexpr (!kBf) {
+    if constexpr (!kPlanes) {
 #pragma unroll
       for (int q = 0; q < DP / 8; ++q) {
         const float4 v = *reinterpret_cast<const float4*>(yrow + 8 * q + 4 * h);
@@ -645,32 +592,24 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   };
   // MFMA number k (0 <= k < NMAIN) of one logits tile (32 keys x 32 queries) of query block
   // rb.  Plane products run from the lowest weight to hi*hi (COARSE: hi*hi first, it is what
-  // the early test looks at); those below 2^-16 (2^-24 with three planes) are skipped.
+  // the early test looks at); lo*lo (2^-22) is left out.
   auto mfma_k = [&](int k, f32x16 acc, const KeyRegs& kr, int rb) {
-    if constexpr (!kBf) {
+    if constexpr (!kPlanes) {
       return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ya[k], xs[rb][k], acc, 0, 0, 0);
     } else {
       const int prod = k / G::KK16, kk = k % G::KK16;
-      // NP == 2: (1,0) (0,1) (0,0);  NP == 3: (2,0) (1,1) (0,2) (1,0) (0,1) (0,0)
+      // (key plane, query plane): (lo,hi) (hi,lo) (hi,hi)
       int pa, pb;
-      if (NP == 2 && COARSE) {  // (0,0) first: it is tested before the cross products run
+      if (COARSE) {  // (hi,hi) first: it is tested before the cross products run
         pa = (prod == 1) ? 1 : 0;
         pb = (prod == 2) ? 1 : 0;
-      } else if (NP == 2) {
+      } else {
         pa = (prod == 0) ? 1 : 0;
         pb = (prod == 1) ? 1 : 0;
-      } else {
-        pa = (prod == 0) ? 2 : ((prod == 1 || prod == 3) ? 1 : 0);
-        pb = (prod == 2) ? 2 : ((prod == 1 || prod == 4) ? 1 : 0);
       }
-      if constexpr (PREC == kH3)
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr.yq[pa][kk]),
-                                                      __builtin_bit_cast(f16x8, xq[rb][pb][kk]),
-                                                      acc, 0, 0, 0);
-      else
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kr.yq[pa][kk]),
-                                                       __builtin_bit_cast(bf16x8, xq[rb][pb][kk]),
-                                                       acc, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr.yq[pa][kk]),
+                                                    __builtin_bit_cast(f16x8, xq[rb][pb][kk]), acc,
+                                                    0, 0, 0);
     }
   };
   // BIASC: the key bias of sub-tile js as the accumulator layout holds it (register r of lane
@@ -851,6 +790,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   static_assert(!BIASC || (NSUB * RB) % 2 == 0, "units per tile must be even");
 
   bool prev_coarse = false;  // COARSE: the previous unit ended after its hi*hi product
+  unsigned n_ended = 0;      // COARSE: units of this wavefront that ended there
   // ---- steady state: the soft-max of the previous logits tile rides between the MFMAs ----
   for (int t = 1; t < ntiles; ++t) {
     if constexpr (!KPF) stage_load(j_begin + (t + 1) * G::JT, nxt);
@@ -957,6 +897,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
           for (int p = 6; p < kPieces; ++p) step(p, soft, full);
           if (soft) softmax_tail(st, prev_rb);
           prev_coarse = !full;
+          n_ended += full ? 0u : 1u;
           FS_SCHED_FENCE();
           continue;
         }
@@ -996,6 +937,14 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     f32x16 v16;
     if constexpr (VEC) v16 = load_v16(nx2, NSUB - 1);  // after rotate(): the tile just finished
     softmax(R1, RB - 1, v16);
+  }
+
+  if constexpr (COARSE) {  // unit counts of this wavefront for the variant choice on the device
+    if (args.sel != nullptr && lane == 0 && ntiles > 1) {
+      const int slot = blockIdx.x % kSelSlots;
+      atomicAdd(&args.sel[kSelEnded + slot], n_ended);
+      atomicAdd(&args.sel[kSelUnits + slot], (unsigned)((ntiles - 1) * NSUB * RB));
+    }
   }
 
 #pragma unroll

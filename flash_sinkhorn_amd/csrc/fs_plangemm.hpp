@@ -38,10 +38,10 @@ namespace fs {
 
 constexpr int kPgKeys = 256;          // keys per tile
 constexpr int kPgRows = 32;           // query rows per workgroup
-constexpr float kPgLazyThresh = 8.0f; // exponentials stay below 2^8 relative to the running maximum
-// exponentials are taken 2^7 up before the fp16 split and the reported maximum 7 down, as in
-// plan_tile_kernel: a probability keeps a nonzero fp16 image down to 2^-31 of the row's largest
-constexpr float kPgUp = 7.0f;
+constexpr float kPgLazyThresh = 4.0f; // exponentials stay below 2^4 relative to the running maximum
+// exponentials are taken 2^11 up before the fp16 split and the reported maximum 11 down, as in
+// plan_tile_kernel: a probability keeps a nonzero fp16 image down to 2^-35 of the row's largest
+constexpr float kPgUp = 11.0f;
 
 // Largest |rowscale[r] * src[r, c]| (rowscale may be null): one partial maximum per block.
 __global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ src,

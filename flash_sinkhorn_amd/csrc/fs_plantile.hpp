@@ -9,7 +9,7 @@
 //   logits   3 fp16 MFMA products per 16 columns, then one fp32 MFMA that adds the key bias
 //            and subtracts the block's running maximum (both in units of the raw products);
 //   soft-max lane-private and lazy: the running maximum moves only when a tile exceeds it by
-//            2^8, so the probabilities stay below 2^8 and are fp16-safe;
+//            2^4, so the exponentials stay below 2^4 (2^15 after the shift below): fp16-safe;
 //   values   (kMat) the lane's own 16 probabilities are, as they stand, its B operands of the
 //            two 16-key steps; they are split into hi / lo fp16 and multiplied with the V^T
 //            operands that transpose_planes_f16_kernel laid out in MFMA order in global memory
@@ -31,12 +31,12 @@
 
 namespace fs {
 
-constexpr float kPtLazyThresh = 8.0f;  // exponentials stay below 2^8 relative to the running maximum
-// The exponentials are taken 2^7 up before they are cut into fp16 planes (values up to 2^15), and
-// the maximum a row reports is lowered by the same 7: the pair (maximum, sums) means the same
-// thing, while a probability keeps a nonzero fp16 image down to 2^-31 of the row's largest one
+constexpr float kPtLazyThresh = 4.0f;  // exponentials stay below 2^4 relative to the running maximum
+// The exponentials are taken 2^11 up before they are cut into fp16 planes (values up to 2^15), and
+// the maximum a row reports is lowered by the same 11: the pair (maximum, sums) means the same
+// thing, while a probability keeps a nonzero fp16 image down to 2^-35 of the row's largest one
 // instead of 2^-24 (a tail of many far keys would otherwise be rounded away one-sidedly).
-constexpr float kPtUp = 7.0f;
+constexpr float kPtUp = 11.0f;
 
 template <int DP, int RB, int MODE>
 __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void plan_tile_kernel(const LaunchArgs args) {

@@ -468,6 +468,9 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
 template <bool HAS_O>
 __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int dp, int items0,
                                                      int items1) {
+  if constexpr (!HAS_O) {  // the launch that follows both variants of a device-chosen step
+    if (args.sel != nullptr && blockIdx.x == 0 && threadIdx.x < 64) coarse_decide(args.sel, threadIdx.x);
+  }
   int it = blockIdx.x * 256 + threadIdx.x;
   if (it >= items0 + items1) return;  // the other side may have nothing to merge
   const bool second = it >= items0;
@@ -498,6 +501,12 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
   } else {
     epilogue_scalar(sd.ep, row, M, s, o);
   }
+}
+
+// The decision alone, for a step whose launch split no keys (no merge follows).
+template <int T>
+__global__ __launch_bounds__(64) void coarse_decide_kernel(unsigned* state) {
+  coarse_decide(state, threadIdx.x);
 }
 
 // kArgmax: merge the partial (largest value, key) pairs of the key splits; equal values keep

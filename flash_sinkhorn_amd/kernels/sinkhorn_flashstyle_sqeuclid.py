@@ -10,7 +10,9 @@ potentials f_hat = f - alpha, g_hat = g - beta, one half-update is
     f_hat_i = -eps * damping * LSE_j[ 2*cost_scale*x_i.y_j/eps + g_hat_j/eps + log b_j ].
 Triton tuning keywords (block_*, num_warps, num_stages, autotune) are accepted
 and ignored; ``use_exp2`` selects nothing (the kernels work in base 2, which is
-the same function); ``allow_tf32=False`` means strict fp32 MFMA operands.
+the same function); ``allow_tf32`` selects nothing either unless
+``_lib.STRICT_OPERANDS = "fp32_mfma"`` asks for fp32 MFMA operands under ``allow_tf32=False``:
+the default two-plane fp16 operands are fp32-grade and the fastest mode.
 """
 from __future__ import annotations
 
@@ -119,8 +121,9 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
     """One launch on already contiguous fp32 operands.  With shift_x/shift_y the
     unbalanced shift correction is applied inside the epilogue.  When every paired argument
     is the same tensor (the self problem OT(x, x)) the library computes the one distinct
-    half-update and the same tensor is returned twice.  ``coarse`` sets
-    ``FS_FLAG_COARSE_TEST`` (tiles tested after their hi*hi plane product)."""
+    half-update and the same tensor is returned twice.  ``coarse``: True sets
+    ``FS_FLAG_COARSE_TEST`` (tiles tested after their hi*hi plane product), "auto"
+    ``FS_FLAG_COARSE_AUTO`` (the device decides; needs ``prepared``)."""
     n, d = x.shape
     m = y.shape[0]
     f_out = torch.empty((n,), device=x.device, dtype=torch.float32)
@@ -129,8 +132,7 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
     g_out = f_out if self_problem else torch.empty((m,), device=x.device, dtype=torch.float32)
     wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_SYMMETRIC_STEP, x, y,
                                            _lib.flags(use_exp2, allow_tf32), prepared)
-    if coarse:
-        fl |= _lib.FS_FLAG_COARSE_TEST
+    fl |= _lib.coarse_flag(coarse)
     rc = _lib.lib().fs_symmetric_step(
         x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), f_out.data_ptr(), g_out.data_ptr(), _lib.ptr(shift_x),
@@ -161,8 +163,7 @@ def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale,
     eps_a, alpha_a, df_a, dg_a = (arr(*[float(s[i]) for s in steps]) for i in range(4))
     wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_SYMMETRIC_STEP, x, y,
                                            _lib.flags(use_exp2, allow_tf32), prepared)
-    if coarse:
-        fl |= _lib.FS_FLAG_COARSE_TEST
+    fl |= _lib.coarse_flag(coarse)
     rc = _lib.lib().fs_symmetric_steps(
         x.data_ptr(), y.data_ptr(), f_hat.data_ptr(), g_hat.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), f_work[0].data_ptr(), g_work[0].data_ptr(), f_work[1].data_ptr(),

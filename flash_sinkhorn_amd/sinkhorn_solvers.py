@@ -21,22 +21,21 @@ from flash_sinkhorn_amd.kernels._common import (
 
 __all__ = ["sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric"]
 
-# Long fixed-eps solves on large clouds run on rows and keys grouped by k-means cluster, and
-# time a few steps with and without FS_FLAG_COARSE_TEST to pick the faster kernel variant: with
+# Long fixed-eps solves on large clouds run on rows and keys grouped by k-means cluster, with the
+# kernel variant that tests a tile after its hi*hi plane product (FS_FLAG_COARSE_TEST): with
 # neighbouring rows next to each other, whole key tiles fall below the 2^-40 criterion for all
-# rows of a workgroup at once, which the coarse test turns into fewer MFMAs.  The potentials
-# come back in the caller's order; values agree with the unordered solve to fp32 rounding.
+# rows of a workgroup at once, which the coarse test turns into fewer MFMAs.  Whether the
+# variant stays is decided on the device from the share of tiles that end at the test in the
+# first steps (FS_FLAG_COARSE_AUTO): no timing, no host read-back, the same inputs take the
+# same path on every run.  The potentials come back in the caller's order; values agree with
+# the unordered solve to fp32 rounding.
 CLUSTER_ORDER = os.environ.get("FLASH_SINKHORN_CLUSTER_ORDER", "1") != "0"
-# None: time both variants in the first steps of such a solve; True / False: no timing
+# None: the device decides; True / False: the coarse variant on every step / on none
 COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_TEST", ""))
-# measured on the benchmark's mixtures at d = 64: below about 40,000 rows per cloud the ordering
-# and the timed steps cost more than the coarse variant returns (25,000: +4 %; 32,768: even)
+# measured on 8-component Gaussian mixtures at d = 64: below about 40,000 rows per cloud the
+# ordering costs more than the coarse variant returns (25,000: +4 %; 32,768: even)
 _CLUSTER_MIN_ROWS = 40000
 _CLUSTER_MIN_STEPS = 24
-# what the last symmetric solve did: {"cluster_order": bool, "coarse_test": bool}
-LAST_SOLVE = {"cluster_order": False, "coarse_test": False}
-_TUNE_STEPS = 3  # steps timed per variant
-_RETUNE_AFTER = 24  # steps between the first choice and the second one of a long run
 
 
 def _cluster_order(pts: torch.Tensor, k: int = 16, iters: int = 4) -> torch.Tensor:
@@ -166,7 +165,7 @@ def sinkhorn_flashstyle_symmetric(
     f_init: Optional[torch.Tensor] = None, g_init: Optional[torch.Tensor] = None,
     label_x: Optional[torch.Tensor] = None, label_y: Optional[torch.Tensor] = None,
     label_cost_matrix: Optional[torch.Tensor] = None, lambda_x: float = 1.0,
-    lambda_y: float = 0.0,
+    lambda_y: float = 0.0, solve_info: Optional[dict] = None,
 ):
     """GeomLoss-style symmetric (Jacobi, averaged) Sinkhorn with an eps schedule.
 
@@ -179,6 +178,9 @@ def sinkhorn_flashstyle_symmetric(
     snapshot.  ``f_init``/``g_init`` warm-start (standard potentials).
     Returns (f, g[, f_prelast, g_prelast][, n_iters_used]); the prelast pair is
     only returned when ``return_prelast and last_extrapolation``.
+    ``solve_info`` (not in the reference): a dict that receives ``cluster_order`` (rows were
+    grouped by cluster), ``coarse`` (False, True or "auto") and ``prepared`` (the operand
+    planes, whose ``variant_state()`` tells what the device chose).
     """
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
         _symmetric_step_raw, _symmetric_steps_raw, flashsinkhorn_lse,
@@ -221,15 +223,16 @@ def sinkhorn_flashstyle_symmetric(
     # stay equal under the Jacobi iteration, so every step computes one half-update.
     if (fused and not use_labels and f_init is None and g_init is None and rho_x == rho_y
             and xf.data_ptr() == yf.data_ptr() and xf.shape == yf.shape
-            and (a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape))):
+            and (a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape
+                            and a.stride() == b.stride()))):
         yf, beta, log_b, g_hat = xf, alpha, log_a, f_hat
 
     # cluster order (see CLUSTER_ORDER): every per-row array is permuted, the results are
     # put back in the caller's order at the end
     inv_x = inv_y = None
-    coarse = [False, False]  # [variant in use, still to be tuned]
-    if (CLUSTER_ORDER and fused and not use_labels and not allow_tf32 and _lib.TILE_SKIP
-            and _lib.STRICT_OPERANDS == "fp16x2" and xf.shape[1] <= 64
+    coarse = False
+    if (CLUSTER_ORDER and fused and not use_labels and _lib.TILE_SKIP
+            and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
             and min(xf.shape[0], yf.shape[0]) >= _CLUSTER_MIN_ROWS
             and len(eps_list) >= _CLUSTER_MIN_STEPS
             and all(e == eps_list[0] for e in eps_list)):
@@ -248,7 +251,7 @@ def sinkhorn_flashstyle_symmetric(
             inv_y[perm_y] = torch.arange(perm_y.numel(), device=perm_y.device)
             yf, beta, log_b, g_hat = (yf[perm_y].contiguous(), beta[perm_y], log_b[perm_y],
                                       g_hat[perm_y])
-        coarse[0], coarse[1] = bool(COARSE_TEST), COARSE_TEST is None
+        coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
 
     # operand planes are converted once for the whole loop
     prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32))
@@ -260,7 +263,7 @@ def sinkhorn_flashstyle_symmetric(
                 xf, yf, f_hat, g_hat, log_a, log_b, e, cost_scale=cost_scale, alpha=w,
                 damping_f=damp_f, damping_g=damp_g,
                 shift_x=alpha if damp_f < 1.0 else None, shift_y=beta if damp_g < 1.0 else None,
-                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=coarse[0])
+                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=coarse)
         # two launches, raw-bias kernel, averaging and shift correction on the host
         kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
                   _prepared=prepared)
@@ -281,42 +284,11 @@ def sinkhorn_flashstyle_symmetric(
                 f_hat, g_hat = jacobi(f_hat, g_hat, e, w)
             return f_hat, g_hat
         steps = [(e, w, dampening(e, rho_x), dampening(e, rho_y)) for e, w in run]
-
-        def launch(f_hat, g_hat, part, variant):
-            return _symmetric_steps_raw(
-                xf, yf, f_hat, g_hat, log_a, log_b, part, cost_scale=cost_scale,
-                shift_x=alpha if rho_x is not None else None,
-                shift_y=beta if rho_y is not None else None,
-                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=variant)
-
-        def tune(f_hat, g_hat, window):
-            # the steps of `window` alternate between the two variants (all of them steps of
-            # the solve), each timed on the stream; the coarse variant takes the earlier step
-            # of each pair (early steps get faster as the plan sharpens)
-            ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(window) + 1)]
-            stream = torch.cuda.current_stream(xf.device)  # the stream the launches go to
-            ev[0].record(stream)
-            for i in range(len(window)):
-                f_hat, g_hat = launch(f_hat, g_hat, window[i:i + 1], i % 2 == 0)
-                ev[i + 1].record(stream)
-            ev[-1].synchronize()
-            took = [ev[i].elapsed_time(ev[i + 1]) for i in range(len(window))]
-            return f_hat, g_hat, sum(took[0::2]) < 0.98 * sum(took[1::2])
-
-        if coarse[1] and len(steps) >= 2 * _TUNE_STEPS + 2:
-            # first choice after the very first step (it starts from flat potentials); a long
-            # run chooses again some thirty steps in: a device that was idle before the solve
-            # takes that long to settle, and the first choice may have seen it cold
-            w = 2 * _TUNE_STEPS
-            f_hat, g_hat = launch(f_hat, g_hat, steps[:1], False)
-            f_hat, g_hat, coarse[0] = tune(f_hat, g_hat, steps[1:1 + w])
-            steps = steps[1 + w:]
-            if len(steps) >= _RETUNE_AFTER + 2 * w:
-                f_hat, g_hat = launch(f_hat, g_hat, steps[:_RETUNE_AFTER], coarse[0])
-                f_hat, g_hat, coarse[0] = tune(f_hat, g_hat, steps[_RETUNE_AFTER:_RETUNE_AFTER + w])
-                steps = steps[_RETUNE_AFTER + w:]
-            coarse[1] = False
-        return launch(f_hat, g_hat, steps, coarse[0])
+        return _symmetric_steps_raw(
+            xf, yf, f_hat, g_hat, log_a, log_b, steps, cost_scale=cost_scale,
+            shift_x=alpha if rho_x is not None else None,
+            shift_y=beta if rho_y is not None else None,
+            allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=coarse)
 
     # the initial full step and the averaged steps, cut where a convergence check looks at
     # the potentials
@@ -344,7 +316,8 @@ def sinkhorn_flashstyle_symmetric(
     out = (f_hat + alpha, g_hat + beta)
     if return_prelast and last_extrapolation:
         out = out + (f_prelast, g_prelast)
-    LAST_SOLVE["cluster_order"], LAST_SOLVE["coarse_test"] = inv_x is not None, coarse[0]
+    if solve_info is not None:
+        solve_info.update(cluster_order=inv_x is not None, coarse=coarse, prepared=prepared)
     if inv_x is not None:  # back to the caller's row order
         out = tuple(t[inv_x if i % 2 == 0 else inv_y] for i, t in enumerate(out))
     if return_n_iters:

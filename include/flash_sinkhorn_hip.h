@@ -15,16 +15,15 @@
  *    returns without synchronising; the library keeps no mutable global state
  *  - return value: FS_OK or a negative FS_ERR_* code (fs_error_string names it)
  *  - flags: FS_FLAG_EXP2 is accepted for interface parity (the kernels always
- *    work in base 2, which is the same function).  Operand precision of the
- *    log-sum-exp kernels (everything accumulates in fp32):
+ *    work in base 2, which is the same function).  Operand precision (everything
+ *    accumulates in fp32):
  *      default                    operands as two fp16 planes (22 significand bits) of
  *                                 the matrix scaled by a power of two, three MFMA
  *                                 products: error at or below that of fp32 MFMA operands
- *      FS_FLAG_BF16X3_OPERANDS    three bf16 planes, six products: same accuracy class,
- *                                 no dependence on the dynamic range inside a matrix
  *      FS_FLAG_FP32_MFMA          fp32 operands on v_mfma_f32_32x32x2_f32
- *      FS_FLAG_REDUCED_OPERANDS   two bf16 planes, three products (~2^-17 relative
- *                                 per product): the counterpart of allow_tf32=True
+ *      FS_FLAG_REDUCED_OPERANDS   permission to use less precise operands (the counterpart of
+ *                                 allow_tf32=True); accepted and not acted on: the default
+ *                                 mode is the fastest one on this machine
  *    The d <= 128 log-sum-exp kernel leaves out the exponentials of a 32 x 32 logits tile
  *    whose every entry lies more than 2^40 below its row's running maximum (they cannot
  *    change the fp32 row sums); FS_FLAG_NO_TILE_SKIP computes them all the same.
@@ -36,10 +35,16 @@
  *    within fp32 rounding of the full computation.  It pays when rows and keys are ordered so
  *    that neighbouring rows have neighbouring keys (e.g. sorted by cluster) and the plan is
  *    peaked; on other inputs the test costs about 10 %.  Ignored where it does not apply.
- *    The gradient, the plan-vector / plan-matrix products, mat5 and the c-transform, and for
- *    d > 128 the log-sum-exp as well, run on the two-plane fp16 operands by default and with
- *    FS_FLAG_REDUCED_OPERANDS, and on fp32 MFMA operands with FS_FLAG_FP32_MFMA or
- *    FS_FLAG_BF16X3_OPERANDS.
+ *    FS_FLAG_COARSE_AUTO (with FS_FLAG_OPERANDS_PREPARED, same conditions) leaves that choice to
+ *    the device: every step enqueues both variants and a word of state next to the prepared
+ *    planes says which one runs (the workgroups of the other return at once).  The coarse
+ *    variant runs first and counts the tiles that end at its test; after each of its first
+ *    three launches the step's merge kernel switches to the plain variant for good if fewer than
+ *    40 % did.  The state is reset by fs_prepare_operands.  Nothing is read back or timed on
+ *    the host: the same inputs take the same path on every run, and the calls can be captured
+ *    into a graph.
+ *    Every operation runs on the two-plane fp16 operands by default and on fp32 MFMA operands
+ *    with FS_FLAG_FP32_MFMA (the c-transform at d > 128: fp16 planes in either case).
  */
 #ifndef FLASH_SINKHORN_HIP_H
 #define FLASH_SINKHORN_HIP_H
@@ -62,10 +67,11 @@ extern "C" {
 #define FS_FLAG_EXP2 1u
 #define FS_FLAG_REDUCED_OPERANDS 2u
 #define FS_FLAG_FP32_MFMA 4u
-#define FS_FLAG_BF16X3_OPERANDS 8u
+/* 8u: unused (three-plane bf16 operands in ABI version 1) */
 #define FS_FLAG_OPERANDS_PREPARED 16u
 #define FS_FLAG_NO_TILE_SKIP 32u
 #define FS_FLAG_COARSE_TEST 64u
+#define FS_FLAG_COARSE_AUTO 128u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0
@@ -94,6 +100,17 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d);
  */
 int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
                         uint32_t flags, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Byte offset, inside a workspace that fs_prepare_operands(x, y, ...) has filled, of the state
+ * FS_FLAG_COARSE_AUTO keeps (0 when the configuration has none).  Six 32-bit words a caller
+ * may read for diagnostics once the stream has drained: [0] the variant the steps run now
+ * (0: coarse tile test, 1: plain), [1] decisions taken so far, [2..3] a 64-bit count of the
+ * 32 x 32 logits tiles that ended at the coarse test, [4..5] of the tiles it tested.  Host
+ * arithmetic only.  No counterpart in the reference.
+ */
+size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
+                               uint32_t flags);
 
 /*
  * out[i] = -eps*damping * LSE_j[ coord_scale * x_i.y_j / eps + bias[j] ]
@@ -265,7 +282,7 @@ int fs_mat5(const float* x, const float* y, const float* f_ott, const float* g_o
  *   min_out[i] = min_j [-coord_scale x_i.y_j + bias_j],  argmin_out[i] = the smallest j
  * attaining it (int64).  The caller passes bias_j = cost_scale |y_j|^2 - psi_j and adds
  * cost_scale |x_i|^2 to min_out.  Runs on the two-plane fp16 operands (fp32 MFMA operands for
- * d <= 128 with FS_FLAG_FP32_MFMA or FS_FLAG_BF16X3_OPERANDS).
+ * d <= 128 with FS_FLAG_FP32_MFMA).
  * Replaces c_transform_kernel (kernels/c_transform_sqeuclid.py:219-354, kernel 117-214).
  */
 int fs_c_transform(const float* x, const float* y, const float* bias, float* min_out,

@@ -80,19 +80,24 @@ def test_config3_solve_and_gradient_properties(c3):
     assert torch.isfinite(gy).all()
 
 
-@pytest.mark.parametrize("order,coarse", [(True, True), (True, False), (False, None)])
+@pytest.mark.parametrize("order,coarse", [(True, True), (True, False), (True, None), (False, None)])
 def test_config3_solve_variants_match_oracle_rows(c3, monkeypatch, order, coarse):
     """The same solve on rows grouped by cluster with the coarse tile test forced on, forced off,
-    and in the caller's order on the plain kernel: sampled rows of the final extrapolation step
+    chosen on the device, and in the caller's order on the plain kernel: sampled rows of the final extrapolation step
     (f = softmin of the pre-extrapolation g, g likewise) against the dense fp64 oracle."""
     import flash_sinkhorn_amd.sinkhorn_solvers as solvers
     x, y, a, b, (X, Y, A, B) = c3
     monkeypatch.setattr(solvers, "CLUSTER_ORDER", order)
     monkeypatch.setattr(solvers, "COARSE_TEST", coarse)
+    info = {}
     f, g, fp, gp = solvers.sinkhorn_flashstyle_symmetric(
         X, Y, A, B, use_epsilon_scaling=False, eps=EPS, n_iters=100, allow_tf32=False,
-        return_prelast=True)
-    assert solvers.LAST_SOLVE == {"cluster_order": order, "coarse_test": bool(order and coarse)}
+        return_prelast=True, solve_info=info)
+    assert info["cluster_order"] == order
+    assert info["coarse"] == (False if not order else ("auto" if coarse is None else coarse))
+    if order and coarse is None:  # on these mixtures the device keeps the coarse variant
+        state = info["prepared"].variant_state()
+        assert not state["plain_selected"] and state["tiles_ended"] > 0.5 * state["tiles_tested"]
     rows = np.random.default_rng(2).choice(50_000, 96, replace=False)
     want_f = oracle.softmin(x[rows], y, gp.cpu().numpy(), np.log(b), EPS)
     want_g = oracle.softmin(y[rows], x, fp.cpu().numpy(), np.log(a), EPS)

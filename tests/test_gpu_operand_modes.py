@@ -1,10 +1,11 @@
-"""The non-default operand modes of the C ABI against the fp64 oracle.
+"""The non-default operand mode of the C ABI against the fp64 oracle.
 
-``FS_FLAG_FP32_MFMA`` and ``FS_FLAG_BF16X3_OPERANDS`` (Python: ``_lib.STRICT_OPERANDS``) route
-d <= 128 log-sum-exp launches to the fp32 / three-plane bf16 variants of the pipelined kernel
-and every d > 128 operation to the column-sliced fp32-MFMA kernels; ``allow_tf32=True``
-(``FS_FLAG_REDUCED_OPERANDS``) selects two bf16 planes for d <= 128.  Strict modes are held to
-the rel 1e-4 bar of the default mode; the reduced mode to 2e-3 (its products carry ~2^-17).
+``FS_FLAG_FP32_MFMA`` (Python: ``_lib.STRICT_OPERANDS = "fp32_mfma"`` with ``allow_tf32=False``)
+routes d <= 128 log-sum-exp launches to the fp32 variant of the pipelined kernel, the d <= 128
+products to ``stream_kernel`` and every d > 128 operation to the column-sliced fp32-MFMA
+kernels, all held to the rel 1e-4 bar of the default mode.  ``allow_tf32=True``
+(``FS_FLAG_REDUCED_OPERANDS``) is a permission the library does not use: same kernels, same
+numbers as the default.
 """
 import numpy as np
 import pytest
@@ -38,7 +39,7 @@ def problem(n, m, d, seed=0):
     return x, y, a, b, f_hat, g_hat
 
 
-@pytest.fixture(params=["fp32_mfma", "bf16x3"])
+@pytest.fixture(params=["fp32_mfma"])
 def strict_mode(request, monkeypatch):
     from flash_sinkhorn_amd import _lib
     monkeypatch.setattr(_lib, "STRICT_OPERANDS", request.param)
@@ -58,8 +59,8 @@ def test_symmetric_step_in_strict_modes(strict_mode, n, m, d):
 
 @pytest.mark.parametrize("n,m,d", SHAPES)
 def test_products_on_fp32_mfma(strict_mode, n, m, d):
-    """With either strict flag every product runs on fp32 MFMA operands: `stream_kernel` for
-    d <= 128, `sliced_kernel` beyond."""
+    """With the flag every product runs on fp32 MFMA operands: `stream_kernel` for d <= 128,
+    `sliced_kernel` beyond."""
     from flash_sinkhorn_amd.kernels.apply_flash import (
         apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
     from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
@@ -96,14 +97,19 @@ def test_products_on_fp32_mfma(strict_mode, n, m, d):
 
 
 @pytest.mark.parametrize("n,m,d", SHAPES)
-def test_symmetric_step_with_reduced_operands(n, m, d):
+def test_symmetric_step_with_allow_tf32_is_the_default_kernel(n, m, d):
+    """allow_tf32=True (the reference's and this API's default) gets the same kernel as
+    allow_tf32=False: bit-equal results, within 1e-4 of the oracle."""
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
     x, y, a, b, fh, gh = problem(n, m, d, seed=3)
     la, lb = np.log(a), np.log(b)
     wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, 0.3, 1.0, 0.5, 1.0, 1.0)
-    gf, gg = _symmetric_step_raw(*dev(x, y, fh, gh, la, lb), 0.3, cost_scale=1.0, alpha=0.5,
-                                 damping_f=1.0, damping_g=1.0, allow_tf32=True)
-    assert rel_err(gf, wf) < 2e-3 and rel_err(gg, wg) < 2e-3
+    args = dev(x, y, fh, gh, la, lb)
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0)
+    gf, gg = _symmetric_step_raw(*args, 0.3, allow_tf32=True, **kw)
+    sf, sg = _symmetric_step_raw(*args, 0.3, allow_tf32=False, **kw)
+    assert rel_err(gf, wf) < RTOL and rel_err(gg, wg) < RTOL
+    assert torch.equal(gf, sf) and torch.equal(gg, sg)
 
 
 def test_tile_skip_leaves_results_unchanged(monkeypatch):

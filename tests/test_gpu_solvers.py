@@ -34,7 +34,7 @@ def test_symmetric_solver_vs_reference_golden(golden):
     assert rel_err(f, golden["sym_smalleps_f"]) < 2e-4
     # fp16 inputs are cast to fp32 by the launchers (reference test uses fp16 x, y)
     f16, g16 = solve(X.half(), Y.half(), A, B, use_epsilon_scaling=False, eps=0.5, n_iters=3)
-    assert rel_err(f16, golden["sym_fixed_f"]) < 2e-3
+    assert rel_err(f16, golden["sym_fixed_f"]) < 2e-3  # the rounding of the inputs to fp16
 
 
 def test_fused_equals_separate_and_exp2_flag():
@@ -244,10 +244,9 @@ def test_prepared_operands_give_identical_results(n, m, d):
         o0 = flashsinkhorn_lse_fused(q, k, pot, lw, 0.2, allow_tf32=False)
         o1 = flashsinkhorn_lse_fused(q, k, pot, lw, 0.2, allow_tf32=False, _prepared=prep)
         assert torch.equal(o0, o1)
-    # a different precision request does not match the prepared planes: falls back to converting
+    # allow_tf32=True is served by the same planes
     o2 = flashsinkhorn_lse_fused(X, Y, G, LB, 0.2, allow_tf32=True, _prepared=prep)
-    want = oracle.lse_shifted_fused(x, y, gh, np.log(b), 0.2)
-    assert rel_err(o2, want) < 1e-3
+    assert torch.equal(o2, flashsinkhorn_lse_fused(X, Y, G, LB, 0.2, allow_tf32=False))
 
 @pytest.mark.parametrize("n,m,d", [(3000, 4100, 64), (129, 1000, 3), (5000, 300, 128), (260, 260, 32)])
 def test_launches_are_repeatable_on_one_workspace(n, m, d):
@@ -592,8 +591,8 @@ def test_coarse_tile_test_leaves_results_unchanged(n, m, d, eps, sort):
 @pytest.mark.parametrize("variant", [True, False, None])
 def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
     """Long fixed-eps solves on large clouds run on rows grouped by k-means cluster and hand the
-    potentials back in the caller's order; with the coarse tile test forced on, off, or chosen by
-    timing, the result is the unordered solve's to rounding."""
+    potentials back in the caller's order; with the coarse tile test forced on, off, or chosen on
+    the device, the result is the unordered solve's to rounding."""
     import flash_sinkhorn_amd.sinkhorn_solvers as solvers
     rng = np.random.default_rng(32)
     n, m, d = 16500, 16400, 8
@@ -605,15 +604,20 @@ def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
     kw = dict(use_epsilon_scaling=False, eps=0.05, n_iters=26, allow_tf32=False,
               return_prelast=True)
     monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
-    want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
-    assert not solvers.LAST_SOLVE["cluster_order"]
+    info = {}
+    want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
+    assert not info["cluster_order"] and info["coarse"] is False
     monkeypatch.setattr(solvers, "CLUSTER_ORDER", True)
     monkeypatch.setattr(solvers, "_CLUSTER_MIN_ROWS", 16384)  # the default only orders larger clouds
     monkeypatch.setattr(solvers, "COARSE_TEST", variant)
-    got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
-    assert solvers.LAST_SOLVE["cluster_order"]
-    if variant is not None:
-        assert solvers.LAST_SOLVE["coarse_test"] == variant
+    got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
+    assert info["cluster_order"]
+    assert info["coarse"] == ("auto" if variant is None else variant)
+    state = info["prepared"].variant_state()
+    if variant is None:  # the device looked at the first three steps and took a decision
+        assert state["decisions"] == 3 and state["tiles_tested"] > 0
+    else:
+        assert state["decisions"] == 0 and state["tiles_tested"] == 0
     for u, v in zip(got, want):
         assert rel_err(u, v.cpu().numpy()) < 2e-5
     # the self problem keeps its single half-update per step under the ordering
@@ -634,3 +638,46 @@ def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
     want2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
     for u, v in zip(got2, want2):
         assert float((u - v).abs().max()) < 2e-6 * scale
+
+
+def test_variant_choice_on_the_device():
+    """FS_FLAG_COARSE_AUTO: every step enqueues both kernel variants and a word next to the
+    prepared planes says which runs.  On rows sorted by cluster with a peaked plan most tiles end
+    at the coarse test and the variant stays; on an unsorted cloud few do and the third decision
+    at the latest switches to the plain kernel for good.  Either way the potentials equal those
+    of the forced variants to rounding, and a second run takes the same path bit for bit."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_steps_raw
+    rng = np.random.default_rng(35)
+    n, m, d, eps = 6000, 5200, 64, 0.01
+    x, lx = _clustered(rng, n, d)
+    y, ly = _clustered(rng, m, d)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    steps = [(eps, 1.0, 1.0, 1.0)] + [(eps, 0.5, 1.0, 1.0)] * 7
+    for sort in (True, False):
+        xs, ys = (x[np.argsort(lx, kind="stable")], y[np.argsort(ly, kind="stable")]) if sort else \
+            (rng.standard_normal((n, d)).astype(np.float32), rng.standard_normal((m, d)).astype(np.float32))
+        fh = (-(xs * xs).sum(1)).astype(np.float32)
+        gh = (-(ys * ys).sum(1)).astype(np.float32)
+        X, Y, F, G, LA, LB = dev(xs, ys, fh, gh, np.log(a), np.log(b))
+        runs = {}
+        for coarse in ("auto", "auto", True, False):
+            prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+            out = _symmetric_steps_raw(X, Y, F, G, LA, LB, steps, cost_scale=1.0, prepared=prep,
+                                       allow_tf32=False, coarse=coarse)
+            st = prep.variant_state()
+            if coarse == "auto":
+                assert st["decisions"] >= 1 and st["tiles_tested"] > 0
+                share = st["tiles_ended"] / st["tiles_tested"]
+                # sorted clusters keep the coarse variant, the unsorted cloud leaves it
+                assert st["plain_selected"] == (not sort), (sort, st)
+                assert (share >= 0.4) == sort, (sort, share)
+                if "auto" in runs:  # same path, same bits
+                    assert torch.equal(out[0], runs["auto"][0]) and torch.equal(out[1], runs["auto"][1])
+            else:
+                assert st["decisions"] == 0
+            runs[coarse] = out
+        for k in (0, 1):
+            ref = runs[False][k].cpu().numpy()
+            assert rel_err(runs["auto"][k], ref) < 2e-6 and rel_err(runs[True][k], ref) < 2e-6
