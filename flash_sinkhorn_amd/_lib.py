@@ -51,6 +51,7 @@ _SIGNATURES = {
     "fs_lse": (ctypes.c_int, [_P] * 4 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_lse_fused": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_symmetric_step": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + _TAIL),
+    "fs_symmetric_step_noalloc": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + [_U, _P]),
     "fs_symmetric_steps": (ctypes.c_int, [_P] * 12 + [_I] * 3 + [_P] * 4 + [ctypes.c_int, _F] + _TAIL),
     "fs_schur_matvec": (ctypes.c_int, [_P] * 11 + [_I] * 3 + [_F, _F] + _TAIL),
     "fs_cg_init": (ctypes.c_int, [_P] * 5 + [_I, _F, _F, _P]),

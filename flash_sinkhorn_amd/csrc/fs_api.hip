@@ -4,14 +4,40 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <mutex>
 
 #include "flash_sinkhorn_hip.h"
 #include "fs_common.hpp"
 #include "fs_dispatch.hpp"
 #include "fs_stream.hpp"
 
+// Scratch of fs_symmetric_step_noalloc: lives in the code object, one copy per GPU that loads
+// the library, held until the process ends.  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels and copies get the per-device address it returns.
+constexpr size_t kScratchBytes = (size_t)48 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 namespace fs {
 namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // address of `scratch` on each device, looked up once
+std::mutex g_scratch_mutex;
+
+// Address of the built-in scratch buffer on the current device (set-up on the first call there).
+int scratch_on_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FS_ERR_LAUNCH_FAILED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr)
+      return FS_ERR_LAUNCH_FAILED;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return FS_OK;
+}
 
 constexpr int kMaxStreamD = 128;    // register-stationary streaming kernels
 constexpr int kMaxSlicedD = 16384;  // widest supported rows
@@ -896,6 +922,7 @@ const char* fs_error_string(int code) {
     case FS_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
     case FS_ERR_LAUNCH_FAILED: return "kernel launch failed";
     case FS_ERR_UNSUPPORTED: return "unsupported configuration";
+    case FS_ERR_SCRATCH_TOO_SMALL: return "problem too large for the built-in scratch buffer";
   }
   return "unknown error";
 }
@@ -1016,6 +1043,27 @@ int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const 
   s[1] = lse_side(y, x, f_hat, kLog2e / eps, log_a, kLog2e, m, n, qs);
   lse_epilogue(s[1], g_out, g_hat, alpha, eps, damp_g, shift_y);
   return run_stream(kLse, false, s, 2, d, workspace, workspace_bytes, (hipStream_t)stream, flags);
+}
+
+int fs_symmetric_step_noalloc(const float* x, const float* y, const float* f_hat,
+                              const float* g_hat, const float* log_a, const float* log_b,
+                              float* f_out, float* g_out, const float* shift_x,
+                              const float* shift_y, int64_t n, int64_t m, int64_t d, float eps,
+                              float alpha, float damp_f, float damp_g, float coord_scale,
+                              uint32_t flags, void* stream) {
+  if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
+  if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
+  const size_t need = fs_workspace_bytes(FS_OP_SYMMETRIC_STEP, n, m, d);
+  if (need == 0 || need > kScratchBytes) return FS_ERR_SCRATCH_TOO_SMALL;
+  void* buf = nullptr;
+  const int rc = scratch_on_current_device(&buf);
+  if (rc != FS_OK) return rc;
+  // the call writes its own operand planes (which also resets the variant-choice state) and
+  // every partial row before reading it: nothing in the buffer has to be cleared beforehand
+  flags &= ~(uint32_t)(FS_FLAG_OPERANDS_PREPARED | FS_FLAG_COARSE_AUTO);
+  return fs_symmetric_step(x, y, f_hat, g_hat, log_a, log_b, f_out, g_out, shift_x, shift_y, n, m,
+                           d, eps, alpha, damp_f, damp_g, coord_scale, flags, buf, kScratchBytes,
+                           stream);
 }
 
 int fs_symmetric_steps(const float* x, const float* y, const float* f_hat, const float* g_hat,

@@ -13,6 +13,7 @@
  *    outputs and the workspace (size from fs_workspace_bytes)
  *  - all work is enqueued on `stream` (a hipStream_t passed as void*) and
  *    returns without synchronising; the library keeps no mutable global state
+ *    (fs_symmetric_step_noalloc remembers, per device, the address of its built-in buffer)
  *  - return value: FS_OK or a negative FS_ERR_* code (fs_error_string names it)
  *  - flags: FS_FLAG_EXP2 is accepted for interface parity (the kernels always
  *    work in base 2, which is the same function).  Operand precision (everything
@@ -63,6 +64,7 @@ extern "C" {
 #define FS_ERR_WORKSPACE_TOO_SMALL (-4)
 #define FS_ERR_LAUNCH_FAILED (-5)
 #define FS_ERR_UNSUPPORTED (-6)
+#define FS_ERR_SCRATCH_TOO_SMALL (-7)
 
 #define FS_FLAG_EXP2 1u
 #define FS_FLAG_REDUCED_OPERANDS 2u
@@ -151,6 +153,28 @@ int fs_symmetric_step(const float* x, const float* y, const float* f_hat, const 
                       int64_t n, int64_t m, int64_t d, float eps, float alpha, float damp_f,
                       float damp_g, float coord_scale, uint32_t flags, void* workspace,
                       size_t workspace_bytes, void* stream);
+
+/*
+ * fs_symmetric_step without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  The scratch the kernels need (operand planes and
+ * partial soft-max rows) lives in a buffer of FS_NOALLOC_SCRATCH_BYTES that is part of the
+ * library's code object: every GPU the library runs on holds its own copy until the process
+ * ends.  The call allocates and frees nothing; the first call on a device looks up that
+ * device's buffer address (callers that will capture make one call before capture starts).
+ * Problems with fs_workspace_bytes(FS_OP_SYMMETRIC_STEP, n, m, d) above the buffer size return
+ * FS_ERR_SCRATCH_TOO_SMALL.  The device the pointers and the stream belong to must be the
+ * current one.  All calls on one GPU share the one buffer: calls that overlap in time on one GPU
+ * (two streams, two threads) race; calls ordered on one stream do not.  FS_FLAG_OPERANDS_PREPARED
+ * and FS_FLAG_COARSE_AUTO are ignored (every call writes its own operand planes).
+ */
+#define FS_NOALLOC_SCRATCH_BYTES ((size_t)48 << 20)
+int fs_symmetric_step_noalloc(const float* x, const float* y, const float* f_hat,
+                              const float* g_hat, const float* log_a, const float* log_b,
+                              float* f_out, float* g_out, const float* shift_x,
+                              const float* shift_y, int64_t n, int64_t m, int64_t d, float eps,
+                              float alpha, float damp_f, float damp_g, float coord_scale,
+                              uint32_t flags, void* stream);
 
 /*
  * n_steps Jacobi steps of fs_symmetric_step back to back, enqueued by one call: step s runs

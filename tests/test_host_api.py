@@ -35,6 +35,11 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
                           0, None, 0, None) == -3
     assert L.fs_apply_mat(fake, fake, fake, fake, fake, fake, fake, fake, fake, 8, 8, 4, 4, 0.1,
                           2.0, 0, 0, None, 0, None) == -3  # scale with axis=0
+    # the entry point with the built-in scratch buffer refuses what does not fit it, on the host
+    assert L.fs_workspace_bytes(_lib.OP_SYMMETRIC_STEP, 8192, 8192, 1536) > 48 << 20
+    assert L.fs_symmetric_step_noalloc(fake, fake, fake, fake, fake, fake, fake, fake, None, None,
+                                       8192, 8192, 1536, 0.1, 0.5, 1.0, 1.0, 2.0, 0, None) == -7
+    assert L.fs_error_string(-7) == b"problem too large for the built-in scratch buffer"
     # a split launch without workspace is refused, not launched
     n = m = 50000
     need = L.fs_workspace_bytes(_lib.OP_LSE, n, m, 64)
