@@ -877,8 +877,12 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   return FS_OK;
 }
 
+// Launch planning counts work items (rows x 4-column groups of the padded row) and workgroups
+// in 32-bit ints: sizes whose counts would not fit are refused.
 bool bad_sizes(int64_t n, int64_t m, int64_t d) {
-  return n <= 0 || m <= 0 || d <= 0 || n > (1 << 30) || m > (1 << 30) || d > (1 << 20);
+  if (n <= 0 || m <= 0 || d <= 0 || n > (1 << 30) || m > (1 << 30) || d > (1 << 20)) return true;
+  const int64_t dp = d <= 128 ? 128 : ((d + 1535) / 1536) * 1536;
+  return std::max(n, m) * (dp / 4) > (int64_t)INT32_MAX;
 }
 
 Side lse_side(const float* q, const float* k, const float* kb0, float kc0, const float* kb1,

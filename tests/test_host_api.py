@@ -35,6 +35,10 @@ def test_c_abi_rejects_bad_arguments_before_any_launch():
                           0, None, 0, None) == -3
     assert L.fs_apply_mat(fake, fake, fake, fake, fake, fake, fake, fake, fake, 8, 8, 4, 4, 0.1,
                           2.0, 0, 0, None, 0, None) == -3  # scale with axis=0
+    # sizes whose work-item counts overflow 32-bit launch planning (rows x padded columns / 4)
+    assert L.fs_lse(fake, fake, fake, fake, 70_000_000, 8, 128, 0.1, 2.0, 1.0, 0, None, 0, None) == -2
+    assert L.fs_lse(fake, fake, fake, fake, 8, 3_000_000, 4096, 0.1, 2.0, 1.0, 0, None, 0, None) == -2
+    assert L.fs_workspace_bytes(_lib.OP_LSE, 70_000_000, 8, 128) == 0
     # the entry point with the built-in scratch buffer refuses what does not fit it, on the host
     assert L.fs_workspace_bytes(_lib.OP_SYMMETRIC_STEP, 8192, 8192, 1536) > 48 << 20
     assert L.fs_symmetric_step_noalloc(fake, fake, fake, fake, fake, fake, fake, fake, None, None,
