@@ -17,8 +17,9 @@ operand planes, row order and kernel variant the solve used.
   algorithmic work of a launch   4*n*m*d matrix flop (2*n*m*d per half-update) + 2*n*m exp2
   executed work                  the fp16 two-plane mode runs three 16-bit MFMA products per
                                  algorithmic product; the variant with the coarse tile test ends
-                                 a 32x32 tile after its hi*hi product (1 of 3) when no logit of
-                                 it can matter, and counts such tiles on the device
+                                 a 32x32 tile after its hi*hi product (1 of 3, plus one MFMA for
+                                 the bias bound) when no logit of it can matter, and counts such
+                                 tiles on the device
   roofline.achieved              EXECUTED 16-bit MFMA flop / launch time, against the published
                                  dense fp16 peak (2516.6 TFLOP/s); roofline.frac = their ratio.
                                  roofline.algorithmic_tflops = 4*n*m*d / launch time is what a
@@ -233,14 +234,16 @@ def main():
             r.update(achieved=r["algorithmic_tflops"], peak=FP32_MFMA_PEAK_TFLOPS,
                      peak_note="published dense fp32 MFMA peak; executed = algorithmic flop")
         else:
-            # three plane products per tile; a tile that ends at the coarse test ran one, and a
-            # workgroup of that variant first runs the hi*hi product of one sampled tile per
-            # row block (as many tiles as it has first tiles, which the test does not see)
+            # three plane products per tile in the plain kernel.  The variant with the coarse tile
+            # test runs, for every tile, the hi*hi product plus one more 16-column MFMA step that
+            # carries the bias bound, and the two cross products only for tiles that go on (the
+            # few tiles per workgroup that seed the running maxima, under 1 %, are not counted).
             products = 3.0 * tiles_all
             if counts is not None and counts["tiles_tested"] > 0 and not counts["plain_selected"]:
-                products += -2.0 * counts["tiles_ended"] + (tiles_all - counts["tiles_tested"])
+                went_on = 1.0 - counts["tiles_ended"] / counts["tiles_tested"]
+                products = tiles_all * (1.0 + 16.0 / dp + 2.0 * went_on)
                 r["coarse_test"] = {
-                    "share_of_tested_tiles_ended": counts["tiles_ended"] / counts["tiles_tested"],
+                    "share_of_tested_tiles_ended": 1.0 - went_on,
                     "mfma_products_per_tile": products / tiles_all}
             executed = products * flop_per_tile_product
             r.update(achieved=executed / (ms * 1e-3) / 1e12, peak=F16_MFMA_PEAK_TFLOPS,

@@ -755,6 +755,13 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   // pipelined LSE kernel: the 16-bit plane modes take any d <= 128, the fp32 mode needs aligned rows
   const bool lse2 = vec_lse2 || (mode == kLse && !fam.sliced && (prec != 0 || (aligned && dp >= 16)));
   const int dp2 = cfg.dp;
+  // the kernel variant with the coarse tile test: asked for, or left to the device.  The device's
+  // choice lives in state that belongs to prepared planes (a call that writes its own planes
+  // would start it afresh), so without them FS_FLAG_COARSE_AUTO means the plain kernel.
+  const bool can_coarse = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && !(flags & FS_FLAG_NO_TILE_SKIP);
+  const bool coarse = (flags & FS_FLAG_COARSE_TEST) && can_coarse;
+  const bool auto_sel = (flags & FS_FLAG_COARSE_AUTO) && can_coarse && !coarse && prepared;
+  if (coarse || auto_sel) rb = 2;  // that kernel works on two row blocks per wavefront
   PlaneSet ps;
   ps.n = 0;
   ps.end = 0;
@@ -809,24 +816,21 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   if (total <= 0) return FS_OK;
 
   int rc;
-  bool auto_sel = false;
   if (fam.sliced) {
     rc = launch_sliced(mode, a, fam.nw, fam.nsl, total, st);
   } else if (lse2) {
     rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
     a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
-    const bool can_coarse = mode == kLse && prec == 3 && dp2 <= 64 && !(flags & FS_FLAG_NO_TILE_SKIP);
-    const bool coarse = (flags & FS_FLAG_COARSE_TEST) && can_coarse;
-    // device-chosen variant: both are enqueued, the one the state word names runs; the state
-    // belongs to prepared planes (a call that writes its own planes would start it afresh)
-    auto_sel = (flags & FS_FLAG_COARSE_AUTO) && can_coarse && !coarse && prepared;
+    // device-chosen variant: both are enqueued, the one the state word names runs
     if (auto_sel) {
       a.sel = select_state(ps, ws);
+      a.sel_pred = 1;
       a.sel_want = 1u;
       if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, false, false, total, st);
       a.sel_want = 0u;
       if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, false, true, total, st);
     } else if (rc == FS_OK) {
+      if (coarse && prepared) a.sel = select_state(ps, ws);  // the forced variant counts as well
       rc = launch_lse2(a, dp2, rb, prec, mode == kVec, coarse, total, st);
     }
   } else
@@ -849,7 +853,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
                        a);
     return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
   }
-  if (auto_sel && !any_split) {  // no merge launch to carry the decision
+  if (a.sel != nullptr && !any_split) {  // no merge launch to carry the decision
     hipLaunchKernelGGL((coarse_decide_kernel<0>), dim3(1), dim3(64), 0, st, a.sel);
     if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
   }

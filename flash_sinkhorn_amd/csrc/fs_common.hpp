@@ -101,11 +101,12 @@ struct LaunchArgs {
   float out_scale;  // finish_argmax_kernel: units of the partial values (1, or the plane scale)
   float skip_log2;  // lse2_kernel: tiles whose logits all lie this far (base 2, negative) below
                     // the running maxima skip their exponentials; -inf-like to switch it off
-  // lse2_kernel, variant chosen on the device: a launch with `sel` set runs only when
-  // sel[kSelWord] == sel_want (its workgroups return at once otherwise).  The variant with the
-  // coarse tile test counts its units into the slots of the same state block.
+  // Log-sum-exp kernels, variant chosen on the device: a launch with `sel` and `sel_pred` set
+  // runs only when sel[kSelWord] == sel_want (its workgroups return at once otherwise).  The
+  // variant with the coarse tile test counts its units into the slots of the same state block.
   unsigned* sel;
   unsigned sel_want;
+  int sel_pred;  // 0: the launch runs whatever the state says (it still counts into it)
 };
 
 // Device state of the variant choice (unsigned words), zeroed when the operand planes are

@@ -1,13 +1,14 @@
 // Instantiations and dispatch of the software-pipelined log-sum-exp kernel.
 #include "fs_lse2.hpp"
+#include "fs_lsecoarse.hpp"
 
 #include "fs_dispatch.hpp"
 
 namespace fs {
 
-template <int DP, int RB, int PREC, bool VEC, bool COARSE = false>
+template <int DP, int RB, int PREC, bool VEC>
 static int launch_cfg(const LaunchArgs& a, int blocks, hipStream_t st) {
-  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC, VEC, COARSE>), dim3(blocks), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((lse2_kernel<DP, RB, PREC, VEC>), dim3(blocks), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
@@ -47,18 +48,20 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
-// fp16 planes, log-sum-exp, rows of at most 64 columns: the variants with the coarse test
+// fp16 planes, log-sum-exp, rows of at most 64 columns: the pipelined kernel with the coarse
+// tile test (two blocks of 32 query rows per wavefront: the launch must be planned with rb = 2)
+template <int DP>
+static int launch_coarse_dp(const LaunchArgs& a, int blocks, hipStream_t st) {
+  hipLaunchKernelGGL((lse_coarse_kernel<DP>), dim3(blocks), dim3(256), 0, st, a);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
 static int launch_coarse(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
+  if (rb != 2) return FS_ERR_BAD_ARGUMENT;
   switch (dp) {
-    case 16:
-      return rb >= 2 ? launch_cfg<16, 2, kH3, false, true>(a, blocks, st)
-                     : launch_cfg<16, 1, kH3, false, true>(a, blocks, st);
-    case 32:
-      return rb >= 2 ? launch_cfg<32, 2, kH3, false, true>(a, blocks, st)
-                     : launch_cfg<32, 1, kH3, false, true>(a, blocks, st);
-    case 64:
-      return rb >= 2 ? launch_cfg<64, 2, kH3, false, true>(a, blocks, st)
-                     : launch_cfg<64, 1, kH3, false, true>(a, blocks, st);
+    case 16: return launch_coarse_dp<16>(a, blocks, st);
+    case 32: return launch_coarse_dp<32>(a, blocks, st);
+    case 64: return launch_coarse_dp<64>(a, blocks, st);
   }
   return FS_ERR_UNSUPPORTED;
 }

@@ -166,7 +166,7 @@ struct SoftmaxStage {
 // VEC: the plan-vector product (kVec) on the same pipeline: next to the row sums the kernel
 // keeps o_i = sum_j p_ij v_j, with v staged through LDS beside the key bias.  Two-plane modes
 // at d <= 64 only (the bias-as-accumulator-start variants).
-template <int DP, int RB, int PREC, bool VEC = false, bool COARSE = false>
+template <int DP, int RB, int PREC, bool VEC = false>
 __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   using G = Geo2<DP, PREC>;
   constexpr int NP = G::NP;
@@ -183,16 +183,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // bias MFMA (64 of 448 MFMA cycles per unit at d = 64) out of the loop.
   constexpr bool BIASC = (PREC == kH3) && KPF;
   static_assert(!VEC || BIASC, "the vector mode rides on the bias-as-accumulator-start pipeline");
-  // fp16 planes, log-sum-exp: the hi*hi product of a unit runs first and is tested before the two
-  // cross products.  |x_hi.y_lo + x_lo.y_hi| has a bound per query row that needs no look at the
-  // keys (planes hold |values| < 2^15, a lo part is at most 2^-11 of its hi part), so a unit
-  // whose hi*hi logits all lie below (running max - skip distance - bound) can end there: none
-  // of its full logits would have passed the test that lets a unit's exponentials be left out.
-  // Before its first tile such a workgroup also runs 64 keys sampled evenly from the whole key
-  // set and keeps only their largest logit per row: a key chunk that holds none of a row's
-  // near keys (rows and keys sorted by cluster) would otherwise measure its tiles against its
-  // own, far too low, maximum and skip nothing.
-  static_assert(!COARSE || (BIASC && PREC == kH3 && !VEC), "coarse test: fp16 planes, d <= 64");
   // Two-plane modes bring key tiles into LDS with direct global->LDS loads (no staging
   // registers, no ds_write): rows are unpadded and 16-byte piece p of row r sits in slot
   // p ^ swz(r), which keeps the b128 reads of 16 consecutive rows conflict free.  With the
@@ -207,7 +197,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   __shared__ __attribute__((aligned(16))) float lds_v[VEC ? NBUF : 1][VEC ? 256 : 4];  // VEC: v_j
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
-  if (args.sel != nullptr && args.sel[kSelWord] != args.sel_want) return;
+  if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;
@@ -261,29 +251,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 #pragma unroll
         for (int kk = 0; kk < G::KK16; ++kk)
           xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qrow + p * (DP / 2) + 8 * kk + 4 * h);
-    }
-  }
-
-  // COARSE: bound on the two cross products of a row, in accumulator units.  With X, Y the scaled
-  // matrices (|.| < 2^15) and hi/lo their planes: |Y_lo| <= 8 (half an ulp of [2^14, 2^15)) and
-  // |X_lo| <= 2^-11 |X_hi| (+ 2^-24 for subnormal hi), hence
-  //   sum_k |Y_lo X_hi| + |Y_hi X_lo| <= (8 + 16) * (1 + 2^-10) * sum_k |X_hi| + DP * 2^-9,
-  // rounded up generously; one base-2 unit of slack covers the fp32 roundings of the chain.
-  const bool coarse_on = COARSE && args.skip_log2 > -1.0e30f;  // wave-uniform
-  float corr[RB];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    corr[rb] = 0.f;
-    if constexpr (COARSE) {
-      float l1 = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < G::KK16; ++kk) {
-        const f16x8 hv = __builtin_bit_cast(f16x8, xq[rb][0][kk]);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) l1 += fabsf((float)hv[e]);
-      }
-      l1 += xor32(l1);
-      corr[rb] = 24.5f * l1 + (float)DP * 0x1p-9f + inv_lscale;
     }
   }
 
@@ -591,22 +558,15 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     kr.ab = h ? 1.0f : b;
   };
   // MFMA number k (0 <= k < NMAIN) of one logits tile (32 keys x 32 queries) of query block
-  // rb.  Plane products run from the lowest weight to hi*hi (COARSE: hi*hi first, it is what
-  // the early test looks at); lo*lo (2^-22) is left out.
+  // rb.  Plane products run from the lowest weight to hi*hi; lo*lo (2^-22) is left out.
   auto mfma_k = [&](int k, f32x16 acc, const KeyRegs& kr, int rb) {
     if constexpr (!kPlanes) {
       return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ya[k], xs[rb][k], acc, 0, 0, 0);
     } else {
       const int prod = k / G::KK16, kk = k % G::KK16;
       // (key plane, query plane): (lo,hi) (hi,lo) (hi,hi)
-      int pa, pb;
-      if (COARSE) {  // (hi,hi) first: it is tested before the cross products run
-        pa = (prod == 1) ? 1 : 0;
-        pb = (prod == 2) ? 1 : 0;
-      } else {
-        pa = (prod == 0) ? 1 : 0;
-        pb = (prod == 1) ? 1 : 0;
-      }
+      const int pa = (prod == 0) ? 1 : 0;
+      const int pb = (prod == 1) ? 1 : 0;
       return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kr.yq[pa][kk]),
                                                     __builtin_bit_cast(f16x8, xq[rb][pb][kk]), acc,
                                                     0, 0, 0);
@@ -687,51 +647,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     if (NBUF == 2) nxt = c;
   };
 
-  // ---- COARSE: running max of 64 keys sampled from the whole key set (sums start empty) ----
-  bool seeded = false;
-  if constexpr (COARSE) {
-    if (coarse_on) {
-      const int stride = sd.nk / G::JT;  // sampled keys: 0, stride, 2 stride, ...
-      {
-        const int j = min(tid, G::JT - 1) * stride;
-        float b = kc0 * sd.kb0[j] + (has_kb1 ? kc1 * kb1p[j] : 0.f);
-        b += (has_kb2 ? kc2 * kb2p[j] : 0.f);
-        lds_b[0][tid] = fmaxf(b, kNegBig) * inv_lscale;
-      }
-#pragma unroll
-      for (int c = 0; c < PER_THREAD; ++c) {
-        const int idx = tid + 256 * c;
-        const int r = idx / C16_PER_ROW;
-        const int piece = (idx % C16_PER_ROW) ^ swz(r);
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(krows + (size_t)(r * stride) *
-                                                                 (size_t)krow_words + piece * 4),
-            (__attribute__((address_space(3))) void*)(&lds_k[0][(c * 256 + wave * 64) * 4]), 16, 0,
-            0);
-      }
-      wait_all_vm();
-      __syncthreads();
-#pragma unroll
-      for (int js = 0; js < NSUB; ++js) {
-        load_keys(K[0], 0, js);
-        wait_lds();
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          const float m = column_max(chain(K[0], rb, 0, js));
-          run_m[rb] = js == 0 ? m : fmaxf(run_m[rb], m);
-        }
-      }
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        float c = -run_m[rb] * lscale;
-        asm volatile("" : "+v"(c));  // rounded once, see softmax()
-        run_c[rb] = c;
-      }
-      seeded = true;
-      __syncthreads();  // buffer 0 is free again
-    }
-  }
-
   // ---- prologue: tile 0 into buffer 0; with KPF tile 1 is already on its way ----
   stage_load(j_begin, 0);
   stage_store(0);
@@ -768,7 +683,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         const f32x16 acc = add_bias(chain(kr, rb, cur, js), kr, rb);
         f32x16 v16;
         if constexpr (VEC) v16 = load_v16(cur, js);
-        if (js == 0 && !seeded) softmax_first(acc, rb, v16); else softmax(acc, rb, v16);
+        if (js == 0) softmax_first(acc, rb, v16); else softmax(acc, rb, v16);
       }
     }
     if constexpr (!KPF) {
@@ -789,8 +704,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   if constexpr (BIASC) R0 = load_bias16(cur, 0);
   static_assert(!BIASC || (NSUB * RB) % 2 == 0, "units per tile must be even");
 
-  bool prev_coarse = false;  // COARSE: the previous unit ended after its hi*hi product
-  unsigned n_ended = 0;      // COARSE: units of this wavefront that ended there
   // ---- steady state: the soft-max of the previous logits tile rides between the MFMAs ----
   for (int t = 1; t < ntiles; ++t) {
     if constexpr (!KPF) stage_load(j_begin + (t + 1) * G::JT, nxt);
@@ -823,18 +736,10 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         FS_SCHED_FENCE();
         // MFMAs of piece p of this unit, the pipeline's memory traffic, and (soft) piece p
         // of the previous unit's soft-max
-        // MFMAs of piece p.  COARSE: hi*hi in pieces 0..3, nothing in 4 and 5 (the soft-max
-        // pieces there cover the wait for the test's input), the cross products in 6..11.
-        auto k_first = [](int p) {
-          if (!COARSE) return (p * NMAIN) / kPieces;
-          constexpr int HH = G::KK16;  // MFMAs of one plane product
-          return p < 4 ? (p * HH) / 4 : (p < 6 ? HH : HH + ((p - 6) * 2 * HH) / 6);
-        };
-        auto step = [&](int p, bool soft, bool mfmas = true) {
-          if (mfmas) {
+        auto k_first = [](int p) { return (p * NMAIN) / kPieces; };  // MFMAs of piece p
+        auto step = [&](int p, bool soft) {
 #pragma unroll
-            for (int k = k_first(p); k < k_first(p + 1); ++k) acc = mfma_k(k, acc, kr, rb);
-          }
+          for (int k = k_first(p); k < k_first(p + 1); ++k) acc = mfma_k(k, acc, kr, rb);
           if constexpr (KPF) {
             // LDS / global traffic of the pipeline, placed where it has the whole unit to land
             if (js == 0 && rb == 0 && p == 0) stage_store(nxt);                   // tile t+1
@@ -873,34 +778,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
           if (soft) softmax_piece(p, st, acc_prev, prev_rb, vsrc);
           FS_SCHED_FENCE();
         };
-        if constexpr (COARSE) {
-          // a previous unit that ended at the coarse stage has no soft-max at all
-#pragma unroll
-          for (int p = 0; p < kMaxPieces; ++p) step(p, !prev_coarse);
-          bool soft = false;
-          if (!prev_coarse) soft = wave_any(st.mx - run_m[prev_rb] > skip_below);
-#pragma unroll
-          for (int p = kMaxPieces; p < 6; ++p) step(p, soft);
-          bool full = true;
-          if (coarse_on) {
-            const float thr = run_m[rb] + skip_below - corr[rb];
-            const float m0 = fmaxf(fmaxf(acc[0], acc[1]), acc[2]);
-            const float m1 = fmaxf(fmaxf(acc[3], acc[4]), acc[5]);
-            const float m2 = fmaxf(fmaxf(acc[6], acc[7]), acc[8]);
-            const float m3 = fmaxf(fmaxf(acc[9], acc[10]), acc[11]);
-            const float m4 = fmaxf(fmaxf(acc[12], acc[13]), acc[14]);
-            const float m5 = fmaxf(fmaxf(m0, m1), acc[15]);
-            full = wave_any(fmaxf(m5, fmaxf(fmaxf(m2, m3), m4)) > thr);
-          }
-          FS_SCHED_FENCE();
-#pragma unroll
-          for (int p = 6; p < kPieces; ++p) step(p, soft, full);
-          if (soft) softmax_tail(st, prev_rb);
-          prev_coarse = !full;
-          n_ended += full ? 0u : 1u;
-          FS_SCHED_FENCE();
-          continue;
-        }
 #pragma unroll
         for (int p = 0; p < kMaxPieces; ++p) step(p, true);
         // Every logit of the previous unit more than 2^40 (LaunchArgs::skip_log2) below its
@@ -937,14 +814,6 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     f32x16 v16;
     if constexpr (VEC) v16 = load_v16(nx2, NSUB - 1);  // after rotate(): the tile just finished
     softmax(R1, RB - 1, v16);
-  }
-
-  if constexpr (COARSE) {  // unit counts of this wavefront for the variant choice on the device
-    if (args.sel != nullptr && lane == 0 && ntiles > 1) {
-      const int slot = blockIdx.x % kSelSlots;
-      atomicAdd(&args.sel[kSelEnded + slot], n_ended);
-      atomicAdd(&args.sel[kSelUnits + slot], (unsigned)((ntiles - 1) * NSUB * RB));
-    }
   }
 
 #pragma unroll

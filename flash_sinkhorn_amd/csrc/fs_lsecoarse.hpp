@@ -1,0 +1,528 @@
+// Log-sum-exp kernel with the coarse tile test as a software pipeline (fp16 planes, d <= 64).
+//
+// Operands are two fp16 planes (hi, lo) per matrix; a logit needs the three plane products
+// hi*hi + hi*lo + lo*hi.  The hi*hi product alone (a third of the MFMAs) already tells whether
+// a 32 x 32 logits tile can matter: with B_i a bound on the two cross products of query row i
+// (it needs no look at the keys, see `corr` below) and b~_j an upper bound of the key bias,
+//     hi*hi_ij + b~_j + B_i  <  M_i - 2^40 distance   for every i, j of the tile
+// means no logit of the tile could change the fp32 row sums, and the tile ends there.
+// The bias bound rides in the same MFMA chain: b~_j = bmax + 2^18 a_j with bmax the largest
+// bias of the 32-key sub-tile and a_j <= 0 one fp16 number per key, (b_j - bmax) / 2^18 rounded
+// towards zero, multiplied in by one more 16-column MFMA step (keys: eight copies of a_j,
+// queries: eight times 2^15); bmax itself moves to the other side of the comparison.  A unit
+// that goes on gets b_j - 2^18 a_j added in fp32, which restores the exact bias.
+//
+// A wavefront owns 64 query rows (two blocks of 32) whose planes stay in registers, and walks
+// its key chunk in 32-key sub-tiles ("unit": 32 keys x 32 queries).  One step per sub-tile s:
+//   1. the hi*hi products of the two units of sub-tile s+1 go to the matrix pipe (ten MFMAs,
+//      two independent chains), and between them in program order sit
+//   2. the tests of the two units of sub-tile s, whose products finished during the last step:
+//      a wavefront issues in order, so only work placed between MFMAs runs in their shadow;
+//   3. for a unit of s that goes on, in a block of its own: the cross products khi*qlo and
+//      klo*qhi and the exact key bias (one fp32 MFMA) on top of its hi*hi product, then the
+//      soft-max.
+// Nothing a conditional block computes outlives it except the running (maximum, sum) of the
+// rows: no accumulator tile is carried across a branch, so the register allocator never has
+// to reconcile two versions of one (four tiles hold the hi*hi products of two sub-tiles, and
+// they are only ever written unconditionally).  Only the hi plane of a sub-tile is read from
+// LDS up front (two sub-tiles ahead); a unit that goes on reads both planes and the per-key
+// biases of its sub-tile again.  The running maximum of a row starts from 64 keys sampled
+// evenly over the whole key set, so that a key chunk without any of the row's near keys is
+// measured against a meaningful maximum from its first tile on.  A unit that ends costs five
+// MFMAs, a 16-value maximum and a ballot.
+//
+// Everything LDS-related is written out by hand (ds_read / ds_write / s_waitcnt / s_barrier):
+// key tiles arrive by direct global->LDS loads two tiles ahead, and the compiler, which
+// cannot tell a read of one ring buffer from the loads still filling another, would make
+// every LDS access wait for all of them.
+#pragma once
+
+#include <type_traits>
+
+#include "fs_common.hpp"
+#include "fs_stream.hpp"
+
+namespace fs {
+
+#define FS_LC_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+template <int DP>
+__global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs args) {
+  static_assert(DP == 16 || DP == 32 || DP == 64, "two-plane rows of at most 64 columns");
+  constexpr int RB = 2;                // blocks of 32 query rows per wavefront
+  constexpr int JT = 64;               // keys per tile
+  constexpr int KK16 = DP / 16;        // MFMAs of one plane product
+  constexpr int ROWW = DP;             // 32-bit words per two-plane row
+  constexpr int PPR = ROWW / 4;        // 16-byte pieces per row
+  constexpr int PER_THREAD = JT * PPR / 256;
+  constexpr int NBUF = 4;              // ring of key tiles in LDS: tile t+3 is requested during tile t
+
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][JT * ROWW];
+  __shared__ __attribute__((aligned(16))) float lds_b[NBUF][JT + 4];  // [JT]: b_j - 2^18 a_j, then bmax of the two sub-tiles
+  __shared__ __attribute__((aligned(16))) unsigned lds_a[NBUF][JT * 4];  // eight copies of a_j (fp16) per key
+
+  // variant chosen on the device: the launch of the variant that was not chosen ends here
+  if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
+
+  int bid = blockIdx.x;
+  const bool second = bid >= args.blocks0;
+  if (second) bid -= args.blocks0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+
+  const int split = bid % sd.splits;
+  const int ig = bid / sd.splits;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int h = lane >> 5;
+  const int row0 = (ig * 4 + wave) * (32 * RB);
+  const int j_begin = split * sd.chunk;
+  const int j_end = min(sd.nk, j_begin + sd.chunk);
+  const int ntiles = (j_end - j_begin + JT - 1) / JT;
+
+  // MFMAs produce raw products of the scaled planes; lscale turns them into base-2 logits
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
+  const float inv_lscale = 1.0f / lscale;
+  const float skip_below = args.skip_log2 * inv_lscale;  // the 2^40 distance in raw units (< 0)
+
+  // ---- stationary query planes: [block][plane][16-column step] ----
+  u32x4 xq[RB][2][KK16];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = min(row0 + rb * 32 + li, sd.nq - 1);
+    const unsigned* qrow = sd.qplanes + (size_t)row * (size_t)ROWW;
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk)
+        xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qrow + p * (DP / 2) + 8 * kk + 4 * h);
+  }
+
+  // Bound on the two cross products of a row, in raw units.  With X, Y the scaled matrices
+  // (|.| < 2^15) and hi/lo their planes: |Y_lo| <= 8 (half an ulp of [2^14, 2^15)) and
+  // |X_lo| <= 2^-11 |X_hi| (+ 2^-24 for subnormal hi), hence
+  //   sum_k |Y_lo X_hi| + |Y_hi X_lo| <= (8 + 16) * (1 + 2^-10) * sum_k |X_hi| + DP * 2^-9,
+  // rounded up generously; one base-2 unit of slack covers the fp32 roundings of the chain.
+  float corr[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float l1 = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) {
+      const f16x8 hv = __builtin_bit_cast(f16x8, xq[rb][0][kk]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) l1 += fabsf((float)hv[e]);
+    }
+    l1 += xor32(l1);
+    corr[rb] = 24.5f * l1 + (float)DP * 0x1p-9f + inv_lscale;
+  }
+
+  // run_m: running maximum in raw units; run_c = -run_m * lscale as rounded once, the offset
+  // every exponent of the row uses (rescaling by differences of run_c stays consistent)
+  float run_m[RB], run_s[RB], run_c[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) run_m[rb] = run_s[rb] = run_c[rb] = 0.f;
+
+  // ---- LDS access by hand ----
+  auto lds_addr = [](const void* p) {
+    return (unsigned)(size_t)(const __attribute__((address_space(3))) void*)p;
+  };
+  auto ds_read16 = [&](const unsigned* p) -> u32x4 {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+    return v;
+  };
+  auto ds_read4 = [&](const float* p) -> float {
+    float v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+    return v;
+  };
+  auto ds_write4 = [&](float* p, float v) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(lds_addr(p)), "v"(v) : "memory");
+  };
+  auto ds_write16 = [&](unsigned* p, u32x4 v) {
+    asm volatile("ds_write_b128 %0, %1" : : "v"(lds_addr(p)), "v"(v) : "memory");
+  };
+  auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xC07F); };   // lgkmcnt(0)
+  // The compiler takes the result of a hand-written ds_read for valid right after the
+  // statement.  Passing the registers through an empty statement placed after the wait makes
+  // every later use depend on a point behind it.
+  auto pin4 = [](u32x4& v) { asm volatile("" : "+v"(v)); };
+  auto pin1 = [](float& v) { asm volatile("" : "+v"(v)); };
+  auto wait_all = [&]() { __builtin_amdgcn_s_waitcnt(0x0070); };   // vmcnt(0) and lgkmcnt(0)
+  // everything but the newest key tile has landed (loads complete in issue order), and lgkmcnt(0)
+  auto wait_older_tiles = [&]() { __builtin_amdgcn_s_waitcnt(0x0070 | PER_THREAD); };
+  auto barrier = [&]() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  auto swz = [&](int r) {  // slot permutation of LDS row r
+    return PPR >= 16 ? (r & 15) : (PPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3));
+  };
+
+  // ---- key tiles: lane idx of instruction c fills LDS slot idx and fetches the piece that
+  // belongs there (slot = piece ^ swz(row)); the plane buffers end in zero rows, so tiles past
+  // the chunk are fetched like any other and masked by their bias ----
+  const unsigned* kp[PER_THREAD];
+#pragma unroll
+  for (int c = 0; c < PER_THREAD; ++c) {
+    const int idx = tid + 256 * c;
+    const int r = idx / PPR;
+    const int piece = (idx % PPR) ^ swz(r);
+    kp[c] = sd.kplanes + (size_t)(j_begin + r) * (size_t)ROWW + piece * 4;
+  }
+  auto issue_tile = [&](int buf) {  // the next tile in sequence
+#pragma unroll
+    for (int c = 0; c < PER_THREAD; ++c) {
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)kp[c],
+          (__attribute__((address_space(3))) void*)(&lds_k[buf][(c * 256 + wave * 64) * 4]), 16, 0,
+          0);
+      kp[c] += JT * ROWW;
+    }
+  };
+
+  // ---- key bias: wavefront 0 fetches the raw terms of key j0 + lane a tile ahead and writes
+  // the combined value (raw units) and the maximum of each 32-key sub-tile before the barrier
+  // that publishes the tile ----
+  const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
+  const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
+  const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
+  const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
+  float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f;
+  bool st_live = false;
+  auto bias_load = [&](int j) {  // j: the key this lane stages (every wavefront loads, so that
+                                 // all of them count the same loads in flight; wavefront 0 stores)
+    const int jj = max(0, min(j, j_end - 1));
+    st_b0 = sd.kb0[jj];
+    st_b1 = kb1p[jj];
+    st_b2 = kb2p[jj];
+    st_live = j < j_end;
+  };
+  auto bias_store = [&](int buf) {
+    if (wave == 0) {
+      float b = kc0 * st_b0 + (has_kb1 ? kc1 * st_b1 : 0.f);
+      b += (has_kb2 ? kc2 * st_b2 : 0.f);
+      b = st_live ? fmaxf(b, kNegBig) : 2.0f * kNegBig;
+      b = fmaxf(b * inv_lscale, -3.0e38f);
+      float mx = b;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      // a_j: (b - bmax) / 2^18 as fp16, rounded towards zero (never below the true value)
+      const float rel = fmaxf((b - mx) * 0x1p-18f, -65504.0f);
+      _Float16 ah = (_Float16)rel;
+      if ((float)ah < rel)  // negative and one step too low: the next fp16 towards zero
+        ah = __builtin_bit_cast(_Float16, (unsigned short)(__builtin_bit_cast(unsigned short, ah) - 1));
+      const unsigned aw = (unsigned)__builtin_bit_cast(unsigned short, ah) * 0x00010001u;
+      ds_write16(&lds_a[buf][lane * 4], u32x4{aw, aw, aw, aw});
+      ds_write4(&lds_b[buf][lane], b - (float)ah * 0x1p18f);
+      if (li == 0) ds_write4(&lds_b[buf][JT + h], mx);
+    }
+  };
+
+  auto mfma16 = [](const u32x4& a, const u32x4& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  };
+  // 16-byte piece (plane, step kk, half h) of key row js*32 + li
+  auto read_plane = [&](u32x4 (&dst)[KK16], int buf, int js, int plane) {
+    const unsigned* yrow = lds_k[buf] + (js * 32 + li) * ROWW;
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) {
+      const int piece = plane * (DP / 8) + 2 * kk + h;
+      dst[kk] = ds_read16(yrow + ((piece ^ swz(li)) << 2));  // swz(js*32 + li) == swz(li)
+    }
+  };
+  // v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its
+  // second: (a, b) = (t, t) becomes (low half twice, high half twice)
+  auto swap_halves = [&](float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  };
+  auto max16 = [](const f32x16& a) {
+    const float m0 = fmaxf(fmaxf(a[0], a[1]), a[2]);
+    const float m1 = fmaxf(fmaxf(a[3], a[4]), a[5]);
+    const float m2 = fmaxf(fmaxf(a[6], a[7]), a[8]);
+    const float m3 = fmaxf(fmaxf(a[9], a[10]), a[11]);
+    const float m4 = fmaxf(fmaxf(a[12], a[13]), a[14]);
+    return fmaxf(fmaxf(fmaxf(m0, m1), a[15]), fmaxf(fmaxf(m2, m3), m4));
+  };
+  // the key bias of sub-tile js added to every query column: A = [bias_j, 1], B = [1, 0]
+  auto add_bias = [&](const f32x16& acc, float bias_lane) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(h ? 1.0f : bias_lane, h ? 0.0f : 1.0f, acc, 0, 0, 0);
+  };
+
+  u32x4 KH[2][KK16];  // hi planes of the sub-tile in work and the next one
+  u32x4 KA[2];        // their a_j pieces (the same piece in both half-waves)
+  // query side of the a_j step: 2^15 in the eight slots of the lower half-wave, nothing above
+  const unsigned qcw = h ? 0u : 0x78007800u;
+  const u32x4 QC = {qcw, qcw, qcw, qcw};
+  u32x4 KL[KK16];     // lo plane of the sub-tile in work, read when a unit of it goes on
+  float kbias = 0.f;  // bias of key js*32 + li of that sub-tile, read together with KL
+  float bmax[2] = {0.f, 0.f};  // largest bias of the sub-tiles whose hi planes are in KH
+
+  // ---- running maximum from 64 keys sampled over the whole key set (sums start empty) ----
+  {
+    const int stride = sd.nk / JT;  // sampled keys: 0, stride, 2 stride, ...
+    if (wave == 0) {
+      const int j = lane * stride;
+      float b = kc0 * sd.kb0[j] + (has_kb1 ? kc1 * kb1p[j] : 0.f);
+      b += (has_kb2 ? kc2 * kb2p[j] : 0.f);
+      ds_write4(&lds_b[0][lane], fmaxf(fmaxf(b, kNegBig) * inv_lscale, -3.0e38f));
+    }
+#pragma unroll
+    for (int c = 0; c < PER_THREAD; ++c) {
+      const int idx = tid + 256 * c;
+      const int r = idx / PPR;
+      const int piece = (idx % PPR) ^ swz(r);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(sd.kplanes + (size_t)(r * stride) *
+                                                                          (size_t)ROWW + piece * 4),
+          (__attribute__((address_space(3))) void*)(&lds_k[0][(c * 256 + wave * 64) * 4]), 16, 0, 0);
+    }
+    wait_all();
+    barrier();
+#pragma unroll
+    for (int js = 0; js < 2; ++js) {
+      read_plane(KH[0], 0, js, 0);
+      read_plane(KL, 0, js, 1);
+      kbias = ds_read4(&lds_b[0][js * 32 + li]);
+      wait_lds();
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk) {
+        pin4(KH[0][kk]);
+        pin4(KL[kk]);
+      }
+      pin1(kbias);
+      FS_LC_FENCE();
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK16; ++kk) acc = mfma16(KL[kk], xq[rb][0][kk], acc);
+#pragma unroll
+        for (int kk = 0; kk < KK16; ++kk) acc = mfma16(KH[0][kk], xq[rb][1][kk], acc);
+#pragma unroll
+        for (int kk = 0; kk < KK16; ++kk) acc = mfma16(KH[0][kk], xq[rb][0][kk], acc);
+        acc = add_bias(acc, kbias);
+        float a = max16(acc), b = a;
+        swap_halves(a, b);
+        const float m = fmaxf(a, b);
+        run_m[rb] = js == 0 ? m : fmaxf(run_m[rb], m);
+      }
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      float c = -run_m[rb] * lscale;
+      asm volatile("" : "+v"(c));  // the rounded product itself, nothing fused into later uses
+      run_c[rb] = c;
+    }
+    barrier();  // buffer 0 is free again
+  }
+
+  unsigned n_ended = 0;
+  f32x16 H[4];  // hi*hi products (on top of 2^18 a_j): sub-tile s, row block rb in H[2 (s & 1) + rb]
+
+  // Start of tile t: the bias of tile t+1 goes to LDS and its keys have landed (only those of
+  // tile t+2 may still be in flight); after the barrier tile t+1 is visible and every wavefront
+  // is done with tile t-1, whose buffer takes tile t+3.  The raw bias terms of tile t+2 are
+  // requested before those keys, so that the next round's wait covers them.
+  auto start_of_tile = [&](int t) {
+    bias_store((t + 1) & 3);
+    wait_older_tiles();
+    barrier();
+    bias_load(j_begin + (t + 2) * JT + lane);
+    issue_tile((t + 3) & 3);
+  };
+  // hi plane, a_j piece and bmax of sub-tile js of the tile in buffer b, into register set k
+  auto request = [&](int k, int b, int js) {
+    read_plane(KH[k], b, js, 0);
+    KA[k] = ds_read16(&lds_a[b][(js * 32 + li) * 4]);
+    bmax[k] = ds_read4(&lds_b[b][JT + js]);
+  };
+  auto arrived = [&](int k) {  // after a wait: every later use of set k sits behind this point
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) pin4(KH[k][kk]);
+    pin4(KA[k]);
+    pin1(bmax[k]);
+  };
+
+  // A unit that goes on: the two cross products and the key bias on top of its hi*hi product,
+  // then its soft-max.  Everything it computes lives and dies here.  KX: registers for the hi
+  // plane of the unit's sub-tile, read again from LDS (the set it was multiplied from has
+  // moved on to a later sub-tile).
+  auto go_on = [&](const f32x16& hh, u32x4 (&KX)[KK16], int b, int js, int rb, bool first) {
+    if (first) {  // first unit of the sub-tile to go on
+      read_plane(KX, b, js, 0);
+      read_plane(KL, b, js, 1);
+      kbias = ds_read4(&lds_b[b][js * 32 + li]);
+      wait_lds();
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk) {
+        pin4(KX[kk]);
+        pin4(KL[kk]);
+      }
+      pin1(kbias);
+    }
+    FS_LC_FENCE();
+    f32x16 L = mfma16(KX[0], xq[rb][1][0], hh);
+#pragma unroll
+    for (int kk = 1; kk < KK16; ++kk) L = mfma16(KX[kk], xq[rb][1][kk], L);
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) L = mfma16(KL[kk], xq[rb][0][kk], L);
+    L = add_bias(L, kbias);
+    FS_LC_FENCE();
+    const float mx = max16(L);  // this lane's 16 keys
+    // every logit of the unit more than the 2^40 distance below its row's running maximum:
+    // its exponentials would not change the fp32 row sums
+    if (wave_any(mx - run_m[rb] > skip_below)) {
+      float a = mx, b2 = mx;
+      swap_halves(a, b2);
+      const float m_new = fmaxf(fmaxf(a, b2), run_m[rb]);
+      float cx = -m_new * lscale;
+      asm volatile("" : "+v"(cx));  // rounded once, see run_c
+      float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        ps0 += fast_exp2(__builtin_fmaf(L[r], lscale, cx));
+        ps1 += fast_exp2(__builtin_fmaf(L[r + 1], lscale, cx));
+      }
+      run_s[rb] = run_s[rb] * fast_exp2(cx - run_c[rb]) + (ps0 + ps1);
+      run_m[rb] = m_new;
+      run_c[rb] = cx;
+    }
+  };
+
+  // One step = one 32-key sub-tile s (parity c = s & 1, in LDS buffer b): the hi*hi products of
+  // sub-tile s+1 go to the matrix pipe, with the tests of sub-tile s (whose products finished
+  // during the last step) placed between them in program order; then the units of s that go on.
+  // nb, njs: buffer and sub-tile index of s+2, whose hi plane is requested into the set that
+  // sub-tile s was multiplied from.
+  auto step = [&](auto c_c, int b, int js, int nb, int njs) {
+    constexpr int c = decltype(c_c)::value, n = c ^ 1;
+    wait_lds();  // set n (sub-tile s+1), requested during the last step
+    arrived(n);
+    const float lim = skip_below - bmax[c];  // read before the request below replaces bmax[c]
+    request(c, nb, njs);
+    FS_LC_FENCE();
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.f;
+    const f32x16& t0 = H[2 * c], &t1 = H[2 * c + 1];
+    f32x16 &a = H[2 * n], &bq = H[2 * n + 1];
+    a = mfma16(KA[n], QC, z);
+    FS_LC_FENCE();
+    const float p0 = fmaxf(fmaxf(t0[0], t0[1]), t0[2]), p1 = fmaxf(fmaxf(t0[3], t0[4]), t0[5]);
+    FS_LC_FENCE();
+    bq = mfma16(KA[n], QC, z);
+    FS_LC_FENCE();
+    const float p2 = fmaxf(fmaxf(t0[6], t0[7]), t0[8]), p3 = fmaxf(fmaxf(t0[9], t0[10]), t0[11]);
+    FS_LC_FENCE();
+    a = mfma16(KH[n][0], xq[0][0][0], a);
+    FS_LC_FENCE();
+    const float p4 = fmaxf(fmaxf(t0[12], t0[13]), t0[14]), p5 = fmaxf(fmaxf(p0, p1), t0[15]);
+    FS_LC_FENCE();
+    bq = mfma16(KH[n][0], xq[1][0][0], bq);
+    FS_LC_FENCE();
+    const float mx0 = fmaxf(p5, fmaxf(fmaxf(p2, p3), p4));
+    const bool full0 = wave_any(mx0 > run_m[0] + lim - corr[0]);
+    FS_LC_FENCE();
+    float q0 = 0.f, q1 = 0.f, q2 = 0.f, q3 = 0.f, q4 = 0.f, q5 = 0.f;
+#pragma unroll
+    for (int kk = 1; kk < KK16; ++kk) {
+      a = mfma16(KH[n][kk], xq[0][0][kk], a);
+      FS_LC_FENCE();
+      if (kk == 1) {
+        q0 = fmaxf(fmaxf(t1[0], t1[1]), t1[2]);
+        q1 = fmaxf(fmaxf(t1[3], t1[4]), t1[5]);
+        q2 = fmaxf(fmaxf(t1[6], t1[7]), t1[8]);
+      }
+      FS_LC_FENCE();
+      bq = mfma16(KH[n][kk], xq[1][0][kk], bq);
+      FS_LC_FENCE();
+      if (kk == 1) {
+        q3 = fmaxf(fmaxf(t1[9], t1[10]), t1[11]);
+        q4 = fmaxf(fmaxf(t1[12], t1[13]), t1[14]);
+        q5 = fmaxf(fmaxf(q0, q1), t1[15]);
+      }
+      FS_LC_FENCE();
+    }
+    if (KK16 == 1) {  // narrow rows: no MFMA left to sit behind
+      q0 = fmaxf(fmaxf(t1[0], t1[1]), t1[2]);
+      q1 = fmaxf(fmaxf(t1[3], t1[4]), t1[5]);
+      q2 = fmaxf(fmaxf(t1[6], t1[7]), t1[8]);
+      q3 = fmaxf(fmaxf(t1[9], t1[10]), t1[11]);
+      q4 = fmaxf(fmaxf(t1[12], t1[13]), t1[14]);
+      q5 = fmaxf(fmaxf(q0, q1), t1[15]);
+    }
+    const float mx1 = fmaxf(q5, fmaxf(fmaxf(q2, q3), q4));
+    const bool full1 = wave_any(mx1 > run_m[1] + lim - corr[1]);
+    n_ended += (full0 ? 0u : 1u) + (full1 ? 0u : 1u);
+    FS_LC_FENCE();
+    // the set that sub-tile s+1 was just multiplied from is free until the next step's request
+    if (full0) go_on(t0, KH[n], b, js, 0, true);
+    if (full1) go_on(t1, KH[n], b, js, 1, !full0);
+    FS_LC_FENCE();
+  };
+
+  // ---- prologue: tiles 0 and 1 published, tiles 2 and 3 on their way; hi*hi of sub-tile 0 ----
+  bias_load(j_begin + lane);
+  issue_tile(0);
+  issue_tile(1);
+  bias_store(0);
+  bias_load(j_begin + JT + lane);
+  issue_tile(2);
+  start_of_tile(0);
+  request(0, 0, 0);
+  request(1, 0, 1);
+  wait_lds();
+  arrived(0);
+  arrived(1);
+  FS_LC_FENCE();
+  {
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.f;
+    H[0] = mfma16(KA[0], QC, z);
+    H[1] = mfma16(KA[0], QC, z);
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) {
+      H[0] = mfma16(KH[0][kk], xq[0][0][kk], H[0]);
+      H[1] = mfma16(KH[0][kk], xq[1][0][kk], H[1]);
+    }
+  }
+  for (int t = 0; t < ntiles; ++t) {
+    if (t > 0) start_of_tile(t);
+    const int b = t & 3, nb = (t + 1) & 3;
+    step(std::integral_constant<int, 0>{}, b, 0, nb, 0);  // sub-tile 0: multiplies sub-tile 1, requests (t+1, 0)
+    step(std::integral_constant<int, 1>{}, b, 1, nb, 1);  // sub-tile 1: multiplies (t+1, 0), requests (t+1, 1)
+  }
+  wait_all();  // tiles fetched past the chunk: let them land before the workgroup ends
+
+  // unit counts of this wavefront for the variant choice on the device
+  if (args.sel != nullptr && lane == 0 && ntiles > 0) {
+    const int slot = blockIdx.x % kSelSlots;
+    atomicAdd(&args.sel[kSelEnded + slot], n_ended);
+    atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * 4));
+  }
+
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = row0 + rb * 32 + li;
+    const float s = run_s[rb] + xor32(run_s[rb]);
+    const float M2 = -run_c[rb];
+    if (row < sd.nq && h == 0) {
+      if (sd.splits == 1) {
+        epilogue_scalar(sd.ep, row, M2, s, 0.f);
+      } else {
+        const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
+      }
+    }
+  }
+}
+
+}  // namespace fs

@@ -614,10 +614,11 @@ def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
     assert info["cluster_order"]
     assert info["coarse"] == ("auto" if variant is None else variant)
     state = info["prepared"].variant_state()
-    if variant is None:  # the device looked at the first three steps and took a decision
-        assert state["decisions"] == 3 and state["tiles_tested"] > 0
-    else:
-        assert state["decisions"] == 0 and state["tiles_tested"] == 0
+    if variant is None:  # the device looked at up to three steps (it stops once it has left
+        # the coarse variant) and counted tiles
+        assert 1 <= state["decisions"] <= 3 and state["tiles_tested"] > 0
+    else:  # a forced coarse variant counts its tiles too, the plain kernel has nothing to count
+        assert (state["tiles_tested"] > 0) == variant
     for u, v in zip(got, want):
         assert rel_err(u, v.cpu().numpy()) < 2e-5
     # the self problem keeps its single half-update per step under the ordering
@@ -676,7 +677,7 @@ def test_variant_choice_on_the_device():
                 if "auto" in runs:  # same path, same bits
                     assert torch.equal(out[0], runs["auto"][0]) and torch.equal(out[1], runs["auto"][1])
             else:
-                assert st["decisions"] == 0
+                assert (st["tiles_tested"] > 0) == coarse
             runs[coarse] = out
         for k in (0, 1):
             ref = runs[False][k].cpu().numpy()
