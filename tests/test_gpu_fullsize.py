@@ -14,6 +14,11 @@ def rel_err(got, want):
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
 
 
+def _fixture(name):
+    import os
+    return np.load(os.path.join(os.path.dirname(__file__), "golden", name))
+
+
 @pytest.fixture(scope="module")
 def c3():
     x, y, a, b = make_inputs(50_000, 50_000, 64)
@@ -105,6 +110,58 @@ def test_config3_solve_variants_match_oracle_rows(c3, monkeypatch, order, coarse
     assert rel_err(g.cpu().numpy()[rows], want_g) < 1e-4
 
 
+@pytest.mark.parametrize("order,coarse", [(True, None), (True, True), (True, False), (False, None)])
+def test_config3_solve_against_the_fp64_oracle_solve(c3, monkeypatch, order, coarse):
+    """The headline solve (100 iterations at eps = 0.01, 102 Jacobi steps at n = m = 50,000,
+    d = 64) as a whole against the fp64 oracle's own 102 steps, cached in
+    tests/golden/oracle_config3.npz: loss, all four potential vectors on every row, and 256
+    sampled rows of grad_x, for every kernel variant the solver can pick."""
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    from flash_sinkhorn_amd.kernels import sinkhorn_geomloss_online_grad_sqeuclid
+    x, y, a, b, (X, Y, A, B) = c3
+    fix = _fixture("oracle_config3.npz")
+    monkeypatch.setattr(solvers, "CLUSTER_ORDER", order)
+    monkeypatch.setattr(solvers, "COARSE_TEST", coarse)
+    f, g, fp, gp = solvers.sinkhorn_flashstyle_symmetric(
+        X, Y, A, B, use_epsilon_scaling=False, eps=EPS, n_iters=100, allow_tf32=False,
+        return_prelast=True)
+    loss = float((A.double() * f.double()).sum() + (B.double() * g.double()).sum())
+    assert abs(loss - float(fix["loss"])) < 1e-4 * abs(float(fix["loss"]))
+    for got, key in ((f, "f"), (g, "g"), (fp, "f_prelast"), (gp, "g_prelast")):
+        assert rel_err(got.cpu().numpy(), fix[key]) < 1e-4, key
+    # grad_x from the solver's own pre-extrapolation potentials.  The soft-max weights at
+    # eps = 0.01 sit on a few keys with logits of order 1e5 (base 2), where fp32 resolves 0.008:
+    # (1) any fp32 evaluation of a logit carries that much noise, 1 % on an individual weight,
+    #     whichever way it is computed: `noise` below is what the dense fp32 numpy formula shows
+    #     against fp64 on the same potentials;
+    # (2) an error of 1e-6 relative in a potential moves a logit by 0.06, so the gradient of any
+    #     fp32 solve differs from the fp64 solve's by what `inherited` shows: the fp64 formula
+    #     fed with THIS solve's fp32 potentials against the fixture.
+    # The kernel is held to 1e-4 plus three times (1) against the fp64 formula on its own
+    # potentials, and to that plus (2) against the fixture.
+    rows = fix["rows"]
+    gx, _ = sinkhorn_geomloss_online_grad_sqeuclid(X, Y, A, B, fp, gp, eps=EPS, allow_tf32=False,
+                                                   compute_grad_y=False)
+    want = fix["grad_x_rows"]
+    gpn = gp.cpu().numpy().astype(np.float64)
+    c = oracle.sqeuclid_cost(x[rows], y)
+    lg = (gpn[None, :] - c) / EPS + np.log(b.astype(np.float64))[None, :]
+    w = np.exp(lg - lg.max(1, keepdims=True))
+    w /= w.sum(1, keepdims=True)
+    inherited = 2.0 * a[rows, None].astype(np.float64) * (x[rows].astype(np.float64)
+                                                          - w @ y.astype(np.float64))
+    floor = rel_err(inherited, want)
+    fp32_gx, _ = oracle.grad_barycentric(x[rows], y, a[rows], b, fp.cpu().numpy()[rows],
+                                         gp.cpu().numpy(), EPS, dtype=np.float32)
+    noise = rel_err(fp32_gx, inherited)
+    err_same, err_fix = rel_err(gx.cpu().numpy()[rows], inherited), rel_err(gx.cpu().numpy()[rows], want)
+    print(f"config3 grad_x rows: kernel vs fp64 formula on its potentials {err_same:.2e}, dense fp32 "
+          f"formula {noise:.2e}, fp64 formula on these potentials vs fixture {floor:.2e}, kernel vs "
+          f"fixture {err_fix:.2e}")
+    assert err_same < 1e-4 + 3.0 * noise
+    assert err_fix < 1e-4 + 3.0 * noise + 1.5 * floor
+
+
 def test_config2_loss_and_potentials():
     """Benchmark configuration 2 (n=m=10,000, d=64, eps=0.01, 100 iterations) against the fp64
     oracle on all rows; the oracle side is cached in tests/golden/oracle_config2.npz."""
@@ -127,10 +184,6 @@ def test_config2_loss_and_potentials():
                       n_iters=100, allow_tf32=False)(X, Y)
     assert abs(float(deb) - float(fix["loss_debiased"])) < 1e-4 * abs(float(fix["loss_debiased"]))
 
-
-def _fixture(name):
-    import os
-    return np.load(os.path.join(os.path.dirname(__file__), "golden", name))
 
 
 def test_config1_debiased_loss_and_gradient():
