@@ -144,14 +144,16 @@ def _symmetric_step_raw(x, y, f_hat, g_hat, log_a, log_b, eps, *, cost_scale, al
 
 def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale, shift_x=None,
                          shift_y=None, allow_tf32=True, use_exp2=True, prepared=None,
-                         coarse=False):
+                         coarse=False, with_previous=False):
     """``steps`` = [(eps, alpha, damping_f, damping_g), ...] run back to back by one library call
     (``fs_symmetric_steps``): the per-step host work is a kernel launch, not a Python round
-    trip.  Operands as for ``_symmetric_step_raw``; returns the potentials of the last step."""
+    trip.  Operands as for ``_symmetric_step_raw``; returns the potentials of the last step,
+    with ``with_previous`` followed by those the last step started from (its input: the two
+    work vectors alternate, so the one before last is still intact)."""
     import ctypes
     k = len(steps)
     if k == 0:
-        return f_hat, g_hat
+        return (f_hat, g_hat, f_hat, g_hat) if with_previous else (f_hat, g_hat)
     n, d = x.shape
     m = y.shape[0]
     self_problem = (y is x and g_hat is f_hat and log_b is log_a and shift_y is shift_x
@@ -172,18 +174,24 @@ def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale,
     _lib.check(rc, "fs_symmetric_steps")
     last = (k - 1) & 1
     f_out = f_work[last]
-    return f_out, (f_out if self_problem else g_work[last])
+    out = (f_out, f_out if self_problem else g_work[last])
+    if with_previous:
+        f_prev = f_work[last ^ 1] if k > 1 else f_hat
+        out = out + (f_prev, f_prev if self_problem else (g_work[last ^ 1] if k > 1 else g_hat))
+    return out
 
 
 def _self_pair_steps_raw(x, y, fx_hat, fy_hat, log_a, log_b, steps, *, cost_scale, shift_x=None,
-                         shift_y=None, allow_tf32=True, use_exp2=True, prepared=None):
+                         shift_y=None, allow_tf32=True, use_exp2=True, prepared=None,
+                         with_previous=False):
     """The self problems OT(x, x; a) and OT(y, y; b) advanced together (``fs_self_pair_steps``):
     ``steps`` = [(eps_x, eps_y, alpha, damping_x, damping_y), ...], one launch per step for both.
-    ``prepared`` must have been built with ``self_pair=True``.  Returns (fx_hat, fy_hat)."""
+    ``prepared`` must have been built with ``self_pair=True``.  Returns (fx_hat, fy_hat), with
+    ``with_previous`` followed by the pair the last step started from."""
     import ctypes
     k = len(steps)
     if k == 0:
-        return fx_hat, fy_hat
+        return (fx_hat, fy_hat, fx_hat, fy_hat) if with_previous else (fx_hat, fy_hat)
     n, d = x.shape
     m = y.shape[0]
     fx_work = [torch.empty((n,), device=x.device, dtype=torch.float32) for _ in range(2)]
@@ -207,7 +215,10 @@ def _self_pair_steps_raw(x, y, fx_hat, fy_hat, log_a, log_b, steps, *, cost_scal
         k, 2.0 * float(cost_scale), fl, wp, wn, _lib.stream_of(x))
     _lib.check(rc, "fs_self_pair_steps")
     last = (k - 1) & 1
-    return fx_work[last], fy_work[last]
+    out = (fx_work[last], fy_work[last])
+    if with_previous:
+        out = out + ((fx_work[last ^ 1], fy_work[last ^ 1]) if k > 1 else (fx_hat, fy_hat))
+    return out
 
 
 def flashsinkhorn_symmetric_step(

@@ -13,7 +13,7 @@ from typing import Optional, Sequence, Tuple
 
 import torch
 
-from flash_sinkhorn_amd import _lib
+from flash_sinkhorn_amd import _graphs, _lib
 from flash_sinkhorn_amd.kernels._common import (
     _f32c, augment_label_cost, dampening, epsilon_schedule, label_cost_active, log_weights,
     max_diameter,
@@ -253,8 +253,14 @@ def sinkhorn_flashstyle_symmetric(
                                       g_hat[perm_y])
         coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
 
-    # operand planes are converted once for the whole loop
-    prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32))
+    # operand planes are converted once for the whole loop, when the first launch needs them
+    # (a run replayed from a graph has planes of its own)
+    made = []
+
+    def planes():
+        if not made:
+            made.append(_lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32)))
+        return made[0]
 
     def jacobi(f_hat, g_hat, e, w):
         damp_f, damp_g = dampening(e, rho_x), dampening(e, rho_y)
@@ -263,10 +269,10 @@ def sinkhorn_flashstyle_symmetric(
                 xf, yf, f_hat, g_hat, log_a, log_b, e, cost_scale=cost_scale, alpha=w,
                 damping_f=damp_f, damping_g=damp_g,
                 shift_x=alpha if damp_f < 1.0 else None, shift_y=beta if damp_g < 1.0 else None,
-                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=coarse)
+                allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=planes(), coarse=coarse)
         # two launches, raw-bias kernel, averaging and shift correction on the host
         kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
-                  _prepared=prepared)
+                  _prepared=planes())
         f_c = flashsinkhorn_lse(xf, yf, (g_hat + e * log_b) / e, e, damping=damp_f, **kw)
         g_c = flashsinkhorn_lse(yf, xf, (f_hat + e * log_a) / e, e, damping=damp_g, **kw)
         if damp_f < 1.0:
@@ -277,47 +283,82 @@ def sinkhorn_flashstyle_symmetric(
             return f_c, g_c
         return (1.0 - w) * f_hat + w * f_c, (1.0 - w) * g_hat + w * g_c
 
-    def jacobi_run(f_hat, g_hat, run):
-        """Consecutive steps [(eps, weight), ...]: one library call when fused."""
+    def jacobi_run(f_hat, g_hat, run, with_previous=False):
+        """Consecutive steps [(eps, weight), ...]: one library call when fused, replayed from a
+        HIP graph on small problems (``_graphs``).  ``with_previous``: also the potentials the
+        last step started from."""
         if not fused:
+            f_prev, g_prev = f_hat, g_hat
             for e, w in run:
+                f_prev, g_prev = f_hat, g_hat
                 f_hat, g_hat = jacobi(f_hat, g_hat, e, w)
-            return f_hat, g_hat
-        steps = [(e, w, dampening(e, rho_x), dampening(e, rho_y)) for e, w in run]
-        return _symmetric_steps_raw(
-            xf, yf, f_hat, g_hat, log_a, log_b, steps, cost_scale=cost_scale,
-            shift_x=alpha if rho_x is not None else None,
-            shift_y=beta if rho_y is not None else None,
-            allow_tf32=allow_tf32, use_exp2=use_exp2, prepared=prepared, coarse=coarse)
+            return (f_hat, g_hat, f_prev, g_prev) if with_previous else (f_hat, g_hat)
+        steps = tuple((e, w, dampening(e, rho_x), dampening(e, rho_y)) for e, w in run)
+        shift_x = alpha if rho_x is not None else None
+        shift_y = beta if rho_y is not None else None
+        kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
+                  with_previous=with_previous)
+        if coarse is False and _graphs.eligible(xf.shape[0], yf.shape[0], len(steps), xf.device):
+            aliased = yf is xf and log_b is log_a and g_hat is f_hat and beta is alpha
+            flag_bits = _lib.flags(use_exp2, allow_tf32)
+
+            def enqueue(xs, ys, fs, gs, las, lbs, sx, sy):
+                if aliased:
+                    ys, gs, lbs, sy = xs, fs, las, sx
+                own = _lib.PreparedOperands(xs, ys, flag_bits)
+                out = _symmetric_steps_raw(xs, ys, fs, gs, las, lbs, steps, shift_x=sx,
+                                           shift_y=sy, prepared=own, **kw)
+                return out[0::2] if aliased else out  # one vector per pair when both are one
+
+            key = ("symmetric", xf.device.index, tuple(xf.shape), tuple(yf.shape), steps,
+                   float(cost_scale), shift_x is not None, shift_y is not None, flag_bits, aliased,
+                   with_previous)
+            none = None
+            out = _graphs.run(key, enqueue, [
+                xf, none if aliased else yf, f_hat, none if aliased else g_hat, log_a,
+                none if aliased else log_b, shift_x, none if aliased else shift_y])
+            if aliased:
+                out = tuple(t for t in out for _ in (0, 1))
+            return out
+        return _symmetric_steps_raw(xf, yf, f_hat, g_hat, log_a, log_b, steps, shift_x=shift_x,
+                                    shift_y=shift_y, prepared=planes(), coarse=coarse, **kw)
 
     # the initial full step and the averaged steps, cut where a convergence check looks at
     # the potentials
     used = 0
     prev_f = prev_g = None
-    run = [(eps_list[0], 1.0)]
-    for idx, e in enumerate(eps_list):
-        run.append((e, 0.5))
-        check = threshold is not None and (idx + 1) % check_every == 0
-        if check or idx + 1 == len(eps_list):
-            f_hat, g_hat = jacobi_run(f_hat, g_hat, run)
-            used += len(run)
-            run = []
-        if check:
-            if prev_f is not None and _max_change(f_hat, g_hat, prev_f, prev_g) < threshold:
-                break
-            prev_f, prev_g = f_hat.clone(), g_hat.clone()
-
     f_prelast = g_prelast = None
-    if last_extrapolation:
-        f_prelast, g_prelast = f_hat + alpha, g_hat + beta
-        f_hat, g_hat = jacobi(f_hat, g_hat, eps_list[-1], 1.0)
-        used += 1
+    run = [(eps_list[0], 1.0)]
+    if threshold is None and last_extrapolation:
+        # nothing looks at the potentials on the way: the whole solve, extrapolation step
+        # included, is one run (one library call, or one graph replay)
+        run += [(e, 0.5) for e in eps_list] + [(eps_list[-1], 1.0)]
+        f_hat, g_hat, f_pre, g_pre = jacobi_run(f_hat, g_hat, run, with_previous=True)
+        f_prelast, g_prelast = f_pre + alpha, g_pre + beta
+        used = len(run)
+    else:
+        for idx, e in enumerate(eps_list):
+            run.append((e, 0.5))
+            check = threshold is not None and (idx + 1) % check_every == 0
+            if check or idx + 1 == len(eps_list):
+                f_hat, g_hat = jacobi_run(f_hat, g_hat, run)
+                used += len(run)
+                run = []
+            if check:
+                if prev_f is not None and _max_change(f_hat, g_hat, prev_f, prev_g) < threshold:
+                    break
+                prev_f, prev_g = f_hat.clone(), g_hat.clone()
+        if last_extrapolation:
+            f_prelast, g_prelast = f_hat + alpha, g_hat + beta
+            f_hat, g_hat = jacobi(f_hat, g_hat, eps_list[-1], 1.0)
+            used += 1
 
     out = (f_hat + alpha, g_hat + beta)
     if return_prelast and last_extrapolation:
         out = out + (f_prelast, g_prelast)
     if solve_info is not None:
-        solve_info.update(cluster_order=inv_x is not None, coarse=coarse, prepared=prepared)
+        solve_info.update(cluster_order=inv_x is not None, coarse=coarse,
+                          prepared=made[0] if made else None)
     if inv_x is not None:  # back to the caller's row order
         out = tuple(t[inv_x if i % 2 == 0 else inv_y] for i, t in enumerate(out))
     if return_n_iters:
@@ -369,13 +410,28 @@ def sinkhorn_flashstyle_symmetric_self_pair(
     fx, fy = -alpha_x, -alpha_y
     shift_x = alpha_x if rho is not None else None
     shift_y = alpha_y if rho is not None else None
-    prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32), self_pair=True)
+    flag_bits = _lib.flags(use_exp2, allow_tf32)
     kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
+    made = []
 
-    def pair(fx, fy, steps):  # steps: [(eps_x, eps_y, weight)]
-        full = [(e1, e2, w, dampening(e1, rho), dampening(e2, rho)) for e1, e2, w in steps]
+    def pair(fx, fy, steps, with_previous=False):  # steps: [(eps_x, eps_y, weight)]
+        full = tuple((e1, e2, w, dampening(e1, rho), dampening(e2, rho)) for e1, e2, w in steps)
+        if _graphs.eligible(max(xf.shape[0], yf.shape[0]), max(xf.shape[0], yf.shape[0]),
+                            len(full), xf.device):
+            def enqueue(xs, ys, fxs, fys, las, lbs, sxs, sys_):
+                own = _lib.PreparedOperands(xs, ys, flag_bits, self_pair=True)
+                return _self_pair_steps_raw(xs, ys, fxs, fys, las, lbs, full, shift_x=sxs,
+                                            shift_y=sys_, prepared=own,
+                                            with_previous=with_previous, **kw)
+
+            key = ("self pair", xf.device.index, tuple(xf.shape), tuple(yf.shape), full,
+                   float(cost_scale), shift_x is not None, flag_bits, with_previous)
+            return _graphs.run(key, enqueue, [xf, yf, fx, fy, log_a, log_b, shift_x, shift_y])
+        if not made:  # operand planes of both clouds, converted once for the whole loop
+            made.append(_lib.PreparedOperands(xf, yf, flag_bits, self_pair=True))
         return _self_pair_steps_raw(xf, yf, fx, fy, log_a, log_b, full, shift_x=shift_x,
-                                    shift_y=shift_y, prepared=prepared, **kw)
+                                    shift_y=shift_y, prepared=made[0],
+                                    with_previous=with_previous, **kw)
 
     def alone(pts, f, log_w, shift, steps):  # steps: [(eps, weight)]
         full = [(e, w, dampening(e, rho), dampening(e, rho)) for e, w in steps]
@@ -385,16 +441,21 @@ def sinkhorn_flashstyle_symmetric_self_pair(
     sx = [(ex[0], 1.0)] + [(e, 0.5) for e in ex]
     sy = [(ey[0], 1.0)] + [(e, 0.5) for e in ey]
     k = min(len(sx), len(sy))
-    fx, fy = pair(fx, fy, [(sx[i][0], sy[i][0], sx[i][1]) for i in range(k)])
-    if len(sx) > k:
-        fx = alone(xf, fx, log_a, shift_x, sx[k:])
-    if len(sy) > k:
-        fy = alone(yf, fy, log_b, shift_y, sy[k:])
-
     pre_x = pre_y = None
-    if last_extrapolation:
-        pre_x, pre_y = fx + alpha_x, fy + alpha_y
-        fx, fy = pair(fx, fy, [(ex[-1], ey[-1], 1.0)])
+    both = [(sx[i][0], sy[i][0], sx[i][1]) for i in range(k)]
+    if len(sx) == len(sy) and last_extrapolation:
+        # equal schedules: the whole solve, extrapolation step included, is one run
+        fx, fy, px, py = pair(fx, fy, both + [(ex[-1], ey[-1], 1.0)], with_previous=True)
+        pre_x, pre_y = px + alpha_x, py + alpha_y
+    else:
+        fx, fy = pair(fx, fy, both)
+        if len(sx) > k:
+            fx = alone(xf, fx, log_a, shift_x, sx[k:])
+        if len(sy) > k:
+            fy = alone(yf, fy, log_b, shift_y, sy[k:])
+        if last_extrapolation:
+            pre_x, pre_y = fx + alpha_x, fy + alpha_y
+            fx, fy = pair(fx, fy, [(ex[-1], ey[-1], 1.0)])
     out_x = (fx + alpha_x,) * 2
     out_y = (fy + alpha_y,) * 2
     if return_prelast and last_extrapolation:

@@ -682,3 +682,54 @@ def test_variant_choice_on_the_device():
         for k in (0, 1):
             ref = runs[False][k].cpu().numpy()
             assert rel_err(runs["auto"][k], ref) < 2e-6 and rel_err(runs[True][k], ref) < 2e-6
+
+
+def test_graph_replays_equal_eager_solves(monkeypatch):
+    """Small solves are captured into a HIP graph on their second call and replayed afterwards.
+    Every call (eager, capturing, replaying) is compared with the launch-by-launch solve of the
+    same inputs, bit for bit, with eager work and synchronisations between the calls and fresh
+    input values each time; then the same through SamplesLoss(debias=True) with a backward pass
+    (xy solve and the paired self solves, each with a graph of its own)."""
+    from flash_sinkhorn_amd import SamplesLoss, _graphs
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    rng = np.random.default_rng(41)
+    n, m, d = 700, 650, 5
+    kw = dict(use_epsilon_scaling=False, eps=0.05, n_iters=12, allow_tf32=False, return_prelast=True)
+    _graphs.clear()
+    scratch = torch.zeros(1 << 16, device="cuda")
+    for call in range(5):
+        x, y, a, b = inputs(50 + call, n, m, d)
+        X, Y, A, B = dev(x, y, a, b)
+        monkeypatch.setattr(_graphs, "ENABLED", False)
+        want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+        want_self = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, reach=1.2, **kw)
+        monkeypatch.setattr(_graphs, "ENABLED", True)
+        got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+        scratch.add_(1.0).mul_(0.5)  # unrelated eager work between replays
+        torch.cuda.synchronize()
+        got_self = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, reach=1.2, **kw)
+        for u, v in zip(got + got_self, want + want_self):
+            assert torch.equal(u, v), call
+    keys = [k[0] for k in _graphs._cache]
+    assert keys.count("symmetric") == 2 and all(e.graph is not None for e in _graphs._cache.values())
+    # through the public loss: value and gradient, replay after replay
+    loss_fn = SamplesLoss("sinkhorn", blur=0.2, debias=True, use_epsilon_scaling=False, eps=0.04,
+                          n_iters=10, allow_tf32=False)
+    for call in range(4):
+        x, y, _, _ = inputs(70 + call, n, n, d)
+        outs = []
+        for enabled in (False, True):
+            monkeypatch.setattr(_graphs, "ENABLED", enabled)
+            X = torch.from_numpy(x).cuda().requires_grad_(True)
+            Y = torch.from_numpy(y).cuda()
+            loss = loss_fn(X, Y)
+            (gx,) = torch.autograd.grad(loss, X)
+            torch.cuda.synchronize()
+            outs.append((loss.detach(), gx))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1]), call
+    assert any(k[0] == "self pair" for k in _graphs._cache)
+    x, y, a, b = oracle_small = inputs(90, n, m, d)
+    f, g, fp, gp = solvers.sinkhorn_flashstyle_symmetric(*dev(x, y, a, b), **kw)  # a replay
+    wf, wg, wfp, wgp = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=0.05,
+                                                 n_iters=12, return_prelast=True)
+    assert rel_err(f, wf) < RTOL and rel_err(g, wg) < RTOL and rel_err(fp, wfp) < RTOL
