@@ -48,6 +48,7 @@ _SIGNATURES = {
     "fs_workspace_bytes": (_Z, [ctypes.c_int, _I, _I, _I]),
     "fs_prepare_operands": (ctypes.c_int, [_P] * 2 + [_I] * 3 + _TAIL),
     "fs_variant_state_offset": (_Z, [_P] * 2 + [_I] * 3 + [_U]),
+    "fs_best_keys_offset": (_Z, [_P] * 2 + [_I] * 3 + [_U, ctypes.c_int]),
     "fs_lse": (ctypes.c_int, [_P] * 4 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_lse_fused": (ctypes.c_int, [_P] * 5 + [_I] * 3 + [_F] * 3 + _TAIL),
     "fs_symmetric_step": (ctypes.c_int, [_P] * 10 + [_I] * 3 + [_F] * 5 + _TAIL),
@@ -155,9 +156,20 @@ class PreparedOperands:
         self.d = d
         self.state_offset = int(L.fs_variant_state_offset(x.data_ptr(), y.data_ptr(), n, m, d,
                                                           flag_bits))
+        self._keys_at = [(int(L.fs_best_keys_offset(x.data_ptr(), y.data_ptr(), n, m, d, flag_bits, w)),
+                          rows) for w, rows in ((0, n), (1, m))]
         check(L.fs_prepare_operands(x.data_ptr(), y.data_ptr(), n, m, d, flag_bits,
                                     self.ws.data_ptr(), nbytes, stream_of(x)),
               "fs_prepare_operands")
+
+    def best_keys(self, which: int) -> Optional[torch.Tensor]:
+        """View (int32, one entry per row of x for ``which`` = 0, of y for 1) of the keys the
+        kernel with the coarse tile test starts its rows from; None when the configuration keeps
+        none.  Whatever a caller writes there, results stay exact: a diagnostic and test hook."""
+        off, rows = self._keys_at[which]
+        if off == 0:
+            return None
+        return self.ws[off:off + 4 * rows].view(torch.int32)
 
     def variant_state(self) -> dict:
         """What ``FS_FLAG_COARSE_AUTO`` has done on these planes so far (reads the device: a

@@ -121,7 +121,7 @@ SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam, int rb_f
 size_t side_ws_floats(int mode, const SidePlan& p, int64_t nq, int dp) {
   if (p.splits <= 1) return 0;
   size_t f = (size_t)p.splits * (size_t)nq * 2;
-  if (mode == kVec) f += (size_t)p.splits * (size_t)nq;
+  if (mode == kVec || mode == kLse) f += (size_t)p.splits * (size_t)nq;  // kLse: Side::part_best
   if (mode == kMat || mode == kMat5) f += (size_t)p.splits * (size_t)nq * (size_t)dp;
   return (f + 3) & ~(size_t)3;  // keep the next region 16-byte aligned
 }
@@ -196,8 +196,14 @@ struct PlaneSet {
   size_t aux_off, end;
 };
 
-size_t plane_bytes(int64_t rows, const LseConfig& c) {
+// Bytes of one matrix's planes alone, and of its whole region: the planes, then one int per row
+// (the key behind the row's largest logit, kept from launch to launch of lse_coarse_kernel).
+size_t planes_only_bytes(int64_t rows, const LseConfig& c) {
   return (((size_t)(rows + kPlanePadRowsApi) * (size_t)c.np * (size_t)(c.dp / 2) * 4) + 15) & ~(size_t)15;
+}
+
+size_t plane_bytes(int64_t rows, const LseConfig& c) {
+  return planes_only_bytes(rows, c) + (((size_t)rows * sizeof(int) + 15) & ~(size_t)15);
 }
 
 // Distinct (pointer, rows) operands among up to four candidates, in canonical order.
@@ -250,6 +256,13 @@ const unsigned* plane_of(const PlaneSet& ps, void* ws, const float* src, int row
   return nullptr;
 }
 
+int* best_keys_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float* src, int rows) {
+  for (int i = 0; i < ps.n; ++i)
+    if (ps.src[i] == src && ps.rows[i] == rows)
+      return reinterpret_cast<int*>(static_cast<char*>(ws) + ps.off[i] + planes_only_bytes(rows, c));
+  return nullptr;
+}
+
 // Writes the planes (and, for fp16, the scales) of every matrix of the set.
 int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws, hipStream_t st) {
   if (ps.n == 0) return FS_OK;
@@ -265,7 +278,8 @@ int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws
       rc = launch_split_planes_f16(ps.src[i], reinterpret_cast<unsigned*>(base + ps.off[i]),
                                    ps.rows[i], (int)d, c.dp, partial + 256 * i, scales + i,
                                    two ? nullptr : scales + 1, c.gemm ? 1 : 0,
-                                   i == 0 ? select_state(ps, ws) : nullptr, st);
+                                   i == 0 ? select_state(ps, ws) : nullptr,
+                                   best_keys_of(ps, c, ws, ps.src[i], ps.rows[i]), st);
   }
   return rc;
 }
@@ -525,7 +539,7 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
       rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
-                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, nullptr, st);
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, nullptr, nullptr, st);
   }
   if (rc == FS_OK) rc = launch_plan_gemm(a, mat5, cb, total, st);
   if (rc != FS_OK) return rc;
@@ -663,7 +677,7 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     if (rc == FS_OK) rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
       rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
-                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, nullptr, st);
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, nullptr, nullptr, st);
   }
   for (int s = 0; s < nsides && rc == FS_OK && has_o; ++s) {
     const Side& sd = sides[s];
@@ -704,15 +718,16 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
 size_t pt_ws_bytes(int mode, int64_t n, int64_t m, int64_t d, bool both, bool either,
                    const Family& fam) {
   const int dpk = std::max(padded_d(d), 16);
-  const size_t planes =
-      (size_t)(n + m + 2 * kPlanePadRowsApi) * 2 * (dpk / 2) * 4 + 64 + kPlaneAuxBytes;
+  LseConfig c;
+  c.gemm = false; c.prec = 3; c.dp = dpk; c.np = 2;
+  const size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes;
   auto side = [&](int64_t nq, int64_t nk) {
     size_t b = 0;
     for (int rb = 1; rb <= 2; ++rb)
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dpk) * sizeof(float));
     if (mode == kMat || mode == kMat5) b += pt_vt_bytes(nk, dpk) + kPgAuxBytes;
     if (mode == kMat5)  // planes of the second operand, aux, row bounds
-      b += (size_t)(nq + kPlanePadRowsApi) * 2 * (dpk / 2) * 4 + kPlaneAuxBytes + ((size_t)nq + 64) * 4 + 64;
+      b += plane_bytes(nq, c) + kPlaneAuxBytes + ((size_t)nq + 64) * 4 + 64;
     return b + 16;
   };
   if (both) return planes + side(n, m) + side(m, n) + 64;
@@ -786,6 +801,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     sd.splits = p.splits;
     sd.chunk = p.chunk;
     sd.igroups = p.igroups;
+    sd.best_key = nullptr;
+    sd.part_best = nullptr;
     sd.part_ms = nullptr;
     sd.part_o = nullptr;
     if (p.splits > 1) {
@@ -793,6 +810,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       sd.part_ms = wsp;
       size_t off = (size_t)p.splits * (size_t)sd.nq * 2;
       if (mode != kLse) sd.part_o = wsp + ((off + 3) & ~(size_t)3);
+      else sd.part_best = reinterpret_cast<int*>(wsp + off);
       wsp += side_ws_floats(mode, p, sd.nq, dp);
     }
     vec_ok = vec_ok && aligned16(sd.q) && aligned16(sd.k) && aligned16(sd.ep.out);
@@ -805,6 +823,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       sd.plane_scale = plane_scales(ps, ws);
       sd.ps_q = plane_index(ps, sd.q, sd.nq);
       sd.ps_k = plane_index(ps, sd.k, sd.nk);
+      if (coarse || auto_sel) sd.best_key = best_keys_of(ps, cfg, ws, sd.q, sd.nq);
     }
     a.side[s] = sd;
   }
@@ -959,8 +978,11 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     return b * sizeof(float);
   };
   size_t planes = 0;  // two fp16 planes of x and y for the pipelined LSE kernel
-  if (mode == kLse && !fam.sliced)
-    planes = (size_t)(n + m + 2 * kPlanePadRowsApi) * 2 * (std::max(dp, 16) / 2) * 4 + 64 + kPlaneAuxBytes;
+  if (mode == kLse && !fam.sliced) {
+    LseConfig c;
+    c.gemm = false; c.prec = 3; c.dp = std::max(dp, 16); c.np = 2;
+    planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes;
+  }
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
@@ -997,6 +1019,19 @@ size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_
   PlaneSet ps;
   if (make_plane_set(ptrs, rows, 2, cfg, ps) != FS_OK || ps.n == 0) return 0;
   return ps.aux_off + (2 * 256 + 8) * sizeof(float);
+}
+
+size_t fs_best_keys_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
+                           uint32_t flags, int which) {
+  if (!x || !y || bad_sizes(n, m, d) || d > kMaxSlicedD || (which != 0 && which != 1)) return 0;
+  const LseConfig cfg = lse_config(d, flags);
+  if (cfg.gemm || cfg.dp > 64) return 0;
+  const float* ptrs[2] = {x, y};
+  const int rows[2] = {(int)n, (int)m};
+  PlaneSet ps;
+  if (make_plane_set(ptrs, rows, 2, cfg, ps) != FS_OK || ps.n == 0) return 0;
+  const int i = plane_index(ps, ptrs[which], rows[which]);
+  return ps.off[i] + planes_only_bytes(rows[which], cfg);
 }
 
 int fs_lse(const float* x, const float* y, const float* bias, float* out, int64_t n, int64_t m,

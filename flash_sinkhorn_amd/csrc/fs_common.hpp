@@ -87,6 +87,12 @@ struct Side {
   const float* q2norm2;        // mat5: |q2_i|^2 per row [nq]
   const float* kmax2;          // mat5: 64 partial maxima of |k_j|^2
   float* part_ms;       // [splits, nq, 2] partial (M, s) when splits > 1
+  // lse_coarse_kernel: per query row, the key that held the row's largest logit in the last
+  // launch over these operands (-1: none yet).  The current logit of that key is where the
+  // row's running maximum starts: a lower bound of the new maximum whatever the entry holds.
+  int* best_key;        // [nq] or null
+  int* part_best;       // [splits, nq] when splits > 1: the key behind a partial M, -1 when no
+                        // key of the chunk exceeded the starting value
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;
 };
@@ -115,11 +121,13 @@ struct LaunchArgs {
 constexpr int kSelWord = 0, kSelDecisions = 1, kSelCumEnded = 2, kSelCumUnits = 4;  // totals: u64
 constexpr int kSelSlots = 64, kSelEnded = 8, kSelUnits = kSelEnded + kSelSlots;
 constexpr int kSelWords = kSelUnits + kSelSlots;
-constexpr unsigned kSelDecideSteps = 3;  // the first launches of the coarse variant decide
+constexpr unsigned kSelDecideSteps = 3;  // which counted launch of the coarse variant decides
 constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
 
-// One wavefront: add the launch's counters to the totals, clear them, and while decisions are
-// still open leave the coarse variant when too few units ended at its test.
+// One wavefront: add the launch's counters to the totals and clear them.  Only workgroups whose
+// rows all started from a key of the previous launch count, and the share of ended units climbs
+// over the first launches that have such keys: the kSelDecideSteps-th launch with counts decides,
+// and leaves the coarse variant when too few of its units ended at the test.
 __device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
   unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane];
   st[kSelEnded + lane] = 0u;
@@ -134,9 +142,11 @@ __device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
     unsigned long long* cum = reinterpret_cast<unsigned long long*>(st + kSelCumEnded);
     cum[0] += es;
     cum[1] += us;
-    if (st[kSelDecisions] < kSelDecideSteps) {
-      st[kSelDecisions] += 1u;
-      if (es * 100ull < us * (unsigned long long)kSelMinPercent) st[kSelWord] = 1u;
+    const unsigned seen = st[kSelDecisions];
+    if (seen < kSelDecideSteps) {  // the share of the last of these launches decides
+      st[kSelDecisions] = seen + 1u;
+      if (seen + 1u == kSelDecideSteps && es * 100ull < us * (unsigned long long)kSelMinPercent)
+        st[kSelWord] = 1u;
     }
   }
 }

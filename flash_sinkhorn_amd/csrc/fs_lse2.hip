@@ -40,11 +40,11 @@ int launch_absmax(const float* a, long long na, const float* b, long long nb, fl
 
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
-                            int chunked, unsigned* clear_state, hipStream_t st) {
+                            int chunked, unsigned* clear_state, int* best_keys, hipStream_t st) {
   const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
   const int grid = (int)((items + 255) / 256);
   hipLaunchKernelGGL(split_planes_f16_kernel, dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp,
-                     partial_max, scale_out, scale_out2, chunked, clear_state);
+                     partial_max, scale_out, scale_out2, chunked, clear_state, best_keys);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

@@ -92,12 +92,14 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ a
 // x[rows, d] (fp32) -> two packed fp16 planes [rows + kPlanePadRows][2][DP/2] of scale*x, zero
 // padded to DP columns and in the trailing rows.  scale is derived from the partial maxima of
 // absmax_kernel; block 0 also publishes it in *scale_out for the consuming kernel and clears
-// the kSelWords words at `clear_state` (the variant-choice state that belongs to the planes).
+// the kSelWords words at `clear_state` (the variant-choice state that belongs to the planes);
+// `best_keys` (one int per row, may be null) is reset to -1.
 // With `chunked` the two planes are interleaved per 32 columns (layout of lse_gemm_kernel).
 __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     const float* __restrict__ src, unsigned* __restrict__ dst, int rows, int d, int dp,
     const float* __restrict__ partial_max, float* __restrict__ scale_out,
-    float* __restrict__ scale_out2, int chunked, unsigned* __restrict__ clear_state) {
+    float* __restrict__ scale_out2, int chunked, unsigned* __restrict__ clear_state,
+    int* __restrict__ best_keys) {
   __shared__ float red[4];
   float m = partial_max[threadIdx.x];  // kAbsmaxBlocks == blockDim.x
 #pragma unroll
@@ -113,6 +115,7 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
 
   const int per_row = dp / 4;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (best_keys != nullptr && idx < rows) best_keys[idx] = -1;  // new planes: no key known yet
   if (idx >= (long long)(rows + kPlanePadRows) * per_row) return;
   const int r = (int)(idx / per_row);
   const int c4 = (int)(idx % per_row) * 4;

@@ -262,8 +262,53 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   float kbias = 0.f;  // bias of key js*32 + li of that sub-tile, read together with KL
   float bmax[2] = {0.f, 0.f};  // largest bias of the sub-tiles whose hi planes are in KH
 
-  // ---- running maximum from 64 keys sampled over the whole key set (sums start empty) ----
-  {
+  // ---- where the running maxima start (sums start empty) ----
+  // A row whose largest logit of the last launch sat at key j starts from its current logit at
+  // j, computed here on the vector pipe from the same planes: whatever the potentials did since,
+  // this is a logit of the row, hence a lower bound of its new maximum, and close to it once
+  // the potentials settle.  (Any index inside the key set keeps the result exact; a stale one
+  // only costs tests that pass.)  The sum of the fp32 roundings of the two routes to a logit is
+  // far below corr / 64, which is taken off together with one base-2 unit.
+  const bool track = sd.best_key != nullptr;
+  int best_j[RB];
+  float warm[RB];
+  bool have = track;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    best_j[rb] = -1;
+    warm[rb] = -3.0e38f;
+    if (track) {
+      const int row = min(row0 + rb * 32 + li, sd.nq - 1);
+      const int j = sd.best_key[row];
+      have = have && j >= 0;
+      const int jc = min(max(j, 0), sd.nk - 1);
+      const unsigned* krow = sd.kplanes + (size_t)jc * (size_t)ROWW + 4 * h;
+      float dot = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk) {
+        const u32x4 khi = *reinterpret_cast<const u32x4*>(krow + 8 * kk);
+        const u32x4 klo = *reinterpret_cast<const u32x4*>(krow + DP / 2 + 8 * kk);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          // (words copied out first: a bit cast applied to a vector element reads element 0)
+          const unsigned khw = khi[w], klw = klo[w], qhw = xq[rb][0][kk][w], qlw = xq[rb][1][kk][w];
+          const f16x2 kh = __builtin_bit_cast(f16x2, khw), kl = __builtin_bit_cast(f16x2, klw);
+          const f16x2 qh = __builtin_bit_cast(f16x2, qhw), ql = __builtin_bit_cast(f16x2, qlw);
+          dot = __builtin_amdgcn_fdot2(kh, qh, dot, false);
+          dot = __builtin_amdgcn_fdot2(kh, ql, dot, false);
+          dot = __builtin_amdgcn_fdot2(kl, qh, dot, false);
+        }
+      }
+      dot += xor32(dot);
+      float b = kc0 * sd.kb0[jc] + (has_kb1 ? kc1 * kb1p[jc] : 0.f);
+      b += (has_kb2 ? kc2 * kb2p[jc] : 0.f);
+      b = fmaxf(fmaxf(b, kNegBig) * inv_lscale, -3.0e38f);
+      if (j >= 0) warm[rb] = fmaxf(dot + b - (corr[rb] * 0x1p-6f + inv_lscale), -3.0e38f);
+    }
+  }
+  // a workgroup with a row that has no key yet also samples 64 keys spread over the whole key set
+  const bool cold = __syncthreads_or(have ? 0 : 1) != 0;
+  if (cold) {
     const int stride = sd.nk / JT;  // sampled keys: 0, stride, 2 stride, ...
     if (wave == 0) {
       const int j = lane * stride;
@@ -308,19 +353,31 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
 #pragma unroll
         for (int kk = 0; kk < KK16; ++kk) acc = mfma16(KH[0][kk], xq[rb][0][kk], acc);
         acc = add_bias(acc, kbias);
-        float a = max16(acc), b = a;
+        const float mx = max16(acc);
+        float a = mx, b = mx;
         swap_halves(a, b);
         const float m = fmaxf(a, b);
+        if (track && (js == 0 || wave_any(m > run_m[rb]))) {  // as in go_on below
+          int rr = 0;
+#pragma unroll
+          for (int r = 1; r < 16; ++r) rr = (acc[r] == mx) ? r : rr;
+          if (js == 0 || m > run_m[rb])
+            best_j[rb] = (mx == m) ? (js * 32 + 8 * (rr >> 2) + 4 * h + (rr & 3)) * stride : -1;
+        }
         run_m[rb] = js == 0 ? m : fmaxf(run_m[rb], m);
       }
     }
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      float c = -run_m[rb] * lscale;
-      asm volatile("" : "+v"(c));  // the rounded product itself, nothing fused into later uses
-      run_c[rb] = c;
-    }
     barrier();  // buffer 0 is free again
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    if (!cold || warm[rb] > run_m[rb]) {  // the row's key of the last launch stays until exceeded
+      run_m[rb] = warm[rb];
+      best_j[rb] = -1;
+    }
+    float c = -run_m[rb] * lscale;
+    asm volatile("" : "+v"(c));  // the rounded product itself, nothing fused into later uses
+    run_c[rb] = c;
   }
 
   unsigned n_ended = 0;
@@ -354,7 +411,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // then its soft-max.  Everything it computes lives and dies here.  KX: registers for the hi
   // plane of the unit's sub-tile, read again from LDS (the set it was multiplied from has
   // moved on to a later sub-tile).
-  auto go_on = [&](const f32x16& hh, u32x4 (&KX)[KK16], int b, int js, int rb, bool first) {
+  auto go_on = [&](const f32x16& hh, u32x4 (&KX)[KK16], int b, int js, int rb, bool first, int kbase) {
     if (first) {  // first unit of the sub-tile to go on
       read_plane(KX, b, js, 0);
       read_plane(KL, b, js, 1);
@@ -382,6 +439,14 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
       float a = mx, b2 = mx;
       swap_halves(a, b2);
       const float m_new = fmaxf(fmaxf(a, b2), run_m[rb]);
+      if (track && wave_any(m_new > run_m[rb])) {
+        // the maximum of a row moves: the half-wave that holds the new one notes its key (register
+        // r of a lane is key 8 (r / 4) + 4 h + r % 4 of the sub-tile), the other half forgets its own
+        int rr = 0;
+#pragma unroll
+        for (int r = 1; r < 16; ++r) rr = (L[r] == mx) ? r : rr;
+        if (m_new > run_m[rb]) best_j[rb] = (mx == m_new) ? kbase + 8 * (rr >> 2) + 4 * h + (rr & 3) : -1;
+      }
       float cx = -m_new * lscale;
       asm volatile("" : "+v"(cx));  // rounded once, see run_c
       float ps0 = 0.f, ps1 = 0.f;
@@ -401,7 +466,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // during the last step) placed between them in program order; then the units of s that go on.
   // nb, njs: buffer and sub-tile index of s+2, whose hi plane is requested into the set that
   // sub-tile s was multiplied from.
-  auto step = [&](auto c_c, int b, int js, int nb, int njs) {
+  auto step = [&](auto c_c, int b, int js, int nb, int njs, int kbase) {
     constexpr int c = decltype(c_c)::value, n = c ^ 1;
     wait_lds();  // set n (sub-tile s+1), requested during the last step
     arrived(n);
@@ -463,8 +528,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     n_ended += (full0 ? 0u : 1u) + (full1 ? 0u : 1u);
     FS_LC_FENCE();
     // the set that sub-tile s+1 was just multiplied from is free until the next step's request
-    if (full0) go_on(t0, KH[n], b, js, 0, true);
-    if (full1) go_on(t1, KH[n], b, js, 1, !full0);
+    if (full0) go_on(t0, KH[n], b, js, 0, true, kbase);
+    if (full1) go_on(t1, KH[n], b, js, 1, !full0, kbase);
     FS_LC_FENCE();
   };
 
@@ -497,13 +562,15 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   for (int t = 0; t < ntiles; ++t) {
     if (t > 0) start_of_tile(t);
     const int b = t & 3, nb = (t + 1) & 3;
-    step(std::integral_constant<int, 0>{}, b, 0, nb, 0);  // sub-tile 0: multiplies sub-tile 1, requests (t+1, 0)
-    step(std::integral_constant<int, 1>{}, b, 1, nb, 1);  // sub-tile 1: multiplies (t+1, 0), requests (t+1, 1)
+    const int kb = j_begin + t * JT;
+    step(std::integral_constant<int, 0>{}, b, 0, nb, 0, kb);  // sub-tile 0: multiplies sub-tile 1, requests (t+1, 0)
+    step(std::integral_constant<int, 1>{}, b, 1, nb, 1, kb + 32);  // sub-tile 1: multiplies (t+1, 0), requests (t+1, 1)
   }
   wait_all();  // tiles fetched past the chunk: let them land before the workgroup ends
 
-  // unit counts of this wavefront for the variant choice on the device
-  if (args.sel != nullptr && lane == 0 && ntiles > 0) {
+  // unit counts of this wavefront for the variant choice on the device; a workgroup that had
+  // to sample its starting values says nothing about the launches that follow
+  if (args.sel != nullptr && lane == 0 && ntiles > 0 && !(track && cold)) {
     const int slot = blockIdx.x % kSelSlots;
     atomicAdd(&args.sel[kSelEnded + slot], n_ended);
     atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * 4));
@@ -514,12 +581,17 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     const int row = row0 + rb * 32 + li;
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float M2 = -run_c[rb];
+    int bj = best_j[rb];
+    const int oj = __shfl_xor(bj, 32, 64);
+    if (bj < 0) bj = oj;
     if (row < sd.nq && h == 0) {
       if (sd.splits == 1) {
         epilogue_scalar(sd.ep, row, M2, s, 0.f);
+        if (track && bj >= 0) sd.best_key[row] = bj;
       } else {
         const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
         *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
+        if (sd.part_best != nullptr) sd.part_best[pr] = bj;
       }
     }
   }

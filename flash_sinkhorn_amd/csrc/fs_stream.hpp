@@ -499,6 +499,21 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
   if constexpr (HAS_O) {
     epilogue_vec4(sd.ep, sd.q, args.d, args.vec_ok != 0, row, col, M, s, O);
   } else {
+    if (sd.best_key != nullptr && sd.part_best != nullptr) {
+      // the key behind the largest partial maximum that a key of its chunk attained
+      float bm = -3.0e38f;
+      int bj = -1;
+      for (int sp = 0; sp < sd.splits; ++sp) {
+        const size_t pr = (size_t)sp * sd.nq + row;
+        const int j = sd.part_best[pr];
+        const float m = sd.part_ms[2 * pr];
+        if (j >= 0 && m > bm) {
+          bm = m;
+          bj = j;
+        }
+      }
+      if (bj >= 0) sd.best_key[row] = bj;  // no chunk exceeded the starting value: the old key stays
+    }
     epilogue_scalar(sd.ep, row, M, s, o);
   }
 }

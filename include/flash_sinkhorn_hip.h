@@ -31,17 +31,25 @@
  *    FS_FLAG_COARSE_TEST (log-sum-exp entry points, default operand mode, d <= 64) applies the
  *    same 2^40 criterion one stage earlier: the hi*hi plane product of a tile is tested
  *    against the running maximum, lowered by a per-row bound on the two cross products, and a
- *    tile that fails ends there (4 of its 12 MFMAs); a workgroup first takes the largest
- *    logit of 64 keys sampled from the whole key set as its running maximum.  Results stay
- *    within fp32 rounding of the full computation.  It pays when rows and keys are ordered so
- *    that neighbouring rows have neighbouring keys (e.g. sorted by cluster) and the plan is
- *    peaked; on other inputs the test costs about 10 %.  Ignored where it does not apply.
+ *    tile that fails ends there (5 MFMAs instead of 13 at d = 64).  What the test can end
+ *    depends on where a row's running maximum starts.  With FS_FLAG_OPERANDS_PREPARED the
+ *    workspace keeps one int per row next to the planes: the key that held the row's largest
+ *    logit in the last launch over these operands.  The row's current logit at that key, a
+ *    lower bound of its new maximum whatever the potentials did in between, is where the
+ *    running maximum starts; once the potentials settle it is the maximum, and on a peaked
+ *    plan nearly every tile ends at the test, sorted rows or not.  Any content of that array
+ *    leaves the results exact (indices are clamped into the key set); fs_prepare_operands
+ *    resets it, and a row without a key starts from the largest logit of 64 keys sampled from
+ *    the whole key set.  Results stay within fp32 rounding of the full computation.  On a
+ *    flat plan, where every tile matters, the test costs about 20 %.  Ignored where it does
+ *    not apply.
  *    FS_FLAG_COARSE_AUTO (with FS_FLAG_OPERANDS_PREPARED, same conditions) leaves that choice to
  *    the device: every step enqueues both variants and a word of state next to the prepared
  *    planes says which one runs (the workgroups of the other return at once).  The coarse
- *    variant runs first and counts the tiles that end at its test; after each of its first
- *    three launches the step's merge kernel switches to the plain variant for good if fewer than
- *    40 % did.  The state is reset by fs_prepare_operands.  Nothing is read back or timed on
+ *    variant runs first and counts the tiles that end at its test in workgroups whose rows all
+ *    started from a key of the launch before; the third launch with such counts decides: if
+ *    fewer than 40 % of its tiles ended, the step's merge kernel switches to the plain variant
+ *    for good.  The state is reset by fs_prepare_operands.  Nothing is read back or timed on
  *    the host: the same inputs take the same path on every run, and the calls can be captured
  *    into a graph.
  *    Every operation runs on the two-plane fp16 operands by default and on fp32 MFMA operands
@@ -113,6 +121,16 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
  */
 size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
                                uint32_t flags);
+
+/*
+ * Byte offset, inside the same workspace, of the per-row keys FS_FLAG_COARSE_TEST starts from:
+ * one int32 per row of x (which = 0) or of y (which = 1), the key of the other matrix (or of
+ * the same one, for a self problem) that held the row's largest logit in the last launch with
+ * that matrix as the stationary one; -1: none yet.  0 when the configuration keeps none.
+ * Diagnostics and tests only; host arithmetic only.  No counterpart in the reference.
+ */
+size_t fs_best_keys_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
+                           uint32_t flags, int which);
 
 /*
  * out[i] = -eps*damping * LSE_j[ coord_scale * x_i.y_j / eps + bias[j] ]
