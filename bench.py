@@ -11,9 +11,10 @@ Operand modes (results are fp32 in both):
                             of fp32 MFMA operands; allow_tf32=True runs the same kernels
   fp32_mfma (--mode ...)    fp32 operands on v_mfma_f32_32x32x2_f32
 
-roofline (dominant kernel: lse2_kernel, one launch = both half-updates of a symmetric step, with
-its small merge kernel): the launch is timed with HIP events on the launch stream, on the
-operand planes, row order and kernel variant the solve used.
+roofline (dominant kernel: lse_coarse_kernel, or lse2_kernel when the plain variant runs; one
+launch = both half-updates of a symmetric step, with its small merge kernel): the launch is timed
+with HIP events on the launch stream, on prepared operand planes and with the kernel variant
+the solve used, after the eight launches in which the rows' starting keys settle.
   algorithmic work of a launch   4*n*m*d matrix flop (2*n*m*d per half-update) + 2*n*m exp2
   executed work                  the fp16 two-plane mode runs three 16-bit MFMA products per
                                  algorithmic product; the variant with the coarse tile test ends
@@ -24,9 +25,9 @@ operand planes, row order and kernel variant the solve used.
                                  dense fp16 peak (2516.6 TFLOP/s); roofline.frac = their ratio.
                                  roofline.algorithmic_tflops = 4*n*m*d / launch time is what a
                                  user gets (it counts flop the coarse test never ran).
-The solver groups rows by k-means cluster and lets the device decide, from the share of tiles that
-end at the coarse test in the first steps, which kernel variant runs; value_data_independent_ms
-is the same solve with that switched off (caller's row order, plain kernel on every tile).
+The solver lets the device decide, from the share of tiles that end at the coarse test, which
+kernel variant runs; value_plain_kernel_ms is the same solve with the plain kernel on every
+tile, which is what a plan too flat for the test to end anything costs.
 cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores on a
 bounded sample and scaled to the metric's unit.
 """
@@ -47,11 +48,10 @@ MODES = ["strict", "fp32_mfma"]
 FP32_MFMA_PEAK_TFLOPS = 157.3
 F16_MFMA_PEAK_TFLOPS = 2516.6
 EXP2_PER_S = 18.6e12  # v_exp_f32 lanes per second measured on the box (half rate)
-# Memory-side bytes per lse2_kernel launch of the default workload (rows in cluster order, coarse
-# tile test), from two rocprofv3 --pmc runs: FETCH_SIZE 113,782 KiB x 2.0 and WRITE_SIZE
-# 12,510 KiB x 1.0; the factors are what the same counters read for the 256 MiB device copy of
-# --copy-calibration (half the bytes copied, and all of them).
-MEASURED_TRAFFIC_BYTES = {"strict": int((113782 * 2.0 + 12510) * 1024)}
+# Memory-side bytes per lse_coarse_kernel launch of the default workload, from two rocprofv3 --pmc
+# runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each times the factor that the same
+# counter shows for the 256 MiB device copy of --copy-calibration); see profiles/.
+MEASURED_TRAFFIC_BYTES = {}
 
 
 def gmm_cloud(rng, n, d, k=8):
@@ -185,26 +185,22 @@ def main():
     coarse_ran = (solve_info["coarse"] is True
                   or (chosen is not None and not chosen["plain_selected"]))
 
-    # dominant kernel: symmetric-step launches on prepared operand planes, in the row order and
-    # with the kernel variant of the solve, timed with events on the launch stream
+    # dominant kernel: symmetric-step launches on prepared operand planes with the kernel variant
+    # of the solve, timed with events on the launch stream
     alpha = (X * X).sum(1).contiguous()
     beta = (Y * Y).sum(1).contiguous()
     la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
     fh, gh = (f - alpha).contiguous(), (g - beta).contiguous()
-    plain_ops = (X, Y, fh, gh, la, lb)
-    ordered_ops = plain_ops
-    if solve_info["cluster_order"]:
-        px, py = solvers._cluster_order(X), solvers._cluster_order(Y)
-        ordered_ops = (X[px].contiguous(), Y[py].contiguous(), fh[px].contiguous(),
-                       gh[py].contiguous(), la[px].contiguous(), lb[py].contiguous())
+    ops = (X, Y, fh, gh, la, lb)
 
-    def launch_ms(mode, ops, coarse=False, reps=20):
+    def launch_ms(mode, coarse=False, reps=20):
         """(ms per launch, device counters of the coarse variant over the timed launches)"""
         set_mode(mode)
         prep = _lib.PreparedOperands(ops[0], ops[1], _lib.flags(True, False))
         kw = dict(cost_scale=1.0, allow_tf32=False, prepared=prep, coarse=coarse)
         steps = [(EPS, 0.5, 1.0, 1.0)] * reps
-        _symmetric_steps_raw(*ops, steps[:4], **kw)  # also the launches that take the decision
+        # the launches that take the decision, and in which the rows' starting keys settle
+        _symmetric_steps_raw(*ops, steps[:8], **kw)
         torch.cuda.synchronize()
         before = prep.variant_state()
         stream = torch.cuda.current_stream(dev)
@@ -225,9 +221,11 @@ def main():
 
     def roofline_for(mode, ms, counts):
         r = {"bound": "mfma", "unit": "TFLOP/s",
-             "kernel": "lse2_kernel (+ its merge kernel): one launch = both half-updates of a "
-                       "symmetric step on prepared operand planes; algorithmic work 4*n*m*d flop "
-                       "+ 2*n*m exp2",
+             "kernel": ("lse_coarse_kernel" if counts is not None and counts["tiles_tested"] > 0
+                        and not counts["plain_selected"] else "lse2_kernel")
+                       + " (+ its merge kernel): one launch = both half-updates of a symmetric "
+                         "step on prepared operand planes; algorithmic work 4*n*m*d flop + 2*n*m "
+                         "exp2",
              "launch_ms": ms, "algorithmic_tflops": flop / (ms * 1e-3) / 1e12,
              "exp_per_s": 2.0 * n * m / (ms * 1e-3)}
         if mode == "fp32_mfma":
@@ -236,8 +234,7 @@ def main():
         else:
             # three plane products per tile in the plain kernel.  The variant with the coarse tile
             # test runs, for every tile, the hi*hi product plus one more 16-column MFMA step that
-            # carries the bias bound, and the two cross products only for tiles that go on (the
-            # few tiles per workgroup that seed the running maxima, under 1 %, are not counted).
+            # carries the bias bound, and the two cross products only for tiles that go on.
             products = 3.0 * tiles_all
             if counts is not None and counts["tiles_tested"] > 0 and not counts["plain_selected"]:
                 went_on = 1.0 - counts["tiles_ended"] / counts["tiles_tested"]
@@ -257,7 +254,7 @@ def main():
         return r
 
     as_solved = "auto" if solve_info["coarse"] == "auto" else bool(solve_info["coarse"])
-    main_ms, main_counts = launch_ms(args.mode, ordered_ops, coarse=as_solved)
+    main_ms, main_counts = launch_ms(args.mode, coarse=as_solved)
     line = {
         "metric": "ms per 100 symmetric Sinkhorn iterations (n=m=50k, d=64, fp32)",
         "value": ms_per_step, "unit": "ms", "n_gpus": 1, "steps": args.steps,
@@ -270,7 +267,6 @@ def main():
                                "8-component Gaussian mixtures, uniform weights, eps=0.01, "
                                "100 iterations + init + extrapolation = 102 steps",
                    "operand_mode": args.mode,
-                   "rows_in_cluster_order": solve_info["cluster_order"],
                    "kernel_variant": "coarse tile test" if coarse_ran else "plain",
                    "variant_chosen_by": ("device counters" if solve_info["coarse"] == "auto"
                                          else "caller"),
@@ -286,24 +282,24 @@ def main():
     rf["frac_of_serial_mfma_exp_roofline"] = (t_mfma + t_exp) / ms_per_step
 
     if not args.no_extras:
-        solvers_order = solvers.CLUSTER_ORDER
-        # the data-independent figure: caller's row order, plain kernel on every tile
-        solvers.CLUSTER_ORDER = False
-        line["value_data_independent_ms"], _ = timed_solves(max(2, args.steps // 2), 1)
-        solvers.CLUSTER_ORDER = solvers_order
+        # the plan-independent figure: the plain kernel on every tile
+        forced = solvers.COARSE_TEST
+        solvers.COARSE_TEST = False
+        line["value_plain_kernel_ms"], _ = timed_solves(max(2, args.steps // 2), 1)
+        solvers.COARSE_TEST = forced
         # the 101-step variant (no extrapolation step) that the reference's README times
         line["value_without_last_extrapolation_ms"], _ = timed_solves(
             max(2, args.steps // 2), 1, last_extrapolation=False)
-        plain_ms, _ = launch_ms(args.mode, plain_ops)
+        plain_ms, _ = launch_ms(args.mode)
         _lib.TILE_SKIP = False
-        every_exp_ms, _ = launch_ms(args.mode, plain_ops, reps=10)
+        every_exp_ms, _ = launch_ms(args.mode, reps=10)
         _lib.TILE_SKIP = True
         rf["other_launches"] = {
-            "caller_order_plain_kernel": {
+            "plain_kernel": {
                 "launch_ms": plain_ms, **{k: v for k, v in roofline_for(
                     args.mode, plain_ms, None).items() if k in ("achieved", "frac",
                                                                 "algorithmic_tflops")}},
-            "caller_order_plain_kernel_every_exp": {
+            "plain_kernel_every_exp": {
                 "launch_ms": every_exp_ms, **{k: v for k, v in roofline_for(
                     args.mode, every_exp_ms, None).items() if k in ("achieved", "frac",
                                                                     "algorithmic_tflops")}},
@@ -311,7 +307,7 @@ def main():
                     "whose logits all lie 2^40 below their rows' running maxima (exact in "
                     "fp32); every_exp computes those too"}
         other = "fp32_mfma" if args.mode == "strict" else "strict"
-        o_ms, _ = launch_ms(other, plain_ops, reps=5)
+        o_ms, _ = launch_ms(other, reps=5)
         orf = roofline_for(other, o_ms, None)
         line["other_operand_mode"] = {"mode": other, "launch_ms": o_ms,
                                       "ms_per_100_iters_est": o_ms * (ITERS + 2),

@@ -21,39 +21,20 @@ from flash_sinkhorn_amd.kernels._common import (
 
 __all__ = ["sinkhorn_flashstyle_alternating", "sinkhorn_flashstyle_symmetric"]
 
-# Long fixed-eps solves on large clouds run on rows and keys grouped by k-means cluster, with the
-# kernel variant that tests a tile after its hi*hi plane product (FS_FLAG_COARSE_TEST): with
-# neighbouring rows next to each other, whole key tiles fall below the 2^-40 criterion for all
-# rows of a workgroup at once, which the coarse test turns into fewer MFMAs.  Whether the
-# variant stays is decided on the device from the share of tiles that end at the test in the
-# first steps (FS_FLAG_COARSE_AUTO): no timing, no host read-back, the same inputs take the
-# same path on every run.  The potentials come back in the caller's order; values agree with
-# the unordered solve to fp32 rounding.
-CLUSTER_ORDER = os.environ.get("FLASH_SINKHORN_CLUSTER_ORDER", "1") != "0"
+# Fixed-eps solves on large clouds run the kernel variant that tests a 32 x 32 logits tile after
+# its hi*hi plane product (FS_FLAG_COARSE_TEST).  Each row's running maximum starts from the row's
+# logit at the key that held its maximum in the step before, so on a peaked plan (small eps)
+# nearly every tile ends at that test from the third step on, whatever the order of the rows.
+# Whether the variant stays is decided on the device from the share of tiles that end at the
+# test (FS_FLAG_COARSE_AUTO): no timing, no host read-back, the same inputs take the same path
+# on every run; on a flat plan the third counted step switches to the plain kernel for good.
 # None: the device decides; True / False: the coarse variant on every step / on none
 COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_TEST", ""))
-# measured on 8-component Gaussian mixtures at d = 64: below about 40,000 rows per cloud the
-# ordering costs more than the coarse variant returns (25,000: +4 %; 32,768: even)
-_CLUSTER_MIN_ROWS = 40000
-_CLUSTER_MIN_STEPS = 24
-
-
-def _cluster_order(pts: torch.Tensor, k: int = 16, iters: int = 4) -> torch.Tensor:
-    """Permutation that groups the rows of ``pts`` by k-means cluster (Lloyd iterations from
-    evenly spaced rows; GEMM-shaped updates, no host synchronisation)."""
-    n = pts.shape[0]
-    centres = pts[torch.arange(k, device=pts.device) * (n // k)].clone()
-    labels = None
-    for it in range(iters + 1):
-        score = (centres * centres).sum(dim=1)[None, :] - 2.0 * (pts @ centres.T)
-        labels = score.argmin(dim=1)
-        if it == iters:
-            break
-        onehot = torch.nn.functional.one_hot(labels, k).to(pts.dtype)
-        count = onehot.sum(dim=0)
-        mean = (onehot.T @ pts) / count.clamp_min(1.0)[:, None]
-        centres = torch.where(count[:, None] > 0, mean, centres)
-    return torch.argsort(labels, stable=True)
+# measured on 8-component Gaussian mixtures at d = 8, 32, 64 and eps = 0.01: from about 20,000
+# rows per cloud on the coarse variant is the faster one (25,000: 1.1-1.2x, 50,000: 1.3-1.6x,
+# 100,000: 1.4-1.8x); below, its start-up per key chunk outweighs what the test saves
+_COARSE_MIN_ROWS = 24000
+_COARSE_MIN_STEPS = 8
 
 # Reference switches from the one-launch step to two launches at this n
 # (sinkhorn_solvers.py:463-468).  Both give the same numbers; here the one-launch
@@ -178,8 +159,8 @@ def sinkhorn_flashstyle_symmetric(
     snapshot.  ``f_init``/``g_init`` warm-start (standard potentials).
     Returns (f, g[, f_prelast, g_prelast][, n_iters_used]); the prelast pair is
     only returned when ``return_prelast and last_extrapolation``.
-    ``solve_info`` (not in the reference): a dict that receives ``cluster_order`` (rows were
-    grouped by cluster), ``coarse`` (False, True or "auto") and ``prepared`` (the operand
+    ``solve_info`` (not in the reference): a dict that receives ``coarse`` (the kernel variant
+    of the steps: False, True or "auto") and ``prepared`` (the operand
     planes, whose ``variant_state()`` tells what the device chose).
     """
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (
@@ -227,32 +208,14 @@ def sinkhorn_flashstyle_symmetric(
                             and a.stride() == b.stride()))):
         yf, beta, log_b, g_hat = xf, alpha, log_a, f_hat
 
-    # cluster order (see CLUSTER_ORDER): every per-row array is permuted, the results are
-    # put back in the caller's order at the end
-    inv_x = inv_y = None
+    # the kernel variant with the coarse tile test (see COARSE_TEST)
     coarse = False
-    if (CLUSTER_ORDER and fused and not use_labels and _lib.TILE_SKIP
+    if (fused and not use_labels and _lib.TILE_SKIP
             and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
-            and min(xf.shape[0], yf.shape[0]) >= _CLUSTER_MIN_ROWS
-            and len(eps_list) >= _CLUSTER_MIN_STEPS
+            and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
+            and len(eps_list) >= _COARSE_MIN_STEPS
             and all(e == eps_list[0] for e in eps_list)):
-        # the aliased form set up above; x passed twice with two weight vectors is not it
-        self_problem = yf is xf and log_b is log_a and g_hat is f_hat and beta is alpha
-        perm_x = _cluster_order(xf)
-        inv_x = torch.empty_like(perm_x)
-        inv_x[perm_x] = torch.arange(perm_x.numel(), device=perm_x.device)
-        xf, alpha, log_a, f_hat = (xf[perm_x].contiguous(), alpha[perm_x], log_a[perm_x],
-                                   f_hat[perm_x])
-        if self_problem:
-            yf, beta, log_b, g_hat, inv_y = xf, alpha, log_a, f_hat, inv_x
-        else:
-            perm_y = _cluster_order(yf)
-            inv_y = torch.empty_like(perm_y)
-            inv_y[perm_y] = torch.arange(perm_y.numel(), device=perm_y.device)
-            yf, beta, log_b, g_hat = (yf[perm_y].contiguous(), beta[perm_y], log_b[perm_y],
-                                      g_hat[perm_y])
         coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
-
     # operand planes are converted once for the whole loop, when the first launch needs them
     # (a run replayed from a graph has planes of its own)
     made = []
@@ -357,10 +320,7 @@ def sinkhorn_flashstyle_symmetric(
     if return_prelast and last_extrapolation:
         out = out + (f_prelast, g_prelast)
     if solve_info is not None:
-        solve_info.update(cluster_order=inv_x is not None, coarse=coarse,
-                          prepared=made[0] if made else None)
-    if inv_x is not None:  # back to the caller's row order
-        out = tuple(t[inv_x if i % 2 == 0 else inv_y] for i, t in enumerate(out))
+        solve_info.update(coarse=coarse, prepared=made[0] if made else None)
     if return_n_iters:
         out = out + (used,)
     return out

@@ -641,11 +641,11 @@ def test_coarse_test_starts_rows_from_the_keys_of_the_last_step(n, m, d, eps):
     check(fh2, gh2, F2, G2)
 
 
-@pytest.mark.parametrize("variant", [True, False, None])
-def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
-    """Long fixed-eps solves on large clouds run on rows grouped by k-means cluster and hand the
-    potentials back in the caller's order; with the coarse tile test forced on, off, or chosen on
-    the device, the result is the unordered solve's to rounding."""
+@pytest.mark.parametrize("variant", [True, None])
+def test_solver_with_the_coarse_tile_test_equals_the_plain_solve(monkeypatch, variant):
+    """Fixed-eps solves on large clouds run the kernel variant with the coarse tile test, forced
+    or chosen on the device; the potentials are the plain solve's to rounding, for two clouds,
+    for the self problem (one half-update per step) and for one cloud with two weight vectors."""
     import flash_sinkhorn_amd.sinkhorn_solvers as solvers
     rng = np.random.default_rng(32)
     n, m, d = 16500, 16400, 8
@@ -656,40 +656,34 @@ def test_cluster_ordered_solve_equals_unordered(monkeypatch, variant):
     X, Y, A, B = dev(x, y, a / a.sum(), b / b.sum())
     kw = dict(use_epsilon_scaling=False, eps=0.05, n_iters=26, allow_tf32=False,
               return_prelast=True)
-    monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
+    monkeypatch.setattr(solvers, "COARSE_TEST", False)
     info = {}
     want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
-    assert not info["cluster_order"] and info["coarse"] is False
-    monkeypatch.setattr(solvers, "CLUSTER_ORDER", True)
-    monkeypatch.setattr(solvers, "_CLUSTER_MIN_ROWS", 16384)  # the default only orders larger clouds
+    assert info["coarse"] is False
+    wu = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, **kw)
+    A2 = torch.flip(A, dims=[0]).contiguous()
+    want2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
     monkeypatch.setattr(solvers, "COARSE_TEST", variant)
     got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
-    assert info["cluster_order"]
+    assert info["coarse"] is False  # the default only switches on larger clouds
+    monkeypatch.setattr(solvers, "_COARSE_MIN_ROWS", 16384)
+    got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
     assert info["coarse"] == ("auto" if variant is None else variant)
     state = info["prepared"].variant_state()
-    if variant is None:  # the device looked at up to three steps (it stops once it has left
-        # the coarse variant) and counted tiles
-        assert 1 <= state["decisions"] <= 3 and state["tiles_tested"] > 0
-    else:  # a forced coarse variant counts its tiles too, the plain kernel has nothing to count
-        assert (state["tiles_tested"] > 0) == variant
+    assert state["tiles_tested"] > 0
+    if variant is None:  # the third counted step decided
+        assert state["decisions"] == 3
     for u, v in zip(got, want):
         assert rel_err(u, v.cpu().numpy()) < 2e-5
-    # the self problem keeps its single half-update per step under the ordering
+    # the self problem keeps its single half-update per step
     ws = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, **kw)
-    monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
-    wu = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A, **kw)
     # these potentials are small differences of shifted potentials of size |x|^2
     scale = float((X * X).sum(dim=1).max())
     for u, v in zip(ws, wu):
         assert float((u - v).abs().max()) < 2e-6 * scale
     assert float((ws[0] - ws[1]).abs().max()) == 0.0
     # one cloud passed twice with two weight vectors is an ordinary two-sided problem
-    monkeypatch.setattr(solvers, "CLUSTER_ORDER", True)
-    monkeypatch.setattr(solvers, "_CLUSTER_MIN_ROWS", 16384)
-    A2 = torch.flip(A, dims=[0]).contiguous()
     got2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
-    monkeypatch.setattr(solvers, "CLUSTER_ORDER", False)
-    want2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
     for u, v in zip(got2, want2):
         assert float((u - v).abs().max()) < 2e-6 * scale
 

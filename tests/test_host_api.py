@@ -264,25 +264,6 @@ def test_custom_operators_are_registered_with_shape_inference():
     assert out.shape == (m,) and piz.shape == (n,)
 
 
-def test_cluster_order_is_a_permutation_that_groups_clusters():
-    """`_cluster_order` (plain torch, runs on the CPU too): a permutation of the rows under which
-    well separated clusters come out as contiguous runs."""
-    import numpy as np
-    import torch
-    from flash_sinkhorn_amd.sinkhorn_solvers import _cluster_order
-    rng = np.random.default_rng(5)
-    k, n, d = 6, 3000, 5
-    centres = rng.standard_normal((k, d)) * 50.0
-    lab = rng.integers(0, k, n)
-    pts = torch.from_numpy((centres[lab] + rng.standard_normal((n, d))).astype(np.float32))
-    perm = _cluster_order(pts).numpy()
-    assert sorted(perm.tolist()) == list(range(n))
-    runs = 1 + int((np.diff(lab[perm]) != 0).sum())
-    assert runs <= 16  # at most one run per k-means centre
-    same = torch.zeros(40, 3)
-    assert _cluster_order(same, k=4).tolist() == list(range(40))  # ties keep the caller's order
-
-
 def test_solvers_refuse_cpu_tensors_before_touching_them():
     import torch
     from flash_sinkhorn_amd.sinkhorn_solvers import (
