@@ -118,6 +118,11 @@ SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam, int rb_f
   return p;
 }
 
+// Per-tile records of the key bias for lse_coarse_kernel (see coarse_bias_kernel).
+size_t coarse_aux_bytes(int64_t nk) {
+  return (size_t)(ceil_div(nk, 64) + kAuxPadTiles) * kAuxWords * sizeof(unsigned);
+}
+
 size_t side_ws_floats(int mode, const SidePlan& p, int64_t nq, int dp) {
   if (p.splits <= 1) return 0;
   size_t f = (size_t)p.splits * (size_t)nq * 2;
@@ -791,6 +796,14 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     if (!fam.sliced && plans[s].rb != rb) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam, rb);
     need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
   }
+  // lse_coarse_kernel: per-tile records of the key bias, behind the partial rows
+  const size_t aux_off = need;
+  size_t aux_bytes[2] = {0, 0};
+  if (coarse || auto_sel)
+    for (int s = 0; s < nsides; ++s) {
+      aux_bytes[s] = coarse_aux_bytes(sides[s].nk);
+      need += aux_bytes[s];
+    }
   if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
   float* wsp = reinterpret_cast<float*>(static_cast<char*>(ws) + need_planes_end);
   bool any_split = false;
@@ -803,6 +816,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     sd.igroups = p.igroups;
     sd.best_key = nullptr;
     sd.part_best = nullptr;
+    sd.key_aux = nullptr;
     sd.part_ms = nullptr;
     sd.part_o = nullptr;
     if (p.splits > 1) {
@@ -823,7 +837,10 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       sd.plane_scale = plane_scales(ps, ws);
       sd.ps_q = plane_index(ps, sd.q, sd.nq);
       sd.ps_k = plane_index(ps, sd.k, sd.nk);
-      if (coarse || auto_sel) sd.best_key = best_keys_of(ps, cfg, ws, sd.q, sd.nq);
+      if (coarse || auto_sel) {
+        sd.best_key = best_keys_of(ps, cfg, ws, sd.q, sd.nq);
+        sd.key_aux = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + aux_off + (s == 1 ? aux_bytes[0] : 0));
+      }
     }
     a.side[s] = sd;
   }
@@ -983,6 +1000,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     c.gemm = false; c.prec = 3; c.dp = std::max(dp, 16); c.np = 2;
     planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes;
   }
+  if (mode == kLse && !fam.sliced) planes += coarse_aux_bytes(n) + coarse_aux_bytes(m);
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;

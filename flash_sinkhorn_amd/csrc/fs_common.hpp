@@ -93,6 +93,10 @@ struct Side {
   int* best_key;        // [nq] or null
   int* part_best;       // [splits, nq] when splits > 1: the key behind a partial M, -1 when no
                         // key of the chunk exceeded the starting value
+  // lse_coarse_kernel: per 64-key tile, what coarse_bias_kernel derives from the key bias, in
+  // the layout the tile's LDS buffer takes (kAuxWords words per tile, kAuxPadTiles tiles past
+  // the last key)
+  unsigned* key_aux;
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;
 };
@@ -114,6 +118,10 @@ struct LaunchArgs {
   unsigned sel_want;
   int sel_pred;  // 0: the launch runs whatever the state says (it still counts into it)
 };
+
+// Per 64-key tile record of coarse_bias_kernel: eight fp16 copies of a_j per key (4 words each),
+// then b_j - 2^18 a_j per key, then the largest bias of each 32-key sub-tile, padded to 16 bytes.
+constexpr int kAuxA = 0, kAuxB = 256, kAuxMax = 320, kAuxWords = 324, kAuxPadTiles = 4;
 
 // Device state of the variant choice (unsigned words), zeroed when the operand planes are
 // written: which variant runs (0: coarse tile test, 1: plain), how many decisions were taken,

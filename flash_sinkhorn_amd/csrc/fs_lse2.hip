@@ -58,6 +58,11 @@ static int launch_coarse_dp(const LaunchArgs& a, int blocks, hipStream_t st) {
 
 static int launch_coarse(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
   if (rb != 2) return FS_ERR_BAD_ARGUMENT;
+  // the per-tile records of the key bias, for both sides (tiles past the last key included)
+  const int tiles0 = (a.side[0].nk + 63) / 64 + kAuxPadTiles;
+  const int tiles1 = blocks > a.blocks0 ? (a.side[1].nk + 63) / 64 + kAuxPadTiles : 0;
+  hipLaunchKernelGGL((coarse_bias_kernel<0>), dim3(tiles0 + tiles1), dim3(64), 0, st, a, tiles0);
+  if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
   switch (dp) {
     case 16: return launch_coarse_dp<16>(a, blocks, st);
     case 32: return launch_coarse_dp<32>(a, blocks, st);

@@ -14,22 +14,31 @@
 //
 // A wavefront owns 64 query rows (two blocks of 32) whose planes stay in registers, and walks
 // its key chunk in 32-key sub-tiles ("unit": 32 keys x 32 queries).  One step per sub-tile s:
-//   1. the hi*hi products of the two units of sub-tile s+1 go to the matrix pipe (ten MFMAs,
-//      two independent chains), and between them in program order sit
+//   1. the hi*hi products of the two units of sub-tile s+1 go to the matrix pipe (the a_j step,
+//      then two independent chains of four MFMAs), and between them in program order sit
 //   2. the tests of the two units of sub-tile s, whose products finished during the last step:
 //      a wavefront issues in order, so only work placed between MFMAs runs in their shadow;
 //   3. for a unit of s that goes on, in a block of its own: the cross products khi*qlo and
 //      klo*qhi and the exact key bias (one fp32 MFMA) on top of its hi*hi product, then the
 //      soft-max.
 // Nothing a conditional block computes outlives it except the running (maximum, sum) of the
-// rows: no accumulator tile is carried across a branch, so the register allocator never has
-// to reconcile two versions of one (four tiles hold the hi*hi products of two sub-tiles, and
-// they are only ever written unconditionally).  Only the hi plane of a sub-tile is read from
-// LDS up front (two sub-tiles ahead); a unit that goes on reads both planes and the per-key
-// biases of its sub-tile again.  The running maximum of a row starts from 64 keys sampled
-// evenly over the whole key set, so that a key chunk without any of the row's near keys is
-// measured against a meaningful maximum from its first tile on.  A unit that ends costs five
-// MFMAs, a 16-value maximum and a ballot.
+// rows and the key of the maximum: no accumulator tile is carried across a branch, so the
+// register allocator never has to reconcile two versions of one (four tiles hold the hi*hi
+// products of two sub-tiles, and they are only ever written unconditionally).  Only the hi
+// plane of a sub-tile is read from LDS up front (two sub-tiles ahead); a unit that goes on
+// reads both planes and the per-key biases of its sub-tile again.  A unit that ends costs
+// four and a half MFMAs (the a_j step serves both row blocks), a 16-value maximum and a ballot.
+//
+// What the test can end depends on where a row's running maximum starts.  The launch keeps,
+// per row, the key that held the row's largest logit (Side::best_key, merged over the key
+// chunks by finish_kernel), and the next launch over the same planes starts the row from its
+// current logit at that key: a lower bound of the new maximum by construction, and the maximum
+// itself once the potentials settle.  Rows without a key (the first launch on new planes)
+// start from the largest logit of 64 keys sampled evenly over the whole key set, so that a key
+// chunk without any of the row's near keys is measured against a meaningful maximum from its
+// first tile on.  The key-side quantities of the test (a_j, b_j - 2^18 a_j, bmax per sub-tile)
+// are the same for every workgroup: coarse_bias_kernel writes them once per launch, per 64-key
+// tile, in the layout of the tile's LDS record.
 //
 // Everything LDS-related is written out by hand (ds_read / ds_write / s_waitcnt / s_barrier):
 // key tiles arrive by direct global->LDS loads two tiles ahead, and the compiler, which
@@ -46,6 +55,47 @@ namespace fs {
 
 #define FS_LC_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// What lse_coarse_kernel needs of the key bias, once per launch instead of once per workgroup:
+// one wavefront per 64-key tile writes the tile's record (layout: kAux* in fs_common.hpp) in raw
+// units: a_j as eight fp16 copies, b_j - 2^18 a_j, and the largest bias of each 32-key
+// sub-tile.  Keys past the end of the key set get a bias that masks them.  T only makes this a
+// template (header-defined kernel).
+template <int T>
+__global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, int tiles0) {
+  // variant chosen on the device: nothing reads the records when the plain kernel runs
+  if (args.sel_pred && args.sel[kSelWord] != 0u) return;
+  int tile = blockIdx.x;
+  const bool second = tile >= tiles0;
+  if (second) tile -= tiles0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const int lane = threadIdx.x, li = lane & 31, h = lane >> 5;
+  const int j = tile * 64 + lane;
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
+  const float inv_lscale = 1.0f / lscale;
+  float b = 2.0f * kNegBig;
+  if (j < sd.nk) {
+    b = sd.kc0 * sd.kb0[j];
+    if (sd.kb1) b += sd.kc1 * sd.kb1[j];
+    if (sd.kb2) b += sd.kc2 * sd.kb2[j];
+    b = fmaxf(b, kNegBig);
+  }
+  b = fmaxf(b * inv_lscale, -3.0e38f);
+  float mx = b;
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  // a_j: (b - bmax) / 2^18 as fp16, rounded towards zero (never below the true value)
+  const float rel = fmaxf((b - mx) * 0x1p-18f, -65504.0f);
+  _Float16 ah = (_Float16)rel;
+  if ((float)ah < rel)  // negative and one step too low: the next fp16 towards zero
+    ah = __builtin_bit_cast(_Float16, (unsigned short)(__builtin_bit_cast(unsigned short, ah) - 1));
+  const unsigned aw = (unsigned)__builtin_bit_cast(unsigned short, ah) * 0x00010001u;
+  unsigned* rec = sd.key_aux + (size_t)tile * kAuxWords;
+  *reinterpret_cast<u32x4*>(rec + kAuxA + lane * 4) = u32x4{aw, aw, aw, aw};
+  rec[kAuxB + lane] = __builtin_bit_cast(unsigned, b - (float)ah * 0x1p18f);
+  if (li == 0) rec[kAuxMax + h] = __builtin_bit_cast(unsigned, mx);
+  if (lane < kAuxWords - kAuxMax - 2) rec[kAuxMax + 2 + lane] = 0u;
+}
+
 template <int DP>
 __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs args) {
   static_assert(DP == 16 || DP == 32 || DP == 64, "two-plane rows of at most 64 columns");
@@ -58,8 +108,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   constexpr int NBUF = 4;              // ring of key tiles in LDS: tile t+3 is requested during tile t
 
   __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][JT * ROWW];
-  __shared__ __attribute__((aligned(16))) float lds_b[NBUF][JT + 4];  // [JT]: b_j - 2^18 a_j, then bmax of the two sub-tiles
-  __shared__ __attribute__((aligned(16))) unsigned lds_a[NBUF][JT * 4];  // eight copies of a_j (fp16) per key
+  // per tile: eight copies of a_j (fp16) per key, b_j - 2^18 a_j per key, bmax of the two sub-tiles
+  __shared__ __attribute__((aligned(16))) unsigned lds_aux[NBUF][kAuxWords];
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
@@ -184,43 +234,27 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     }
   };
 
-  // ---- key bias: wavefront 0 fetches the raw terms of key j0 + lane a tile ahead and writes
-  // the combined value (raw units) and the maximum of each 32-key sub-tile before the barrier
-  // that publishes the tile ----
+  // ---- key bias: coarse_bias_kernel has written, per 64-key tile, the record that the tile's
+  // LDS buffer takes (a_j, b_j - 2^18 a_j, bmax; raw units); wavefront 0 brings it in with two
+  // direct loads, issued before the tile's keys so that the same wait covers both ----
   const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
   const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
   const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
   const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
-  float st_b0 = 0.f, st_b1 = 0.f, st_b2 = 0.f;
-  bool st_live = false;
-  auto bias_load = [&](int j) {  // j: the key this lane stages (every wavefront loads, so that
-                                 // all of them count the same loads in flight; wavefront 0 stores)
-    const int jj = max(0, min(j, j_end - 1));
-    st_b0 = sd.kb0[jj];
-    st_b1 = kb1p[jj];
-    st_b2 = kb2p[jj];
-    st_live = j < j_end;
-  };
-  auto bias_store = [&](int buf) {
+  const unsigned* auxp = sd.key_aux + (size_t)(j_begin / JT) * kAuxWords + lane * 4;
+  auto issue_aux = [&](int buf) {  // the next tile in sequence
     if (wave == 0) {
-      float b = kc0 * st_b0 + (has_kb1 ? kc1 * st_b1 : 0.f);
-      b += (has_kb2 ? kc2 * st_b2 : 0.f);
-      b = st_live ? fmaxf(b, kNegBig) : 2.0f * kNegBig;
-      b = fmaxf(b * inv_lscale, -3.0e38f);
-      float mx = b;
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-      // a_j: (b - bmax) / 2^18 as fp16, rounded towards zero (never below the true value)
-      const float rel = fmaxf((b - mx) * 0x1p-18f, -65504.0f);
-      _Float16 ah = (_Float16)rel;
-      if ((float)ah < rel)  // negative and one step too low: the next fp16 towards zero
-        ah = __builtin_bit_cast(_Float16, (unsigned short)(__builtin_bit_cast(unsigned short, ah) - 1));
-      const unsigned aw = (unsigned)__builtin_bit_cast(unsigned short, ah) * 0x00010001u;
-      ds_write16(&lds_a[buf][lane * 4], u32x4{aw, aw, aw, aw});
-      ds_write4(&lds_b[buf][lane], b - (float)ah * 0x1p18f);
-      if (li == 0) ds_write4(&lds_b[buf][JT + h], mx);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)auxp,
+          (__attribute__((address_space(3))) void*)(&lds_aux[buf][0]), 16, 0, 0);
+      if (lane < (kAuxWords - 256) / 4)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(auxp + 256),
+            (__attribute__((address_space(3))) void*)(&lds_aux[buf][256]), 16, 0, 0);
     }
+    auxp += kAuxWords;
   };
+  auto lds_b = [&](int buf, int k) { return reinterpret_cast<const float*>(&lds_aux[buf][kAuxB + k]); };
 
   auto mfma16 = [](const u32x4& a, const u32x4& b, const f32x16& c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
@@ -314,7 +348,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
       const int j = lane * stride;
       float b = kc0 * sd.kb0[j] + (has_kb1 ? kc1 * kb1p[j] : 0.f);
       b += (has_kb2 ? kc2 * kb2p[j] : 0.f);
-      ds_write4(&lds_b[0][lane], fmaxf(fmaxf(b, kNegBig) * inv_lscale, -3.0e38f));
+      ds_write4(reinterpret_cast<float*>(&lds_aux[0][kAuxB + lane]),
+                fmaxf(fmaxf(b, kNegBig) * inv_lscale, -3.0e38f));
     }
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
@@ -332,7 +367,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     for (int js = 0; js < 2; ++js) {
       read_plane(KH[0], 0, js, 0);
       read_plane(KL, 0, js, 1);
-      kbias = ds_read4(&lds_b[0][js * 32 + li]);
+      kbias = ds_read4(lds_b(0, js * 32 + li));
       wait_lds();
 #pragma unroll
       for (int kk = 0; kk < KK16; ++kk) {
@@ -383,22 +418,20 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   unsigned n_ended = 0;
   f32x16 H[4];  // hi*hi products (on top of 2^18 a_j): sub-tile s, row block rb in H[2 (s & 1) + rb]
 
-  // Start of tile t: the bias of tile t+1 goes to LDS and its keys have landed (only those of
-  // tile t+2 may still be in flight); after the barrier tile t+1 is visible and every wavefront
-  // is done with tile t-1, whose buffer takes tile t+3.  The raw bias terms of tile t+2 are
-  // requested before those keys, so that the next round's wait covers them.
+  // Start of tile t: the keys and the bias record of tile t+1 have landed (only those of tile t+2
+  // may still be in flight); after the barrier tile t+1 is visible and every wavefront is done
+  // with tile t-1, whose buffer takes tile t+3.
   auto start_of_tile = [&](int t) {
-    bias_store((t + 1) & 3);
     wait_older_tiles();
     barrier();
-    bias_load(j_begin + (t + 2) * JT + lane);
+    issue_aux((t + 3) & 3);
     issue_tile((t + 3) & 3);
   };
   // hi plane, a_j piece and bmax of sub-tile js of the tile in buffer b, into register set k
   auto request = [&](int k, int b, int js) {
     read_plane(KH[k], b, js, 0);
-    KA[k] = ds_read16(&lds_a[b][(js * 32 + li) * 4]);
-    bmax[k] = ds_read4(&lds_b[b][JT + js]);
+    KA[k] = ds_read16(&lds_aux[b][kAuxA + (js * 32 + li) * 4]);
+    bmax[k] = ds_read4(lds_b(b, JT + js));
   };
   auto arrived = [&](int k) {  // after a wait: every later use of set k sits behind this point
 #pragma unroll
@@ -415,7 +448,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     if (first) {  // first unit of the sub-tile to go on
       read_plane(KX, b, js, 0);
       read_plane(KL, b, js, 1);
-      kbias = ds_read4(&lds_b[b][js * 32 + li]);
+      kbias = ds_read4(lds_b(b, js * 32 + li));
       wait_lds();
 #pragma unroll
       for (int kk = 0; kk < KK16; ++kk) {
@@ -534,11 +567,11 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   };
 
   // ---- prologue: tiles 0 and 1 published, tiles 2 and 3 on their way; hi*hi of sub-tile 0 ----
-  bias_load(j_begin + lane);
+  issue_aux(0);
   issue_tile(0);
+  issue_aux(1);
   issue_tile(1);
-  bias_store(0);
-  bias_load(j_begin + JT + lane);
+  issue_aux(2);
   issue_tile(2);
   start_of_tile(0);
   request(0, 0, 0);

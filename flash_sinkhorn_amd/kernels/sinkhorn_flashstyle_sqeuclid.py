@@ -183,11 +183,12 @@ def _symmetric_steps_raw(x, y, f_hat, g_hat, log_a, log_b, steps, *, cost_scale,
 
 def _self_pair_steps_raw(x, y, fx_hat, fy_hat, log_a, log_b, steps, *, cost_scale, shift_x=None,
                          shift_y=None, allow_tf32=True, use_exp2=True, prepared=None,
-                         with_previous=False):
+                         with_previous=False, coarse=False):
     """The self problems OT(x, x; a) and OT(y, y; b) advanced together (``fs_self_pair_steps``):
     ``steps`` = [(eps_x, eps_y, alpha, damping_x, damping_y), ...], one launch per step for both.
     ``prepared`` must have been built with ``self_pair=True``.  Returns (fx_hat, fy_hat), with
-    ``with_previous`` followed by the pair the last step started from."""
+    ``with_previous`` followed by the pair the last step started from.  ``coarse`` as in
+    ``_symmetric_step_raw``."""
     import ctypes
     k = len(steps)
     if k == 0:
@@ -208,6 +209,7 @@ def _self_pair_steps_raw(x, y, fx_hat, fy_hat, log_a, log_b, steps, *, cost_scal
                   + int(L.fs_workspace_bytes(_lib.OP_SYMMETRIC_STEP, m, m, d)))
         _keep = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
         wp, wn, fl = _keep.data_ptr(), nbytes, flag_bits
+    fl |= _lib.coarse_flag(coarse)
     rc = _lib.lib().fs_self_pair_steps(
         x.data_ptr(), y.data_ptr(), fx_hat.data_ptr(), fy_hat.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), fx_work[0].data_ptr(), fy_work[0].data_ptr(), fx_work[1].data_ptr(),

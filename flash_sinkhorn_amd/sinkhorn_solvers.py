@@ -373,6 +373,13 @@ def sinkhorn_flashstyle_symmetric_self_pair(
     flag_bits = _lib.flags(use_exp2, allow_tf32)
     kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2)
     made = []
+    # the kernel variant with the coarse tile test, under the single-problem solver's conditions
+    coarse = False
+    if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
+            and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
+            and min(len(ex), len(ey)) >= _COARSE_MIN_STEPS
+            and all(e == ex[0] for e in ex) and all(e == ey[0] for e in ey)):
+        coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
 
     def pair(fx, fy, steps, with_previous=False):  # steps: [(eps_x, eps_y, weight)]
         full = tuple((e1, e2, w, dampening(e1, rho), dampening(e2, rho)) for e1, e2, w in steps)
@@ -391,7 +398,7 @@ def sinkhorn_flashstyle_symmetric_self_pair(
             made.append(_lib.PreparedOperands(xf, yf, flag_bits, self_pair=True))
         return _self_pair_steps_raw(xf, yf, fx, fy, log_a, log_b, full, shift_x=shift_x,
                                     shift_y=shift_y, prepared=made[0],
-                                    with_previous=with_previous, **kw)
+                                    with_previous=with_previous, coarse=coarse, **kw)
 
     def alone(pts, f, log_w, shift, steps):  # steps: [(eps, weight)]
         full = [(e, w, dampening(e, rho), dampening(e, rho)) for e, w in steps]

@@ -686,6 +686,14 @@ def test_solver_with_the_coarse_tile_test_equals_the_plain_solve(monkeypatch, va
     got2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
     for u, v in zip(got2, want2):
         assert float((u - v).abs().max()) < 2e-6 * scale
+    # the paired self problems of a debiased divergence take the same variant
+    px, py = solvers.sinkhorn_flashstyle_symmetric_self_pair(X, A, Y, B, **kw)
+    monkeypatch.setattr(solvers, "COARSE_TEST", False)
+    qx, qy = solvers.sinkhorn_flashstyle_symmetric_self_pair(X, A, Y, B, **kw)
+    for u, v in zip(px + py, qx + qy):
+        assert float((u - v).abs().max()) < 2e-6 * scale
+    for u, v in zip(px, wu):
+        assert float((u - v).abs().max()) < 2e-6 * scale
 
 
 def test_variant_choice_on_the_device():
