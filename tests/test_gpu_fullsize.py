@@ -199,7 +199,7 @@ def test_config1_debiased_loss_and_gradient():
     # the debiased loss is a difference of three O(1) costs: 1e-4 of it plus fp32 round-off
     # of the undebiased terms
     assert abs(float(loss.detach()) - want) <= 1e-4 * abs(want) + 2e-6
-    assert rel_err(gx.detach().cpu().numpy(), fix["grad_x"]) < 2e-4
+    assert rel_err(gx.detach().cpu().numpy(), fix["grad_x"]) < 1e-4
 
 
 @pytest.mark.parametrize("tag,kw", [("reach", dict(reach=1.0)),
@@ -239,7 +239,7 @@ def test_config5_large_d_loss_gradient_and_hvp():
     want = float(fix["loss_debiased"])
     assert abs(float(loss.detach()) - want) <= 1e-4 * abs(want) + 1e-6 * float(fix["loss_xy"])
     g = gx.detach().cpu().numpy().astype(np.float64)
-    assert rel_err(g[rows], fix["grad_x_debiased_rows"].astype(np.float64)) < 2e-4
+    assert rel_err(g[rows], fix["grad_x_debiased_rows"].astype(np.float64)) < 1e-4
     assert abs(np.linalg.norm(g) - float(fix["grad_x_norm"])) < 1e-4 * float(fix["grad_x_norm"])
 
     X2 = torch.from_numpy(x).cuda().requires_grad_(True)
@@ -250,5 +250,5 @@ def test_config5_large_d_loss_gradient_and_hvp():
                    fix["grad_x_xy_rows"].astype(np.float64)) < 1e-4
     (hv,) = torch.autograd.grad((g1 * V).sum(), X2)
     h = hv.cpu().numpy().astype(np.float64)
-    assert rel_err(h[rows], fix["hvp_rows"].astype(np.float64)) < 2e-4
+    assert rel_err(h[rows], fix["hvp_rows"].astype(np.float64)) < 1e-4
     assert abs(np.linalg.norm(h) - float(fix["hvp_norm"])) < 1e-4 * float(fix["hvp_norm"])

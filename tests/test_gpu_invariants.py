@@ -80,7 +80,7 @@ def test_large_d_gradient_matches_oracle(d):
     _, _, fp, gp = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=0.2,
                                              n_iters=10, return_prelast=True)
     want, _ = oracle.grad_barycentric(x, y, a, b, fp, gp, 0.2)
-    assert rel_err(gx, want) < 2e-4
+    assert rel_err(gx, want) < 1e-4
     f, g = solve(X.detach(), Y, A, B, **kw)
     wf, wg = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=0.2, n_iters=10)
     assert rel_err(f, wf) < 1e-4 and rel_err(g, wg) < 1e-4
@@ -144,8 +144,8 @@ def test_otdd_label_cost_solver_loss_and_gradient(lam_x, d):
     c_yy, gyy_1, gyy_2 = ot(y, y, b, b, ly, ly)
     want = c_xy - 0.5 * c_xx - 0.5 * c_yy
     assert abs(float(loss.detach()) - want) < 1e-4 * max(abs(want), abs(c_xy) * 1e-2)
-    assert rel_err(gx, gx_xy - 0.5 * (gxx_1 + gxx_2)) < 3e-4
-    assert rel_err(gy, gy_xy - 0.5 * (gyy_1 + gyy_2)) < 3e-4
+    assert rel_err(gx, gx_xy - 0.5 * (gxx_1 + gxx_2)) < 1e-4
+    assert rel_err(gy, gy_xy - 0.5 * (gyy_1 + gyy_2)) < 1e-4
     with pytest.raises(NotImplementedError):
         (g1,) = torch.autograd.grad(L(X, Y, label_x=LX, label_y=LY), X, create_graph=True)
         torch.autograd.grad(g1.sum(), X)

@@ -31,7 +31,11 @@ def test_symmetric_solver_vs_reference_golden(golden):
     f, g = solve(X, Y, A, B, blur=0.5, scaling=0.7, allow_tf32=False)
     assert rel_err(f, golden["sym_scaling_f"]) < RTOL and rel_err(g, golden["sym_scaling_g"]) < RTOL
     f, g = solve(X, Y, A, B, use_epsilon_scaling=False, eps=0.05, n_iters=20, allow_tf32=False)
+    # the golden vector is the reference's own fp32 torch run, 1.5e-4 from the fp64 answer at
+    # this eps; against the fp64 oracle the bar is 1e-4
     assert rel_err(f, golden["sym_smalleps_f"]) < 2e-4
+    wf, wg = oracle.sinkhorn_symmetric(x, y, a, b, use_epsilon_scaling=False, eps=0.05, n_iters=20)
+    assert rel_err(f, wf) < RTOL and rel_err(g, wg) < RTOL
     # fp16 inputs are cast to fp32 by the launchers (reference test uses fp16 x, y)
     f16, g16 = solve(X.half(), Y.half(), A, B, use_epsilon_scaling=False, eps=0.5, n_iters=3)
     assert rel_err(f16, golden["sym_fixed_f"]) < 2e-3  # the rounding of the inputs to fp16
@@ -129,7 +133,7 @@ def test_samples_loss_value_and_gradient_config1_shape():
                        use_epsilon_scaling=False, eps=0.01, n_iters=100, allow_tf32=False)(X, Y)
     (gx,) = torch.autograd.grad(loss, X)
     assert abs(float(loss) - want) <= 1e-4 * max(abs(want), 1e-3) + 2e-6
-    assert rel_err(gx, want_gx) < 2e-4
+    assert rel_err(gx, want_gx) < RTOL
 
 
 def test_samples_loss_api_forms():
@@ -166,18 +170,22 @@ def test_hvp_vs_reference_golden_and_oracle(golden):
     A, f, g = golden["hvp_A"], golden["hvp_f_ott"], golden["hvp_g_ott"]
     X, Y, F, G, AA = dev(x, y, f, g, A)
     h, info = hvp(X, Y, F, G, AA, eps=0.2)
+    # the golden vector is the reference's fp32 CG run (1.4e-4 from the fp64 dense solve); the
+    # fp64 oracle, itself pinned by that vector and by finite differences, is the 1e-4 bar
     assert rel_err(h, golden["hvp_plain"]) < 2e-4 and info.cg_converged
+    want, _ = oracle.hvp_x_from_potentials(x, y, f, g, A, eps=0.2)
+    assert rel_err(h, want) < RTOL
     for tag, rx, ry in (("hvp_semi_x", 1.0, None), ("hvp_semi_y", None, 0.5),
                         ("hvp_unbal", 1.0, 2.0)):
         h, info = hvp(X, Y, F, G, AA, eps=0.2, rho_x=rx, rho_y=ry)
-        assert rel_err(h, golden[tag]) < 2e-4
+        assert rel_err(h, golden[tag]) < RTOL
     # half cost and the preconditioned operator: restatement only (see oracle header)
     want, _ = oracle.hvp_x_from_potentials(x, y, f, g, A, eps=0.2, cost_scale=0.5,
                                            preconditioner="jacobi")
     h, _ = hvp(X, Y, F, G, AA, eps=0.2, cost_scale=0.5, preconditioner="jacobi")
-    assert rel_err(h, want) < 2e-4
+    assert rel_err(h, want) < RTOL
     psd, ind, _ = hvp(X, Y, F, G, AA, eps=0.2, return_components=True)
-    assert rel_err(psd + ind, golden["hvp_plain"]) < 2e-4
+    assert rel_err(psd + ind, golden["hvp_plain"]) < 2e-4  # fp32 golden, as above
 
 
 def test_double_backward_equals_direct_hvp():
