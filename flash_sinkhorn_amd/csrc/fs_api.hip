@@ -42,7 +42,7 @@ int scratch_on_current_device(void** out) {
 constexpr int kMaxStreamD = 128;    // register-stationary streaming kernels
 constexpr int kMaxSlicedD = 16384;  // widest supported rows
 constexpr int kSlicedSpan = 1536;   // columns one workgroup of the column-sliced kernels spans
-constexpr int kPlanePadRowsApi = 256;  // must match kPlanePadRows of the plane-splitting kernels
+constexpr int kPlanePadRowsApi = 512;  // must match kPlanePadRows of the plane-splitting kernels
 // after the planes: absmax partials [2][256], plane scales [4] (+4 spare), variant-choice state
 constexpr size_t kPlaneAuxBytes = (2 * 256 + 8 + kSelWords) * sizeof(float);
 static_assert(kSelWords <= 256, "the state is cleared by one workgroup");
@@ -781,7 +781,12 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const bool can_coarse = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && !(flags & FS_FLAG_NO_TILE_SKIP);
   const bool coarse = (flags & FS_FLAG_COARSE_TEST) && can_coarse;
   const bool auto_sel = (flags & FS_FLAG_COARSE_AUTO) && can_coarse && !coarse && prepared;
-  if (coarse || auto_sel) rb = 2;  // that kernel works on two row blocks per wavefront
+  Family fam_plan = fam;
+  if (coarse || auto_sel) {  // that kernel works on two row blocks per wavefront and 128-key tiles
+    rb = 2;
+    fam_plan.jt = 128;
+    for (int s = 0; s < nsides; ++s) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam_plan, rb);
+  }
   PlaneSet ps;
   ps.n = 0;
   ps.end = 0;
@@ -793,7 +798,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const size_t need_planes_end = need;
   for (int s = 0; s < nsides; ++s) {
     // both sides run in one launch and must share the rows-per-wave template
-    if (!fam.sliced && plans[s].rb != rb) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam, rb);
+    if (!fam.sliced && plans[s].rb != rb) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam_plan, rb);
     need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
   }
   // lse_coarse_kernel: per-tile records of the key bias, behind the partial rows

@@ -119,9 +119,11 @@ struct LaunchArgs {
   int sel_pred;  // 0: the launch runs whatever the state says (it still counts into it)
 };
 
-// Per 64-key tile record of coarse_bias_kernel: eight fp16 copies of a_j per key (4 words each),
-// then b_j - 2^18 a_j per key, then the largest bias of each 32-key sub-tile, padded to 16 bytes.
-constexpr int kAuxA = 0, kAuxB = 256, kAuxMax = 320, kAuxWords = 324, kAuxPadTiles = 4;
+// Record of coarse_bias_kernel per 64 keys: eight fp16 copies of a_j per key (4 words each), then
+// b_j - 2^18 a_j per key, then the largest bias of each 32-key sub-tile in the first two of 64
+// words: three parts that one wavefront moves with one full instruction each (16, 4 and 4
+// bytes per lane).
+constexpr int kAuxA = 0, kAuxB = 256, kAuxMax = 320, kAuxWords = 384, kAuxPadTiles = 8;
 
 // Device state of the variant choice (unsigned words), zeroed when the operand planes are
 // written: which variant runs (0: coarse tile test, 1: plain), how many decisions were taken,

@@ -43,7 +43,7 @@ namespace fs {
 
 enum Prec : int { kF32 = 0, kH3 = 3 };
 
-constexpr int kPlanePadRows = 256;  // zero rows after the last row of a plane buffer
+constexpr int kPlanePadRows = 512;  // zero rows after the last row of a plane buffer
 constexpr int kAbsmaxBlocks = 256;  // partial maxima per matrix written by absmax_kernel
 
 

@@ -24,9 +24,10 @@
 // Nothing a conditional block computes outlives it except the running (maximum, sum) of the
 // rows and the key of the maximum: no accumulator tile is carried across a branch, so the
 // register allocator never has to reconcile two versions of one (four tiles hold the hi*hi
-// products of two sub-tiles, and they are only ever written unconditionally).  Only the hi
-// plane of a sub-tile is read from LDS up front (two sub-tiles ahead); a unit that goes on
-// reads both planes and the per-key biases of its sub-tile again.  A unit that ends costs
+// products of two sub-tiles, and they are only ever written unconditionally).  Key tiles hold
+// hi planes only (128 keys, 16 KiB at 64 columns, ring of four, three tiles ahead, one barrier
+// per tile): the few units that go on read the hi plane and the per-key biases of their
+// sub-tile again from LDS and fetch the lo plane from global memory.  A unit that ends costs
 // four and a half MFMAs (the a_j step serves both row blocks), a 16-value maximum and a ballot.
 //
 // What the test can end depends on where a row's running maximum starts.  The launch keeps,
@@ -37,11 +38,11 @@
 // start from the largest logit of 64 keys sampled evenly over the whole key set, so that a key
 // chunk without any of the row's near keys is measured against a meaningful maximum from its
 // first tile on.  The key-side quantities of the test (a_j, b_j - 2^18 a_j, bmax per sub-tile)
-// are the same for every workgroup: coarse_bias_kernel writes them once per launch, per 64-key
-// tile, in the layout of the tile's LDS record.
+// are the same for every workgroup: coarse_bias_kernel writes them once per launch, one record
+// per 64 keys, in the layout the records take in LDS.
 //
 // Everything LDS-related is written out by hand (ds_read / ds_write / s_waitcnt / s_barrier):
-// key tiles arrive by direct global->LDS loads two tiles ahead, and the compiler, which
+// key tiles arrive by direct global->LDS loads three tiles ahead, and the compiler, which
 // cannot tell a read of one ring buffer from the loads still filling another, would make
 // every LDS access wait for all of them.
 #pragma once
@@ -92,24 +93,30 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
   unsigned* rec = sd.key_aux + (size_t)tile * kAuxWords;
   *reinterpret_cast<u32x4*>(rec + kAuxA + lane * 4) = u32x4{aw, aw, aw, aw};
   rec[kAuxB + lane] = __builtin_bit_cast(unsigned, b - (float)ah * 0x1p18f);
-  if (li == 0) rec[kAuxMax + h] = __builtin_bit_cast(unsigned, mx);
-  if (lane < kAuxWords - kAuxMax - 2) rec[kAuxMax + 2 + lane] = 0u;
+  const float mx_sub = __shfl(mx, (lane & 1) * 32, 64);  // lanes 0 and 1: the two sub-tiles' maxima
+  rec[kAuxMax + lane] = lane < 2 ? __builtin_bit_cast(unsigned, mx_sub) : 0u;
 }
 
 template <int DP>
 __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs args) {
   static_assert(DP == 16 || DP == 32 || DP == 64, "two-plane rows of at most 64 columns");
   constexpr int RB = 2;                // blocks of 32 query rows per wavefront
-  constexpr int JT = 64;               // keys per tile
+  constexpr int JT = 128;              // keys per tile: hi planes only, four 32-key sub-tiles
+  constexpr int NSUB = JT / 32;
+  constexpr int NREC = JT / 64;        // bias records (64 keys each) per tile
   constexpr int KK16 = DP / 16;        // MFMAs of one plane product
-  constexpr int ROWW = DP;             // 32-bit words per two-plane row
-  constexpr int PPR = ROWW / 4;        // 16-byte pieces per row
-  constexpr int PER_THREAD = JT * PPR / 256;
+  constexpr int ROWW = DP;             // 32-bit words per two-plane row in global memory
+  constexpr int PPR = ROWW / 4;        // 16-byte pieces per two-plane row
+  constexpr int ROWH = DP / 2;         // words per hi-plane row in LDS
+  constexpr int PPRH = ROWH / 4;       // 16-byte pieces per hi-plane row
+  constexpr int PER_THREAD = JT * PPRH / 256;
+  static_assert(64 * PPR == JT * PPRH, "the 64 sampled two-plane rows fill one tile buffer");
   constexpr int NBUF = 4;              // ring of key tiles in LDS: tile t+3 is requested during tile t
 
-  __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][JT * ROWW];
-  // per tile: eight copies of a_j (fp16) per key, b_j - 2^18 a_j per key, bmax of the two sub-tiles
-  __shared__ __attribute__((aligned(16))) unsigned lds_aux[NBUF][kAuxWords];
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][JT * ROWH];
+  // per 64 keys of a tile: eight copies of a_j (fp16) per key, b_j - 2^18 a_j per key, bmax of
+  // the two sub-tiles
+  __shared__ __attribute__((aligned(16))) unsigned lds_aux[NBUF][NREC * kAuxWords];
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
@@ -208,9 +215,13 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  auto swz = [&](int r) {  // slot permutation of LDS row r
-    return PPR >= 16 ? (r & 15) : (PPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3));
+  // slot permutation of LDS row r when a row has `ppr` 16-byte pieces: b128 reads of 32
+  // consecutive rows at one piece index then spread over all banks
+  auto swz_of = [](int r, int ppr) {
+    return ppr >= 16 ? (r & 15) : (ppr == 8 ? ((r >> 1) & 7) : (ppr == 4 ? ((r >> 2) & 3) : ((r >> 3) & 1)));
   };
+  auto swz = [&](int r) { return swz_of(r, PPR); };    // the sampled two-plane rows
+  auto swzh = [&](int r) { return swz_of(r, PPRH); };  // hi-plane rows of a key tile
 
   // ---- key tiles: lane idx of instruction c fills LDS slot idx and fetches the piece that
   // belongs there (slot = piece ^ swz(row)); the plane buffers end in zero rows, so tiles past
@@ -219,8 +230,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
 #pragma unroll
   for (int c = 0; c < PER_THREAD; ++c) {
     const int idx = tid + 256 * c;
-    const int r = idx / PPR;
-    const int piece = (idx % PPR) ^ swz(r);
+    const int r = idx / PPRH;
+    const int piece = (idx % PPRH) ^ swzh(r);  // a piece of the hi plane, the first half of the row
     kp[c] = sd.kplanes + (size_t)(j_begin + r) * (size_t)ROWW + piece * 4;
   }
   auto issue_tile = [&](int buf) {  // the next tile in sequence
@@ -241,32 +252,48 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
   const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
   const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
-  const unsigned* auxp = sd.key_aux + (size_t)(j_begin / JT) * kAuxWords + lane * 4;
+  const unsigned* auxp = sd.key_aux + (size_t)(j_begin / 64) * kAuxWords + lane * 4;
   auto issue_aux = [&](int buf) {  // the next tile in sequence
-    if (wave == 0) {
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)auxp,
-          (__attribute__((address_space(3))) void*)(&lds_aux[buf][0]), 16, 0, 0);
-      if (lane < (kAuxWords - 256) / 4)
+    if (wave == 0) {  // every instruction with all 64 lanes: 16, 4 and 4 bytes per lane
+#pragma unroll
+      for (int rec = 0; rec < NREC; ++rec) {
+        const unsigned* src = auxp + rec * kAuxWords;  // auxp: word 4 * lane of the record
         __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(auxp + 256),
-            (__attribute__((address_space(3))) void*)(&lds_aux[buf][256]), 16, 0, 0);
+            (const __attribute__((address_space(1))) void*)src,
+            (__attribute__((address_space(3))) void*)(&lds_aux[buf][rec * kAuxWords + kAuxA]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(src - 3 * lane + kAuxB),
+            (__attribute__((address_space(3))) void*)(&lds_aux[buf][rec * kAuxWords + kAuxB]), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(src - 3 * lane + kAuxMax),
+            (__attribute__((address_space(3))) void*)(&lds_aux[buf][rec * kAuxWords + kAuxMax]), 4, 0, 0);
+      }
     }
-    auxp += kAuxWords;
+    auxp += NREC * kAuxWords;
   };
-  auto lds_b = [&](int buf, int k) { return reinterpret_cast<const float*>(&lds_aux[buf][kAuxB + k]); };
+  // word `what` (+ key k of the sub-tile) in the record that holds sub-tile js of buffer buf
+  auto aux_at = [&](int buf, int js, int what) {
+    return &lds_aux[buf][(js >> 1) * kAuxWords + what];
+  };
 
   auto mfma16 = [](const u32x4& a, const u32x4& b, const f32x16& c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   };
-  // 16-byte piece (plane, step kk, half h) of key row js*32 + li
-  auto read_plane = [&](u32x4 (&dst)[KK16], int buf, int js, int plane) {
-    const unsigned* yrow = lds_k[buf] + (js * 32 + li) * ROWW;
+  // 16-byte piece (step kk, half h) of the hi plane of key row js*32 + li of a key tile
+  auto read_hi = [&](u32x4 (&dst)[KK16], int buf, int js) {
+    const unsigned* yrow = lds_k[buf] + (js * 32 + li) * ROWH;
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk)
+      dst[kk] = ds_read16(yrow + (((2 * kk + h) ^ swzh(li)) << 2));  // swzh(js*32 + li) == swzh(li)
+  };
+  // the same of either plane of sampled two-plane row js*32 + li (buffer 0)
+  auto read_sampled = [&](u32x4 (&dst)[KK16], int js, int plane) {
+    const unsigned* yrow = lds_k[0] + (js * 32 + li) * ROWW;
 #pragma unroll
     for (int kk = 0; kk < KK16; ++kk) {
       const int piece = plane * (DP / 8) + 2 * kk + h;
-      dst[kk] = ds_read16(yrow + ((piece ^ swz(li)) << 2));  // swz(js*32 + li) == swz(li)
+      dst[kk] = ds_read16(yrow + ((piece ^ swz(li)) << 2));
     }
   };
   // v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its
@@ -343,7 +370,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // a workgroup with a row that has no key yet also samples 64 keys spread over the whole key set
   const bool cold = __syncthreads_or(have ? 0 : 1) != 0;
   if (cold) {
-    const int stride = sd.nk / JT;  // sampled keys: 0, stride, 2 stride, ...
+    const int stride = sd.nk / 64;  // sampled keys: 0, stride, 2 stride, ...
     if (wave == 0) {
       const int j = lane * stride;
       float b = kc0 * sd.kb0[j] + (has_kb1 ? kc1 * kb1p[j] : 0.f);
@@ -365,9 +392,9 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     barrier();
 #pragma unroll
     for (int js = 0; js < 2; ++js) {
-      read_plane(KH[0], 0, js, 0);
-      read_plane(KL, 0, js, 1);
-      kbias = ds_read4(lds_b(0, js * 32 + li));
+      read_sampled(KH[0], js, 0);
+      read_sampled(KL, js, 1);
+      kbias = ds_read4(reinterpret_cast<const float*>(&lds_aux[0][kAuxB + js * 32 + li]));
       wait_lds();
 #pragma unroll
       for (int kk = 0; kk < KK16; ++kk) {
@@ -429,9 +456,9 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   };
   // hi plane, a_j piece and bmax of sub-tile js of the tile in buffer b, into register set k
   auto request = [&](int k, int b, int js) {
-    read_plane(KH[k], b, js, 0);
-    KA[k] = ds_read16(&lds_aux[b][kAuxA + (js * 32 + li) * 4]);
-    bmax[k] = ds_read4(lds_b(b, JT + js));
+    read_hi(KH[k], b, js);
+    KA[k] = ds_read16(aux_at(b, js, kAuxA + ((js & 1) * 32 + li) * 4));
+    bmax[k] = ds_read4(reinterpret_cast<const float*>(aux_at(b, js, kAuxMax + (js & 1))));
   };
   auto arrived = [&](int k) {  // after a wait: every later use of set k sits behind this point
 #pragma unroll
@@ -446,15 +473,16 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // moved on to a later sub-tile).
   auto go_on = [&](const f32x16& hh, u32x4 (&KX)[KK16], int b, int js, int rb, bool first, int kbase) {
     if (first) {  // first unit of the sub-tile to go on
-      read_plane(KX, b, js, 0);
-      read_plane(KL, b, js, 1);
-      kbias = ds_read4(lds_b(b, js * 32 + li));
+      // the lo plane is not in LDS: the few units that get here fetch it from global memory
+      // (the second half of a key's two-plane row; the compiler places the wait)
+      const unsigned* lrow = sd.kplanes + (size_t)(kbase + li) * (size_t)ROWW + DP / 2 + 4 * h;
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk) KL[kk] = *reinterpret_cast<const u32x4*>(lrow + 8 * kk);
+      read_hi(KX, b, js);
+      kbias = ds_read4(reinterpret_cast<const float*>(aux_at(b, js, kAuxB + (js & 1) * 32 + li)));
       wait_lds();
 #pragma unroll
-      for (int kk = 0; kk < KK16; ++kk) {
-        pin4(KX[kk]);
-        pin4(KL[kk]);
-      }
+      for (int kk = 0; kk < KK16; ++kk) pin4(KX[kk]);
       pin1(kbias);
     }
     FS_LC_FENCE();
@@ -596,8 +624,11 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     if (t > 0) start_of_tile(t);
     const int b = t & 3, nb = (t + 1) & 3;
     const int kb = j_begin + t * JT;
-    step(std::integral_constant<int, 0>{}, b, 0, nb, 0, kb);  // sub-tile 0: multiplies sub-tile 1, requests (t+1, 0)
-    step(std::integral_constant<int, 1>{}, b, 1, nb, 1, kb + 32);  // sub-tile 1: multiplies (t+1, 0), requests (t+1, 1)
+    // sub-tile js multiplies sub-tile js+1 and requests sub-tile js+2 (the last two: of tile t+1)
+    step(std::integral_constant<int, 0>{}, b, 0, b, 2, kb);
+    step(std::integral_constant<int, 1>{}, b, 1, b, 3, kb + 32);
+    step(std::integral_constant<int, 0>{}, b, 2, nb, 0, kb + 64);
+    step(std::integral_constant<int, 1>{}, b, 3, nb, 1, kb + 96);
   }
   wait_all();  // tiles fetched past the chunk: let them land before the workgroup ends
 
@@ -606,7 +637,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   if (args.sel != nullptr && lane == 0 && ntiles > 0 && !(track && cold)) {
     const int slot = blockIdx.x % kSelSlots;
     atomicAdd(&args.sel[kSelEnded + slot], n_ended);
-    atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * 4));
+    atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
   }
 
 #pragma unroll
