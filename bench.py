@@ -117,6 +117,78 @@ def cpu_baseline(x, y, a, b, budget_s=20.0):
     }
 
 
+def cpu_baseline_other_configs():
+    """The numpy fp32 oracle on the host cores at the other four benchmark configurations, per
+    unit of work (--cpu-configs; about three minutes).  Seeds and shapes as in BASELINE's
+    configurations; every figure is wall time of the dense / row-chunked oracle."""
+    import numpy as np
+
+    import oracle
+
+    def timed(fn, reps=1):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2] * 1e3
+
+    out = {}
+    f32 = np.float32
+    # configuration 1: n = m = 2000, d = 3, eps = 0.01, half cost, 100 iterations, the three
+    # solves of a debiased loss, median of 3
+    rng = np.random.default_rng(1)
+    x, y = rng.standard_normal((2000, 3)).astype(f32), rng.standard_normal((2000, 3)).astype(f32)
+    a = np.full(2000, 1 / 2000, f32)
+    kw = dict(use_epsilon_scaling=False, eps=0.01, n_iters=100, cost_scale=0.5, dtype=f32)
+
+    def c1():
+        for p, q in ((x, y), (x, x), (y, y)):
+            oracle.sinkhorn_symmetric(p, q, a, a, **kw)
+    out["c1_debiased_solves_100_iters_ms"] = timed(c1, 3)
+    # configuration 2: n = m = 10,000, d = 64: 5 symmetric iterations timed, scaled to 100 + 2
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((10000, 64)).astype(f32)
+    y = (rng.standard_normal((10000, 64)) + 0.5).astype(f32)
+    a = np.full(10000, 1e-4, f32)
+    la = np.log(a)
+    fh, gh = -(x * x).sum(1), -(y * y).sum(1)
+
+    def c2():
+        for _ in range(5):
+            oracle.symmetric_step(x, y, fh, gh, la, la, 0.01, 1.0, 0.5, 1.0, 1.0, dtype=f32)
+    out["c2_xy_solve_100_iters_ms_from_5_steps"] = timed(c2) / 5 * 102
+    # configuration 4: n = 20,000, m = 30,000, d = 128: one alternating iteration (two half-updates)
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((20000, 128)).astype(f32)
+    y = (1.5 * rng.standard_normal((30000, 128))).astype(f32)
+    a = rng.dirichlet(np.ones(20000)).astype(f32)
+    b = (1.3 * rng.dirichlet(np.ones(30000))).astype(f32)
+    out["c4_one_alternating_iteration_ms"] = timed(lambda: oracle.sinkhorn_alternating(
+        x, y, a, b, eps=0.0025, n_iters=1, reach=1.0, dtype=f32))
+    # configuration 5: n = m = 8192, d = 1536: one gradient (both sides), one plan-vector product
+    # pair (the matrix-vector work of one CG iteration)
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((8192, 1536)) / np.sqrt(1536)).astype(f32)
+    y = (rng.standard_normal((8192, 1536)) / np.sqrt(1536)).astype(f32)
+    a = np.full(8192, 1 / 8192, f32)
+    la = np.log(a)
+    fz = np.zeros(8192, f32)
+    out["c5_one_gradient_ms"] = timed(lambda: oracle.grad_barycentric(x, y, a, a, fz, fz, 0.25,
+                                                                      dtype=f32))
+    fh, gh = -(x * x).sum(1), -(y * y).sum(1)
+    v = rng.standard_normal(8192).astype(f32)
+
+    def c5_cg():
+        w = oracle.apply_plan_vec(x, y, fh, gh, la, la, v, 0.25, 1, dtype=f32)
+        oracle.apply_plan_vec(x, y, fh, gh, la, la, w, 0.25, 0, dtype=f32)
+    out["c5_one_cg_iteration_matvecs_ms"] = timed(c5_cg)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    out.update(cores=cores, cpu_model=cpu_model(), kind="port",
+               note="numpy fp32 oracle, BLAS threads = host default")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -127,6 +199,9 @@ def main():
     ap.add_argument("--d", type=int, default=D)
     ap.add_argument("--mode", choices=MODES, default="strict")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-configs", action="store_true",
+                    help="also time the CPU oracle at the other four benchmark configurations "
+                         "(per unit of work; about three minutes)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the comparison timings (other operand mode, data-independent "
                          "solve, every-exponential launch, 101-step solve)")
@@ -322,6 +397,8 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(x, y, a, b)
+    if args.cpu_configs:
+        line["cpu_baseline_other_configs"] = cpu_baseline_other_configs()
     print(json.dumps(line))
 
 

@@ -65,6 +65,30 @@ def test_unbalanced_symmetric_vs_oracle(kw):
     assert rel_err(f, wf) < RTOL and rel_err(g, wg) < RTOL
 
 
+@pytest.mark.parametrize("rx,ry", [(2.0, 0.7), (0.7, 2.0), (1.5, None), (None, 0.9)])
+def test_unbalanced_symmetric_fixed_point_on_the_gpu(rx, ry):
+    """No oracle involved: the GPU's unbalanced symmetric solver, run to its fixed point, returns
+    potentials whose plan (its marginals taken with the GPU's plan-vector product) satisfies the
+    first-order conditions of the KL-relaxed problem, P 1 = a exp(-f / rho_x) and
+    P^T 1 = b exp(-g / rho_y), a balanced side meaning exp(.) = 1."""
+    from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_symmetric as solve
+    from flash_sinkhorn_amd.kernels.apply_flash import apply_plan_vec_flashstyle as apply_vec
+    x, y, a, b = inputs(33, 300, 260, 8, scale=0.5)
+    b = (b * 1.3).astype(np.float32)
+    eps = 0.5
+    X, Y, A, B = dev(x, y, a, b)
+    f, g = solve(X, Y, A, B, use_epsilon_scaling=False, eps=eps, n_iters=600, allow_tf32=False,
+                 rho_x=rx, rho_y=ry)
+    fh, gh = f - (X * X).sum(1), g - (Y * Y).sum(1)
+    la, lb = torch.log(A), torch.log(B)
+    row = apply_vec(X, Y, fh, gh, la, lb, torch.ones_like(B), eps=eps, axis=1)
+    col = apply_vec(X, Y, fh, gh, la, lb, torch.ones_like(A), eps=eps, axis=0)
+    want_row = A * (torch.exp(-f / rx) if rx is not None else 1.0)
+    want_col = B * (torch.exp(-g / ry) if ry is not None else 1.0)
+    assert float((row - want_row).abs().max()) < 1e-4 * float(want_row.max())
+    assert float((col - want_col).abs().max()) < 1e-4 * float(want_col.max())
+
+
 def test_alternating_solver(golden):
     from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating as solve
     x, y, a, b = inputs(12, 40, 56, 16)
