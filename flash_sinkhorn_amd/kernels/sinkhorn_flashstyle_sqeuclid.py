@@ -62,9 +62,11 @@ def flashsinkhorn_lse(
     cost_scale: float = 1.0, damping: float = 1.0, allow_tf32: bool = True,
     use_exp2: bool = True, block_m: Optional[int] = None, block_n: Optional[int] = None,
     block_k: Optional[int] = None, num_warps: Optional[int] = None, num_stages: int = 2,
-    autotune: bool = True, _prepared: Optional[_lib.PreparedOperands] = None,
+    autotune: bool = True, _prepared: Optional[_lib.PreparedOperands] = None, _coarse=False,
 ) -> torch.Tensor:
-    """out_i = -eps*damping*LSE_j[2*cost_scale*x_i.y_j/eps + bias_j]; returns fp32 [n]."""
+    """out_i = -eps*damping*LSE_j[2*cost_scale*x_i.y_j/eps + bias_j]; returns fp32 [n].
+    ``_prepared`` / ``_coarse`` (not in the reference): operand planes converted up front, and
+    the kernel variant as in ``_symmetric_step_raw``."""
     if not x.is_cuda or not y.is_cuda:
         raise ValueError("x and y must be CUDA tensors")
     if x.ndim != 2 or y.ndim != 2:
@@ -81,6 +83,7 @@ def flashsinkhorn_lse(
     out = torch.empty((n,), device=x.device, dtype=torch.float32)
     wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_LSE, x, y, _lib.flags(use_exp2, allow_tf32),
                                            _prepared)
+    fl |= _lib.coarse_flag(_coarse)
     rc = _lib.lib().fs_lse(
         x.data_ptr(), y.data_ptr(), bias.data_ptr(), out.data_ptr(), n, m, d,
         float(eps), 2.0 * float(cost_scale), float(damping), fl, wp, wn, _lib.stream_of(x))
@@ -93,7 +96,7 @@ def flashsinkhorn_lse_fused(
     cost_scale: float = 1.0, damping: float = 1.0, allow_tf32: bool = True,
     use_exp2: bool = True, block_m: Optional[int] = None, block_n: Optional[int] = None,
     block_k: Optional[int] = None, num_warps: Optional[int] = None, num_stages: int = 2,
-    autotune: bool = True, _prepared: Optional[_lib.PreparedOperands] = None,
+    autotune: bool = True, _prepared: Optional[_lib.PreparedOperands] = None, _coarse=False,
 ) -> torch.Tensor:
     """Same as flashsinkhorn_lse with bias_j = g_hat_j/eps + log_w_j formed in the kernel."""
     if not x.is_cuda or not y.is_cuda:
@@ -108,6 +111,7 @@ def flashsinkhorn_lse_fused(
     out = torch.empty((n,), device=x.device, dtype=torch.float32)
     wp, wn, fl, _keep = _lib.lse_workspace(_lib.OP_LSE, x, y, _lib.flags(use_exp2, allow_tf32),
                                            _prepared)
+    fl |= _lib.coarse_flag(_coarse)
     rc = _lib.lib().fs_lse_fused(
         x.data_ptr(), y.data_ptr(), g_hat.data_ptr(), log_w.data_ptr(), out.data_ptr(), n, m, d,
         float(eps), 2.0 * float(cost_scale), float(damping), fl, wp, wn, _lib.stream_of(x))

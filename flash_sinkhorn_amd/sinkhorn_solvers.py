@@ -110,8 +110,15 @@ def sinkhorn_flashstyle_alternating(
     prev_f, prev_g = (f_hat.clone(), g_hat.clone()) if threshold is not None else (None, None)
     # operand planes are converted once for the whole loop
     prepared = _lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32))
+    # the kernel variant with the coarse tile test (see COARSE_TEST): every half-update starts
+    # its rows from the keys of the same half-update one iteration earlier
+    coarse = False
+    if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
+            and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
+            and int(n_iters) >= _COARSE_MIN_STEPS):
+        coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
     kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
-              _prepared=prepared)
+              _prepared=prepared, _coarse=coarse)
 
     used = 0
     for it in range(int(n_iters)):

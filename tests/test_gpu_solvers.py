@@ -719,9 +719,16 @@ def test_solver_with_the_coarse_tile_test_equals_the_plain_solve(monkeypatch, va
     got2 = solvers.sinkhorn_flashstyle_symmetric(X, X, A, A2, **kw)
     for u, v in zip(got2, want2):
         assert float((u - v).abs().max()) < 2e-6 * scale
-    # the paired self problems of a debiased divergence take the same variant
+    # the alternating solver (both conventions, one of them unbalanced) takes the same variant
+    akw = [dict(eps=0.05, n_iters=10, allow_tf32=False, reach=1.5),
+           dict(eps=0.05, n_iters=10, allow_tf32=False, ott_convention=True)]
+    alt = [solvers.sinkhorn_flashstyle_alternating(X, Y, A, B, **k) for k in akw]
+    # the paired self problems of a debiased divergence too
     px, py = solvers.sinkhorn_flashstyle_symmetric_self_pair(X, A, Y, B, **kw)
     monkeypatch.setattr(solvers, "COARSE_TEST", False)
+    for k, got_alt in zip(akw, alt):
+        for u, v in zip(got_alt, solvers.sinkhorn_flashstyle_alternating(X, Y, A, B, **k)):
+            assert float((u - v).abs().max()) < 2e-6 * scale
     qx, qy = solvers.sinkhorn_flashstyle_symmetric_self_pair(X, A, Y, B, **kw)
     for u, v in zip(px + py, qx + qy):
         assert float((u - v).abs().max()) < 2e-6 * scale
