@@ -93,7 +93,8 @@ Family family_for(int64_t d) {
 }
 
 // Rows per wavefront (RB blocks of 32) and the key split for one side.
-SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam, int rb_force = 0) {
+SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam, int rb_force = 0,
+                   int min_splits = 1) {
   SidePlan p;
   const bool has_o = (mode == kMat || mode == kMat5);
   const int dp = fam.dp;
@@ -113,6 +114,7 @@ SidePlan plan_side(int mode, int64_t nq, int64_t nk, const Family& fam, int rb_f
   const int cap = has_o ? 16 : 64;
   int s = 1;
   while (p.igroups * s < target && s * 2 <= max_splits && s * 2 <= cap) s *= 2;
+  s = std::max(s, min_splits);
   p.chunk = ceil_div(ceil_div(nk, s), jt) * jt;
   p.splits = ceil_div(nk, p.chunk);
   return p;
@@ -199,6 +201,8 @@ struct PlaneSet {
   int rows[2];
   size_t off[2];
   size_t aux_off, end;
+  size_t margin_off, margin_slot;  // two slots of carried margins behind the aux block (0: none)
+  int margin_stride;               // sub-tiles per wavefront row of a slot
 };
 
 // Bytes of one matrix's planes alone, and of its whole region: the planes, then one int per row
@@ -207,8 +211,30 @@ size_t planes_only_bytes(int64_t rows, const LseConfig& c) {
   return (((size_t)(rows + kPlanePadRowsApi) * (size_t)c.np * (size_t)(c.dp / 2) * 4) + 15) & ~(size_t)15;
 }
 
+// One 4-byte value per row, 16-byte aligned; a matrix keeps three such arrays behind its planes:
+// the key behind each row's largest logit, that logit (the merged maximum of the last launch
+// with the matrix as the stationary one), and the row's bias of the last launch as a key.
+size_t row_array_bytes(int64_t rows) { return ((size_t)rows * 4 + 15) & ~(size_t)15; }
+
+// Second copy of two-plane rows of at most 64 columns in MFMA operand order (Side::ktiled),
+// whole blocks of 32 rows.
+size_t tiled_bytes(int64_t rows, const LseConfig& c) {
+  if (c.gemm || c.prec != 3 || c.dp > 64) return 0;
+  return (size_t)ceil_div(rows + kPlanePadRowsApi, 32) * 32 * (size_t)c.dp * 4;
+}
+
 size_t plane_bytes(int64_t rows, const LseConfig& c) {
-  return planes_only_bytes(rows, c) + (((size_t)rows * sizeof(int) + 15) & ~(size_t)15);
+  return planes_only_bytes(rows, c) + 3 * row_array_bytes(rows) + tiled_bytes(rows, c);
+}
+
+// Carried margins of lse_coarse_kernel: per wavefront (64 rows) and 32-key sub-tile two entries.
+// A slot serves any pairing of the set's matrices as (stationary, streamed).
+int margin_stride_for(int64_t max_rows) { return (ceil_div(max_rows, 128) + 1) * 4; }
+size_t margin_slot_bytes(int64_t max_rows, const LseConfig& c) {
+  if (c.gemm || c.prec != 3 || c.dp > 64) return 0;
+  // wavefront rows in whole workgroups of four: the last workgroup's spare wavefronts keep entries too
+  const size_t b = (size_t)ceil_div(max_rows, 256) * 4 * (size_t)margin_stride_for(max_rows) * 8;
+  return b <= ((size_t)128 << 20) ? b : 0;
 }
 
 // Distinct (pointer, rows) operands among up to four candidates, in canonical order.
@@ -216,6 +242,8 @@ int make_plane_set(const float* const* ptrs, const int* rows, int count, const L
                    PlaneSet& ps) {
   ps.n = 0;
   ps.aux_off = ps.end = 0;
+  ps.margin_off = ps.margin_slot = 0;
+  ps.margin_stride = 0;
   if (c.prec == 0) return FS_OK;
   for (int k = 0; k < count; ++k) {
     bool seen = false;
@@ -237,6 +265,12 @@ int make_plane_set(const float* const* ptrs, const int* rows, int count, const L
   }
   ps.aux_off = need;
   ps.end = need + kPlaneAuxBytes;
+  int64_t max_rows = 0;
+  for (int i = 0; i < ps.n; ++i) max_rows = std::max<int64_t>(max_rows, ps.rows[i]);
+  ps.margin_off = ps.end;
+  ps.margin_slot = ps.n > 0 ? margin_slot_bytes(max_rows, c) : 0;
+  ps.margin_stride = margin_stride_for(max_rows);
+  ps.end += 2 * ps.margin_slot;
   return FS_OK;
 }
 
@@ -268,11 +302,30 @@ int* best_keys_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float*
   return nullptr;
 }
 
+float* row_array_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float* src, int rows,
+                    int which) {  // 1: last maxima, 2: last biases
+  int* keys = best_keys_of(ps, c, ws, src, rows);
+  if (keys == nullptr) return nullptr;
+  return reinterpret_cast<float*>(reinterpret_cast<char*>(keys) + which * row_array_bytes(rows));
+}
+
+unsigned* tiled_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float* src, int rows) {
+  if (tiled_bytes(rows, c) == 0) return nullptr;
+  int* keys = best_keys_of(ps, c, ws, src, rows);
+  if (keys == nullptr) return nullptr;
+  return reinterpret_cast<unsigned*>(reinterpret_cast<char*>(keys) + 3 * row_array_bytes(rows));
+}
+
 // Writes the planes (and, for fp16, the scales) of every matrix of the set.
-int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws, hipStream_t st) {
+int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws, hipStream_t st,
+                     bool clear_margins = false) {
   if (ps.n == 0) return FS_OK;
   char* base = static_cast<char*>(ws);
   int rc = FS_OK;
+  if (clear_margins && ps.margin_slot > 0)
+    rc = launch_fill_zero(reinterpret_cast<unsigned*>(base + ps.margin_off),
+                          (long long)(2 * ps.margin_slot / 4), st);
+  if (rc != FS_OK) return rc;
   {
     float* partial = reinterpret_cast<float*>(base + ps.aux_off);
     float* scales = partial + 2 * 256;
@@ -284,7 +337,8 @@ int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws
                                    ps.rows[i], (int)d, c.dp, partial + 256 * i, scales + i,
                                    two ? nullptr : scales + 1, c.gemm ? 1 : 0,
                                    i == 0 ? select_state(ps, ws) : nullptr,
-                                   best_keys_of(ps, c, ws, ps.src[i], ps.rows[i]), st);
+                                   best_keys_of(ps, c, ws, ps.src[i], ps.rows[i]),
+                                   tiled_of(ps, c, ws, ps.src[i], ps.rows[i]), st);
   }
   return rc;
 }
@@ -544,7 +598,7 @@ int run_plan_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
       rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
-                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, nullptr, nullptr, st);
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 1, nullptr, nullptr, nullptr, st);
   }
   if (rc == FS_OK) rc = launch_plan_gemm(a, mat5, cb, total, st);
   if (rc != FS_OK) return rc;
@@ -682,7 +736,7 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
     if (rc == FS_OK) rc = launch_absmax(sd.q2, (long long)sd.nq * d, sd.q2, 0, partial, st);
     if (rc == FS_OK)
       rc = launch_split_planes_f16(sd.q2, reinterpret_cast<unsigned*>(base + q2_off), sd.nq, (int)d,
-                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, nullptr, nullptr, st);
+                                   cfg.dp, partial, partial + 2 * 256, nullptr, 0, nullptr, nullptr, nullptr, st);
   }
   for (int s = 0; s < nsides && rc == FS_OK && has_o; ++s) {
     const Side& sd = sides[s];
@@ -725,7 +779,8 @@ size_t pt_ws_bytes(int mode, int64_t n, int64_t m, int64_t d, bool both, bool ei
   const int dpk = std::max(padded_d(d), 16);
   LseConfig c;
   c.gemm = false; c.prec = 3; c.dp = dpk; c.np = 2;
-  const size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes;
+  const size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes +
+                        2 * margin_slot_bytes(std::max(n, m), c);  // the whole plane set
   auto side = [&](int64_t nq, int64_t nk) {
     size_t b = 0;
     for (int rb = 1; rb <= 2; ++rb)
@@ -782,10 +837,18 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const bool coarse = (flags & FS_FLAG_COARSE_TEST) && can_coarse;
   const bool auto_sel = (flags & FS_FLAG_COARSE_AUTO) && can_coarse && !coarse && prepared;
   Family fam_plan = fam;
+  // carried margins: prepared planes only (they are state)
+  bool margins = (coarse || auto_sel) && prepared;
+  int min_splits[2] = {1, 1};
   if (coarse || auto_sel) {  // that kernel works on two row blocks per wavefront and 128-key tiles
     rb = 2;
     fam_plan.jt = 128;
-    for (int s = 0; s < nsides; ++s) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam_plan, rb);
+    for (int s = 0; s < nsides; ++s) {
+      min_splits[s] = 2;  // the merge kernel carries the margins' state from launch to launch
+      if (sides[s].nk < 2 * 128) margins = false;
+    }
+    for (int s = 0; s < nsides; ++s)
+      plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam_plan, rb, margins ? min_splits[s] : 1);
   }
   PlaneSet ps;
   ps.n = 0;
@@ -798,8 +861,23 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const size_t need_planes_end = need;
   for (int s = 0; s < nsides; ++s) {
     // both sides run in one launch and must share the rows-per-wave template
-    if (!fam.sliced && plans[s].rb != rb) plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam_plan, rb);
+    if (!fam.sliced && plans[s].rb != rb)
+      plans[s] = plan_side(mode, sides[s].nq, sides[s].nk, fam_plan, rb, margins ? min_splits[s] : 1);
     need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
+  }
+  // The sparse form's wavefronts go through several chunks each (at most 2048 sub-tiles: its
+  // list of sub-tiles to visit), few enough that the whole launch is about four per slot of
+  // the chip.
+  int sparse_group[2] = {1, 1};
+  {
+    int64_t waves = 0;
+    for (int s = 0; s < nsides; ++s) {
+      waves += (int64_t)plans[s].igroups * 4;
+      if (plans[s].splits <= 1 || ps.margin_slot == 0 || plans[s].chunk > 65536) margins = false;
+    }
+    const int want = (int)std::max<int64_t>(1, ceil_div(4 * 2048, std::max<int64_t>(waves, 1)));
+    for (int s = 0; s < nsides; ++s)
+      sparse_group[s] = std::max(1, std::min(ceil_div(plans[s].splits, want), 65536 / std::max(plans[s].chunk, 1)));
   }
   // lse_coarse_kernel: per-tile records of the key bias, behind the partial rows
   const size_t aux_off = need;
@@ -822,6 +900,11 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     sd.best_key = nullptr;
     sd.part_best = nullptr;
     sd.key_aux = nullptr;
+    sd.margins = nullptr;
+    sd.sparse_group = 1;
+    sd.ktiled = sd.qtiled = nullptr;
+    sd.m_prev = nullptr;
+    sd.bias_prev = nullptr;
     sd.part_ms = nullptr;
     sd.part_o = nullptr;
     if (p.splits > 1) {
@@ -846,11 +929,35 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
         sd.best_key = best_keys_of(ps, cfg, ws, sd.q, sd.nq);
         sd.key_aux = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + aux_off + (s == 1 ? aux_bytes[0] : 0));
       }
+      if (margins) {
+        sd.margins = reinterpret_cast<float*>(static_cast<char*>(ws) + ps.margin_off + s * ps.margin_slot);
+        sd.margin_stride = ps.margin_stride;
+        sd.sparse_group = sparse_group[s];
+        sd.ktiled = tiled_of(ps, cfg, ws, sd.k, sd.nk);
+        sd.qtiled = tiled_of(ps, cfg, ws, sd.q, sd.nq);
+        sd.m_prev = row_array_of(ps, cfg, ws, sd.q, sd.nq, 1);
+        sd.bias_prev = row_array_of(ps, cfg, ws, sd.k, sd.nk, 2);
+        // what the margins depend on: the pairing of matrices, the scale of the dot products
+        // and the coefficients of the bias terms
+        auto bits = [](float v) { unsigned u; std::memcpy(&u, &v, 4); return u; };
+        unsigned t = 0x9e3779b9u * (unsigned)(1 + sd.ps_q + 2 * sd.ps_k);
+        for (unsigned w : {bits(sd.qscale), bits(sd.kc0), bits(sd.kc1), bits(sd.kc2),
+                           (unsigned)(sd.kb1 != nullptr) + 2u * (unsigned)(sd.kb2 != nullptr),
+                           (unsigned)sd.nq, (unsigned)sd.nk, (unsigned)p.chunk})
+          t = (t ^ w) * 0x85ebca6bu + 0xc2b2ae35u;
+        a.tag[s] = t | 1u;  // never 0, the cleared state
+      }
     }
     a.side[s] = sd;
   }
   if (nsides == 1) a.side[1] = a.side[0];
   a.blocks0 = blocks[0];
+  a.blocks0_sparse = a.blocks_sparse = 0;
+  for (int s = 0; s < nsides; ++s) {
+    const int b = ceil_div(plans[s].igroups * ceil_div(plans[s].splits, sparse_group[s]), 8) * 8;
+    if (s == 0) a.blocks0_sparse = b;
+    a.blocks_sparse += b;
+  }
   a.vec_ok = vec_ok ? 1 : 0;
   a.nss = fam.nss;
   const int total = blocks[0] + blocks[1];
@@ -997,13 +1104,20 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     size_t b = 0;  // the launch may settle on any rows-per-wave count: size for the largest
     for (int rb = 0; rb <= 3; ++rb)
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dp));
+    if (mode == kLse && !fam.sliced && dp <= 64) {  // the plans of lse_coarse_kernel
+      Family f2 = fam;
+      f2.jt = 128;
+      b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, f2, 2), nq, dp));
+      b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, f2, 2, 2), nq, dp));  // with carried margins
+    }
     return b * sizeof(float);
   };
   size_t planes = 0;  // two fp16 planes of x and y for the pipelined LSE kernel
   if (mode == kLse && !fam.sliced) {
     LseConfig c;
     c.gemm = false; c.prec = 3; c.dp = std::max(dp, 16); c.np = 2;
-    planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes;
+    planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes +
+             2 * margin_slot_bytes(std::max(n, m), c);
   }
   if (mode == kLse && !fam.sliced) planes += coarse_aux_bytes(n) + coarse_aux_bytes(m);
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
@@ -1030,7 +1144,7 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
   const int rc = make_plane_set(ptrs, rows, 2, cfg, ps);
   if (rc != FS_OK || ps.n == 0) return rc;
   if (ps.end > workspace_bytes || workspace == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
-  return launch_plane_set(ps, cfg, d, workspace, (hipStream_t)stream);
+  return launch_plane_set(ps, cfg, d, workspace, (hipStream_t)stream, true);
 }
 
 size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,

@@ -97,6 +97,22 @@ struct Side {
   // the layout the tile's LDS buffer takes (kAuxWords words per tile, kAuxPadTiles tiles past
   // the last key)
   unsigned* key_aux;
+  // lse_coarse_kernel, margins carried from launch to launch (all null: none).  margins: per
+  // wavefront (64 query rows) and 32-key sub-tile two entries (one per row block), `margin_stride`
+  // sub-tiles per wavefront: by how much the sub-tile's logits stayed below the point where they
+  // could matter when they were last tested, plus twice the sum of all key-bias changes up to
+  // then, tagged with a generation in the low 8 bits.  m_prev: per query row the merged maximum
+  // of the last launch (base-2 units).  bias_prev: per key the raw bias of the last launch.
+  // Second copy of the key and query planes in MFMA operand order, for kernels that take their
+  // operands straight from global memory: per 32 rows, plane and 16-column step one 1 KiB block
+  // with lane (h, row % 32)'s 16 bytes at 16 * (32 h + row % 32).
+  const unsigned* ktiled;
+  const unsigned* qtiled;
+  float* margins;
+  int margin_stride;
+  int sparse_group;     // key chunks one wavefront of the sparse form goes through
+  float* m_prev;
+  float* bias_prev;
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;
 };
@@ -117,6 +133,8 @@ struct LaunchArgs {
   unsigned* sel;
   unsigned sel_want;
   int sel_pred;  // 0: the launch runs whatever the state says (it still counts into it)
+  unsigned tag[2];  // per side: what the carried margins depend on (operands, scales, coefficients)
+  int blocks0_sparse, blocks_sparse;  // grid of the sparse form of lse_coarse_kernel: side 0, both sides
 };
 
 // Record of coarse_bias_kernel per 64 keys: eight fp16 copies of a_j per key (4 words each), then
@@ -130,7 +148,14 @@ constexpr int kAuxA = 0, kAuxB = 256, kAuxMax = 320, kAuxWords = 384, kAuxPadTil
 // running totals, and per-launch counters spread over kSelSlots slots (slot = workgroup % slots).
 constexpr int kSelWord = 0, kSelDecisions = 1, kSelCumEnded = 2, kSelCumUnits = 4;  // totals: u64
 constexpr int kSelSlots = 64, kSelEnded = 8, kSelUnits = kSelEnded + kSelSlots;
-constexpr int kSelWords = kSelUnits + kSelSlots;
+// carried margins, per side s: running sum of the key-bias changes (float), this launch's largest
+// change (float bits, by atomic max), the tag the margins were taken under, their generation
+// (1..255; 0 never valid), and whether this launch started a generation
+constexpr int kSelCum = kSelUnits + kSelSlots, kSelDmax = kSelCum + 2, kSelTag = kSelDmax + 2;
+constexpr int kSelGen = kSelTag + 2, kSelBump = kSelGen + 2;
+constexpr int kSelMode = kSelBump + 2;  // per side: the last launch ran in the sparse form
+constexpr int kSelWords = kSelMode + 2;
+constexpr int kMarginGroups = 4;  // a key chunk holds at most 64 * kMarginGroups / 2 sub-tiles
 constexpr unsigned kSelDecideSteps = 3;  // which counted launch of the coarse variant decides
 constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
 
@@ -138,6 +163,29 @@ constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units en
 // rows all started from a key of the previous launch count, and the share of ended units climbs
 // over the first launches that have such keys: the kSelDecideSteps-th launch with counts decides,
 // and leaves the coarse variant when too few of its units ended at the test.
+// After a launch that used carried margins: this launch's bias change joins the running sum.
+// Which form of lse_coarse_kernel runs for a side: the sparse one once the side's largest bias
+// change since its last launch is below 32 base-2 units (margins then outlast many launches),
+// and on until it is above 128 again; the pipelined one before, and when a generation starts.
+// lscale: base-2 units per raw unit.
+__device__ __forceinline__ bool margins_settled(const unsigned* st, int side, float lscale) {
+  if (st[kSelBump + side] != 0u || st[kSelGen + side] > 255u) return false;
+  const float d = __builtin_bit_cast(float, st[kSelDmax + side]) * lscale;
+  return d < (st[kSelMode + side] != 0u ? 128.0f : 32.0f);  // false when d is not a number
+}
+
+__device__ __forceinline__ void margins_commit(unsigned* st, int lane, bool settled) {
+  if (lane < 2) {
+    st[kSelMode + lane] = settled ? 1u : 0u;
+    const float cum = st[kSelBump + lane] ? 0.f
+                                          : __builtin_bit_cast(float, st[kSelCum + lane]) +
+                                                __builtin_bit_cast(float, st[kSelDmax + lane]);
+    st[kSelCum + lane] = __builtin_bit_cast(unsigned, cum);
+    st[kSelDmax + lane] = 0u;
+    st[kSelBump + lane] = 0u;
+  }
+}
+
 __device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
   unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane];
   st[kSelEnded + lane] = 0u;

@@ -14,11 +14,14 @@ int launch_sliced(int mode, const LaunchArgs& a, int nw, int nsl, int blocks, hi
 // split per matrix, which also writes the matrix's power-of-two scale to *scale_out and clears
 // the variant-choice state at clear_state (kSelWords words; may be null) and resets best_keys
 // (one int per row; may be null) to -1.
+// n 32-bit words at p (16-byte aligned) set to zero by a kernel (graph-capture safe).
+int launch_fill_zero(unsigned* p, long long n, hipStream_t st);
 int launch_absmax(const float* a, long long na, const float* b, long long nb, float* partial,
                   hipStream_t st);
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
-                            int chunked, unsigned* clear_state, int* best_keys, hipStream_t st);
+                            int chunked, unsigned* clear_state, int* best_keys, unsigned* tiled,
+                            hipStream_t st);
 // GEMM-style LSE kernel for 128 < d <= 1536 on chunked fp16 planes; Side::splits counts
 // partial rows (twice the workgroup-level key splits).
 int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st);  // kLse, kVec, kArgmax

@@ -38,13 +38,21 @@ int launch_absmax(const float* a, long long na, const float* b, long long nb, fl
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
+int launch_fill_zero(unsigned* p, long long n, hipStream_t st) {
+  if (n <= 0) return FS_OK;
+  const long long grid = (n / 4 + 256) / 256;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)grid), dim3(256), 0, st, p, n);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
-                            int chunked, unsigned* clear_state, int* best_keys, hipStream_t st) {
+                            int chunked, unsigned* clear_state, int* best_keys, unsigned* tiled,
+                            hipStream_t st) {
   const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
   const int grid = (int)((items + 255) / 256);
   hipLaunchKernelGGL(split_planes_f16_kernel, dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp,
-                     partial_max, scale_out, scale_out2, chunked, clear_state, best_keys);
+                     partial_max, scale_out, scale_out2, chunked, clear_state, best_keys, tiled);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
@@ -52,7 +60,10 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
 // tile test (two blocks of 32 query rows per wavefront: the launch must be planned with rb = 2)
 template <int DP>
 static int launch_coarse_dp(const LaunchArgs& a, int blocks, hipStream_t st) {
-  hipLaunchKernelGGL((lse_coarse_kernel<DP>), dim3(blocks), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((lse_coarse_kernel<DP, false>), dim3(blocks), dim3(256), 0, st, a);
+  // with carried margins both forms are enqueued; per side, the one the state words name runs
+  if (a.side[0].margins != nullptr)
+    hipLaunchKernelGGL((lse_coarse_kernel<DP, true>), dim3(a.blocks_sparse), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

@@ -93,13 +93,24 @@ __global__ __launch_bounds__(256) void absmax_kernel(const float* __restrict__ a
 // padded to DP columns and in the trailing rows.  scale is derived from the partial maxima of
 // absmax_kernel; block 0 also publishes it in *scale_out for the consuming kernel and clears
 // the kSelWords words at `clear_state` (the variant-choice state that belongs to the planes);
-// `best_keys` (one int per row, may be null) is reset to -1.
+// `best_keys` (may be null) starts three arrays of one value per row, (rows + 3) & ~3 values apart:
+// the keys (reset to -1), the rows' last maxima (3e38) and the rows' last biases as keys (0).
 // With `chunked` the two planes are interleaved per 32 columns (layout of lse_gemm_kernel).
+// `tiled` (may be null; not with `chunked`): a second copy in MFMA operand order, see Side::ktiled.
+__global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* __restrict__ p, long long n) {
+  const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i + 3 < n) {
+    *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
+  } else {
+    for (long long k = i; k < n; ++k) p[k] = 0u;
+  }
+}
+
 __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     const float* __restrict__ src, unsigned* __restrict__ dst, int rows, int d, int dp,
     const float* __restrict__ partial_max, float* __restrict__ scale_out,
     float* __restrict__ scale_out2, int chunked, unsigned* __restrict__ clear_state,
-    int* __restrict__ best_keys) {
+    int* __restrict__ best_keys, unsigned* __restrict__ tiled) {
   __shared__ float red[4];
   float m = partial_max[threadIdx.x];  // kAbsmaxBlocks == blockDim.x
 #pragma unroll
@@ -115,7 +126,12 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
 
   const int per_row = dp / 4;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (best_keys != nullptr && idx < rows) best_keys[idx] = -1;  // new planes: no key known yet
+  if (best_keys != nullptr && idx < rows) {  // new planes: the three per-row arrays behind them
+    const int stride = (rows + 3) & ~3;
+    best_keys[idx] = -1;                                                  // no key known yet
+    reinterpret_cast<float*>(best_keys)[stride + idx] = 3.0e38f;          // no maximum known yet
+    reinterpret_cast<float*>(best_keys)[2 * stride + idx] = 0.f;          // no bias seen yet
+  }
   if (idx >= (long long)(rows + kPlanePadRows) * per_row) return;
   const int r = (int)(idx / per_row);
   const int c4 = (int)(idx % per_row) * 4;
@@ -136,6 +152,14 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
   } else {
     *reinterpret_cast<uint2*>(o + c4 / 2) = make_uint2(h01, h23);
     *reinterpret_cast<uint2*>(o + dp / 2 + c4 / 2) = make_uint2(l01, l23);
+    if (tiled != nullptr) {
+      // the same words in MFMA operand order: per 32 rows [plane][16-column step][half h][row % 32]
+      // 16 bytes; word w of a plane row belongs to step w / 8, half (w / 4) % 2
+      const int w = c4 / 2, kk16 = dp / 16;
+      unsigned* t = tiled + ((size_t)(r / 32) * 2 * kk16 + w / 8) * 256 + (((w >> 2) & 1) * 32 + r % 32) * 4 + (w & 3);
+      *reinterpret_cast<uint2*>(t) = make_uint2(h01, h23);
+      *reinterpret_cast<uint2*>(t + (size_t)kk16 * 256) = make_uint2(l01, l23);
+    }
   }
 }
 

@@ -469,7 +469,14 @@ template <bool HAS_O>
 __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int dp, int items0,
                                                      int items1) {
   if constexpr (!HAS_O) {  // the launch that follows both variants of a device-chosen step
-    if (args.sel != nullptr && blockIdx.x == 0 && threadIdx.x < 64) coarse_decide(args.sel, threadIdx.x);
+    if (args.sel != nullptr && blockIdx.x == 0 && threadIdx.x < 64) {
+      coarse_decide(args.sel, threadIdx.x);
+      if (args.side[0].margins != nullptr) {
+        const Side& ms = args.side[threadIdx.x & 1];
+        const float lscale = ms.qscale / (ms.plane_scale[ms.ps_q] * ms.plane_scale[ms.ps_k]);
+        margins_commit(args.sel, threadIdx.x, margins_settled(args.sel, threadIdx.x & 1, lscale));
+      }
+    }
   }
   int it = blockIdx.x * 256 + threadIdx.x;
   if (it >= items0 + items1) return;  // the other side may have nothing to merge
@@ -514,6 +521,7 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
       }
       if (bj >= 0) sd.best_key[row] = bj;  // no chunk exceeded the starting value: the old key stays
     }
+    if (sd.m_prev != nullptr) sd.m_prev[row] = M;
     epilogue_scalar(sd.ep, row, M, s, o);
   }
 }
