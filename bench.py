@@ -274,8 +274,9 @@ def main():
         prep = _lib.PreparedOperands(ops[0], ops[1], _lib.flags(True, False))
         kw = dict(cost_scale=1.0, allow_tf32=False, prepared=prep, coarse=coarse)
         steps = [(EPS, 0.5, 1.0, 1.0)] * reps
-        # the launches that take the decision, and in which the rows' starting keys settle
-        _symmetric_steps_raw(*ops, steps[:8], **kw)
+        # the launches that take the decision, in which the rows' starting keys settle and after
+        # which the kernel with the coarse tile test runs in its sparse form
+        _symmetric_steps_raw(*ops, steps[:16], **kw)
         torch.cuda.synchronize()
         before = prep.variant_state()
         stream = torch.cuda.current_stream(dev)
@@ -285,7 +286,8 @@ def main():
         e1.record(stream)
         torch.cuda.synchronize()
         after = prep.variant_state()
-        counts = {k: (after[k] - before[k]) / reps for k in ("tiles_ended", "tiles_tested")}
+        counts = {k: (after[k] - before[k]) / reps
+                  for k in ("tiles_ended", "tiles_tested", "tiles_skipped")}
         counts["plain_selected"] = after["plain_selected"]
         return e0.elapsed_time(e1) / reps, counts
 
@@ -308,22 +310,28 @@ def main():
                      peak_note="published dense fp32 MFMA peak; executed = algorithmic flop")
         else:
             # three plane products per tile in the plain kernel.  The variant with the coarse tile
-            # test runs, for every tile, the hi*hi product plus one more 16-column MFMA step that
-            # carries the bias bound, and the two cross products only for tiles that go on.
+            # test runs, for every tile it visits, the hi*hi product plus one more 16-column MFMA
+            # step that carries the bias bound, and the two cross products only for tiles that go
+            # on; its sparse form does not visit tiles whose carried margin still holds.
             products = 3.0 * tiles_all
             if counts is not None and counts["tiles_tested"] > 0 and not counts["plain_selected"]:
                 went_on = 1.0 - counts["tiles_ended"] / counts["tiles_tested"]
-                products = tiles_all * (1.0 + 16.0 / dp + 2.0 * went_on)
+                visited = 1.0 - counts["tiles_skipped"] / counts["tiles_tested"]
+                products = tiles_all * (visited * (1.0 + 16.0 / dp) + 2.0 * went_on)
                 r["coarse_test"] = {
-                    "share_of_tested_tiles_ended": 1.0 - went_on,
+                    "share_of_tiles_not_visited": 1.0 - visited,
+                    "share_of_tiles_ended_at_the_test": visited - went_on,
+                    "share_of_tiles_in_full": went_on,
                     "mfma_products_per_tile": products / tiles_all}
+                if visited < 0.5:
+                    r["kernel"] = r["kernel"].replace("lse_coarse_kernel", "lse_coarse_kernel, sparse form")
             executed = products * flop_per_tile_product
             r.update(achieved=executed / (ms * 1e-3) / 1e12, peak=F16_MFMA_PEAK_TFLOPS,
                      executed_flop_per_launch=executed,
                      peak_note="published dense fp16 MFMA peak; achieved counts the 16-bit MFMA "
                                "flop the launch executed (three plane products per algorithmic "
-                               "product, one for tiles that end at the coarse test, padding of "
-                               "d to the MFMA width included)")
+                               "product, one for tiles that end at the coarse test, none for "
+                               "tiles not visited, padding of d to the MFMA width included)")
         r["frac"] = r["achieved"] / r["peak"]
         r["traffic"] = MEASURED_TRAFFIC_BYTES.get(mode) if (n, m, d) == (N, M, D) else None
         return r

@@ -176,11 +176,13 @@ class PreparedOperands:
         diagnostic, not part of any solve): which variant the steps now run, and how many
         32 x 32 logits tiles of the coarse variant ended at its test."""
         if self.state_offset == 0:
-            return {"plain_selected": True, "decisions": 0, "tiles_ended": 0, "tiles_tested": 0}
-        w = self.ws[self.state_offset:self.state_offset + 24].cpu().view(torch.int32).tolist()
+            return {"plain_selected": True, "decisions": 0, "tiles_ended": 0, "tiles_tested": 0,
+                    "tiles_skipped": 0}
+        w = self.ws[self.state_offset:self.state_offset + 32].cpu().view(torch.int32).tolist()
         u = [v & 0xFFFFFFFF for v in w]
         return {"plain_selected": u[0] != 0, "decisions": u[1],
-                "tiles_ended": u[2] | (u[3] << 32), "tiles_tested": u[4] | (u[5] << 32)}
+                "tiles_ended": u[2] | (u[3] << 32), "tiles_tested": u[4] | (u[5] << 32),
+                "tiles_skipped": u[6] | (u[7] << 32)}
 
     def serves(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int) -> bool:
         # the workspace layout depends on the set of matrices, so the call must name the same set

@@ -930,7 +930,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
         sd.key_aux = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + aux_off + (s == 1 ? aux_bytes[0] : 0));
       }
       if (margins) {
-        sd.margins = reinterpret_cast<float*>(static_cast<char*>(ws) + ps.margin_off + s * ps.margin_slot);
+        // (slot and state words go with the matrix that holds the query rows)
+        sd.margins = reinterpret_cast<float*>(static_cast<char*>(ws) + ps.margin_off + sd.ps_q * ps.margin_slot);
         sd.margin_stride = ps.margin_stride;
         sd.sparse_group = sparse_group[s];
         sd.ktiled = tiled_of(ps, cfg, ws, sd.k, sd.nk);

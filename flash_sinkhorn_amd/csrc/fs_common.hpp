@@ -148,13 +148,17 @@ constexpr int kAuxA = 0, kAuxB = 256, kAuxMax = 320, kAuxWords = 384, kAuxPadTil
 // running totals, and per-launch counters spread over kSelSlots slots (slot = workgroup % slots).
 constexpr int kSelWord = 0, kSelDecisions = 1, kSelCumEnded = 2, kSelCumUnits = 4;  // totals: u64
 constexpr int kSelSlots = 64, kSelEnded = 8, kSelUnits = kSelEnded + kSelSlots;
-// carried margins, per side s: running sum of the key-bias changes (float), this launch's largest
+// carried margins, per matrix of the plane set in the role of the query rows (Side::ps_q):
+// running sum of the key-bias changes (float), this launch's largest
 // change (float bits, by atomic max), the tag the margins were taken under, their generation
 // (1..255; 0 never valid), and whether this launch started a generation
 constexpr int kSelCum = kSelUnits + kSelSlots, kSelDmax = kSelCum + 2, kSelTag = kSelDmax + 2;
 constexpr int kSelGen = kSelTag + 2, kSelBump = kSelGen + 2;
-constexpr int kSelMode = kSelBump + 2;  // per side: the last launch ran in the sparse form
-constexpr int kSelWords = kSelMode + 2;
+constexpr int kSelMode = kSelBump + 2;  // likewise: the last launch ran in the sparse form
+constexpr int kSelSkip = kSelMode + 2;  // per-launch slots: units the sparse form did not visit
+constexpr int kSelCumSkipped = 6;       // their running total (u64), part of kSelCumEnded's
+constexpr int kSelWords = kSelSkip + kSelSlots;
+static_assert(kSelWords <= 256, "one workgroup clears the state block");
 constexpr int kMarginGroups = 4;  // a key chunk holds at most 64 * kMarginGroups / 2 sub-tiles
 constexpr unsigned kSelDecideSteps = 3;  // which counted launch of the coarse variant decides
 constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
@@ -175,7 +179,7 @@ __device__ __forceinline__ bool margins_settled(const unsigned* st, int side, fl
 }
 
 __device__ __forceinline__ void margins_commit(unsigned* st, int lane, bool settled) {
-  if (lane < 2) {
+  {
     st[kSelMode + lane] = settled ? 1u : 0u;
     const float cum = st[kSelBump + lane] ? 0.f
                                           : __builtin_bit_cast(float, st[kSelCum + lane]) +
@@ -187,19 +191,22 @@ __device__ __forceinline__ void margins_commit(unsigned* st, int lane, bool sett
 }
 
 __device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
-  unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane];
+  unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane], k = st[kSelSkip + lane];
   st[kSelEnded + lane] = 0u;
   st[kSelUnits + lane] = 0u;
-  unsigned long long es = e, us = u;
+  st[kSelSkip + lane] = 0u;
+  unsigned long long es = e, us = u, ks = k;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     es += __shfl_xor(es, o, 64);
     us += __shfl_xor(us, o, 64);
+    ks += __shfl_xor(ks, o, 64);
   }
   if (lane == 0 && us > 0) {
     unsigned long long* cum = reinterpret_cast<unsigned long long*>(st + kSelCumEnded);
     cum[0] += es;
     cum[1] += us;
+    cum[2] += ks;
     const unsigned seen = st[kSelDecisions];
     if (seen < kSelDecideSteps) {  // the share of the last of these launches decides
       st[kSelDecisions] = seen + 1u;

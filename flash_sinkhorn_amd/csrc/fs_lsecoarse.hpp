@@ -100,7 +100,7 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
   // (raw units), and the generation of the margins: a launch whose tag differs from the one the
   // margins were taken under (other operands, eps, coefficients) starts a new one.
   if (sd.bias_prev != nullptr && args.sel != nullptr) {
-    const int side = second ? 1 : 0;
+    const int side = sd.ps_q;  // the margins' state goes with the matrix that holds the query rows
     float dch = 0.f;
     if (j < sd.nk) {
       dch = fabsf(b - sd.bias_prev[j]);
@@ -111,8 +111,8 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
     for (int o = 32; o > 0; o >>= 1) dch = fmaxf(dch, __shfl_xor(dch, o, 64));
     if (lane == 0) {
       atomicMax(&args.sel[kSelDmax + side], __builtin_bit_cast(unsigned, dch));
-      if (tile == 0 && args.sel[kSelTag + side] != args.tag[side]) {
-        args.sel[kSelTag + side] = args.tag[side];
+      if (tile == 0 && args.sel[kSelTag + side] != args.tag[second ? 1 : 0]) {
+        args.sel[kSelTag + side] = args.tag[second ? 1 : 0];
         // entries carry the generation in 8 bits and are cleared only with the planes: after 255
         // generations the margins of this side stay off (256 matches no entry)
         args.sel[kSelGen + side] = min(args.sel[kSelGen + side] + 1u, 256u);
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // one runs for a side.
   if (sd.margins != nullptr) {
     const bool settled = margins_settled(
-        args.sel, second ? 1 : 0, sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]));
+        args.sel, sd.ps_q, sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]));
     if (settled != SPARSE) return;
   }
 
@@ -674,7 +674,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     // twice the running sum.  That needs every row of the wavefront to start where its last
     // maximum says (checked against the maximum the merge kernel kept); a wavefront where it does
     // not hold visits everything and only writes entries.
-    const int side_i = second ? 1 : 0;
+    const int side_i = sd.ps_q;
     const unsigned* st = args.sel;
     const unsigned gen = st[kSelGen + side_i];
     const float dnow = __builtin_bit_cast(float, st[kSelDmax + side_i]);
@@ -881,6 +881,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   if (args.sel != nullptr && lane == 0 && ntiles > 0 && !(track && cold)) {
     const int slot = blockIdx.x % kSelSlots;
         atomicAdd(&args.sel[kSelEnded + slot], n_ended + n_skipped);
+    if (SPARSE) atomicAdd(&args.sel[kSelSkip + slot], n_skipped);
     atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
   }
 

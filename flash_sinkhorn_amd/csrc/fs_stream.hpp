@@ -471,10 +471,11 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
   if constexpr (!HAS_O) {  // the launch that follows both variants of a device-chosen step
     if (args.sel != nullptr && blockIdx.x == 0 && threadIdx.x < 64) {
       coarse_decide(args.sel, threadIdx.x);
-      if (args.side[0].margins != nullptr) {
-        const Side& ms = args.side[threadIdx.x & 1];
+      // lanes 0 and 1: the sides of this launch (the second one only when it has rows to merge)
+      if (args.side[0].margins != nullptr && (threadIdx.x == 0 || (threadIdx.x == 1 && items1 > 0))) {
+        const Side& ms = args.side[threadIdx.x];
         const float lscale = ms.qscale / (ms.plane_scale[ms.ps_q] * ms.plane_scale[ms.ps_k]);
-        margins_commit(args.sel, threadIdx.x, margins_settled(args.sel, threadIdx.x & 1, lscale));
+        margins_commit(args.sel, ms.ps_q, margins_settled(args.sel, ms.ps_q, lscale));
       }
     }
   }

@@ -113,11 +113,12 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
 
 /*
  * Byte offset, inside a workspace that fs_prepare_operands(x, y, ...) has filled, of the state
- * FS_FLAG_COARSE_AUTO keeps (0 when the configuration has none).  Six 32-bit words a caller
+ * FS_FLAG_COARSE_AUTO keeps (0 when the configuration has none).  Eight 32-bit words a caller
  * may read for diagnostics once the stream has drained: [0] the variant the steps run now
  * (0: coarse tile test, 1: plain), [1] decisions taken so far, [2..3] a 64-bit count of the
- * 32 x 32 logits tiles that ended at the coarse test, [4..5] of the tiles it tested.  Host
- * arithmetic only.  No counterpart in the reference.
+ * 32 x 32 logits tiles that ended at the coarse test or were not visited at all, [4..5] of all
+ * tiles of those launches, [6..7] of the tiles not visited (carried margins, part of [2..3]).
+ * Host arithmetic only.  No counterpart in the reference.
  */
 size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
                                uint32_t flags);

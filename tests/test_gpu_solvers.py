@@ -674,6 +674,110 @@ def test_coarse_test_starts_rows_from_the_keys_of_the_last_step(n, m, d, eps):
     check(fh2, gh2, F2, G2)
 
 
+@pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2500, 2300, 20, 0.05), (1200, 9000, 33, 0.02)])
+def test_carried_margins_leave_every_step_unchanged(n, m, d, eps):
+    """On prepared planes the kernel with the coarse tile test carries margins from launch to
+    launch and, once the potentials move little, runs in a sparse form that visits only the
+    tiles whose margin may have been used up.  Every step of a long sequence must equal the plain
+    launch on the same inputs, and the oracle: while the potentials settle, when they are then
+    disturbed a little (the sparse form stays, with many margins used up), a lot (back to the
+    pipelined form), when the kept keys are overwritten with arbitrary numbers, and when eps
+    changes (margins of another problem must not be used)."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    rng = np.random.default_rng(41)
+    x, _ = _clustered(rng, n, d)
+    y, _ = _clustered(rng, m, d)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = (rng.random(m) + 0.5).astype(np.float32)
+    b /= b.sum()
+    la, lb = np.log(a), np.log(b)
+    fh = (-(x * x).sum(1)).astype(np.float32)
+    gh = (-(y * y).sum(1)).astype(np.float32)
+    X, Y, F, G, LA, LB = dev(x, y, fh, gh, la, lb)
+    prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    worst = [0.0]
+
+    def step(F_in, G_in, e, with_oracle=False):
+        f1, g1 = _symmetric_step_raw(X, Y, F_in, G_in, LA, LB, e, coarse=True, prepared=prep, **kw)
+        f0, g0 = _symmetric_step_raw(X, Y, F_in, G_in, LA, LB, e, coarse=False, **kw)
+        err = max(rel_err(f1, f0.cpu().numpy()), rel_err(g1, g0.cpu().numpy()))
+        worst[0] = max(worst[0], err)
+        assert err < 2e-6, err
+        if with_oracle:
+            wf, wg = oracle.symmetric_step(x, y, F_in.cpu().numpy(), G_in.cpu().numpy(), la, lb, e,
+                                           1.0, 0.5, 1.0, 1.0)
+            assert rel_err(f1, wf) < RTOL and rel_err(g1, wg) < RTOL
+        return f1, g1
+
+    def skipped():
+        return prep.variant_state()["tiles_skipped"]
+
+    for it in range(30):  # settles: the sparse form takes over
+        F, G = step(F, G, eps, with_oracle=it in (0, 29))
+    s0, t0 = skipped(), prep.variant_state()["tiles_tested"]
+    assert s0 > 0
+    F, G = step(F, G, eps)
+    st = prep.variant_state()
+    assert st["tiles_skipped"] > s0  # a settled step skips tiles
+    # a disturbance of about 60 base-2 units: many margins are used up, the sparse form stays
+    amp = 60.0 * eps * np.log(2.0)
+    G2 = G + torch.from_numpy((amp * (2 * rng.random(m) - 1)).astype(np.float32)).cuda()
+    F2 = F + torch.from_numpy((amp * (2 * rng.random(n) - 1)).astype(np.float32)).cuda()
+    F, G = step(F2, G2, eps, with_oracle=True)
+    for it in range(4):
+        F, G = step(F, G, eps)
+    # a large one: back to the pipelined form, then settling again
+    G2 = G + torch.from_numpy((3.0 * rng.standard_normal(m)).astype(np.float32)).cuda()
+    F2 = F + torch.from_numpy((3.0 * rng.standard_normal(n)).astype(np.float32)).cuda()
+    F, G = step(F2, G2, eps, with_oracle=True)
+    for it in range(12):
+        F, G = step(F, G, eps)
+    s1 = skipped()
+    F, G = step(F, G, eps)
+    assert skipped() > s1  # sparse again
+    # arbitrary numbers in the key arrays: rows no longer start where their last maximum says
+    prep.best_keys(0).copy_(torch.from_numpy(rng.integers(-5, m + 5, n).astype(np.int32)))
+    prep.best_keys(1).copy_(torch.from_numpy(rng.integers(-2**31, 2**31 - 1, m).astype(np.int32)))
+    F, G = step(F, G, eps, with_oracle=True)
+    F, G = step(F, G, eps)
+    # another eps on the same planes, and back
+    for e in (2.0 * eps, 2.0 * eps, eps, eps, eps):
+        F, G = step(F, G, e, with_oracle=(e != eps))
+    print("largest difference to the plain launch", worst[0])
+
+
+def test_carried_margins_with_one_sided_launches():
+    """The alternating solver's half-updates are one-sided launches on shared prepared planes: the
+    margins' state goes with the matrix that holds the query rows, so both directions settle into
+    the sparse form, and every half-update equals the plain launch."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import flashsinkhorn_lse_fused
+    rng = np.random.default_rng(42)
+    n, m, d, eps = 2600, 3100, 48, 0.02
+    x, _ = _clustered(rng, n, d)
+    y, _ = _clustered(rng, m, d)
+    la = np.log(np.full(n, 1.0 / n, np.float32))
+    lb = np.log(np.full(m, 1.0 / m, np.float32))
+    X, Y, LA, LB = dev(x, y, la, lb)
+    F = -(X * X).sum(1)
+    G = -(Y * Y).sum(1)
+    prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+    for it in range(40):
+        for q, k, lw, out in ((X, Y, LB, "f"), (Y, X, LA, "g")):
+            pot = G if out == "f" else F
+            got = flashsinkhorn_lse_fused(q, k, pot, lw, eps, allow_tf32=False, _prepared=prep, _coarse=True)
+            want = flashsinkhorn_lse_fused(q, k, pot, lw, eps, allow_tf32=False)
+            assert rel_err(got, want.cpu().numpy()) < 2e-6
+            if out == "f":
+                F = 0.5 * (F + got)  # damped, so that the sequence settles
+            else:
+                G = 0.5 * (G + got)
+    st = prep.variant_state()
+    assert st["tiles_skipped"] > 0
+
+
 @pytest.mark.parametrize("variant", [True, None])
 def test_solver_with_the_coarse_tile_test_equals_the_plain_solve(monkeypatch, variant):
     """Fixed-eps solves on large clouds run the kernel variant with the coarse tile test, forced
