@@ -3,6 +3,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -211,9 +212,10 @@ size_t planes_only_bytes(int64_t rows, const LseConfig& c) {
   return (((size_t)(rows + kPlanePadRowsApi) * (size_t)c.np * (size_t)(c.dp / 2) * 4) + 15) & ~(size_t)15;
 }
 
-// One 4-byte value per row, 16-byte aligned; a matrix keeps three such arrays behind its planes:
+// One 4-byte value per row, 16-byte aligned; a matrix keeps four such arrays behind its planes:
 // the key behind each row's largest logit, that logit (the merged maximum of the last launch
-// with the matrix as the stationary one), and the row's bias of the last launch as a key.
+// with the matrix as the stationary one), the row's bias of the last launch as a key, and where
+// the row's running maximum starts in the launch under way.
 size_t row_array_bytes(int64_t rows) { return ((size_t)rows * 4 + 15) & ~(size_t)15; }
 
 // Second copy of two-plane rows of at most 64 columns in MFMA operand order (Side::ktiled),
@@ -224,7 +226,7 @@ size_t tiled_bytes(int64_t rows, const LseConfig& c) {
 }
 
 size_t plane_bytes(int64_t rows, const LseConfig& c) {
-  return planes_only_bytes(rows, c) + 3 * row_array_bytes(rows) + tiled_bytes(rows, c);
+  return planes_only_bytes(rows, c) + 4 * row_array_bytes(rows) + tiled_bytes(rows, c);
 }
 
 // Carried margins of lse_coarse_kernel: per wavefront (64 rows) and 32-key sub-tile two entries.
@@ -303,7 +305,7 @@ int* best_keys_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float*
 }
 
 float* row_array_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float* src, int rows,
-                    int which) {  // 1: last maxima, 2: last biases
+                    int which) {  // 1: last maxima, 2: last biases, 3: this launch's starting values
   int* keys = best_keys_of(ps, c, ws, src, rows);
   if (keys == nullptr) return nullptr;
   return reinterpret_cast<float*>(reinterpret_cast<char*>(keys) + which * row_array_bytes(rows));
@@ -313,7 +315,7 @@ unsigned* tiled_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float
   if (tiled_bytes(rows, c) == 0) return nullptr;
   int* keys = best_keys_of(ps, c, ws, src, rows);
   if (keys == nullptr) return nullptr;
-  return reinterpret_cast<unsigned*>(reinterpret_cast<char*>(keys) + 3 * row_array_bytes(rows));
+  return reinterpret_cast<unsigned*>(reinterpret_cast<char*>(keys) + 4 * row_array_bytes(rows));
 }
 
 // Writes the planes (and, for fp16, the scales) of every matrix of the set.
@@ -901,6 +903,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     sd.part_best = nullptr;
     sd.key_aux = nullptr;
     sd.margins = nullptr;
+    sd.seed = nullptr;
     sd.sparse_group = 1;
     sd.ktiled = sd.qtiled = nullptr;
     sd.m_prev = nullptr;
@@ -927,6 +930,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       sd.ps_k = plane_index(ps, sd.k, sd.nk);
       if (coarse || auto_sel) {
         sd.best_key = best_keys_of(ps, cfg, ws, sd.q, sd.nq);
+        sd.seed = row_array_of(ps, cfg, ws, sd.q, sd.nq, 3);
         sd.key_aux = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + aux_off + (s == 1 ? aux_bytes[0] : 0));
       }
       if (margins) {

@@ -113,6 +113,7 @@ struct Side {
   int sparse_group;     // key chunks one wavefront of the sparse form goes through
   float* m_prev;
   float* bias_prev;
+  float* seed;          // per query row: where this launch's running maximum starts (raw units)
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;
 };

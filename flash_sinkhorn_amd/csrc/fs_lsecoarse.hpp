@@ -61,10 +61,77 @@ namespace fs {
 // units: a_j as eight fp16 copies, b_j - 2^18 a_j, and the largest bias of each 32-key
 // sub-tile.  Keys past the end of the key set get a bias that masks them.  T only makes this a
 // template (header-defined kernel).
+//
+// The blocks behind the tiles (64 query rows each, side 0 first: seed_blocks0 of them) compute
+// where the rows' running maxima start.  A row whose largest logit of the last launch sat at key
+// j starts from its current logit at j, computed on the vector pipe from the same planes:
+// whatever the potentials did since, this is a logit of the row, hence a lower bound of its new
+// maximum, and close to it once the potentials settle.  (Any index inside the key set keeps the
+// result exact; a stale one only costs tests that pass.)  The sum of the fp32 roundings of the
+// two routes to a logit is far below 1/64 of the row's bound on its cross products, which is taken
+// off together with one base-2 unit.  A row without a key gets -3e38.
 template <int T>
-__global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, int tiles0) {
+__global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, int tiles0, int tiles_all,
+                                                         int seed_blocks0, int dp) {
   // variant chosen on the device: nothing reads the records when the plain kernel runs
   if (args.sel_pred && args.sel[kSelWord] != 0u) return;
+  if ((int)blockIdx.x >= tiles_all) {
+    int blk = blockIdx.x - tiles_all;
+    const bool second_s = blk >= seed_blocks0;
+    if (second_s) blk -= seed_blocks0;
+    const Side& ss = second_s ? args.side[1] : args.side[0];
+    if (ss.seed == nullptr) return;
+    // eight lanes per row, 16 bytes of each plane per lane (whole cache lines per row), eight rows
+    // per pass
+    const int lane = threadIdx.x, piece = lane & 7, sub = lane >> 3;
+    const float inv_ls = ss.plane_scale[ss.ps_q] * ss.plane_scale[ss.ps_k] / ss.qscale;
+    const bool has_piece = piece * 4 < dp / 2;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+      const int row = blk * 64 + pass * 8 + sub;
+      const int rc = min(row, ss.nq - 1);
+      const int j = ss.best_key[rc];
+      const int jc = min(max(j, 0), ss.nk - 1);
+      float dot = 0.f, l1 = 0.f;
+      if (has_piece) {
+        const unsigned* q = ss.qplanes + (size_t)rc * (size_t)dp + piece * 4;
+        const unsigned* k = ss.kplanes + (size_t)jc * (size_t)dp + piece * 4;
+        const u32x4 qh4 = *reinterpret_cast<const u32x4*>(q);
+        const u32x4 ql4 = *reinterpret_cast<const u32x4*>(q + dp / 2);
+        const u32x4 kh4 = *reinterpret_cast<const u32x4*>(k);
+        const u32x4 kl4 = *reinterpret_cast<const u32x4*>(k + dp / 2);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // (words copied out first: a bit cast applied to a vector element reads element 0)
+          const unsigned qhw = qh4[e], qlw = ql4[e], khw = kh4[e], klw = kl4[e];
+          const f16x2 qh = __builtin_bit_cast(f16x2, qhw), ql = __builtin_bit_cast(f16x2, qlw);
+          const f16x2 kh = __builtin_bit_cast(f16x2, khw), kl = __builtin_bit_cast(f16x2, klw);
+          dot = __builtin_amdgcn_fdot2(kh, qh, dot, false);
+          dot = __builtin_amdgcn_fdot2(kh, ql, dot, false);
+          dot = __builtin_amdgcn_fdot2(kl, qh, dot, false);
+          l1 += fabsf((float)qh[0]) + fabsf((float)qh[1]);
+        }
+      }
+#pragma unroll
+      for (int o = 4; o > 0; o >>= 1) {
+        dot += __shfl_xor(dot, o, 64);
+        l1 += __shfl_xor(l1, o, 64);
+      }
+      if (piece == 0 && row < ss.nq) {
+        float w = -3.0e38f;
+        if (j >= 0) {
+          const float corr = 24.5f * l1 + (float)dp * 0x1p-9f + inv_ls;  // as in lse_coarse_kernel
+          float b = ss.kc0 * ss.kb0[jc];
+          if (ss.kb1) b += ss.kc1 * ss.kb1[jc];
+          if (ss.kb2) b += ss.kc2 * ss.kb2[jc];
+          b = fmaxf(fmaxf(b, kNegBig) * inv_ls, -3.0e38f);
+          w = fmaxf(dot + b - (corr * 0x1p-6f + inv_ls), -3.0e38f);
+        }
+        ss.seed[row] = w;
+      }
+    }
+    return;
+  }
   int tile = blockIdx.x;
   const bool second = tile >= tiles0;
   if (second) tile -= tiles0;
@@ -385,13 +452,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   float kbias = 0.f;  // bias of key js*32 + li of that sub-tile, read together with KL
   float bmax[2] = {0.f, 0.f};  // largest bias of the sub-tiles whose hi planes are in KH
 
-  // ---- where the running maxima start (sums start empty) ----
-  // A row whose largest logit of the last launch sat at key j starts from its current logit at
-  // j, computed here on the vector pipe from the same planes: whatever the potentials did since,
-  // this is a logit of the row, hence a lower bound of its new maximum, and close to it once
-  // the potentials settle.  (Any index inside the key set keeps the result exact; a stale one
-  // only costs tests that pass.)  The sum of the fp32 roundings of the two routes to a logit is
-  // far below corr / 64, which is taken off together with one base-2 unit.
+  // ---- where the running maxima start (sums start empty): coarse_bias_kernel has computed it ----
   const bool track = sd.best_key != nullptr;
   int best_j[RB];
   float warm[RB];
@@ -401,32 +462,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     best_j[rb] = -1;
     warm[rb] = -3.0e38f;
     if (track) {
-      const int row = min(row0 + rb * 32 + li, sd.nq - 1);
-      const int j = sd.best_key[row];
-      have = have && j >= 0;
-      const int jc = min(max(j, 0), sd.nk - 1);
-      const unsigned* krow = sd.kplanes + (size_t)jc * (size_t)ROWW + 4 * h;
-      float dot = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < KK16; ++kk) {
-        const u32x4 khi = *reinterpret_cast<const u32x4*>(krow + 8 * kk);
-        const u32x4 klo = *reinterpret_cast<const u32x4*>(krow + DP / 2 + 8 * kk);
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          // (words copied out first: a bit cast applied to a vector element reads element 0)
-          const unsigned khw = khi[w], klw = klo[w], qhw = xq[rb][0][kk][w], qlw = xq[rb][1][kk][w];
-          const f16x2 kh = __builtin_bit_cast(f16x2, khw), kl = __builtin_bit_cast(f16x2, klw);
-          const f16x2 qh = __builtin_bit_cast(f16x2, qhw), ql = __builtin_bit_cast(f16x2, qlw);
-          dot = __builtin_amdgcn_fdot2(kh, qh, dot, false);
-          dot = __builtin_amdgcn_fdot2(kh, ql, dot, false);
-          dot = __builtin_amdgcn_fdot2(kl, qh, dot, false);
-        }
-      }
-      dot += xor32(dot);
-      float b = kc0 * sd.kb0[jc] + (has_kb1 ? kc1 * kb1p[jc] : 0.f);
-      b += (has_kb2 ? kc2 * kb2p[jc] : 0.f);
-      b = fmaxf(fmaxf(b, kNegBig) * inv_lscale, -3.0e38f);
-      if (j >= 0) warm[rb] = fmaxf(dot + b - (corr[rb] * 0x1p-6f + inv_lscale), -3.0e38f);
+      warm[rb] = sd.seed[min(row0 + rb * 32 + li, sd.nq - 1)];
+      have = have && warm[rb] > -3.0e38f;
     }
   }
   // a workgroup with a row that has no key yet also samples 64 keys spread over the whole key set
