@@ -868,8 +868,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     need += side_ws_floats(mode, plans[s], sides[s].nq, dp) * sizeof(float);
   }
   // The sparse form's wavefronts go through several chunks each (at most 2048 sub-tiles: its
-  // list of sub-tiles to visit), few enough that the whole launch is about four per slot of
-  // the chip.
+  // list of sub-tiles to visit): eight key ranges, one per XCD and its L2, or more when the
+  // launch would otherwise be fewer than about four wavefronts per slot of the chip.
   int sparse_group[2] = {1, 1};
   {
     int64_t waves = 0;
@@ -877,7 +877,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       waves += (int64_t)plans[s].igroups * 4;
       if (plans[s].splits <= 1 || ps.margin_slot == 0 || plans[s].chunk > 65536) margins = false;
     }
-    const int want = (int)std::max<int64_t>(1, ceil_div(4 * 2048, std::max<int64_t>(waves, 1)));
+    const int want = (int)std::max<int64_t>(8, ceil_div(4 * 2048, std::max<int64_t>(waves, 1)));
     for (int s = 0; s < nsides; ++s)
       sparse_group[s] = std::max(1, std::min(ceil_div(plans[s].splits, want), 65536 / std::max(plans[s].chunk, 1)));
   }
