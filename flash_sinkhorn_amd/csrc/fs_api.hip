@@ -318,13 +318,15 @@ unsigned* tiled_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float
   return reinterpret_cast<unsigned*>(reinterpret_cast<char*>(keys) + 4 * row_array_bytes(rows));
 }
 
-// Writes the planes (and, for fp16, the scales) of every matrix of the set.
+// Writes the planes (and, for fp16, the scales) of every matrix of the set.  `keep`: the planes
+// outlive the call (fs_prepare_operands): the carried margins start empty and the second copy
+// in operand order, which only launches on kept planes read, is written too.
 int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws, hipStream_t st,
-                     bool clear_margins = false) {
+                     bool keep = false) {
   if (ps.n == 0) return FS_OK;
   char* base = static_cast<char*>(ws);
   int rc = FS_OK;
-  if (clear_margins && ps.margin_slot > 0)
+  if (keep && ps.margin_slot > 0)
     rc = launch_fill_zero(reinterpret_cast<unsigned*>(base + ps.margin_off),
                           (long long)(2 * ps.margin_slot / 4), st);
   if (rc != FS_OK) return rc;
@@ -340,7 +342,7 @@ int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws
                                    two ? nullptr : scales + 1, c.gemm ? 1 : 0,
                                    i == 0 ? select_state(ps, ws) : nullptr,
                                    best_keys_of(ps, c, ws, ps.src[i], ps.rows[i]),
-                                   tiled_of(ps, c, ws, ps.src[i], ps.rows[i]), st);
+                                   keep ? tiled_of(ps, c, ws, ps.src[i], ps.rows[i]) : nullptr, st);
   }
   return rc;
 }

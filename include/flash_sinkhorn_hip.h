@@ -40,9 +40,15 @@
  *    plan nearly every tile ends at the test, sorted rows or not.  Any content of that array
  *    leaves the results exact (indices are clamped into the key set); fs_prepare_operands
  *    resets it, and a row without a key starts from the largest logit of 64 keys sampled from
- *    the whole key set.  Results stay within fp32 rounding of the full computation.  On a
- *    flat plan, where every tile matters, the test costs about 20 %.  Ignored where it does
- *    not apply.
+ *    the whole key set.  With prepared operands the workspace also carries, per 64 query rows
+ *    and 32 keys, by how much a tile that ended at the test stayed clear of mattering, together
+ *    with the running sum of the largest key-bias changes of the launches so far: as long as
+ *    twice the bias change accumulated since a tile's test is below its margin, the tile would
+ *    end again, and the launch does not visit it.  The margins are dropped when the operands'
+ *    pairing, eps or the bias coefficients change; overwritten keys only cost visits.  Once the
+ *    potentials of a solve move little, nine tiles in ten are not visited on a peaked plan.
+ *    Results stay within fp32 rounding of the full computation.  On a flat plan, where every
+ *    tile matters, the test costs about 20 %.  Ignored where it does not apply.
  *    FS_FLAG_COARSE_AUTO (with FS_FLAG_OPERANDS_PREPARED, same conditions) leaves that choice to
  *    the device: every step enqueues both variants and a word of state next to the prepared
  *    planes says which one runs (the workgroups of the other return at once).  The coarse
