@@ -170,13 +170,15 @@ constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units en
 // and leaves the coarse variant when too few of its units ended at the test.
 // After a launch that used carried margins: this launch's bias change joins the running sum.
 // Which form of lse_coarse_kernel runs for a side: the sparse one once the side's largest bias
-// change since its last launch is below 32 base-2 units (margins then outlast many launches),
-// and on until it is above 128 again; the pipelined one before, and when a generation starts.
+// change since its last launch is below 256 base-2 units (the change about halves from step to
+// step of a solve, so margins of a few times that outlast the rest of it; on a peaked plan most
+// are larger), and on until it is above 1024 again; the pipelined one before, and when a
+// generation starts.
 // lscale: base-2 units per raw unit.
 __device__ __forceinline__ bool margins_settled(const unsigned* st, int side, float lscale) {
   if (st[kSelBump + side] != 0u || st[kSelGen + side] > 255u) return false;
   const float d = __builtin_bit_cast(float, st[kSelDmax + side]) * lscale;
-  return d < (st[kSelMode + side] != 0u ? 128.0f : 32.0f);  // false when d is not a number
+  return d < (st[kSelMode + side] != 0u ? 1024.0f : 256.0f);  // false when d is not a number
 }
 
 __device__ __forceinline__ void margins_commit(unsigned* st, int lane, bool settled) {

@@ -674,7 +674,8 @@ def test_coarse_test_starts_rows_from_the_keys_of_the_last_step(n, m, d, eps):
     check(fh2, gh2, F2, G2)
 
 
-@pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2500, 2300, 20, 0.05), (1200, 9000, 33, 0.02)])
+@pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2500, 2300, 20, 0.05), (1200, 9000, 33, 0.02),
+                                       (2600, 2200, 8, 0.05)])
 def test_carried_margins_leave_every_step_unchanged(n, m, d, eps):
     """On prepared planes the kernel with the coarse tile test carries margins from launch to
     launch and, once the potentials move little, runs in a sparse form that visits only the
@@ -729,10 +730,10 @@ def test_carried_margins_leave_every_step_unchanged(n, m, d, eps):
     for it in range(4):
         F, G = step(F, G, eps)
     # a large one: back to the pipelined form, then settling again
-    G2 = G + torch.from_numpy((3.0 * rng.standard_normal(m)).astype(np.float32)).cuda()
-    F2 = F + torch.from_numpy((3.0 * rng.standard_normal(n)).astype(np.float32)).cuda()
+    G2 = G + torch.from_numpy((20.0 * rng.standard_normal(m)).astype(np.float32)).cuda()
+    F2 = F + torch.from_numpy((20.0 * rng.standard_normal(n)).astype(np.float32)).cuda()
     F, G = step(F2, G2, eps, with_oracle=True)
-    for it in range(12):
+    for it in range(16):
         F, G = step(F, G, eps)
     s1 = skipped()
     F, G = step(F, G, eps)
