@@ -177,7 +177,9 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) dch = fmaxf(dch, __shfl_xor(dch, o, 64));
     if (lane == 0) {
-      atomicMax(&args.sel[kSelDmax + side], __builtin_bit_cast(unsigned, dch));
+      // (most wavefronts find a larger value already there; a stale read only costs an atomic)
+      const unsigned dbits = __builtin_bit_cast(unsigned, dch);
+      if (dbits > args.sel[kSelDmax + side]) atomicMax(&args.sel[kSelDmax + side], dbits);
       if (tile == 0 && args.sel[kSelTag + side] != args.tag[second ? 1 : 0]) {
         args.sel[kSelTag + side] = args.tag[second ? 1 : 0];
         // entries carry the generation in 8 bits and are cleared only with the planes: after 255

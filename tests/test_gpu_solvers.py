@@ -841,6 +841,33 @@ def test_solver_with_the_coarse_tile_test_equals_the_plain_solve(monkeypatch, va
         assert float((u - v).abs().max()) < 2e-6 * scale
 
 
+@pytest.mark.parametrize("extra", [dict(), dict(reach=1.5), dict(reach_x=0.8, reach_y=2.0)])
+def test_long_solves_with_carried_margins_equal_the_plain_solve(monkeypatch, extra):
+    """Sixty fixed-eps iterations, balanced and unbalanced: most of them run in the sparse form of
+    the kernel with the coarse tile test (tiles skipped on their carried margins), and the
+    potentials are the plain solve's to rounding."""
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    rng = np.random.default_rng(43)
+    n, m, d = 16500, 17000, 24
+    x, _ = _clustered(rng, n, d)
+    y, _ = _clustered(rng, m, d)
+    a = rng.random(n).astype(np.float32) + 0.5
+    b = rng.random(m).astype(np.float32) + 0.5
+    X, Y, A, B = dev(x, y, a / a.sum(), b / b.sum())
+    kw = dict(use_epsilon_scaling=False, eps=0.05, n_iters=60, allow_tf32=False, **extra)
+    monkeypatch.setattr(solvers, "_COARSE_MIN_ROWS", 16384)
+    monkeypatch.setattr(solvers, "COARSE_TEST", False)
+    want = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+    monkeypatch.setattr(solvers, "COARSE_TEST", None)
+    info = {}
+    got = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
+    assert info["coarse"] == "auto"
+    state = info["prepared"].variant_state()
+    assert not state["plain_selected"] and state["tiles_skipped"] > 0.3 * state["tiles_tested"]
+    for u, v in zip(got, want):
+        assert rel_err(u, v.cpu().numpy()) < 2e-5
+
+
 def test_variant_choice_on_the_device():
     """FS_FLAG_COARSE_AUTO: every step enqueues both kernel variants and a word next to the
     prepared planes says which runs.  Each row's running maximum starts from its logit at the key
