@@ -333,6 +333,7 @@ def main():
                                "product, one for tiles that end at the coarse test, none for "
                                "tiles not visited, padding of d to the MFMA width included)")
         r["frac"] = r["achieved"] / r["peak"]
+        r["frac_algorithmic"] = r["algorithmic_tflops"] / r["peak"]  # counts work the launch did not have to do
         r["traffic"] = MEASURED_TRAFFIC_BYTES.get(mode) if (n, m, d) == (N, M, D) else None
         return r
 

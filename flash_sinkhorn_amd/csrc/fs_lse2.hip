@@ -72,10 +72,10 @@ static int launch_coarse(const LaunchArgs& a, int dp, int rb, int blocks, hipStr
   // the per-tile records of the key bias, for both sides (tiles past the last key included)
   const int tiles0 = (a.side[0].nk + 63) / 64 + kAuxPadTiles;
   const int tiles1 = blocks > a.blocks0 ? (a.side[1].nk + 63) / 64 + kAuxPadTiles : 0;
-  // behind them, per 64 query rows one block that computes where the rows' maxima start
+  // behind them, per 8 query rows one block that computes where the rows' maxima start
   const bool seeds = a.side[0].seed != nullptr;
-  const int sb0 = seeds ? (a.side[0].nq + 63) / 64 : 0;
-  const int sb1 = seeds && blocks > a.blocks0 ? (a.side[1].nq + 63) / 64 : 0;
+  const int sb0 = seeds ? (a.side[0].nq + 7) / 8 : 0;
+  const int sb1 = seeds && blocks > a.blocks0 ? (a.side[1].nq + 7) / 8 : 0;
   hipLaunchKernelGGL((coarse_bias_kernel<0>), dim3(tiles0 + tiles1 + sb0 + sb1), dim3(64), 0, st, a,
                      tiles0, tiles0 + tiles1, sb0, dp);
   if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;

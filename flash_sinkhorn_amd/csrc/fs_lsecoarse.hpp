@@ -62,7 +62,7 @@ namespace fs {
 // sub-tile.  Keys past the end of the key set get a bias that masks them.  T only makes this a
 // template (header-defined kernel).
 //
-// The blocks behind the tiles (64 query rows each, side 0 first: seed_blocks0 of them) compute
+// The blocks behind the tiles (8 query rows each, side 0 first: seed_blocks0 of them) compute
 // where the rows' running maxima start.  A row whose largest logit of the last launch sat at key
 // j starts from its current logit at j, computed on the vector pipe from the same planes:
 // whatever the potentials did since, this is a logit of the row, hence a lower bound of its new
@@ -81,17 +81,19 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
     if (second_s) blk -= seed_blocks0;
     const Side& ss = second_s ? args.side[1] : args.side[0];
     if (ss.seed == nullptr) return;
-    // eight lanes per row, 16 bytes of each plane per lane (whole cache lines per row), eight rows
-    // per pass
+    // eight lanes per row, 16 bytes of each plane per lane (whole cache lines per row); one
+    // short wavefront per eight rows, so that the launch is as long as one chain of loads
     const int lane = threadIdx.x, piece = lane & 7, sub = lane >> 3;
     const float inv_ls = ss.plane_scale[ss.ps_q] * ss.plane_scale[ss.ps_k] / ss.qscale;
     const bool has_piece = piece * 4 < dp / 2;
-#pragma unroll
-    for (int pass = 0; pass < 8; ++pass) {
-      const int row = blk * 64 + pass * 8 + sub;
+    {
+      const int row = blk * 8 + sub;
       const int rc = min(row, ss.nq - 1);
       const int j = ss.best_key[rc];
       const int jc = min(max(j, 0), ss.nk - 1);
+      float b = ss.kc0 * ss.kb0[jc];  // (every lane of the row: the loads go out with the planes')
+      if (ss.kb1) b += ss.kc1 * ss.kb1[jc];
+      if (ss.kb2) b += ss.kc2 * ss.kb2[jc];
       float dot = 0.f, l1 = 0.f;
       if (has_piece) {
         const unsigned* q = ss.qplanes + (size_t)rc * (size_t)dp + piece * 4;
@@ -121,9 +123,6 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
         float w = -3.0e38f;
         if (j >= 0) {
           const float corr = 24.5f * l1 + (float)dp * 0x1p-9f + inv_ls;  // as in lse_coarse_kernel
-          float b = ss.kc0 * ss.kb0[jc];
-          if (ss.kb1) b += ss.kc1 * ss.kb1[jc];
-          if (ss.kb2) b += ss.kc2 * ss.kb2[jc];
           b = fmaxf(fmaxf(b, kNegBig) * inv_ls, -3.0e38f);
           w = fmaxf(dot + b - (corr * 0x1p-6f + inv_ls), -3.0e38f);
         }

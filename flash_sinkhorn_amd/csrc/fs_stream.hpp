@@ -488,40 +488,45 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
   const int row = it / per_row;
   const int col = (it % per_row) * 4;
   if (row >= sd.nq) return;
+  // (loops unrolled so that the loads of several key splits are in flight together: the merge
+  // is a chain of memory round trips and nothing else)
   float M = -3.0e38f;
+#pragma unroll 8
   for (int sp = 0; sp < sd.splits; ++sp)
     M = fmaxf(M, sd.part_ms[2 * ((size_t)sp * sd.nq + row)]);
   float s = 0.f, o = 0.f;
   float4 O = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int sp = 0; sp < sd.splits; ++sp) {
-    const size_t pr = (size_t)sp * sd.nq + row;
-    const float w = exp2f(sd.part_ms[2 * pr] - M);
-    s += w * sd.part_ms[2 * pr + 1];
-    if constexpr (HAS_O) {
+  if constexpr (HAS_O) {
+    for (int sp = 0; sp < sd.splits; ++sp) {
+      const size_t pr = (size_t)sp * sd.nq + row;
+      const float w = exp2f(sd.part_ms[2 * pr] - M);
+      s += w * sd.part_ms[2 * pr + 1];
       const float4 v = *reinterpret_cast<const float4*>(&sd.part_o[pr * dp + col]);
       O.x += w * v.x; O.y += w * v.y; O.z += w * v.z; O.w += w * v.w;
-    } else if (sd.part_o) {
-      o += w * sd.part_o[pr];
     }
-  }
-  if constexpr (HAS_O) {
     epilogue_vec4(sd.ep, sd.q, args.d, args.vec_ok != 0, row, col, M, s, O);
   } else {
-    if (sd.best_key != nullptr && sd.part_best != nullptr) {
-      // the key behind the largest partial maximum that a key of its chunk attained
-      float bm = -3.0e38f;
-      int bj = -1;
-      for (int sp = 0; sp < sd.splits; ++sp) {
-        const size_t pr = (size_t)sp * sd.nq + row;
+    // the sums, and the key behind the largest partial maximum that a key of its chunk attained
+    const bool keys = sd.best_key != nullptr && sd.part_best != nullptr;
+    const bool has_o = sd.part_o != nullptr;
+    float bm = -3.0e38f;
+    int bj = -1;
+#pragma unroll 8
+    for (int sp = 0; sp < sd.splits; ++sp) {
+      const size_t pr = (size_t)sp * sd.nq + row;
+      const float2 ms = *reinterpret_cast<const float2*>(&sd.part_ms[2 * pr]);
+      const float w = exp2f(ms.x - M);
+      s += w * ms.y;
+      if (has_o) o += w * sd.part_o[pr];
+      if (keys) {
         const int j = sd.part_best[pr];
-        const float m = sd.part_ms[2 * pr];
-        if (j >= 0 && m > bm) {
-          bm = m;
+        if (j >= 0 && ms.x > bm) {
+          bm = ms.x;
           bj = j;
         }
       }
-      if (bj >= 0) sd.best_key[row] = bj;  // no chunk exceeded the starting value: the old key stays
     }
+    if (keys && bj >= 0) sd.best_key[row] = bj;  // no chunk exceeded the starting value: the old key stays
     if (sd.m_prev != nullptr) sd.m_prev[row] = M;
     epilogue_scalar(sd.ep, row, M, s, o);
   }
