@@ -217,6 +217,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // sparse form: per wavefront, which sub-tiles it visits (bit 2 k of word g: sub-tile 32 g + k)
   constexpr int kActWords = 64;
   __shared__ unsigned long long lds_act[SPARSE ? 4 : 1][SPARSE ? kActWords : 1];
+  __shared__ unsigned lds_cnt[4];  // sparse form: the workgroup's unit counts, wavefronts done
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
@@ -246,6 +247,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     const int per_xcd = ((sd.igroups * nsplit + 7) / 8);
     bid = (bid % 8) * per_xcd + bid / 8;
     if (bid >= sd.igroups * nsplit) return;
+    if (threadIdx.x < 4) lds_cnt[threadIdx.x] = 0u;
+    __syncthreads();  // the only one of this form
   }
   const int split = SPARSE ? (bid / sd.igroups) * group : bid % nsplit;
   const int ig = SPARSE ? bid % sd.igroups : bid / nsplit;
@@ -916,11 +919,26 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
 
   // unit counts of this wavefront for the variant choice on the device; a workgroup that had
   // to sample its starting values says nothing about the launches that follow
-  if (args.sel != nullptr && lane == 0 && ntiles > 0 && !(track && cold)) {
+  if (args.sel != nullptr && lane == 0 && ntiles > 0) {
     const int slot = blockIdx.x % kSelSlots;
-        atomicAdd(&args.sel[kSelEnded + slot], n_ended + n_skipped);
-    if (SPARSE) atomicAdd(&args.sel[kSelSkip + slot], n_skipped);
-    atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
+    const bool counts = !(track && cold);
+    if constexpr (SPARSE) {
+      // the wavefronts of a workgroup end at different times: they add up in LDS, and the last
+      // one out hands the workgroup's counts to the state words (a quarter of the atomics)
+      if (counts) {
+        atomicAdd(&lds_cnt[0], n_ended + n_skipped);
+        atomicAdd(&lds_cnt[1], n_skipped);
+        atomicAdd(&lds_cnt[2], (unsigned)(ntiles * NSUB * RB));
+      }
+      if (atomicAdd(&lds_cnt[3], 1u) == 3u && lds_cnt[2] != 0u) {
+        atomicAdd(&args.sel[kSelEnded + slot], lds_cnt[0]);
+        atomicAdd(&args.sel[kSelSkip + slot], lds_cnt[1]);
+        atomicAdd(&args.sel[kSelUnits + slot], lds_cnt[2]);
+      }
+    } else if (counts) {
+      atomicAdd(&args.sel[kSelEnded + slot], n_ended);
+      atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
+    }
   }
 
 #pragma unroll
