@@ -675,7 +675,8 @@ def test_coarse_test_starts_rows_from_the_keys_of_the_last_step(n, m, d, eps):
 
 
 @pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2500, 2300, 20, 0.05), (1200, 9000, 33, 0.02),
-                                       (2600, 2200, 8, 0.05)])
+                                       (2600, 2200, 8, 0.05), (300, 260, 16, 0.1), (130, 700, 5, 0.2),
+                                       (64, 257, 64, 0.05)])
 def test_carried_margins_leave_every_step_unchanged(n, m, d, eps):
     """On prepared planes the kernel with the coarse tile test carries margins from launch to
     launch and, once the potentials move little, runs in a sparse form that visits only the
@@ -718,10 +719,11 @@ def test_carried_margins_leave_every_step_unchanged(n, m, d, eps):
     for it in range(30):  # settles: the sparse form takes over
         F, G = step(F, G, eps, with_oracle=it in (0, 29))
     s0, t0 = skipped(), prep.variant_state()["tiles_tested"]
-    assert s0 > 0
+    big = min(n, m) >= 1000  # (small problems may have no tile that can be skipped)
+    assert s0 > 0 or not big
     F, G = step(F, G, eps)
     st = prep.variant_state()
-    assert st["tiles_skipped"] > s0  # a settled step skips tiles
+    assert st["tiles_skipped"] > s0 or not big  # a settled step skips tiles
     # a disturbance of about 60 base-2 units: many margins are used up, the sparse form stays
     amp = 60.0 * eps * np.log(2.0)
     G2 = G + torch.from_numpy((amp * (2 * rng.random(m) - 1)).astype(np.float32)).cuda()
@@ -737,7 +739,7 @@ def test_carried_margins_leave_every_step_unchanged(n, m, d, eps):
         F, G = step(F, G, eps)
     s1 = skipped()
     F, G = step(F, G, eps)
-    assert skipped() > s1  # sparse again
+    assert skipped() > s1 or not big  # sparse again
     # arbitrary numbers in the key arrays: rows no longer start where their last maximum says
     prep.best_keys(0).copy_(torch.from_numpy(rng.integers(-5, m + 5, n).astype(np.int32)))
     prep.best_keys(1).copy_(torch.from_numpy(rng.integers(-2**31, 2**31 - 1, m).astype(np.int32)))
