@@ -160,7 +160,6 @@ constexpr int kSelSkip = kSelMode + 2;  // per-launch slots: units the sparse fo
 constexpr int kSelCumSkipped = 6;       // their running total (u64), part of kSelCumEnded's
 constexpr int kSelWords = kSelSkip + kSelSlots;
 static_assert(kSelWords <= 256, "one workgroup clears the state block");
-constexpr int kMarginGroups = 4;  // a key chunk holds at most 64 * kMarginGroups / 2 sub-tiles
 constexpr unsigned kSelDecideSteps = 3;  // which counted launch of the coarse variant decides
 constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
 
