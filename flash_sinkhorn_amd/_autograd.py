@@ -63,14 +63,14 @@ class _SinkhornGradFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, y, a, b, f_grad, g_grad, grad_scale, eps: float,
                 config: _SinkhornConfig, compute_grad_x: bool, compute_grad_y: bool,
-                label_x=None, label_y=None, label_cost_matrix=None):
+                label_x=None, label_y=None, label_cost_matrix=None, seed_keys=None):
         gx, gy = sinkhorn_geomloss_online_grad_sqeuclid(
             x, y, a, b, f_grad, g_grad, eps=float(eps), allow_tf32=config.allow_tf32,
             use_exp2=config.use_exp2, grad_scale=grad_scale,
             compute_grad_x=bool(compute_grad_x), compute_grad_y=bool(compute_grad_y),
             cost_scale=config.cost_scale, label_x=label_x, label_y=label_y,
             label_cost_matrix=label_cost_matrix, lambda_x=config.lambda_x,
-            lambda_y=config.lambda_y)
+            lambda_y=config.lambda_y, _seed_keys=seed_keys)
         ctx.save_for_backward(x, y, a, b, f_grad, g_grad, grad_scale)
         ctx.eps = float(eps)
         ctx.config = config
@@ -105,7 +105,7 @@ class _SinkhornGradFn(torch.autograd.Function):
                     allow_tf32=False,  # second order needs full fp32 operands
                     use_exp2=cfg.use_exp2)
                 out_x = hvp * grad_scale
-        return (out_x,) + (None,) * 13
+        return (out_x,) + (None,) * 14
 
 
 class _SinkhornCostFn(torch.autograd.Function):
@@ -118,6 +118,7 @@ class _SinkhornCostFn(torch.autograd.Function):
         problem (with ``return_prelast=config.last_extrapolation``), when the caller has already
         run the solve (the two self terms of a debiased loss are solved together)."""
         eps_last = float(eps_list[-1])
+        seed_keys = None
         if presolved is not None:
             if config.last_extrapolation:
                 f_cost, g_cost, f_grad, g_grad = presolved
@@ -133,8 +134,9 @@ class _SinkhornCostFn(torch.autograd.Function):
             f_grad, g_grad = f_cost, g_cost
             balanced_formula = True
         else:
+            info = {}
             out = sinkhorn_flashstyle_symmetric(
-                x, y, a, b, blur=config.blur, scaling=config.scaling,
+                x, y, a, b, solve_info=info, blur=config.blur, scaling=config.scaling,
                 use_epsilon_scaling=config.use_epsilon_scaling, eps=config.eps,
                 n_iters=config.n_iters, allow_tf32=config.allow_tf32, use_exp2=config.use_exp2,
                 cost_scale=config.cost_scale, rho_x=config.rho_x, rho_y=config.rho_y,
@@ -150,10 +152,18 @@ class _SinkhornCostFn(torch.autograd.Function):
                 f_grad, g_grad = f_cost, g_cost
             # <a,f>+<b,g> unless BOTH marginals are relaxed
             balanced_formula = config.rho_x is None or config.rho_y is None
+            # the keys behind the rows' largest logits, where the solve kept them: a hint from
+            # which the gradient's sweep recognises the tiles that cannot matter
+            prep = info.get("prepared")
+            if prep is not None and info.get("coarse"):
+                kx, ky = prep.best_keys(0), prep.best_keys(1)
+                if kx is not None and ky is not None:
+                    seed_keys = (kx.clone(), ky.clone())
 
         ctx.save_for_backward(x, y, a, b, f_cost, g_cost, f_grad, g_grad)
         ctx.eps = eps_last
         ctx.config = config
+        ctx.seed_keys = seed_keys
         labelled = config.backend != "alternating"  # the alternating backend takes no labels
         ctx.labels = (label_x, label_y, label_cost_matrix) if labelled else (None, None, None)
         if balanced_formula:
@@ -170,7 +180,7 @@ class _SinkhornCostFn(torch.autograd.Function):
         if x.requires_grad or y.requires_grad:
             gx, gy = _SinkhornGradFn.apply(x, y, a, b, f_grad, g_grad, grad_out, ctx.eps,
                                            ctx.config, x.requires_grad, y.requires_grad,
-                                           *ctx.labels)
+                                           *ctx.labels, ctx.seed_keys)
             grad_x = gx if x.requires_grad else None
             grad_y = gy if y.requires_grad else None
         if a.requires_grad:

@@ -59,6 +59,7 @@ _SIGNATURES = {
     "fs_cg_update": (ctypes.c_int, [_P] * 5 + [_I, _P]),
     "fs_self_pair_steps": (ctypes.c_int, [_P] * 12 + [_I] * 3 + [_P] * 5 + [ctypes.c_int, _F] + _TAIL),
     "fs_grad": (ctypes.c_int, [_P] * 13 + [_I] * 3 + [_F] * 2 + _TAIL),
+    "fs_grad_seeded": (ctypes.c_int, [_P] * 13 + [_I] * 3 + [_F] * 2 + [_P] * 2 + _TAIL),
     "fs_apply_vec": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + [ctypes.c_int] + _TAIL),
     "fs_apply_mat": (ctypes.c_int, [_P] * 9 + [_I] * 4 + [_F] * 2 + [ctypes.c_int] + _TAIL),
     "fs_mat5": (ctypes.c_int, [_P] * 8 + [_I] * 3 + [_F] * 2 + _TAIL),

@@ -688,7 +688,7 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
   bool vec_ok = (d % 4 == 0);
-  bool any_split = false;
+  bool any_split = false, any_seed = false;
   int blocks[2] = {0, 0};
   for (int s = 0; s < nsides; ++s) {
     Side& sd = sides[s];
@@ -722,6 +722,11 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
       sd.kmax2 = reinterpret_cast<const float*>(base + bounds_off);
       sd.q2norm2 = sd.kmax2 + 64;
     }
+    // a caller that knows, per query row, a key with a large logit (the carried keys of a solve):
+    // the rows' running maxima start from their logits at those keys
+    sd.seed = (sd.best_key != nullptr && mode != kArgmax)
+                  ? row_array_of(ps, cfg, ws, sd.q, sd.nq, 3) : nullptr;
+    any_seed = any_seed || sd.seed != nullptr;
     blocks[s] = p.igroups * p.splits;
     a.side[s] = sd;
   }
@@ -732,6 +737,7 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   if (total <= 0) return FS_OK;
 
   if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
+  if (any_seed && rc == FS_OK) rc = launch_row_seeds(a, dpk, nsides, st);
   if (mat5 && rc == FS_OK) {
     const Side& sd = sides[0];
     float* partial = reinterpret_cast<float*>(base + q2_off + plane_bytes(sd.nq, cfg));
@@ -1322,6 +1328,16 @@ int fs_grad(const float* x, const float* y, const float* f, const float* g, cons
             const float* grad_scale, float* grad_x, float* grad_y, int64_t n, int64_t m,
             int64_t d, float eps, float cost_scale, uint32_t flags, void* workspace,
             size_t workspace_bytes, void* stream) {
+  return fs_grad_seeded(x, y, f, g, log_a, log_b, a, b, x2, y2, grad_scale, grad_x, grad_y, n, m, d,
+                        eps, cost_scale, nullptr, nullptr, flags, workspace, workspace_bytes, stream);
+}
+
+int fs_grad_seeded(const float* x, const float* y, const float* f, const float* g,
+                   const float* log_a, const float* log_b, const float* a, const float* b,
+                   const float* x2, const float* y2, const float* grad_scale, float* grad_x,
+                   float* grad_y, int64_t n, int64_t m, int64_t d, float eps, float cost_scale,
+                   const int* keys_x, const int* keys_y, uint32_t flags, void* workspace,
+                   size_t workspace_bytes, void* stream) {
   (void)flags;
   if (!x || !y || !f || !g || !log_a || !log_b || !a || !b || !x2 || !y2)
     return FS_ERR_NULL_POINTER;
@@ -1336,6 +1352,7 @@ int fs_grad(const float* x, const float* y, const float* f, const float* g, cons
     sd.kb2 = log_b; sd.kc2 = kLog2e;
     sd.ep.kind = kEpiGrad; sd.ep.out = grad_x; sd.ep.w = a; sd.ep.grad_scale = grad_scale;
     sd.ep.gcoef = 2.0f * cost_scale;
+    sd.best_key = const_cast<int*>(keys_x);  // read only
   }
   if (grad_y) {
     Side& sd = s[ns++];
@@ -1343,6 +1360,7 @@ int fs_grad(const float* x, const float* y, const float* f, const float* g, cons
     sd.kb2 = log_a; sd.kc2 = kLog2e;
     sd.ep.kind = kEpiGrad; sd.ep.out = grad_y; sd.ep.w = b; sd.ep.grad_scale = grad_scale;
     sd.ep.gcoef = 2.0f * cost_scale;
+    sd.best_key = const_cast<int*>(keys_y);
   }
   if (ns == 0) return FS_OK;
   return run_stream(kMat, false, s, ns, d, workspace, workspace_bytes, (hipStream_t)stream, flags);

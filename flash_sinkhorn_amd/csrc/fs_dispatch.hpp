@@ -18,6 +18,9 @@ int launch_sliced(int mode, const LaunchArgs& a, int nw, int nsl, int blocks, hi
 int launch_fill_zero(unsigned* p, long long n, hipStream_t st);
 int launch_absmax(const float* a, long long na, const float* b, long long nb, float* partial,
                   hipStream_t st);
+// The seed part of coarse_bias_kernel alone: per side with Side::seed set, where each query row's
+// running maximum starts (its logit at the key Side::best_key names).
+int launch_row_seeds(const LaunchArgs& a, int dp, int nsides, hipStream_t st);
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
                             int chunked, unsigned* clear_state, int* best_keys, unsigned* tiled,

@@ -67,6 +67,15 @@ static int launch_coarse_dp(const LaunchArgs& a, int blocks, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
+int launch_row_seeds(const LaunchArgs& a, int dp, int nsides, hipStream_t st) {
+  const int sb0 = (a.side[0].nq + 7) / 8;
+  const int sb1 = nsides > 1 ? (a.side[1].nq + 7) / 8 : 0;
+  LaunchArgs b = a;
+  b.sel_pred = 0;
+  hipLaunchKernelGGL((coarse_bias_kernel<0>), dim3(sb0 + sb1), dim3(64), 0, st, b, 0, 0, sb0, dp);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
 static int launch_coarse(const LaunchArgs& a, int dp, int rb, int blocks, hipStream_t st) {
   if (rb != 2) return FS_ERR_BAD_ARGUMENT;
   // the per-tile records of the key bias, for both sides (tiles past the last key included)

@@ -37,6 +37,7 @@ constexpr float kPtLazyThresh = 4.0f;  // exponentials stay below 2^4 relative t
 // thing, while a probability keeps a nonzero fp16 image down to 2^-35 of the row's largest one
 // instead of 2^-24 (a tail of many far keys would otherwise be rounded away one-sidedly).
 constexpr float kPtUp = 11.0f;
+constexpr float kPtSkipBelow = -40.0f;  // base-2 units
 
 template <int DP, int RB, int MODE>
 __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void plan_tile_kernel(const LaunchArgs args) {
@@ -198,6 +199,28 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
     }
   }
 
+  // Where the running maxima start: 0 and the first tile's largest logit, or, when the caller
+  // knew a key with a large logit for every row of this wavefront, the logits at those keys
+  // (coarse_bias_kernel's seed blocks): a lower bound of the row's largest logit, from which
+  // the skip below recognises tiles that cannot matter before the largest one has come by.
+  bool seeded = false;
+  if constexpr (MODE != kArgmax) {
+    if (sd.seed != nullptr) {
+      float sv[RB];
+      bool ok = true;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        sv[rb] = sd.seed[min(row0 + rb * 32 + li, sd.nq - 1)];
+        ok = ok && sv[rb] > -3.0e38f;
+      }
+      seeded = __builtin_amdgcn_ballot_w64(ok) == ~0ull;
+      if (seeded) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) run_m[rb] = sv[rb];
+      }
+    }
+  }
+
   // ---- prologue: tiles 0 and 1 on their way, bias (and v) of tile 0 ----
   RawBias raw_next[NSUB];
 #pragma unroll
@@ -344,7 +367,10 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
         float tmax = fmaxf(acc[0], acc[1]);
 #pragma unroll
         for (int r = 2; r < 16; ++r) tmax = fmaxf(tmax, acc[r]);
-        const bool first = (t == 0 && js == 0);
+        const bool first = (t == 0 && js == 0 && !seeded);
+        // every logit of the unit 2^40 below the running maximum (itself never above the row's
+        // largest logit): its exponentials could not change the fp32 sums
+        if (!first && !wave_any(tmax * lscale > kPtSkipBelow)) continue;
         float cc = 0.f;
         if (first || wave_any(tmax * lscale > kPtLazyThresh)) {
           float a = tmax, b = tmax;

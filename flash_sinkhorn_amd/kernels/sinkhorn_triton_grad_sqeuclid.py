@@ -31,7 +31,7 @@ def sinkhorn_geomloss_online_grad_sqeuclid(
     compute_grad_x: bool = True, compute_grad_y: bool = True, cost_scale: float = 1.0,
     label_x: Optional[torch.Tensor] = None, label_y: Optional[torch.Tensor] = None,
     label_cost_matrix: Optional[torch.Tensor] = None, lambda_x: float = 1.0,
-    lambda_y: float = 0.0,
+    lambda_y: float = 0.0, _seed_keys=None,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
     """Returns (grad_x [n,d] or None, grad_y [m,d] or None), fp32.  ``grad_scale`` is a
     one-element device tensor read by the kernel (no host sync)."""
@@ -81,13 +81,22 @@ def sinkhorn_geomloss_online_grad_sqeuclid(
     gx = torch.empty((n, d), device=x.device, dtype=torch.float32) if compute_grad_x else None
     gy = torch.empty((m, d), device=x.device, dtype=torch.float32) if compute_grad_y else None
     ws = _lib.workspace(_lib.OP_GRAD, n, m, d, x.device)
-    rc = _lib.lib().fs_grad(
+    # _seed_keys: (int32 [n], int32 [m]) keys with a large logit per row, as a solve with the
+    # coarse tile test leaves them (PreparedOperands.best_keys); a hint, results do not depend on it
+    kx = ky = None
+    if _seed_keys is not None:
+        kx, ky = _seed_keys
+        if (kx is None or ky is None or kx.numel() != n or ky.numel() != m
+                or kx.dtype != torch.int32 or ky.dtype != torch.int32):
+            kx = ky = None
+    rc = _lib.lib().fs_grad_seeded(
         xf.data_ptr(), yf.data_ptr(), ff.data_ptr(), gf.data_ptr(), log_a.data_ptr(),
         log_b.data_ptr(), af.data_ptr(), bf.data_ptr(), x2.data_ptr(), y2.data_ptr(),
         _lib.ptr(grad_scale), _lib.ptr(gx), _lib.ptr(gy), n, m, d, float(eps), float(cost_scale),
+        _lib.ptr(kx), _lib.ptr(ky),
         _lib.flags(use_exp2, allow_tf32), _lib.ptr(ws), 0 if ws is None else ws.numel(),
         _lib.stream_of(x))
-    _lib.check(rc, "fs_grad")
+    _lib.check(rc, "fs_grad_seeded")
     if use_labels:
         # The kernel returned 2cs*gs*w*(q' - bar(k')) on the augmented rows.  The reference's
         # result is 2*lambda_x*cs*gs*w*(q - bar(k)) on the first d columns (:277-283); with

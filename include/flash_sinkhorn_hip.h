@@ -295,6 +295,23 @@ int fs_grad(const float* x, const float* y, const float* f, const float* g, cons
             size_t workspace_bytes, void* stream);
 
 /*
+ * fs_grad with a hint, no counterpart in the reference: keys_x[i] (keys_y[j]) names a row of y
+ * (of x) at which row i of x (row j of y) has a large logit, typically the carried keys that a
+ * solve with FS_FLAG_COARSE_TEST left in its prepared workspace (fs_best_keys_offset), or NULL.
+ * The rows' running maxima start from their logits at these keys, so that tiles that cannot
+ * matter are recognised from the first tile on; any content leaves the results exact (indices
+ * are clamped into range, negative ones mean "none").  d <= 128 in the default operand mode;
+ * ignored elsewhere.
+ */
+int fs_grad_seeded(const float* x, const float* y, const float* f, const float* g,
+                   const float* log_a, const float* log_b, const float* a, const float* b,
+                   const float* x2, const float* y2, const float* grad_scale, float* grad_x,
+                   float* grad_y, int64_t n, int64_t m, int64_t d, float eps, float cost_scale,
+                   const int* keys_x, const int* keys_y, uint32_t flags, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+
+/*
  * axis=1: out[i] = sum_j P_ij vec[j];  axis=0: out[j] = sum_i P_ij vec[i], with
  * P_ij = exp(log_a_i + log_b_j + (f_hat_i + g_hat_j + coord_scale x_i.y_j)/eps).
  * Replaces apply_plan_vec_flashstyle (kernels/apply_flash.py:835-951, kernels 594-832).

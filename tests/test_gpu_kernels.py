@@ -125,6 +125,55 @@ def test_gradient(n, m, d):
     assert gx is None and rel_err(gy, wy) < RTOL
 
 
+@pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2100, 2300, 20, 0.05), (700, 5000, 100, 0.02),
+                                       (129, 1000, 3, 0.05)])
+def test_gradient_on_peaked_plans_with_and_without_key_hints(n, m, d, eps):
+    """The product kernel leaves out 32 x 32 tiles whose logits all lie 2^40 below the rows'
+    running maxima, and starts those maxima from the rows' logits at keys a caller names
+    (fs_grad_seeded).  On a peaked plan (clustered clouds, small eps) the gradient must equal the
+    fp64 oracle with the arg-max keys, with keys of another problem, with arbitrary numbers and
+    without keys, and the hinted and plain results must agree to rounding."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    rng = np.random.default_rng(51)
+    # (norms of order 1: the standard potentials enter the logits as g / eps, and their fp32
+    # rounding must stay far below one logit unit for the comparison to be about the kernel)
+    sc = 0.7 / np.sqrt(d)
+    centres = rng.standard_normal((8, d)) * 2.0
+    x = (sc * (centres[rng.integers(0, 8, n)] + rng.standard_normal((n, d)))).astype(np.float32)
+    y = (sc * (centres[rng.integers(0, 8, m)] + rng.standard_normal((m, d)))).astype(np.float32)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = (rng.random(m) + 0.5).astype(np.float32)
+    b /= b.sum()
+    # potentials of a few symmetric iterations: a peaked plan, not a converged one
+    fh = -(x * x).sum(1).astype(np.float32)
+    gh = -(y * y).sum(1).astype(np.float32)
+    la, lb = np.log(a), np.log(b)
+    for it in range(4):
+        fh, gh = oracle.symmetric_step(x, y, fh, gh, la, lb, eps, 1.0, 1.0 if it == 0 else 0.5, 1.0, 1.0)
+    f = (fh + (x * x).sum(1)).astype(np.float32)
+    g = (gh + (y * y).sum(1)).astype(np.float32)
+    wx, wy = oracle.grad_barycentric(x, y, a, b, f, g, eps, cost_scale=1.0, grad_scale=1.0)
+    logits = (2.0 * x.astype(np.float64) @ y.astype(np.float64).T + gh[None, :]) / eps + lb[None, :]
+    kx_true = logits.argmax(1).astype(np.int32)
+    logits_t = (2.0 * y.astype(np.float64) @ x.astype(np.float64).T + fh[None, :]) / eps + la[None, :]
+    ky_true = logits_t.argmax(1).astype(np.int32)
+    X, Y, A, B, F, G = dev(x, y, a, b, f, g)
+    plain = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False)
+    assert rel_err(plain[0], wx) < RTOL and rel_err(plain[1], wy) < RTOL
+    hints = [(kx_true, ky_true),
+             (rng.integers(0, m, n).astype(np.int32), rng.integers(0, n, m).astype(np.int32)),
+             (rng.integers(-2**31, 2**31 - 1, n).astype(np.int32), np.full(m, -1, np.int32))]
+    for kx, ky in hints:
+        keys = (torch.from_numpy(kx).cuda(), torch.from_numpy(ky).cuda())
+        gx, gy = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False, _seed_keys=keys)
+        assert rel_err(gx, wx) < RTOL and rel_err(gy, wy) < RTOL
+        assert rel_err(gx, plain[0].cpu().numpy()) < RTOL and rel_err(gy, plain[1].cpu().numpy()) < RTOL
+    gx, _ = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False, compute_grad_y=False,
+                 _seed_keys=(torch.from_numpy(kx_true).cuda(), torch.from_numpy(ky_true).cuda()))
+    assert rel_err(gx, wx) < RTOL
+
+
 @pytest.mark.parametrize("n,m,d", SHAPES)
 def test_apply_vec_and_mat(n, m, d):
     from flash_sinkhorn_amd.kernels.apply_flash import (
