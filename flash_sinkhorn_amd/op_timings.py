@@ -3,7 +3,8 @@
 Prints one JSON line per shape with the average launch time (HIP events on the current
 stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop),
 one LSE half-update (2nmd), gradient of one side (4nmd), plan-vector (2nmd), plan-matrix
-(4nmd), mat5 (6nmd) and the hard c-transform (2nmd), followed by end-to-end wall times of the five configurations
+(4nmd), mat5 (6nmd) and the hard c-transform (2nmd); at c3 also the gradient after a solve on clustered clouds,
+with and without the keys the solve carried; then end-to-end wall times of the five configurations
 through the public API (solver loops, autograd, CG included).
 """
 from __future__ import annotations
@@ -130,10 +131,48 @@ def end_to_end(name):
     return out
 
 
+def gradient_after_solve(name):
+    """Both-sides gradient at the potentials of a 100-iteration fixed-eps solve on clustered
+    clouds (8-component Gaussian mixtures, a peaked plan): without hints, and with the keys the
+    solve carried (what the loss's backward passes to fs_grad_seeded)."""
+    import numpy as np
+
+    from flash_sinkhorn_amd import sinkhorn_solvers as solvers
+    n, m, d, eps = SHAPES[name]
+    rng = np.random.default_rng(3)
+
+    def cloud(rows):
+        centres = rng.standard_normal((8, d)).astype(np.float32) * 0.6
+        pts = centres[rng.integers(0, 8, rows)] + 0.25 * rng.standard_normal((rows, d)).astype(np.float32)
+        return torch.from_numpy(pts.astype(np.float32)).cuda()
+
+    X, Y = cloud(n), cloud(m)
+    A = torch.full((n,), 1.0 / n, device="cuda")
+    B = torch.full((m,), 1.0 / m, device="cuda")
+    info = {}
+    f, g = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, use_epsilon_scaling=False, eps=eps,
+                                                 n_iters=100, allow_tf32=False, solve_info=info)[:2]
+    prep = info.get("prepared")
+    keys = None
+    if prep is not None and prep.best_keys(0) is not None:
+        keys = (prep.best_keys(0).clone(), prep.best_keys(1).clone())
+    out = {"shape": name, "workload": "gradient of both sides after a 100-iteration solve, "
+                                      "8-component Gaussian mixtures"}
+    for label, k in (("ms_without_hints", None), ("ms_with_carried_keys", keys)):
+        if label == "ms_with_carried_keys" and k is None:
+            continue
+        out[label] = round(_avg_ms(lambda: sinkhorn_geomloss_online_grad_sqeuclid(
+            X, Y, A, B, f, g, eps=eps, allow_tf32=False, _seed_keys=k), reps=10), 4)
+    return out
+
+
 def main(argv):
     names = [a for a in argv if a in SHAPES] or list(SHAPES)
     for name in names:
         print(json.dumps(kernel_timings(name)), flush=True)
+    for name in names:
+        if name == "c3":
+            print(json.dumps(gradient_after_solve(name)), flush=True)
     for name in names:
         print(json.dumps(end_to_end(name)), flush=True)
 
