@@ -11,12 +11,16 @@ the next replay overwrites them).  Keys hold everything that shapes the launches
 shapes, the per-step (eps, weight, damping) tuples, flags, and which arguments alias.  The first
 call with a key runs eagerly (it also loads the kernels), the second captures, later ones replay;
 an LRU bound keeps the memory of forgotten shapes from piling up.  Nothing is captured while the
-caller is itself capturing.  No counterpart in the reference, whose solver loop launches one
+caller is itself capturing.  An entry's static tensors are written, replayed into and cloned on
+the caller's stream, so an entry belongs to one (thread, stream) pair: both are part of the key,
+and two threads or streams solving the same shape each capture a graph of their own; the cache
+itself is guarded by a lock.  No counterpart in the reference, whose solver loop launches one
 Triton kernel per step (sinkhorn_solvers.py:497-531).
 """
 from __future__ import annotations
 
 import os
+import threading
 from collections import OrderedDict
 from typing import Callable, Optional, Sequence, Tuple
 
@@ -41,6 +45,7 @@ class _Entry:
 
 
 _cache: "OrderedDict[tuple, _Entry]" = OrderedDict()
+_lock = threading.Lock()
 
 
 def eligible(n: int, m: int, n_steps: int, device: torch.device) -> bool:
@@ -49,7 +54,8 @@ def eligible(n: int, m: int, n_steps: int, device: torch.device) -> bool:
 
 
 def clear() -> None:
-    _cache.clear()
+    with _lock:
+        _cache.clear()
 
 
 def run(key: tuple, fn: Callable[..., Tuple[torch.Tensor, ...]],
@@ -57,12 +63,14 @@ def run(key: tuple, fn: Callable[..., Tuple[torch.Tensor, ...]],
     """``fn(*inputs)`` through a graph: ``fn`` must enqueue the same kernels for the same key
     whatever the values in ``inputs`` (contiguous tensors or None), allocate what it needs with
     torch, and return a tuple of tensors."""
-    entry = _cache.get(key)
-    if entry is None:
-        entry = _cache[key] = _Entry()
-        while len(_cache) > MAX_ENTRIES:
-            _cache.popitem(last=False)
-    _cache.move_to_end(key)
+    key = key + (torch.cuda.current_stream().cuda_stream, threading.get_ident())
+    with _lock:
+        entry = _cache.get(key)
+        if entry is None:
+            entry = _cache[key] = _Entry()
+            while len(_cache) > MAX_ENTRIES:
+                _cache.popitem(last=False)
+        _cache.move_to_end(key)
     entry.calls += 1
     if entry.calls == 1:  # eager: loads the kernels, and one-off shapes never pay for a capture
         return fn(*inputs)

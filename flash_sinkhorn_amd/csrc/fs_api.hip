@@ -650,7 +650,8 @@ int pt_rows_per_wave(int64_t nq) { return nq >= 16384 ? 2 : 1; }
 // Workspace: plane region of x and y (the layout of lse2_kernel, so prepared planes serve),
 // then per side the V^T operands with their aux block (kMat), then per side the partial rows.
 int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig& cfg,
-                  const Family& fam, bool prepared, void* ws, size_t ws_bytes, hipStream_t st) {
+                  const Family& fam, bool prepared, uint32_t flags, void* ws, size_t ws_bytes,
+                  hipStream_t st) {
   PlaneSet ps;
   int rc = side_plane_set(sides, nsides, cfg, ps);
   if (rc != FS_OK) return rc;
@@ -687,6 +688,7 @@ int run_plan_tile(int mode, Side* sides, int nsides, int64_t d, const LseConfig&
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;
+  a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
   bool vec_ok = (d % 4 == 0);
   bool any_split = false, any_seed = false;
   int blocks[2] = {0, 0};
@@ -822,7 +824,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   // the plan-vector product at <= 64 columns rides on the pipelined log-sum-exp kernel
   const bool vec_lse2 = mode == kVec && cfg.prec == 3 && cfg.dp <= 64 && !fam.sliced;
   if (mode != kLse && !vec_lse2 && !fam.sliced && cfg.prec == 3)
-    return run_plan_tile(mode, sides, nsides, d, cfg, fam, prepared, ws, ws_bytes, st);
+    return run_plan_tile(mode, sides, nsides, d, cfg, fam, prepared, flags, ws, ws_bytes, st);
   LaunchArgs a;
   std::memset(&a, 0, sizeof(a));
   a.d = (int)d;

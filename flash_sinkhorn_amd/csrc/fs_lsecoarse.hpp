@@ -81,11 +81,11 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
     if (second_s) blk -= seed_blocks0;
     const Side& ss = second_s ? args.side[1] : args.side[0];
     if (ss.seed == nullptr) return;
-    // eight lanes per row, 16 bytes of each plane per lane (whole cache lines per row); one
-    // short wavefront per eight rows, so that the launch is as long as one chain of loads
+    // eight lanes per row, 16 bytes of each plane per lane and 64-column piece of the row (whole
+    // cache lines per row); one short wavefront per eight rows, so that the launch is as long as
+    // one chain of loads
     const int lane = threadIdx.x, piece = lane & 7, sub = lane >> 3;
     const float inv_ls = ss.plane_scale[ss.ps_q] * ss.plane_scale[ss.ps_k] / ss.qscale;
-    const bool has_piece = piece * 4 < dp / 2;
     {
       const int row = blk * 8 + sub;
       const int rc = min(row, ss.nq - 1);
@@ -95,9 +95,10 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
       if (ss.kb1) b += ss.kc1 * ss.kb1[jc];
       if (ss.kb2) b += ss.kc2 * ss.kb2[jc];
       float dot = 0.f, l1 = 0.f;
-      if (has_piece) {
-        const unsigned* q = ss.qplanes + (size_t)rc * (size_t)dp + piece * 4;
-        const unsigned* k = ss.kplanes + (size_t)jc * (size_t)dp + piece * 4;
+      // words [w0, w0 + 4) of each plane: rows wider than 64 columns take more than one round
+      for (int w0 = piece * 4; w0 < dp / 2; w0 += 32) {
+        const unsigned* q = ss.qplanes + (size_t)rc * (size_t)dp + w0;
+        const unsigned* k = ss.kplanes + (size_t)jc * (size_t)dp + w0;
         const u32x4 qh4 = *reinterpret_cast<const u32x4*>(q);
         const u32x4 ql4 = *reinterpret_cast<const u32x4*>(q + dp / 2);
         const u32x4 kh4 = *reinterpret_cast<const u32x4*>(k);
@@ -121,7 +122,8 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
       }
       if (piece == 0 && row < ss.nq) {
         float w = -3.0e38f;
-        if (j >= 0) {
+        // a key that is masked out (bias at the stand-in for -inf) says nothing about the row
+        if (j >= 0 && b > 0.5f * kNegBig) {
           const float corr = 24.5f * l1 + (float)dp * 0x1p-9f + inv_ls;  // as in lse_coarse_kernel
           b = fmaxf(fmaxf(b, kNegBig) * inv_ls, -3.0e38f);
           w = fmaxf(dot + b - (corr * 0x1p-6f + inv_ls), -3.0e38f);

@@ -37,7 +37,6 @@ constexpr float kPtLazyThresh = 4.0f;  // exponentials stay below 2^4 relative t
 // thing, while a probability keeps a nonzero fp16 image down to 2^-35 of the row's largest one
 // instead of 2^-24 (a tail of many far keys would otherwise be rounded away one-sidedly).
 constexpr float kPtUp = 11.0f;
-constexpr float kPtSkipBelow = -40.0f;  // base-2 units
 
 template <int DP, int RB, int MODE>
 __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void plan_tile_kernel(const LaunchArgs args) {
@@ -82,6 +81,8 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
 
   const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = 1.0f / lscale;
+  // base-2 units: -40, or so far down that nothing is skipped (LaunchArgs::skip_log2)
+  const float skip_below = args.skip_log2;
 
   // ---- stationary query planes: [block][plane][16-column step] ----
   u32x4 xq[RB][2][KK16];
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
         const bool first = (t == 0 && js == 0 && !seeded);
         // every logit of the unit 2^40 below the running maximum (itself never above the row's
         // largest logit): its exponentials could not change the fp32 sums
-        if (!first && !wave_any(tmax * lscale > kPtSkipBelow)) continue;
+        if (!first && !wave_any(tmax * lscale > skip_below)) continue;
         float cc = 0.f;
         if (first || wave_any(tmax * lscale > kPtLazyThresh)) {
           float a = tmax, b = tmax;

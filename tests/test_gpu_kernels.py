@@ -174,6 +174,77 @@ def test_gradient_on_peaked_plans_with_and_without_key_hints(n, m, d, eps):
     assert rel_err(gx, wx) < RTOL
 
 
+@pytest.mark.parametrize("d", [100, 128, 72])
+def test_key_hints_on_rows_wider_than_64_columns(d):
+    """64 < d <= 128: the logit at a hinted key must be the dot product over ALL columns.  Every
+    row is hinted at a key whose first 64 columns repeat the row (large positive half dot) and
+    whose other columns oppose it (large negative half dot): the whole logit lies far below the
+    64-column part, and a starting value taken from that part alone would sit above every logit
+    of the row, so that each tile is left out.  Hinted, unhinted and the fp64 oracle must agree."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    rng = np.random.default_rng(61)
+    n = m = 640
+    eps = 0.02
+    x = rng.standard_normal((n, d))
+    x[:, :64] *= 1.6 / np.linalg.norm(x[:, :64], axis=1, keepdims=True)
+    x[:, 64:] *= 0.6 / np.linalg.norm(x[:, 64:], axis=1, keepdims=True)
+    x = x.astype(np.float32)
+    y = np.concatenate([x[:, :64], -3.0 * x[:, 64:]], axis=1)
+    y = (y + 0.01 * rng.standard_normal((m, d))).astype(np.float32)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    la, lb = np.log(a), np.log(b)
+    # potentials that take the key norms out of the logits: what is left is 2 x.y / eps
+    f = (0.02 * rng.standard_normal(n)).astype(np.float32)
+    g = ((y.astype(np.float64) ** 2).sum(1) + 0.02 * rng.standard_normal(m)).astype(np.float32)
+    gh = g - (y.astype(np.float64) ** 2).sum(1)
+    # the half dot of the hinted key exceeds every whole logit of its row by more than 2^40
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    logits = (2.0 * x64 @ y64.T + gh[None, :]) / eps + lb[None, :]
+    half = (2.0 * (x64[:, :64] * y64[:, :64]).sum(1) + gh) / eps + lb
+    assert ((half - logits.max(1)) * np.log2(np.e)).min() > 40.0
+    wx, wy = oracle.grad_barycentric(x, y, a, b, f, g, eps)
+    X, Y, A, B, F, G = dev(x, y, a, b, f, g)
+    plain = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False)
+    own = torch.arange(n, dtype=torch.int32, device="cuda")
+    gx, gy = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False, _seed_keys=(own, own))
+    assert rel_err(gx, wx) < RTOL and rel_err(gy, wy) < RTOL
+    assert rel_err(gx, plain[0].cpu().numpy()) < RTOL and rel_err(gy, plain[1].cpu().numpy()) < RTOL
+
+
+def test_key_hints_that_name_masked_keys():
+    """Hints may name keys that are masked out (potential -inf: bias at the finite stand-in for
+    -inf) or that carry no weight (log-weight floor -100000): such a key says nothing about its
+    row's largest logit, and the result must not depend on it."""
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    rng = np.random.default_rng(62)
+    n, m, d, eps = 700, 900, 64, 0.02
+    sc = 0.7 / np.sqrt(d)
+    centres = rng.standard_normal((6, d)) * 2.0
+    x = (sc * (centres[rng.integers(0, 6, n)] + rng.standard_normal((n, d)))).astype(np.float32)
+    y = (sc * (centres[rng.integers(0, 6, m)] + rng.standard_normal((m, d)))).astype(np.float32)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = (rng.random(m) + 0.5).astype(np.float32)
+    dead = rng.choice(m, 40, replace=False)
+    b[dead[:20]] = 0.0                      # no weight
+    b /= b.sum()
+    f = (0.1 * rng.standard_normal(n)).astype(np.float32)
+    g = (0.1 * rng.standard_normal(m)).astype(np.float32)
+    g[dead[20:]] = -np.inf                  # masked by the potential
+    wx, _ = oracle.grad_barycentric(x, y, a, b, f, g, eps)
+    X, Y, A, B, F, G = dev(x, y, a, b, f, g)
+    plain, _ = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False, compute_grad_y=False)
+    assert rel_err(plain, wx) < RTOL
+    kx = rng.integers(0, m, n).astype(np.int32)
+    kx[::2] = dead[rng.integers(0, 40, len(kx[::2]))]   # every other row is hinted at a dead key
+    keys = (torch.from_numpy(kx).cuda(), torch.zeros(m, dtype=torch.int32, device="cuda"))
+    gx, _ = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False, compute_grad_y=False, _seed_keys=keys)
+    assert torch.isfinite(gx).all()
+    assert rel_err(gx, wx) < RTOL and rel_err(gx, plain.cpu().numpy()) < RTOL
+
+
 @pytest.mark.parametrize("n,m,d", SHAPES)
 def test_apply_vec_and_mat(n, m, d):
     from flash_sinkhorn_amd.kernels.apply_flash import (

@@ -140,3 +140,53 @@ def test_tile_skip_leaves_results_unchanged(monkeypatch):
     assert float((g1 - g0).abs().max()) <= 4e-7 * scale
     wf, wg = oracle.symmetric_step(x, y, fh, gh, la, lb, eps, 1.0, 0.5, 1.0, 1.0)
     assert rel_err(f1, wf) < RTOL and rel_err(g1, wg) < RTOL
+
+
+@pytest.mark.parametrize("d", [64, 100])
+def test_tile_skip_leaves_the_products_unchanged(monkeypatch, d):
+    """The product kernels (gradient, plan * matrix, plan * vector) leave out the same far tiles;
+    FS_FLAG_NO_TILE_SKIP (module switch TILE_SKIP = False) makes them compute every one.  On a
+    peaked plan both launches must agree to fp32 rounding, with values of any magnitude."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels.apply_flash import (
+        apply_plan_mat_flashstyle, apply_plan_vec_flashstyle)
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    rng = np.random.default_rng(22)
+    n, m, eps = 2100, 2600, 0.02
+    sc = 0.7 / np.sqrt(d)
+    centres = rng.standard_normal((8, d)) * 2.0
+    x = (sc * (centres[rng.integers(0, 8, n)] + rng.standard_normal((n, d)))).astype(np.float32)
+    y = (sc * (centres[rng.integers(0, 8, m)] + rng.standard_normal((m, d)))).astype(np.float32)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = np.full(m, 1.0 / m, np.float32)
+    la, lb = np.log(a), np.log(b)
+    fh = -(x * x).sum(1).astype(np.float32)
+    gh = -(y * y).sum(1).astype(np.float32)
+    for it in range(3):
+        fh, gh = oracle.symmetric_step(x, y, fh, gh, la, lb, eps, 1.0, 1.0 if it == 0 else 0.5, 1.0, 1.0)
+    fh, gh = fh.astype(np.float32), gh.astype(np.float32)
+    f = (fh + (x * x).sum(1)).astype(np.float32)
+    g = (gh + (y * y).sum(1)).astype(np.float32)
+    V = (rng.standard_normal((m, d)) * 1e6).astype(np.float32)   # values far from order one
+    v = (rng.standard_normal(m) * 1e6).astype(np.float32)
+    X, Y, A, B, F, G, FH, GH, LA, LB, VM, VV = dev(x, y, a, b, f, g, fh, gh, la, lb, V, v)
+
+    def run():
+        gx, gy = grad(X, Y, A, B, F, G, eps=eps, allow_tf32=False)
+        pm = apply_plan_mat_flashstyle(X, Y, FH, GH, LA, LB, VM, eps=eps, axis=1, allow_tf32=False)
+        pv = apply_plan_vec_flashstyle(X, Y, FH, GH, LA, LB, VV, eps=eps, axis=1, allow_tf32=False)
+        return gx, gy, pm, pv
+
+    monkeypatch.setattr(_lib, "TILE_SKIP", True)
+    with_skip = run()
+    monkeypatch.setattr(_lib, "TILE_SKIP", False)
+    without = run()
+    for got, ref in zip(with_skip, without):
+        assert float((got - ref).abs().max()) <= 2e-6 * float(ref.abs().max())
+    wx, wy = oracle.grad_barycentric(x, y, a, b, f, g, eps)
+    assert rel_err(with_skip[0], wx) < RTOL and rel_err(with_skip[1], wy) < RTOL
+    want = oracle.apply_plan_mat(x, y, fh, gh, la, lb, V, eps, axis=1)
+    assert rel_err(with_skip[2], want) < RTOL
+    want = oracle.apply_plan_vec(x, y, fh, gh, la, lb, v, eps, axis=1)
+    assert rel_err(with_skip[3], want) < RTOL
