@@ -12,6 +12,16 @@
 
 #include "flash_sinkhorn_hip.h"
 
+#ifndef FS_SETTLE
+#define FS_SETTLE 256.0f
+#endif
+#ifndef FS_ENTRIES_BELOW
+#define FS_ENTRIES_BELOW 512.0f
+#endif
+#ifndef FS_ENTRY_MARGIN
+#define FS_ENTRY_MARGIN 1024.0f
+#endif
+
 namespace fs {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -160,6 +170,12 @@ constexpr int kSelSkip = kSelMode + 2;  // per-launch slots: units the sparse fo
 constexpr int kSelCumSkipped = 6;       // their running total (u64), part of kSelCumEnded's
 constexpr int kSelWords = kSelSkip + kSelSlots;
 static_assert(kSelWords <= 256, "one workgroup clears the state block");
+// lse_coarse_kernel leaves margin entries behind once a side's largest bias change is below this
+// many base-2 units (lse_sparse_kernel takes over below 256)
+constexpr float kSettleBelow = FS_SETTLE, kUnsettleAbove = 4.0f * FS_SETTLE;
+constexpr float kEntriesBelow = FS_ENTRIES_BELOW;
+// ... for the units that end at the test by at least this many base-2 units
+constexpr float kEntryMargin = FS_ENTRY_MARGIN;
 constexpr unsigned kSelDecideSteps = 3;  // which counted launch of the coarse variant decides
 constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
 
@@ -177,7 +193,7 @@ constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units en
 __device__ __forceinline__ bool margins_settled(const unsigned* st, int side, float lscale) {
   if (st[kSelBump + side] != 0u || st[kSelGen + side] > 255u) return false;
   const float d = __builtin_bit_cast(float, st[kSelDmax + side]) * lscale;
-  return d < (st[kSelMode + side] != 0u ? 1024.0f : 256.0f);  // false when d is not a number
+  return d < (st[kSelMode + side] != 0u ? kUnsettleAbove : kSettleBelow);  // false when d is not a number
 }
 
 __device__ __forceinline__ void margins_commit(unsigned* st, int lane, bool settled) {
@@ -219,6 +235,43 @@ __device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Smallest value over the wavefront (DPP row shifts, then row broadcasts; lane 63 holds it).
+__device__ __forceinline__ float wave_min_f32(float v) {
+  int x = __builtin_bit_cast(int, v);
+#define FS_MIN_STEP(ctrl, rmask, bmask)                                                          \
+  {                                                                                               \
+    const int o = __builtin_amdgcn_update_dpp(x, x, ctrl, rmask, bmask, false);                   \
+    x = __builtin_bit_cast(int, fminf(__builtin_bit_cast(float, x), __builtin_bit_cast(float, o))); \
+  }
+  FS_MIN_STEP(0x111, 0xf, 0xf)  // row_shr:1
+  FS_MIN_STEP(0x112, 0xf, 0xf)  // row_shr:2
+  FS_MIN_STEP(0x114, 0xf, 0xe)  // row_shr:4
+  FS_MIN_STEP(0x118, 0xf, 0xc)  // row_shr:8
+  FS_MIN_STEP(0x142, 0xa, 0xf)  // row_bcast:15
+  FS_MIN_STEP(0x143, 0xc, 0xf)  // row_bcast:31
+#undef FS_MIN_STEP
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 63));
+}
+
+// Carried margins of lse_coarse_kernel / lse_sparse_kernel.  A unit (32 keys x 32 query rows)
+// that ended at the coarse test with margin mg (how far its bound stayed below the point where
+// a logit could matter, the smallest over its rows; negative: the unit went on) gets the entry
+//   mg - wslack + cum2,   cum2 = 2.002 * (sum of the largest key-bias changes of all launches
+//                                         of this generation up to and including this one),
+// rounded down into the upper 24 bits of a word whose low 8 bits name the generation.  Between
+// two launches a logit rises by at most the largest bias change D, and a row's starting value
+// (its logit at the key that held its maximum) lies at most D + wslack below that maximum: the
+// unit ends again for as long as its entry exceeds the cum2 of the launch that asks.  0: no entry.
+__device__ __forceinline__ unsigned margin_entry(float mg, float wslack, float cum2, unsigned gen) {
+  const float v = mg - wslack + cum2;
+  if (!(mg >= 0.f) || !(v > 0.f) || !(v <= 3.0e38f)) return 0u;
+  return (__builtin_bit_cast(unsigned, v) & ~0xFFu) | gen;
+}
+
+__device__ __forceinline__ bool margin_entry_holds(unsigned w, unsigned gen, unsigned cum2_bits) {
+  return (w & 0xFFu) == gen && (int)(w & ~0xFFu) > (int)cum2_bits;
+}
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 

@@ -1,6 +1,7 @@
 // Instantiations and dispatch of the software-pipelined log-sum-exp kernel.
 #include "fs_lse2.hpp"
 #include "fs_lsecoarse.hpp"
+#include "fs_lsesparse.hpp"
 
 #include "fs_dispatch.hpp"
 
@@ -60,10 +61,10 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
 // tile test (two blocks of 32 query rows per wavefront: the launch must be planned with rb = 2)
 template <int DP>
 static int launch_coarse_dp(const LaunchArgs& a, int blocks, hipStream_t st) {
-  hipLaunchKernelGGL((lse_coarse_kernel<DP, false>), dim3(blocks), dim3(256), 0, st, a);
+  hipLaunchKernelGGL((lse_coarse_kernel<DP>), dim3(blocks), dim3(256), 0, st, a);
   // with carried margins both forms are enqueued; per side, the one the state words name runs
   if (a.side[0].margins != nullptr)
-    hipLaunchKernelGGL((lse_coarse_kernel<DP, true>), dim3(a.blocks_sparse), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((lse_sparse_kernel<DP>), dim3(a.blocks_sparse), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

@@ -192,11 +192,13 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
   }
 }
 
-// SPARSE: the variant for settled potentials.  It carries, per wavefront and sub-tile, by how
-// much the sub-tile's logits stayed below the point where they could matter when they were last
-// tested, and visits only the sub-tiles whose margin the bias changes since then may have used
-// up: no key tiles in LDS, no barriers, every wavefront on its own (see the second main loop).
-template <int DP, bool SPARSE>
+// With carried margins (Side::margins) this kernel is the form for potentials that still move:
+// lse_sparse_kernel, enqueued behind it, runs instead once they have settled (the state words
+// say which of the two runs for a side; the other's workgroups return at once).  In its last
+// launches before that switch (largest bias change below 1024 base-2 units) this form also
+// leaves margin entries behind for the units that end by at least kEntryMargin, so that the first
+// sparse launch finds a list to work from instead of visiting every unit.
+template <int DP>
 __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs args) {
   static_assert(DP == 16 || DP == 32 || DP == 64, "two-plane rows of at most 64 columns");
   constexpr int RB = 2;                // blocks of 32 query rows per wavefront
@@ -212,48 +214,30 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   static_assert(64 * PPR == JT * PPRH, "the 64 sampled two-plane rows fill one tile buffer");
   constexpr int NBUF = 4;              // ring of key tiles in LDS: tile t+3 is requested during tile t
 
-  __shared__ __attribute__((aligned(16))) unsigned lds_k[SPARSE ? 1 : NBUF][SPARSE ? 4 : JT * ROWH];
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[NBUF][JT * ROWH];
   // per 64 keys of a tile: eight copies of a_j (fp16) per key, b_j - 2^18 a_j per key, bmax of
   // the two sub-tiles
-  __shared__ __attribute__((aligned(16))) unsigned lds_aux[SPARSE ? 1 : NBUF][SPARSE ? 4 : NREC * kAuxWords];
-  // sparse form: per wavefront, which sub-tiles it visits (bit 2 k of word g: sub-tile 32 g + k)
-  constexpr int kActWords = 64;
-  __shared__ unsigned long long lds_act[SPARSE ? 4 : 1][SPARSE ? kActWords : 1];
-  __shared__ unsigned lds_cnt[4];  // sparse form: the workgroup's unit counts, wavefronts done
+  __shared__ __attribute__((aligned(16))) unsigned lds_aux[NBUF][NREC * kAuxWords];
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
 
   int bid = blockIdx.x;
-  const int blocks0 = SPARSE ? args.blocks0_sparse : args.blocks0;
-  const bool second = bid >= blocks0;
-  if (second) bid -= blocks0;
+  const bool second = bid >= args.blocks0;
+  if (second) bid -= args.blocks0;
   const Side& sd = second ? args.side[1] : args.side[0];
-  // With carried margins both forms of this kernel are enqueued, and the state words say which
-  // one runs for a side.
+  // With carried margins both forms are enqueued, and the state words say which one runs for a
+  // side: this one while the potentials still move.
+  bool write_entries = false;
   if (sd.margins != nullptr) {
-    const bool settled = margins_settled(
-        args.sel, sd.ps_q, sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]));
-    if (settled != SPARSE) return;
+    const float ls = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
+    if (margins_settled(args.sel, sd.ps_q, ls)) return;
+    // the switch is near (the change about halves from launch to launch): leave entries behind
+    write_entries = args.sel[kSelBump + sd.ps_q] == 0u && args.sel[kSelGen + sd.ps_q] <= 255u &&
+                    __builtin_bit_cast(float, args.sel[kSelDmax + sd.ps_q]) * ls < kEntriesBelow;
   }
-
-  // a wavefront of the sparse form goes through `group` key chunks in a row (what a launch costs
-  // before its first sub-tile is paid once for all of them) and hands the merge kernel one
-  // partial result and group - 1 empty ones
-  const int group = SPARSE ? sd.sparse_group : 1;
-  const int nsplit = (sd.splits + group - 1) / group;
-  if constexpr (SPARSE) {
-    // Workgroups go to the eight XCDs in turn, and each XCD has its own L2: the workgroups of one
-    // XCD take a contiguous run of (key range, row group) pairs, key range slowest, so that those
-    // in flight together fetch the same keys.  (The side's share of the grid is a multiple of 8.)
-    const int per_xcd = ((sd.igroups * nsplit + 7) / 8);
-    bid = (bid % 8) * per_xcd + bid / 8;
-    if (bid >= sd.igroups * nsplit) return;
-    if (threadIdx.x < 4) lds_cnt[threadIdx.x] = 0u;
-    __syncthreads();  // the only one of this form
-  }
-  const int split = SPARSE ? (bid / sd.igroups) * group : bid % nsplit;
-  const int ig = SPARSE ? bid % sd.igroups : bid / nsplit;
+  const int split = bid % sd.splits;
+  const int ig = bid / sd.splits;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -261,7 +245,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   const int h = lane >> 5;
   const int row0 = (ig * 4 + wave) * (32 * RB);
   const int j_begin = split * sd.chunk;
-  const int j_end = min(sd.nk, j_begin + group * sd.chunk);
+  const int j_end = min(sd.nk, j_begin + sd.chunk);
   const int ntiles = (j_end - j_begin + JT - 1) / JT;
 
   // MFMAs produce raw products of the scaled planes; lscale turns them into base-2 logits
@@ -274,21 +258,12 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = min(row0 + rb * 32 + li, sd.nq - 1);
-    if (SPARSE) {  // from the copy in operand order: whole cache lines per load
-      const unsigned* qt = sd.qtiled + (size_t)(row / 32) * (2 * KK16 * 256) + (h * 32 + row % 32) * 4;
+    const unsigned* qrow = sd.qplanes + (size_t)row * (size_t)ROWW;
 #pragma unroll
-      for (int p = 0; p < 2; ++p)
+    for (int p = 0; p < 2; ++p)
 #pragma unroll
-        for (int kk = 0; kk < KK16; ++kk)
-          xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qt + (p * KK16 + kk) * 256);
-    } else {
-      const unsigned* qrow = sd.qplanes + (size_t)row * (size_t)ROWW;
-#pragma unroll
-      for (int p = 0; p < 2; ++p)
-#pragma unroll
-        for (int kk = 0; kk < KK16; ++kk)
-          xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qrow + p * (DP / 2) + 8 * kk + 4 * h);
-    }
+      for (int kk = 0; kk < KK16; ++kk)
+        xq[rb][p][kk] = *reinterpret_cast<const u32x4*>(qrow + p * (DP / 2) + 8 * kk + 4 * h);
   }
 
   // Bound on the two cross products of a row, in raw units.  With X, Y the scaled matrices
@@ -473,12 +448,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     }
   }
   // a workgroup with a row that has no key yet also samples 64 keys spread over the whole key set
-  // (the sparse form, which runs on settled potentials only, does not sample: a wavefront with
-  // such a row starts it from nothing and visits every sub-tile)
-  bool cold;
-  if constexpr (SPARSE) cold = __builtin_amdgcn_ballot_w64(!have) != 0ull;
-  else cold = __syncthreads_or(have ? 0 : 1) != 0;
-  if (!SPARSE && cold) {
+  const bool cold = __syncthreads_or(have ? 0 : 1) != 0;
+  if (cold) {
     const int stride = sd.nk / 64;  // sampled keys: 0, stride, 2 stride, ...
     if (wave == 0) {
       const int j = lane * stride;
@@ -542,13 +513,33 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    if (SPARSE || !cold || warm[rb] > run_m[rb]) {  // the row's key of the last launch stays until exceeded
+    if (!cold || warm[rb] > run_m[rb]) {  // the row's key of the last launch stays until exceeded
       run_m[rb] = warm[rb];
       best_j[rb] = -1;
     }
     float c = -run_m[rb] * lscale;
     asm volatile("" : "+v"(c));  // the rounded product itself, nothing fused into later uses
     run_c[rb] = c;
+  }
+
+  // margin entries of this wavefront (see margin_entry): entry 2 s + rb for sub-tile s of the chunk
+  // (everything here is the same in all lanes and kept in scalar registers)
+  unsigned* ent = nullptr;
+  unsigned far_entry = 0u;
+  const float far_raw = kEntryMargin * inv_lscale;
+  if (write_entries) {
+    const int wrow = __builtin_amdgcn_readfirstlane(row0 / 64);
+    ent = reinterpret_cast<unsigned*>(sd.margins) +
+          ((size_t)wrow * (size_t)sd.margin_stride + (size_t)(j_begin / 32)) * 2;
+    const float cum2 = 2.002f * (__builtin_bit_cast(float, args.sel[kSelCum + sd.ps_q]) +
+                                 __builtin_bit_cast(float, args.sel[kSelDmax + sd.ps_q]));
+    float sl = 0.f;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) sl = fmaxf(sl, corr[rb] * 0x1p-6f + 2.0f * inv_lscale);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sl = fmaxf(sl, __shfl_xor(sl, o, 64));
+    const float wslack = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, sl)));
+    far_entry = margin_entry(far_raw, wslack, cum2, args.sel[kSelGen + sd.ps_q]);
   }
 
   unsigned n_ended = 0;
@@ -698,6 +689,19 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     const bool full1 = wave_any(mx1 > run_m[1] + lim - corr[1]);
     n_ended += (full0 ? 0u : 1u) + (full1 ? 0u : 1u);
     FS_LC_FENCE();
+    if (write_entries) {
+      // (wave-uniform) a unit that ended by at least kEntryMargin gets an entry that says so:
+      // one more comparison per unit, where the exact margin would take a reduction over the
+      // wavefront (lse_sparse_kernel visits the others once and then knows theirs exactly)
+      const bool far0 = !wave_any(mx0 > run_m[0] + lim - corr[0] - far_raw);
+      const bool far1 = !wave_any(mx1 > run_m[1] + lim - corr[1] - far_raw);
+      if (lane == 0) {
+        unsigned* e = ent + (kbase - j_begin) / 16;  // two entries per 32-key sub-tile
+        e[0] = far0 ? far_entry : 0u;
+        e[1] = far1 ? far_entry : 0u;
+      }
+    }
+    FS_LC_FENCE();
     // the set that sub-tile s+1 was just multiplied from is free until the next step's request
     if (full0 || full1) fetch_full(KH[n], b, js, kbase);
     if (full0) unit_full(t0, KH[n], KL, kbias, 0, kbase);
@@ -705,181 +709,6 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     FS_LC_FENCE();
   };
 
-  unsigned n_skipped = 0;  // units the sparse form did not visit
-  if constexpr (SPARSE) {
-    // ---- carried margins ----
-    // An entry holds (margin at the last test) - (the largest starting slack of the wavefront)
-    // + 2 * (sum of the largest key-bias changes of all launches up to that test), with the
-    // generation in its low 8 bits (value rounded down).  Between two launches a logit rises by
-    // at most the largest bias change D, and a row's starting value (its logit at the key that
-    // held its maximum) falls by at most D below that maximum: a sub-tile that ended with margin
-    // mg ends again as long as mg > 2 * (sum of D since) + slack, i.e. while its entry exceeds
-    // twice the running sum.  That needs every row of the wavefront to start where its last
-    // maximum says (checked against the maximum the merge kernel kept); a wavefront where it does
-    // not hold visits everything and only writes entries.
-    const int side_i = sd.ps_q;
-    const unsigned* st = args.sel;
-    const unsigned gen = st[kSelGen + side_i];
-    const float dnow = __builtin_bit_cast(float, st[kSelDmax + side_i]);
-    const float cum = __builtin_bit_cast(float, st[kSelCum + side_i]) + dnow;
-    const float cum2 = 2.002f * cum;  // not finite when a change was not: nothing is valid then
-    const unsigned cum2_bits = __builtin_bit_cast(unsigned, cum2);
-    const int n_sub = ntiles * NSUB;
-    const int n_groups = (n_sub + 31) / 32;   // 64 entries each
-    const bool fits = n_groups <= kActWords;  // else: everything is visited
-    bool ok = track && !cold && fits;
-    float wslack = 0.f;
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const float sl = corr[rb] * 0x1p-6f + 2.0f * inv_lscale;
-      wslack = fmaxf(wslack, sl);
-      const int row = min(row0 + rb * 32 + li, sd.nq - 1);
-      const float mp = sd.m_prev[row] * inv_lscale;
-      ok = ok && (warm[rb] >= mp - 1.001f * dnow - sl);
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) wslack = fmaxf(wslack, __shfl_xor(wslack, o, 64));
-    const bool usable = __builtin_amdgcn_ballot_w64(ok) == ~0ull;
-    // this wavefront's entries: entry 2 s + rb for sub-tile s (counted from its first key)
-    unsigned* ent = reinterpret_cast<unsigned*>(sd.margins) +
-                    ((size_t)(row0 / 64) * (size_t)sd.margin_stride + (size_t)(j_begin / 32)) * 2;
-    auto entry_valid = [&](unsigned w) {
-      return (w & 0xFFu) == gen && (int)(w & ~0xFFu) > (int)cum2_bits;
-    };
-    // sub-tiles of group g that exist
-    auto group_mask = [&](int g) -> unsigned long long {
-      const int left = n_sub - g * 32;
-      return left >= 32 ? 0x5555555555555555ull : (0x5555555555555555ull & ((1ull << (2 * left)) - 1ull));
-    };
-    // ---- which sub-tiles to visit: all but those whose two entries still hold ----
-    if (usable) {
-      for (int g0 = 0; g0 < n_groups; g0 += 4) {
-        unsigned w[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) w[u] = ent[min((g0 + u) * 64 + lane, 2 * n_sub - 1)];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int g = g0 + u;
-          const unsigned long long v =
-              __builtin_amdgcn_ballot_w64(g * 64 + lane < 2 * n_sub && entry_valid(w[u]));
-          if (g < n_groups && lane == 0) lds_act[wave][g] = ~(v & (v >> 1)) & group_mask(g);
-        }
-      }
-    }
-    int g_it = 0;
-    unsigned long long m_it = 0ull;
-    int base_it = 0;
-    // the next sub-tile to visit, or -1
-    auto next = [&]() -> int {
-      while (m_it == 0ull) {
-        if (g_it >= n_groups) return -1;
-        if (usable) {
-          const unsigned long long m = lds_act[wave][g_it];
-          const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)m);
-          const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(m >> 32));
-          m_it = ((unsigned long long)hi << 32) | lo;
-        } else {
-          m_it = group_mask(g_it);
-        }
-        base_it = g_it * 32;
-        ++g_it;
-      }
-      const int bit = __builtin_ctzll(m_it);
-      m_it &= m_it - 1ull;
-      return base_it + (bit >> 1);
-    };
-    auto set_entry = [&](int e, unsigned w) {  // e, w wave-uniform
-      if (lane == 0) ent[e] = w;
-    };
-    // smallest value over the wavefront (DPP row shifts, then row broadcasts; lane 63 holds it)
-    auto wave_min = [&](float v) -> float {
-      int x = __builtin_bit_cast(int, v);
-#define FS_LC_MIN_STEP(ctrl, rmask, bmask)                                                    \
-  {                                                                                           \
-    const int o = __builtin_amdgcn_update_dpp(x, x, ctrl, rmask, bmask, false);                 \
-    x = __builtin_bit_cast(int, fminf(__builtin_bit_cast(float, x), __builtin_bit_cast(float, o))); \
-  }
-      FS_LC_MIN_STEP(0x111, 0xf, 0xf)  // row_shr:1
-      FS_LC_MIN_STEP(0x112, 0xf, 0xf)  // row_shr:2
-      FS_LC_MIN_STEP(0x114, 0xf, 0xe)  // row_shr:4
-      FS_LC_MIN_STEP(0x118, 0xf, 0xc)  // row_shr:8
-      FS_LC_MIN_STEP(0x142, 0xa, 0xf)  // row_bcast:15
-      FS_LC_MIN_STEP(0x143, 0xc, 0xf)  // row_bcast:31
-#undef FS_LC_MIN_STEP
-      return __builtin_bit_cast(float, __builtin_amdgcn_readlane(x, 63));
-    };
-    auto new_entry = [&](float mg) -> unsigned {  // mg < 0: the unit went on
-      const float v = mg - wslack + cum2;
-      if (!(mg >= 0.f) || !(v > 0.f) || !(v <= 3.0e38f)) return 0u;
-      return (__builtin_bit_cast(unsigned, v) & ~0xFFu) | gen;
-    };
-
-    // Operands of a visited sub-tile come straight from global memory (key planes and bias
-    // records are L2 residents), NSET sub-tiles ahead; the slots of a wavefront that has run out
-    // of sub-tiles reload its first one, so that every pass through the loop issues the same loads.
-    // (Nearly every sub-tile that is visited holds a unit that goes on: the lo plane and the
-    // per-key biases come with the set.)
-    constexpr int NSET = 3;
-    u32x4 SH[NSET][KK16], SL[NSET][KK16], SA[NSET];
-    float SB[NSET], SK[NSET];
-    int SS[NSET];
-    auto load_set = [&](u32x4 (&hi)[KK16], u32x4 (&lo)[KK16], u32x4& ka, float& bm, float& kb, int s2) {
-      const int sc = max(s2, 0);
-      const int kbase = j_begin + 32 * sc;
-      const unsigned* blk = sd.ktiled + (size_t)(kbase / 32) * (2 * KK16 * 256) + lane * 4;
-#pragma unroll
-      for (int kk = 0; kk < KK16; ++kk) hi[kk] = *reinterpret_cast<const u32x4*>(blk + kk * 256);
-      const unsigned* rec = sd.key_aux + (size_t)(kbase / 64) * kAuxWords;
-      ka = *reinterpret_cast<const u32x4*>(rec + kAuxA + ((sc & 1) * 32 + li) * 4);
-      bm = __builtin_bit_cast(float, rec[kAuxMax + (sc & 1)]);
-#pragma unroll
-      for (int kk = 0; kk < KK16; ++kk) lo[kk] = *reinterpret_cast<const u32x4*>(blk + (KK16 + kk) * 256);
-      kb = __builtin_bit_cast(float, rec[kAuxB + (sc & 1) * 32 + li]);
-    };
-    auto visit = [&](const u32x4 (&hi)[KK16], const u32x4 (&lo)[KK16], const u32x4& ka, float bm,
-                     float kb, int s2) {
-      const int kbase = j_begin + 32 * s2;
-      const float lim = skip_below - bm;
-      f32x16 z;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) z[r] = 0.f;
-      H[0] = mfma16(ka, QC, z);
-      H[1] = mfma16(ka, QC, z);
-#pragma unroll
-      for (int kk = 0; kk < KK16; ++kk) {
-        H[0] = mfma16(hi[kk], xq[0][0][kk], H[0]);
-        H[1] = mfma16(hi[kk], xq[1][0][kk], H[1]);
-      }
-      const float thr0 = run_m[0] + lim - corr[0], thr1 = run_m[1] + lim - corr[1];
-      const float mx0 = max16(H[0]), mx1 = max16(H[1]);
-      const bool full0 = wave_any(mx0 > thr0), full1 = wave_any(mx1 > thr1);
-      n_ended += (full0 ? 0u : 1u) + (full1 ? 0u : 1u);
-      const float mg0 = full0 ? -1.0f : wave_min(thr0 - mx0);
-      const float mg1 = full1 ? -1.0f : wave_min(thr1 - mx1);
-      if (full0) unit_full(H[0], hi, lo, kb, 0, kbase);
-      if (full1) unit_full(H[1], hi, lo, kb, 1, kbase);
-      set_entry(2 * s2, new_entry(mg0));
-      set_entry(2 * s2 + 1, new_entry(mg1));
-    };
-#pragma unroll
-    for (int i = 0; i < NSET; ++i) {
-      SS[i] = next();
-      load_set(SH[i], SL[i], SA[i], SB[i], SK[i], SS[i]);
-    }
-    int n_visited = 0;
-    while (SS[0] >= 0) {
-#pragma unroll
-      for (int i = 0; i < NSET; ++i) {
-        if (SS[i] >= 0) {
-          visit(SH[i], SL[i], SA[i], SB[i], SK[i], SS[i]);
-          ++n_visited;
-        }
-        SS[i] = SS[i] >= 0 ? next() : -1;
-        load_set(SH[i], SL[i], SA[i], SB[i], SK[i], SS[i]);
-      }
-    }
-    n_skipped = (unsigned)((n_sub - n_visited) * RB);
-  } else {
   // ---- prologue: tiles 0 and 1 published, tiles 2 and 3 on their way; hi*hi of sub-tile 0 ----
   issue_aux(0);
   issue_tile(0);
@@ -916,28 +745,13 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     step(std::integral_constant<int, 0>{}, b, 2, nb, 0, kb + 64);
     step(std::integral_constant<int, 1>{}, b, 3, nb, 1, kb + 96);
   }
-  }
-  if constexpr (!SPARSE) wait_all();  // tiles fetched past the chunk: let them land before the workgroup ends
+  wait_all();  // tiles fetched past the chunk: let them land before the workgroup ends
 
   // unit counts of this wavefront for the variant choice on the device; a workgroup that had
   // to sample its starting values says nothing about the launches that follow
   if (args.sel != nullptr && lane == 0 && ntiles > 0) {
     const int slot = blockIdx.x % kSelSlots;
-    const bool counts = !(track && cold);
-    if constexpr (SPARSE) {
-      // the wavefronts of a workgroup end at different times: they add up in LDS, and the last
-      // one out hands the workgroup's counts to the state words (a quarter of the atomics)
-      if (counts) {
-        atomicAdd(&lds_cnt[0], n_ended + n_skipped);
-        atomicAdd(&lds_cnt[1], n_skipped);
-        atomicAdd(&lds_cnt[2], (unsigned)(ntiles * NSUB * RB));
-      }
-      if (atomicAdd(&lds_cnt[3], 1u) == 3u && lds_cnt[2] != 0u) {
-        atomicAdd(&args.sel[kSelEnded + slot], lds_cnt[0]);
-        atomicAdd(&args.sel[kSelSkip + slot], lds_cnt[1]);
-        atomicAdd(&args.sel[kSelUnits + slot], lds_cnt[2]);
-      }
-    } else if (counts) {
+    if (!(track && cold)) {
       atomicAdd(&args.sel[kSelEnded + slot], n_ended);
       atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
     }
@@ -959,13 +773,6 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
         const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
         *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
         if (sd.part_best != nullptr) sd.part_best[pr] = bj;
-        if constexpr (SPARSE) {  // the other chunks of the group: nothing to merge
-          for (int c = 1; c < group && split + c < sd.splits; ++c) {
-            const size_t pe = (size_t)(split + c) * (size_t)sd.nq + (size_t)row;
-            *reinterpret_cast<float2*>(&sd.part_ms[2 * pe]) = make_float2(-3.0e38f, 0.f);
-            if (sd.part_best != nullptr) sd.part_best[pe] = -1;
-          }
-        }
       }
     }
   }
