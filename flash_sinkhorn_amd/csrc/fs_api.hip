@@ -203,6 +203,7 @@ struct PlaneSet {
   size_t off[2];
   size_t aux_off, end;
   size_t margin_off, margin_slot;  // two slots of carried margins behind the aux block (0: none)
+  size_t queue_off;                // behind them: the work queues of lse_sparse_kernel
   int margin_stride;               // sub-tiles per wavefront row of a slot
 };
 
@@ -239,12 +240,24 @@ size_t margin_slot_bytes(int64_t max_rows, const LseConfig& c) {
   return b <= ((size_t)128 << 20) ? b : 0;
 }
 
+// Everything behind the aux block that belongs to the carried margins: the two slots and the
+// work queues of lse_sparse_kernel.
+// Piece counts of lse_sparse_kernel for one side of a launch: one byte per 64-row group and key
+// range (at most 64 ranges).
+size_t npieces_bytes(int64_t max_rows) { return ((size_t)ceil_div(max_rows, 256) * 4 * 64 + 15) & ~(size_t)15; }
+
+size_t margin_region_bytes(int64_t max_rows, const LseConfig& c) {
+  const size_t slot = margin_slot_bytes(max_rows, c);
+  return slot > 0 ? 2 * slot + kQueueBytes + 2 * npieces_bytes(max_rows) : 0;
+}
+
 // Distinct (pointer, rows) operands among up to four candidates, in canonical order.
 int make_plane_set(const float* const* ptrs, const int* rows, int count, const LseConfig& c,
                    PlaneSet& ps) {
   ps.n = 0;
   ps.aux_off = ps.end = 0;
   ps.margin_off = ps.margin_slot = 0;
+  ps.queue_off = 0;
   ps.margin_stride = 0;
   if (c.prec == 0) return FS_OK;
   for (int k = 0; k < count; ++k) {
@@ -272,7 +285,8 @@ int make_plane_set(const float* const* ptrs, const int* rows, int count, const L
   ps.margin_off = ps.end;
   ps.margin_slot = ps.n > 0 ? margin_slot_bytes(max_rows, c) : 0;
   ps.margin_stride = margin_stride_for(max_rows);
-  ps.end += 2 * ps.margin_slot;
+  ps.queue_off = ps.end + 2 * ps.margin_slot;
+  ps.end += ps.n > 0 ? margin_region_bytes(max_rows, c) : 0;
   return FS_OK;
 }
 
@@ -792,7 +806,7 @@ size_t pt_ws_bytes(int mode, int64_t n, int64_t m, int64_t d, bool both, bool ei
   LseConfig c;
   c.gemm = false; c.prec = 3; c.dp = dpk; c.np = 2;
   const size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes +
-                        2 * margin_slot_bytes(std::max(n, m), c);  // the whole plane set
+                        margin_region_bytes(std::max(n, m), c);  // the whole plane set
   auto side = [&](int64_t nq, int64_t nk) {
     size_t b = 0;
     for (int rb = 1; rb <= 2; ++rb)
@@ -913,6 +927,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
     sd.part_best = nullptr;
     sd.key_aux = nullptr;
     sd.margins = nullptr;
+    sd.npieces = nullptr;
     sd.seed = nullptr;
     sd.sparse_group = 1;
     sd.ktiled = sd.qtiled = nullptr;
@@ -950,6 +965,8 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
         sd.sparse_group = sparse_group[s];
         sd.ktiled = tiled_of(ps, cfg, ws, sd.k, sd.nk);
         sd.qtiled = tiled_of(ps, cfg, ws, sd.q, sd.nq);
+        sd.npieces = reinterpret_cast<unsigned char*>(static_cast<char*>(ws) + ps.queue_off + kQueueBytes) +
+                     (size_t)s * npieces_bytes(std::max(ps.rows[0], ps.n > 1 ? ps.rows[1] : 0));
         sd.m_prev = row_array_of(ps, cfg, ws, sd.q, sd.nq, 1);
         sd.bias_prev = row_array_of(ps, cfg, ws, sd.k, sd.nk, 2);
         // what the margins depend on: the pairing of matrices, the scale of the dot products
@@ -967,12 +984,11 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   }
   if (nsides == 1) a.side[1] = a.side[0];
   a.blocks0 = blocks[0];
-  a.blocks0_sparse = a.blocks_sparse = 0;
-  for (int s = 0; s < nsides; ++s) {
-    const int b = ceil_div(plans[s].igroups * ceil_div(plans[s].splits, sparse_group[s]), 8) * 8;
-    if (s == 0) a.blocks0_sparse = b;
-    a.blocks_sparse += b;
-  }
+  // lse_sparse_kernel: wavefronts that stay and take (row group, key range) items from queues,
+  // two workgroups per CU
+  a.sparse_sides = nsides;
+  a.blocks_sparse = kSparseBlocks;
+  a.queue = margins ? reinterpret_cast<unsigned*>(static_cast<char*>(ws) + ps.queue_off) : nullptr;
   a.vec_ok = vec_ok ? 1 : 0;
   a.nss = fam.nss;
   const int total = blocks[0] + blocks[1];
@@ -1132,7 +1148,7 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
     LseConfig c;
     c.gemm = false; c.prec = 3; c.dp = std::max(dp, 16); c.np = 2;
     planes = plane_bytes(n, c) + plane_bytes(m, c) + 64 + kPlaneAuxBytes +
-             2 * margin_slot_bytes(std::max(n, m), c);
+             margin_region_bytes(std::max(n, m), c);
   }
   if (mode == kLse && !fam.sliced) planes += coarse_aux_bytes(n) + coarse_aux_bytes(m);
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;

@@ -124,6 +124,9 @@ struct Side {
   float* m_prev;
   float* bias_prev;
   float* seed;          // per query row: where this launch's running maximum starts (raw units)
+  // lse_sparse_kernel: per (64-row group, key range) how many of the range's partial results it
+  // wrote (the merge kernel reads only those); index row group * ranges + range
+  unsigned char* npieces;
   float* part_o;        // [splits, nq, DP] partial O when splits > 1 (MAT kinds) or [splits,nq] (VEC)
   Epilogue ep;
 };
@@ -145,8 +148,19 @@ struct LaunchArgs {
   unsigned sel_want;
   int sel_pred;  // 0: the launch runs whatever the state says (it still counts into it)
   unsigned tag[2];  // per side: what the carried margins depend on (operands, scales, coefficients)
-  int blocks0_sparse, blocks_sparse;  // grid of the sparse form of lse_coarse_kernel: side 0, both sides
+  // lse_sparse_kernel: its grid, how many sides it serves, and its work queues (kQueueWords
+  // words per side and XCD, zeroed by coarse_bias_kernel before every launch)
+  int blocks_sparse, sparse_sides;
+  unsigned* queue;
 };
+
+// Work queue of lse_sparse_kernel for one (side, XCD): word 0 counts the base items handed out,
+// word 16 the remainders pushed, word 32 the remainders popped (one cache line each); from word
+// 64 on, kQueueSlots 64-bit slots for the remainders (0: empty, all ones: taken).
+constexpr int kQueueBase = 0, kQueueTail = 16, kQueueHead = 32, kQueueSlot0 = 64, kQueueSlots = 224;
+constexpr int kQueueWords = kQueueSlot0 + 2 * kQueueSlots;
+constexpr size_t kQueueBytes = (size_t)2 * 8 * kQueueWords * 4;
+constexpr int kSparseBlocks = 512;
 
 // Record of coarse_bias_kernel per 64 keys: eight fp16 copies of a_j per key (4 words each), then
 // b_j - 2^18 a_j per key, then the largest bias of each 32-key sub-tile in the first two of 64
@@ -163,12 +177,20 @@ constexpr int kSelSlots = 64, kSelEnded = 8, kSelUnits = kSelEnded + kSelSlots;
 // running sum of the key-bias changes (float), this launch's largest
 // change (float bits, by atomic max), the tag the margins were taken under, their generation
 // (1..255; 0 never valid), and whether this launch started a generation
-constexpr int kSelCum = kSelUnits + kSelSlots, kSelDmax = kSelCum + 2, kSelTag = kSelDmax + 2;
+constexpr int kSelCum = kSelUnits + kSelSlots, kSelTag = kSelCum + 2;
 constexpr int kSelGen = kSelTag + 2, kSelBump = kSelGen + 2;
 constexpr int kSelMode = kSelBump + 2;  // likewise: the last launch ran in the sparse form
 constexpr int kSelSkip = kSelMode + 2;  // per-launch slots: units the sparse form did not visit
 constexpr int kSelCumSkipped = 6;       // their running total (u64), part of kSelCumEnded's
-constexpr int kSelWords = kSelSkip + kSelSlots;
+// likewise (per matrix in the role of the query rows): which kernel wrote the partial results of
+// the launch under way (0: lse2_kernel, 1: lse_coarse_kernel, 2: lse_sparse_kernel), for the merge
+constexpr int kSelForm = kSelSkip + kSelSlots;
+// this launch's largest key-bias change per matrix in the role of the query rows: kDmaxSlots words
+// each (float bits, by atomic max; the wavefronts of coarse_bias_kernel spread over the slots, or
+// a thousand atomics on one word would take longer than the rest of that kernel)
+constexpr int kDmaxSlots = 16;
+constexpr int kSelDmax = kSelForm + 2;
+constexpr int kSelWords = kSelDmax + 2 * kDmaxSlots;
 static_assert(kSelWords <= 256, "one workgroup clears the state block");
 // lse_coarse_kernel leaves margin entries behind once a side's largest bias change is below this
 // many base-2 units (lse_sparse_kernel takes over below 256)
@@ -190,29 +212,49 @@ constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units en
 // are larger), and on until it is above 1024 again; the pipelined one before, and when a
 // generation starts.
 // lscale: base-2 units per raw unit.
+// The launch's largest key-bias change for a side (raw units): the largest of its slots (bit
+// patterns of non-negative floats, or of +inf, order like unsigned integers).
+__device__ __forceinline__ float side_dmax(const unsigned* st, int side) {
+  unsigned m = 0u;
+#pragma unroll
+  for (int i = 0; i < kDmaxSlots; ++i) m = max(m, st[kSelDmax + side * kDmaxSlots + i]);
+  return __builtin_bit_cast(float, m);
+}
+
 __device__ __forceinline__ bool margins_settled(const unsigned* st, int side, float lscale) {
   if (st[kSelBump + side] != 0u || st[kSelGen + side] > 255u) return false;
-  const float d = __builtin_bit_cast(float, st[kSelDmax + side]) * lscale;
+  const float d = side_dmax(st, side) * lscale;
   return d < (st[kSelMode + side] != 0u ? kUnsettleAbove : kSettleBelow);  // false when d is not a number
 }
 
-__device__ __forceinline__ void margins_commit(unsigned* st, int lane, bool settled) {
-  {
-    st[kSelMode + lane] = settled ? 1u : 0u;
-    const float cum = st[kSelBump + lane] ? 0.f
-                                          : __builtin_bit_cast(float, st[kSelCum + lane]) +
-                                                __builtin_bit_cast(float, st[kSelDmax + lane]);
-    st[kSelCum + lane] = __builtin_bit_cast(unsigned, cum);
-    st[kSelDmax + lane] = 0u;
-    st[kSelBump + lane] = 0u;
-  }
-}
-
-__device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
-  unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane], k = st[kSelSkip + lane];
-  st[kSelEnded + lane] = 0u;
-  st[kSelUnits + lane] = 0u;
-  st[kSelSkip + lane] = 0u;
+// What the merge kernel does to the state words after a launch, by one wavefront.  Every word is
+// read before any is written (they live in one buffer, and loads placed behind stores to it would
+// each wait for their own round trip: the chain used to be the longest thing in the kernel).
+//   * the launch's unit counters join the totals and are cleared; the kSelDecideSteps-th launch
+//     with counts decides, and leaves the coarse variant when too few of its units ended;
+//   * per side with carried margins (`commit_sides` of them, their matrices' roles in
+//     `role`, base-2 units per raw unit in `lscale`): the launch's largest bias change joins the
+//     running sum (or starts it, after a launch that began a generation), and the form that ran
+//     is remembered for the hysteresis of margins_settled.
+__device__ __forceinline__ void state_after_launch(unsigned* st, int lane, int commit_sides,
+                                                   const int (&role)[2], const float (&lscale)[2]) {
+  // ---- loads ----
+  const unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane], k = st[kSelSkip + lane];
+  const unsigned long long* cum64 = reinterpret_cast<const unsigned long long*>(st + kSelCumEnded);
+  const unsigned long long c0 = cum64[0], c1 = cum64[1], c2 = cum64[2];
+  const unsigned seen = st[kSelDecisions];
+  unsigned bump[2] = {0u, 0u}, gen[2] = {0u, 0u}, mode[2] = {0u, 0u}, dmax[2] = {0u, 0u}, cum[2] = {0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (i < commit_sides) {
+      bump[i] = st[kSelBump + role[i]];
+      gen[i] = st[kSelGen + role[i]];
+      mode[i] = st[kSelMode + role[i]];
+      cum[i] = st[kSelCum + role[i]];
+    }
+  // (lanes 0..31: the slots of both roles)
+  unsigned dslot = lane < 2 * kDmaxSlots ? st[kSelDmax + lane] : 0u;
+  // ---- the decision ----
   unsigned long long es = e, us = u, ks = k;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -220,17 +262,44 @@ __device__ __forceinline__ void coarse_decide(unsigned* st, int lane) {
     us += __shfl_xor(us, o, 64);
     ks += __shfl_xor(ks, o, 64);
   }
+#pragma unroll
+  for (int o = kDmaxSlots / 2; o > 0; o >>= 1) dslot = max(dslot, (unsigned)__shfl_xor((int)dslot, o, 64));
+  const unsigned d_role0 = (unsigned)__shfl((int)dslot, 0, 64), d_role1 = (unsigned)__shfl((int)dslot, kDmaxSlots, 64);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (i < commit_sides) dmax[i] = role[i] ? d_role1 : d_role0;
+  st[kSelEnded + lane] = 0u;
+  st[kSelUnits + lane] = 0u;
+  st[kSelSkip + lane] = 0u;
+  // the slots of the roles that are committed below start the next launch at zero
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (i < commit_sides && lane >= role[i] * kDmaxSlots && lane < (role[i] + 1) * kDmaxSlots)
+      st[kSelDmax + lane] = 0u;
   if (lane == 0 && us > 0) {
-    unsigned long long* cum = reinterpret_cast<unsigned long long*>(st + kSelCumEnded);
-    cum[0] += es;
-    cum[1] += us;
-    cum[2] += ks;
-    const unsigned seen = st[kSelDecisions];
+    unsigned long long* out = reinterpret_cast<unsigned long long*>(st + kSelCumEnded);
+    out[0] = c0 + es;
+    out[1] = c1 + us;
+    out[2] = c2 + ks;
     if (seen < kSelDecideSteps) {  // the share of the last of these launches decides
       st[kSelDecisions] = seen + 1u;
       if (seen + 1u == kSelDecideSteps && es * 100ull < us * (unsigned long long)kSelMinPercent)
         st[kSelWord] = 1u;
     }
+  }
+  // ---- carried margins ----
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (i < commit_sides && !(i == 1 && role[1] == role[0])) {
+        const float d = __builtin_bit_cast(float, dmax[i]) * lscale[i];
+        const bool settled = bump[i] == 0u && gen[i] <= 255u &&
+                             d < (mode[i] != 0u ? kUnsettleAbove : kSettleBelow);  // margins_settled
+        st[kSelMode + role[i]] = settled ? 1u : 0u;
+        const float cnew = bump[i] ? 0.f : __builtin_bit_cast(float, cum[i]) + __builtin_bit_cast(float, dmax[i]);
+        st[kSelCum + role[i]] = __builtin_bit_cast(unsigned, cnew);
+        st[kSelBump + role[i]] = 0u;
+      }
   }
 }
 

@@ -230,6 +230,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   const bool second = bid >= args.blocks0;
   if (second) bid -= args.blocks0;
   const Side& sd = second ? args.side[1] : args.side[0];
+  // the merge kernel reads the partial results of a launch with carried margins by the kernel
+  // that wrote them: here, one per key chunk
+  if (sd.margins != nullptr && bid == 0 && threadIdx.x == 0) args.sel[kSelForm + sd.ps_q] = 0u;
   const int d = args.d;
 
   const int split = bid % sd.splits;

@@ -75,6 +75,9 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
                                                          int seed_blocks0, int dp) {
   // variant chosen on the device: nothing reads the records when the plain kernel runs
   if (args.sel_pred && args.sel[kSelWord] != 0u) return;
+  if (args.queue != nullptr)  // lse_sparse_kernel's work queues start empty
+    for (int i = blockIdx.x * 64 + threadIdx.x; i < 2 * 8 * kQueueWords; i += gridDim.x * 64)
+      args.queue[i] = 0u;
   if ((int)blockIdx.x >= tiles_all) {
     int blk = blockIdx.x - tiles_all;
     const bool second_s = blk >= seed_blocks0;
@@ -180,7 +183,8 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
     if (lane == 0) {
       // (most wavefronts find a larger value already there; a stale read only costs an atomic)
       const unsigned dbits = __builtin_bit_cast(unsigned, dch);
-      if (dbits > args.sel[kSelDmax + side]) atomicMax(&args.sel[kSelDmax + side], dbits);
+      unsigned* dslot = &args.sel[kSelDmax + side * kDmaxSlots + (tile & (kDmaxSlots - 1))];
+      if (dbits > *dslot) atomicMax(dslot, dbits);
       if (tile == 0 && args.sel[kSelTag + side] != args.tag[second ? 1 : 0]) {
         args.sel[kSelTag + side] = args.tag[second ? 1 : 0];
         // entries carry the generation in 8 bits and are cleared only with the planes: after 255
@@ -234,7 +238,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     if (margins_settled(args.sel, sd.ps_q, ls)) return;
     // the switch is near (the change about halves from launch to launch): leave entries behind
     write_entries = args.sel[kSelBump + sd.ps_q] == 0u && args.sel[kSelGen + sd.ps_q] <= 255u &&
-                    __builtin_bit_cast(float, args.sel[kSelDmax + sd.ps_q]) * ls < kEntriesBelow;
+                    side_dmax(args.sel, sd.ps_q) * ls < kEntriesBelow;
+    if (bid == 0 && threadIdx.x == 0) args.sel[kSelForm + sd.ps_q] = 1u;  // for the merge kernel
   }
   const int split = bid % sd.splits;
   const int ig = bid / sd.splits;
@@ -532,7 +537,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
     ent = reinterpret_cast<unsigned*>(sd.margins) +
           ((size_t)wrow * (size_t)sd.margin_stride + (size_t)(j_begin / 32)) * 2;
     const float cum2 = 2.002f * (__builtin_bit_cast(float, args.sel[kSelCum + sd.ps_q]) +
-                                 __builtin_bit_cast(float, args.sel[kSelDmax + sd.ps_q]));
+                                 side_dmax(args.sel, sd.ps_q));
     float sl = 0.f;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) sl = fmaxf(sl, corr[rb] * 0x1p-6f + 2.0f * inv_lscale);

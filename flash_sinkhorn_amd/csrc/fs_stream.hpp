@@ -470,13 +470,18 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
                                                      int items1) {
   if constexpr (!HAS_O) {  // the launch that follows both variants of a device-chosen step
     if (args.sel != nullptr && blockIdx.x == 0 && threadIdx.x < 64) {
-      coarse_decide(args.sel, threadIdx.x);
-      // lanes 0 and 1: the sides of this launch (the second one only when it has rows to merge)
-      if (args.side[0].margins != nullptr && (threadIdx.x == 0 || (threadIdx.x == 1 && items1 > 0))) {
-        const Side& ms = args.side[threadIdx.x];
-        const float lscale = ms.qscale / (ms.plane_scale[ms.ps_q] * ms.plane_scale[ms.ps_k]);
-        margins_commit(args.sel, ms.ps_q, margins_settled(args.sel, ms.ps_q, lscale));
-      }
+      // the sides of this launch that carry margins (the second one only when it has rows to merge)
+      int role[2] = {0, 0};
+      float ls[2] = {0.f, 0.f};
+      const int commit_sides = args.side[0].margins == nullptr ? 0 : (items1 > 0 ? 2 : 1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if (i < commit_sides) {
+          const Side& ms = args.side[i];
+          role[i] = ms.ps_q;
+          ls[i] = ms.qscale / (ms.plane_scale[ms.ps_q] * ms.plane_scale[ms.ps_k]);
+        }
+      state_after_launch(args.sel, threadIdx.x, commit_sides, role, ls);
     }
   }
   int it = blockIdx.x * 256 + threadIdx.x;
@@ -488,12 +493,22 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
   const int row = it / per_row;
   const int col = (it % per_row) * 4;
   if (row >= sd.nq) return;
+  // lse_sparse_kernel wrote this side's partial results: per key range only as many as its
+  // list had pieces (Side::npieces), in the range's first chunks
+  bool by_range = false;
+  if constexpr (!HAS_O)
+    by_range = sd.npieces != nullptr && args.sel != nullptr && args.sel[kSelForm + sd.ps_q] == 2u;
+  const int rgroup = by_range ? sd.sparse_group : 1;
+  const int nranges = by_range ? (sd.splits + rgroup - 1) / rgroup : sd.splits;
+  const unsigned char* np = by_range ? sd.npieces + (size_t)(row / 64) * nranges : nullptr;
   // (loops unrolled so that the loads of several key splits are in flight together: the merge
   // is a chain of memory round trips and nothing else)
   float M = -3.0e38f;
+  if (!by_range) {
 #pragma unroll 8
-  for (int sp = 0; sp < sd.splits; ++sp)
-    M = fmaxf(M, sd.part_ms[2 * ((size_t)sp * sd.nq + row)]);
+    for (int sp = 0; sp < sd.splits; ++sp)
+      M = fmaxf(M, sd.part_ms[2 * ((size_t)sp * sd.nq + row)]);
+  }
   float s = 0.f, o = 0.f;
   float4 O = make_float4(0.f, 0.f, 0.f, 0.f);
   if constexpr (HAS_O) {
@@ -511,8 +526,7 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
     const bool has_o = sd.part_o != nullptr;
     float bm = -3.0e38f;
     int bj = -1;
-#pragma unroll 8
-    for (int sp = 0; sp < sd.splits; ++sp) {
+    auto merge = [&](int sp) {
       const size_t pr = (size_t)sp * sd.nq + row;
       const float2 ms = *reinterpret_cast<const float2*>(&sd.part_ms[2 * pr]);
       const float w = exp2f(ms.x - M);
@@ -525,6 +539,46 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
           bj = j;
         }
       }
+    };
+    if (by_range) {
+      // one pass, eight ranges at a time: the counts, and the first piece of every range (there
+      // always is one), are loads that wait for nothing; further pieces are rare
+      auto merge_online = [&](float2 ms, int j) {
+        if (ms.x > M) {
+          s = s * exp2f(M - ms.x) + ms.y;
+          M = ms.x;
+        } else {
+          s += ms.y * exp2f(ms.x - M);
+        }
+        if (keys && j >= 0 && ms.x > bm) {
+          bm = ms.x;
+          bj = j;
+        }
+      };
+      for (int r0 = 0; r0 < nranges; r0 += 8) {
+        int cnt[8], pj[8];
+        float2 first[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int r = min(r0 + i, nranges - 1);
+          const size_t pr = (size_t)(r * rgroup) * sd.nq + row;
+          cnt[i] = (r0 + i < nranges) ? (int)np[r] : 0;
+          first[i] = *reinterpret_cast<const float2*>(&sd.part_ms[2 * pr]);
+          pj[i] = keys ? sd.part_best[pr] : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (r0 + i < nranges) merge_online(first[i], pj[i]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          for (int p = 1; p < cnt[i]; ++p) {
+            const size_t pr = (size_t)((r0 + i) * rgroup + p) * sd.nq + row;
+            merge_online(*reinterpret_cast<const float2*>(&sd.part_ms[2 * pr]), keys ? sd.part_best[pr] : -1);
+          }
+      }
+    } else {
+#pragma unroll 8
+      for (int sp = 0; sp < sd.splits; ++sp) merge(sp);
     }
     if (keys && bj >= 0) sd.best_key[row] = bj;  // no chunk exceeded the starting value: the old key stays
     if (sd.m_prev != nullptr) sd.m_prev[row] = M;
@@ -535,7 +589,9 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
 // The decision alone, for a step whose launch split no keys (no merge follows).
 template <int T>
 __global__ __launch_bounds__(64) void coarse_decide_kernel(unsigned* state) {
-  coarse_decide(state, threadIdx.x);
+  const int role[2] = {0, 0};
+  const float ls[2] = {0.f, 0.f};
+  state_after_launch(state, threadIdx.x, 0, role, ls);
 }
 
 // kArgmax: merge the partial (largest value, key) pairs of the key splits; equal values keep
