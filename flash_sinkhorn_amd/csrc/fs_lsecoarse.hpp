@@ -530,7 +530,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
   // margin entries of this wavefront (see margin_entry): entry 2 s + rb for sub-tile s of the chunk
   // (everything here is the same in all lanes and kept in scalar registers)
   unsigned* ent = nullptr;
-  unsigned far_entry = 0u;
+  unsigned far_entry = 0u, gen_word = 0u;
   const float far_raw = kEntryMargin * inv_lscale;
   if (write_entries) {
     const int wrow = __builtin_amdgcn_readfirstlane(row0 / 64);
@@ -544,7 +544,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sl = fmaxf(sl, __shfl_xor(sl, o, 64));
     const float wslack = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, sl)));
-    far_entry = margin_entry(far_raw, wslack, cum2, args.sel[kSelGen + sd.ps_q]);
+    gen_word = args.sel[kSelGen + sd.ps_q];
+    far_entry = margin_entry(far_raw, wslack, cum2, gen_word);
   }
 
   unsigned n_ended = 0;
@@ -702,8 +703,9 @@ __global__ __launch_bounds__(256, 2) void lse_coarse_kernel(const LaunchArgs arg
       const bool far1 = !wave_any(mx1 > run_m[1] + lim - corr[1] - far_raw);
       if (lane == 0) {
         unsigned* e = ent + (kbase - j_begin) / 16;  // two entries per 32-key sub-tile
-        e[0] = far0 ? far_entry : 0u;
-        e[1] = far1 ? far_entry : 0u;
+        // (a unit that went on is marked as such: the generation alone, no margin)
+        e[0] = far0 ? far_entry : (full0 ? gen_word : 0u);
+        e[1] = far1 ? far_entry : (full1 ? gen_word : 0u);
       }
     }
     FS_LC_FENCE();

@@ -57,6 +57,8 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
   constexpr unsigned long long kTaken = ~0ull;
 
   __shared__ unsigned long long lds_act[4][kActWords];
+  // and which of the listed units went on to the soft-max when they were last visited
+  __shared__ unsigned long long lds_full[4][kActWords];
   __shared__ unsigned lds_cnt[4];  // the workgroup's unit counts, wavefronts done
 
   // the device chose the plain kernel: nothing to do
@@ -251,21 +253,32 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
           const int g = g_first + u;
           const unsigned long long v = __builtin_amdgcn_ballot_w64(
               g * 64 + lane < 2 * n_sub && margin_entry_holds(ew[u], gen, cum2_bits));
-          if (g < n_groups && lane == 0)
+          const unsigned long long f = __builtin_amdgcn_ballot_w64(ew[u] == gen);
+          if (g < n_groups && lane == 0) {
             lds_act[wave][g] = listed ? (~(v & usable_bits) & group_mask(g)) : group_mask(g);
+            lds_full[wave][g] = f;
+          }
         }
         for (int g = g_first + kUpFront; g < n_groups; ++g) {  // longer ranges: the rest of the list
           const unsigned w = ent[min(g * 64 + lane, 2 * n_sub - 1)];
           const unsigned long long v = __builtin_amdgcn_ballot_w64(
               g * 64 + lane < 2 * n_sub && margin_entry_holds(w, gen, cum2_bits));
-          if (lane == 0) lds_act[wave][g] = listed ? (~(v & usable_bits) & group_mask(g)) : group_mask(g);
+          const unsigned long long f = __builtin_amdgcn_ballot_w64(w == gen);
+          if (lane == 0) {
+            lds_act[wave][g] = listed ? (~(v & usable_bits) & group_mask(g)) : group_mask(g);
+            lds_full[wave][g] = f;
+          }
         }
       }
-      auto list_word = [&](int g) -> unsigned long long {
-        if (!fits) return group_mask(g);
-        const unsigned long long m = lds_act[wave][g];
+      auto uniform64 = [&](unsigned long long m) -> unsigned long long {
         const unsigned lo32 = (unsigned)uniform((int)(unsigned)m), hi32 = (unsigned)uniform((int)(unsigned)(m >> 32));
         return ((unsigned long long)hi32 << 32) | lo32;
+      };
+      auto list_word = [&](int g) -> unsigned long long {
+        return fits ? uniform64(lds_act[wave][g]) : group_mask(g);
+      };
+      auto full_word = [&](int g) -> unsigned long long {
+        return fits ? uniform64(lds_full[wave][g]) : 0ull;
       };
 
       // run_m: running maximum in raw units; run_c = -run_m * lscale as rounded once, the offset
@@ -285,22 +298,25 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
       unsigned n_ended = 0, n_visited = 0;
 
       // One listed unit: row block rb against the sub-tile whose operands are (hi, lo, ka, bm, kb).
+      // was_full: the unit went on to the soft-max when it was last visited, and will again: no
+      // test, the exact logits right away.
       auto unit = [&](const u32x4 (&hi)[KK16], const u32x4 (&lo)[KK16], const u32x4& ka, float bm,
-                      float kb, int rb, int kbase) -> unsigned {
-        f32x16 z;
+                      float kb, int rb, int kbase, bool was_full) -> unsigned {
+        f32x16 L;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        f32x16 H = mfma16(ka, QC, z);  // 2^18 a_j on every query column
+        for (int r = 0; r < 16; ++r) L[r] = 0.f;
+        L = mfma16(ka, QC, L);  // 2^18 a_j on every query column
 #pragma unroll
-        for (int kk = 0; kk < KK16; ++kk) H = mfma16(hi[kk], xq[rb][0][kk], H);
-        const float thr = run_m[rb] + (skip_below - bm) - corr[rb];
-        const float mxh = max16(H);
-        if (!wave_any(mxh > thr)) {  // ends again: by how much
-          ++n_ended;
-          return margin_entry(wave_min_f32(thr - mxh), wslack, cum2, gen);
+        for (int kk = 0; kk < KK16; ++kk) L = mfma16(hi[kk], xq[rb][0][kk], L);
+        if (!was_full) {
+          const float thr = run_m[rb] + (skip_below - bm) - corr[rb];
+          const float mxh = max16(L);
+          if (!wave_any(mxh > thr)) {  // ends again: by how much
+            ++n_ended;
+            return margin_entry(wave_min_f32(thr - mxh), wslack, cum2, gen);
+          }
         }
         // goes on: the two cross products and the exact key bias on top, then the soft-max
-        f32x16 L = H;
 #pragma unroll
         for (int kk = 0; kk < KK16; ++kk) L = mfma16(hi[kk], xq[rb][1][kk], L);
 #pragma unroll
@@ -310,7 +326,14 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
         const float mx = max16(L);  // this lane's 16 keys
         // every logit of the unit more than the 2^40 distance below its row's running maximum:
         // its exponentials would not change the fp32 row sums
-        if (wave_any(mx - run_m[rb] > skip_below)) {
+        if (!wave_any(mx - run_m[rb] > skip_below)) {
+          // The exact logits say so: the unit gets an entry from them (they rise and the rows'
+          // starting values fall like the bounds of the test do; see margin_entry), and is not
+          // visited again while that holds.
+          ++n_ended;
+          return margin_entry(wave_min_f32(run_m[rb] + skip_below - mx), wslack, cum2, gen);
+        }
+        {
           float a = mx, b2 = mx;
           swap_halves(a, b2);
           const float m_new = fmaxf(fmaxf(a, b2), run_m[rb]);
@@ -335,7 +358,7 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
           run_m[rb] = m_new;
           run_c[rb] = cx;
         }
-        return 0u;  // no entry: the unit is visited again next launch
+        return gen;  // no margin: visited again next launch, and then without the test
       };
 
       // Operands of a listed sub-tile come straight from global memory (key planes and bias
@@ -397,15 +420,18 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
         // ---- walk words [g_it, g_stop) ----
         int base_it = 0;
         unsigned long long m_it = 0ull;
+        unsigned long long f_it = 0ull;
+        // (need: bits 0, 1 = the listed units of the sub-tile, bits 2, 3 = which of them went on last time)
         auto next = [&](unsigned& need) -> int {
           while (m_it == 0ull) {
             if (g_it >= g_stop) return -1;
             m_it = list_word(g_it);
+            f_it = full_word(g_it);
             base_it = g_it * 32;
             ++g_it;
           }
           const int k = __builtin_ctzll(m_it) >> 1;
-          need = (unsigned)(m_it >> (2 * k)) & 3u;
+          need = ((unsigned)(m_it >> (2 * k)) & 3u) | (((unsigned)(f_it >> (2 * k)) & 3u) << 2);
           m_it &= ~(3ull << (2 * k));
           return base_it + k;
         };
@@ -421,12 +447,12 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
             if (SS[i] >= 0) {
               const int kbase = j_begin + 32 * SS[i];
               if (SN[i] & 1u) {
-                const unsigned e = unit(SH[i], SL[i], SA[i], SB[i], SK[i], 0, kbase);
+                const unsigned e = unit(SH[i], SL[i], SA[i], SB[i], SK[i], 0, kbase, (SN[i] & 4u) != 0u);
                 if (lane == 0) ent[2 * SS[i]] = e;
                 ++n_visited;
               }
               if (SN[i] & 2u) {
-                const unsigned e = unit(SH[i], SL[i], SA[i], SB[i], SK[i], 1, kbase);
+                const unsigned e = unit(SH[i], SL[i], SA[i], SB[i], SK[i], 1, kbase, (SN[i] & 8u) != 0u);
                 if (lane == 0) ent[2 * SS[i] + 1] = e;
                 ++n_visited;
               }
