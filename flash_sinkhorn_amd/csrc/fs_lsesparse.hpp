@@ -43,7 +43,7 @@
 namespace fs {
 
 #ifndef FS_PIECE
-#define FS_PIECE 32
+#define FS_PIECE 48
 #endif
 constexpr int kPiece = FS_PIECE;  // units after which a long list is cut (at the next 32 sub-tiles)
 
