@@ -97,11 +97,9 @@ __global__ __launch_bounds__(256, 2) void lse_sparse_kernel(const LaunchArgs arg
 
   unsigned tot_ended = 0, tot_skipped = 0, tot_units = 0;  // over all items of this wavefront
 
-  // half of the workgroups start with either side, so that neither side's last items are left
-  // to a few wavefronts
-  const int first_side = (blockIdx.x >> 3) & 1;
-  for (int pass = 0; pass < args.sparse_sides; ++pass) {
-    const int s_idx = args.sparse_sides == 2 ? (first_side ^ pass) : 0;
+  // one side after the other (with half of the workgroups starting on either side, an XCD's L2
+  // had to hold a key range of each matrix at once, and the launch was slower)
+  for (int s_idx = 0; s_idx < args.sparse_sides; ++s_idx) {
     const Side& sd = args.side[s_idx];
     // ---- the state words: does this form run for the side? ----
     const int side_i = sd.ps_q;  // the margins' state goes with the matrix that holds the query rows
