@@ -23,6 +23,7 @@ FS_FLAG_OPERANDS_PREPARED = 16
 FS_FLAG_NO_TILE_SKIP = 32
 FS_FLAG_COARSE_TEST = 64
 FS_FLAG_COARSE_AUTO = 128
+FS_FLAG_START_PLAIN = 256
 # Every call runs on the two-plane fp16 operands (fp32-grade accuracy, the fastest mode here),
 # whatever allow_tf32 says: permission to reduce precision is not an obligation.
 # STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" makes allow_tf32=False
@@ -141,7 +142,8 @@ class PreparedOperands:
     run on the stream current at construction.
     """
 
-    def __init__(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int, self_pair: bool = False):
+    def __init__(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int, self_pair: bool = False,
+                 start_plain: bool = False):
         n, d = x.shape
         m = y.shape[0]
         L = lib()
@@ -159,7 +161,10 @@ class PreparedOperands:
                                                           flag_bits))
         self._keys_at = [(int(L.fs_best_keys_offset(x.data_ptr(), y.data_ptr(), n, m, d, flag_bits, w)),
                           rows) for w, rows in ((0, n), (1, m))]
-        check(L.fs_prepare_operands(x.data_ptr(), y.data_ptr(), n, m, d, flag_bits,
+        # start_plain: with the kernel variant left to the device, the first steps run the plain
+        # kernel (a schedule that begins at a large eps begins on a flat plan)
+        check(L.fs_prepare_operands(x.data_ptr(), y.data_ptr(), n, m, d,
+                                    flag_bits | (FS_FLAG_START_PLAIN if start_plain else 0),
                                     self.ws.data_ptr(), nbytes, stream_of(x)),
               "fs_prepare_operands")
 

@@ -45,7 +45,8 @@ constexpr int kMaxSlicedD = 16384;  // widest supported rows
 constexpr int kSlicedSpan = 1536;   // columns one workgroup of the column-sliced kernels spans
 constexpr int kPlanePadRowsApi = 512;  // must match kPlanePadRows of the plane-splitting kernels
 // after the planes: absmax partials [2][256], plane scales [4] (+4 spare), variant-choice state
-constexpr size_t kPlaneAuxBytes = (2 * 256 + 8 + kSelWords) * sizeof(float);
+// (a multiple of 256 bytes: the margin entries, queues and their 64-bit slots come right behind)
+constexpr size_t kPlaneAuxBytes = ((2 * 256 + 8 + kSelWords) * sizeof(float) + 255) / 256 * 256;
 static_assert(kSelWords <= 256, "the state is cleared by one workgroup");
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
@@ -240,12 +241,13 @@ size_t margin_slot_bytes(int64_t max_rows, const LseConfig& c) {
   return b <= ((size_t)128 << 20) ? b : 0;
 }
 
-// Everything behind the aux block that belongs to the carried margins: the two slots and the
-// work queues of lse_sparse_kernel.
 // Piece counts of lse_sparse_kernel for one side of a launch: one byte per 64-row group and key
 // range (at most 64 ranges).
 size_t npieces_bytes(int64_t max_rows) { return ((size_t)ceil_div(max_rows, 256) * 4 * 64 + 15) & ~(size_t)15; }
 
+// Everything behind the aux block that belongs to the carried margins: the two slots, the work
+// queues of lse_sparse_kernel (64-bit slots: every part is a multiple of 16 bytes) and its piece
+// counts for either side.
 size_t margin_region_bytes(int64_t max_rows, const LseConfig& c) {
   const size_t slot = margin_slot_bytes(max_rows, c);
   return slot > 0 ? 2 * slot + kQueueBytes + 2 * npieces_bytes(max_rows) : 0;
@@ -336,7 +338,7 @@ unsigned* tiled_of(const PlaneSet& ps, const LseConfig& c, void* ws, const float
 // outlive the call (fs_prepare_operands): the carried margins start empty and the second copy
 // in operand order, which only launches on kept planes read, is written too.
 int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws, hipStream_t st,
-                     bool keep = false) {
+                     bool keep = false, bool start_plain = false) {
   if (ps.n == 0) return FS_OK;
   char* base = static_cast<char*>(ws);
   int rc = FS_OK;
@@ -356,7 +358,8 @@ int launch_plane_set(const PlaneSet& ps, const LseConfig& c, int64_t d, void* ws
                                    two ? nullptr : scales + 1, c.gemm ? 1 : 0,
                                    i == 0 ? select_state(ps, ws) : nullptr,
                                    best_keys_of(ps, c, ws, ps.src[i], ps.rows[i]),
-                                   keep ? tiled_of(ps, c, ws, ps.src[i], ps.rows[i]) : nullptr, st);
+                                   keep ? tiled_of(ps, c, ws, ps.src[i], ps.rows[i]) : nullptr, st,
+                                   start_plain ? 1 : 0);
   }
   return rc;
 }
@@ -1175,7 +1178,8 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
   const int rc = make_plane_set(ptrs, rows, 2, cfg, ps);
   if (rc != FS_OK || ps.n == 0) return rc;
   if (ps.end > workspace_bytes || workspace == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
-  return launch_plane_set(ps, cfg, d, workspace, (hipStream_t)stream, true);
+  return launch_plane_set(ps, cfg, d, workspace, (hipStream_t)stream, true,
+                          (flags & FS_FLAG_START_PLAIN) != 0);
 }
 
 size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,

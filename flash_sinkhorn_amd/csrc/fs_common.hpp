@@ -190,7 +190,13 @@ constexpr int kSelForm = kSelSkip + kSelSlots;
 // a thousand atomics on one word would take longer than the rest of that kernel)
 constexpr int kDmaxSlots = 16;
 constexpr int kSelDmax = kSelForm + 2;
-constexpr int kSelWords = kSelDmax + 2 * kDmaxSlots;
+// likewise per role: margin entries of the current generation exist (lse_coarse_kernel left them
+// behind, or lse_sparse_kernel ran); without them the sparse form would visit every unit
+constexpr int kSelHave = kSelDmax + 2 * kDmaxSlots;
+// the share of units the plain kernel left out in the first launch of its current stretch, in
+// 65536ths plus one (0: not taken yet)
+constexpr int kSelBase = kSelHave + 2;
+constexpr int kSelWords = kSelBase + 1;
 static_assert(kSelWords <= 256, "one workgroup clears the state block");
 // lse_coarse_kernel leaves margin entries behind once a side's largest bias change is below this
 // many base-2 units (lse_sparse_kernel takes over below 256)
@@ -200,6 +206,13 @@ constexpr float kEntriesBelow = FS_ENTRIES_BELOW;
 constexpr float kEntryMargin = FS_ENTRY_MARGIN;
 constexpr unsigned kSelDecideSteps = 3;  // which counted launch of the coarse variant decides
 constexpr unsigned kSelMinPercent = 40;  // keep it while this share of units ends at the test
+// Back to it once the plain kernel leaves out the exponentials of a larger share of its units
+// than in its first launch of this stretch, by this many 65536ths (4 %).  The plain kernel finds
+// its running maxima on the way and always leaves out the padding, so its share says little by
+// itself (1 - 2 % on a flat plan, 7 - 20 % where the coarse variant would end 80 %), but its
+// growth does; measured against the stretch's own first launch, a plan that stays as it is
+// never sends the choice back and forth.
+constexpr unsigned kSelBackStep16 = 2621;
 
 // One wavefront: add the launch's counters to the totals and clear them.  Only workgroups whose
 // rows all started from a key of the previous launch count, and the share of ended units climbs
@@ -222,7 +235,7 @@ __device__ __forceinline__ float side_dmax(const unsigned* st, int side) {
 }
 
 __device__ __forceinline__ bool margins_settled(const unsigned* st, int side, float lscale) {
-  if (st[kSelBump + side] != 0u || st[kSelGen + side] > 255u) return false;
+  if (st[kSelBump + side] != 0u || st[kSelGen + side] > 255u || st[kSelHave + side] == 0u) return false;
   const float d = side_dmax(st, side) * lscale;
   return d < (st[kSelMode + side] != 0u ? kUnsettleAbove : kSettleBelow);  // false when d is not a number
 }
@@ -231,7 +244,9 @@ __device__ __forceinline__ bool margins_settled(const unsigned* st, int side, fl
 // read before any is written (they live in one buffer, and loads placed behind stores to it would
 // each wait for their own round trip: the chain used to be the longest thing in the kernel).
 //   * the launch's unit counters join the totals and are cleared; the kSelDecideSteps-th launch
-//     with counts decides, and leaves the coarse variant when too few of its units ended;
+//     of the coarse variant with counts decides, and leaves it when too few of its units ended;
+//     the plain kernel counts the units whose exponentials it left out, and a launch that left
+//     out clearly more than the first of its stretch hands the next one back to the coarse variant;
 //   * per side with carried margins (`commit_sides` of them, their matrices' roles in
 //     `role`, base-2 units per raw unit in `lscale`): the launch's largest bias change joins the
 //     running sum (or starts it, after a launch that began a generation), and the form that ran
@@ -242,8 +257,9 @@ __device__ __forceinline__ void state_after_launch(unsigned* st, int lane, int c
   const unsigned e = st[kSelEnded + lane], u = st[kSelUnits + lane], k = st[kSelSkip + lane];
   const unsigned long long* cum64 = reinterpret_cast<const unsigned long long*>(st + kSelCumEnded);
   const unsigned long long c0 = cum64[0], c1 = cum64[1], c2 = cum64[2];
-  const unsigned seen = st[kSelDecisions];
+  const unsigned seen = st[kSelDecisions], word = st[kSelWord], base = st[kSelBase];
   unsigned bump[2] = {0u, 0u}, gen[2] = {0u, 0u}, mode[2] = {0u, 0u}, dmax[2] = {0u, 0u}, cum[2] = {0u, 0u};
+  unsigned have[2] = {0u, 0u};
 #pragma unroll
   for (int i = 0; i < 2; ++i)
     if (i < commit_sides) {
@@ -251,6 +267,7 @@ __device__ __forceinline__ void state_after_launch(unsigned* st, int lane, int c
       gen[i] = st[kSelGen + role[i]];
       mode[i] = st[kSelMode + role[i]];
       cum[i] = st[kSelCum + role[i]];
+      have[i] = st[kSelHave + role[i]];
     }
   // (lanes 0..31: the slots of both roles)
   unsigned dslot = lane < 2 * kDmaxSlots ? st[kSelDmax + lane] : 0u;
@@ -281,10 +298,25 @@ __device__ __forceinline__ void state_after_launch(unsigned* st, int lane, int c
     out[0] = c0 + es;
     out[1] = c1 + us;
     out[2] = c2 + ks;
-    if (seen < kSelDecideSteps) {  // the share of the last of these launches decides
-      st[kSelDecisions] = seen + 1u;
-      if (seen + 1u == kSelDecideSteps && es * 100ull < us * (unsigned long long)kSelMinPercent)
-        st[kSelWord] = 1u;
+    if (word == 0u) {
+      if (seen < kSelDecideSteps) {  // the share of the last of these launches decides
+        st[kSelDecisions] = seen + 1u;
+        if (seen + 1u == kSelDecideSteps && es * 100ull < us * (unsigned long long)kSelMinPercent) {
+          st[kSelWord] = 1u;
+          st[kSelBase] = 0u;  // the plain kernel's next launch sets the mark for the way back
+        }
+      }
+    } else {
+      const unsigned share16 = (unsigned)((es << 16) / us);
+      if (base == 0u) {
+        st[kSelBase] = share16 + 1u;
+      } else if (share16 >= base - 1u + kSelBackStep16) {
+        // the plain kernel leaves out clearly more than when this stretch began: the plan has
+        // become peaked (eps went down), and the coarse variant gets its launches with counts again
+        st[kSelWord] = 0u;
+        st[kSelDecisions] = 0u;
+        st[kSelBase] = 0u;
+      }
     }
   }
   // ---- carried margins ----
@@ -293,9 +325,13 @@ __device__ __forceinline__ void state_after_launch(unsigned* st, int lane, int c
     for (int i = 0; i < 2; ++i)
       if (i < commit_sides && !(i == 1 && role[1] == role[0])) {
         const float d = __builtin_bit_cast(float, dmax[i]) * lscale[i];
-        const bool settled = bump[i] == 0u && gen[i] <= 255u &&
+        const bool settled = bump[i] == 0u && gen[i] <= 255u && have[i] != 0u &&
                              d < (mode[i] != 0u ? kUnsettleAbove : kSettleBelow);  // margins_settled
         st[kSelMode + role[i]] = settled ? 1u : 0u;
+        // entries of this generation: none after a launch that began one; there once the sparse
+        // form ran or lse_coarse_kernel left some behind (its own condition, see there)
+        const bool wrote = settled || (bump[i] == 0u && gen[i] <= 255u && d < kEntriesBelow);
+        st[kSelHave + role[i]] = bump[i] != 0u ? 0u : ((have[i] != 0u || wrote) ? 1u : 0u);
         const float cnew = bump[i] ? 0.f : __builtin_bit_cast(float, cum[i]) + __builtin_bit_cast(float, dmax[i]);
         st[kSelCum + role[i]] = __builtin_bit_cast(unsigned, cnew);
         st[kSelBump + role[i]] = 0u;

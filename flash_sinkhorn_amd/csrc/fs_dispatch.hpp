@@ -24,7 +24,7 @@ int launch_row_seeds(const LaunchArgs& a, int dp, int nsides, hipStream_t st);
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
                             int chunked, unsigned* clear_state, int* best_keys, unsigned* tiled,
-                            hipStream_t st);
+                            hipStream_t st, int start_plain = 0);
 // GEMM-style LSE kernel for 128 < d <= 1536 on chunked fp16 planes; Side::splits counts
 // partial rows (twice the workgroup-level key splits).
 int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st);  // kLse, kVec, kArgmax

@@ -49,11 +49,11 @@ int launch_fill_zero(unsigned* p, long long n, hipStream_t st) {
 int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, int dp,
                             const float* partial_max, float* scale_out, float* scale_out2,
                             int chunked, unsigned* clear_state, int* best_keys, unsigned* tiled,
-                            hipStream_t st) {
+                            hipStream_t st, int start_plain) {
   const long long items = (long long)(rows + kPlanePadRows) * (dp / 4);
   const int grid = (int)((items + 255) / 256);
   hipLaunchKernelGGL(split_planes_f16_kernel, dim3(grid), dim3(256), 0, st, src, dst, rows, d, dp,
-                     partial_max, scale_out, scale_out2, chunked, clear_state, best_keys, tiled);
+                     partial_max, scale_out, scale_out2, chunked, clear_state, best_keys, tiled, start_plain);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 

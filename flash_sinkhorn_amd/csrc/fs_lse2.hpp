@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     const float* __restrict__ src, unsigned* __restrict__ dst, int rows, int d, int dp,
     const float* __restrict__ partial_max, float* __restrict__ scale_out,
     float* __restrict__ scale_out2, int chunked, unsigned* __restrict__ clear_state,
-    int* __restrict__ best_keys, unsigned* __restrict__ tiled) {
+    int* __restrict__ best_keys, unsigned* __restrict__ tiled, int start_plain) {
   __shared__ float red[4];
   float m = partial_max[threadIdx.x];  // kAbsmaxBlocks == blockDim.x
 #pragma unroll
@@ -122,7 +122,9 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     *scale_out = sc;
     if (scale_out2) *scale_out2 = sc;  // the same matrix plays both roles
   }
-  if (blockIdx.x == 0 && clear_state != nullptr && threadIdx.x < kSelWords) clear_state[threadIdx.x] = 0u;
+  // (start_plain: the variant choice begins with the plain kernel, see FS_FLAG_START_PLAIN)
+  if (blockIdx.x == 0 && clear_state != nullptr && threadIdx.x < kSelWords)
+    clear_state[threadIdx.x] = (threadIdx.x == kSelWord && start_plain) ? 1u : 0u;
 
   const int per_row = dp / 4;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -255,6 +257,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   if constexpr (PREC == kH3) lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = kPlanes ? 1.0f / lscale : 1.0f;
   const float skip_below = args.skip_log2 * inv_lscale;  // in accumulator units
+  unsigned n_left_out = 0;  // units whose exponentials were not computed
 
   // ---- stationary query operands ----
   float xs[kPlanes ? 1 : RB][kPlanes ? 1 : DP / 2];
@@ -815,6 +818,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         // they are not computed.
         const float mx_rel = BIASC ? st.mx - run_m[prev_rb] : st.mx;
         const bool soft = wave_any(mx_rel > skip_below);
+        n_left_out += soft ? 0u : 1u;
         if constexpr (BIASC) {
           // one branch per piece: a two-sided branch with the MFMAs on both sides makes the
           // compiler move the accumulator tile at the join
@@ -844,6 +848,17 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     f32x16 v16;
     if constexpr (VEC) v16 = load_v16(nx2, NSUB - 1);  // after rotate(): the tile just finished
     softmax(R1, RB - 1, v16);
+  }
+
+  // With the variant chosen on the device, this kernel's own counts (units whose exponentials
+  // it left out, of all its units) tell the merge kernel when the plan has become peaked enough
+  // for the variant with the coarse tile test (a schedule of decreasing eps gets there).
+  if constexpr (PREC == kH3 && !VEC) {
+    if (args.sel != nullptr && args.sel_pred && lane == 0 && ntiles > 0) {
+      const int slot = blockIdx.x % kSelSlots;
+      atomicAdd(&args.sel[kSelEnded + slot], n_left_out);
+      atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
+    }
   }
 
 #pragma unroll

@@ -215,21 +215,28 @@ def sinkhorn_flashstyle_symmetric(
                             and a.stride() == b.stride()))):
         yf, beta, log_b, g_hat = xf, alpha, log_a, f_hat
 
-    # the kernel variant with the coarse tile test (see COARSE_TEST)
+    # the kernel variant with the coarse tile test (see COARSE_TEST).  On a schedule of
+    # decreasing eps the plan is flat for the first steps and peaked for the last ones: the device
+    # starts on the plain kernel and changes over when that kernel leaves out the exponentials
+    # of most of its tiles (forcing the variant applies to fixed-eps solves only).
     coarse = False
+    fixed_eps = all(e == eps_list[0] for e in eps_list)
     if (fused and not use_labels and _lib.TILE_SKIP
             and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
             and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
-            and len(eps_list) >= _COARSE_MIN_STEPS
-            and all(e == eps_list[0] for e in eps_list)):
-        coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
+            and len(eps_list) >= _COARSE_MIN_STEPS):
+        if fixed_eps:
+            coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
+        elif COARSE_TEST is not False:
+            coarse = "auto"
     # operand planes are converted once for the whole loop, when the first launch needs them
     # (a run replayed from a graph has planes of its own)
     made = []
 
     def planes():
         if not made:
-            made.append(_lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32)))
+            made.append(_lib.PreparedOperands(xf, yf, _lib.flags(use_exp2, allow_tf32),
+                                              start_plain=(coarse == "auto" and not fixed_eps)))
         return made[0]
 
     def jacobi(f_hat, g_hat, e, w):
@@ -382,11 +389,14 @@ def sinkhorn_flashstyle_symmetric_self_pair(
     made = []
     # the kernel variant with the coarse tile test, under the single-problem solver's conditions
     coarse = False
+    fixed_eps = all(e == ex[0] for e in ex) and all(e == ey[0] for e in ey)
     if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
             and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
-            and min(len(ex), len(ey)) >= _COARSE_MIN_STEPS
-            and all(e == ex[0] for e in ex) and all(e == ey[0] for e in ey)):
-        coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
+            and min(len(ex), len(ey)) >= _COARSE_MIN_STEPS):
+        if fixed_eps:
+            coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
+        elif COARSE_TEST is not False:
+            coarse = "auto"  # decreasing eps: the device starts on the plain kernel
 
     def pair(fx, fy, steps, with_previous=False):  # steps: [(eps_x, eps_y, weight)]
         full = tuple((e1, e2, w, dampening(e1, rho), dampening(e2, rho)) for e1, e2, w in steps)
@@ -402,7 +412,8 @@ def sinkhorn_flashstyle_symmetric_self_pair(
                    float(cost_scale), shift_x is not None, flag_bits, with_previous)
             return _graphs.run(key, enqueue, [xf, yf, fx, fy, log_a, log_b, shift_x, shift_y])
         if not made:  # operand planes of both clouds, converted once for the whole loop
-            made.append(_lib.PreparedOperands(xf, yf, flag_bits, self_pair=True))
+            made.append(_lib.PreparedOperands(xf, yf, flag_bits, self_pair=True,
+                                              start_plain=(coarse == "auto" and not fixed_eps)))
         return _self_pair_steps_raw(xf, yf, fx, fy, log_a, log_b, full, shift_x=shift_x,
                                     shift_y=shift_y, prepared=made[0],
                                     with_previous=with_previous, coarse=coarse, **kw)

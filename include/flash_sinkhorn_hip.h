@@ -55,9 +55,15 @@
  *    variant runs first and counts the tiles that end at its test in workgroups whose rows all
  *    started from a key of the launch before; the third launch with such counts decides: if
  *    fewer than 40 % of its tiles ended, the step's merge kernel switches to the plain variant
- *    for good.  The state is reset by fs_prepare_operands.  Nothing is read back or timed on
- *    the host: the same inputs take the same path on every run, and the calls can be captured
- *    into a graph.
+ *    while the plan stays as flat.  The plain variant counts in turn the tiles whose
+ *    exponentials it left out (all logits 2^40 below their rows' running maxima), and a launch
+ *    that left out a clearly larger share than the first plain launch of the stretch (by 4 % of
+ *    all tiles) hands the next one back to the coarse variant: a schedule of decreasing eps
+ *    starts flat and ends peaked.  The state is reset by fs_prepare_operands,
+ *    with FS_FLAG_START_PLAIN among its flags to the plain variant (what a caller passes who
+ *    knows that its first steps run at a large eps).  Nothing is read back or timed on the
+ *    host: the same inputs take the same path on every run, and the calls can be captured into
+ *    a graph.
  *    Every operation runs on the two-plane fp16 operands by default and on fp32 MFMA operands
  *    with FS_FLAG_FP32_MFMA (the c-transform at d > 128: fp16 planes in either case).
  */
@@ -88,6 +94,7 @@ extern "C" {
 #define FS_FLAG_NO_TILE_SKIP 32u
 #define FS_FLAG_COARSE_TEST 64u
 #define FS_FLAG_COARSE_AUTO 128u
+#define FS_FLAG_START_PLAIN 256u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0

@@ -924,6 +924,46 @@ def test_variant_choice_on_the_device():
             assert rel_err(runs["auto"][k], ref) < tol and rel_err(runs[True][k], ref) < tol, name
 
 
+def test_variant_follows_a_schedule_of_decreasing_eps(monkeypatch):
+    """eps-scaling (the reference's default schedule) starts on a flat plan and ends on a peaked
+    one.  With the variant left to the device the solve starts on the plain kernel
+    (FS_FLAG_START_PLAIN), which counts the tiles whose exponentials it leaves out; once that
+    share has grown by 4 % of all tiles over the first launch's, the next step runs the variant
+    with the coarse tile test, whose keys and counts then start afresh.  The potentials equal the plain solve's to rounding, the same
+    inputs take the same path twice, and the debiased loss (its self terms on schedules of
+    their own) equals the plain one."""
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    from flash_sinkhorn_amd import SamplesLoss
+    rng = np.random.default_rng(37)
+    n, m, d = 26000, 24500, 16
+    x, _ = _clustered(rng, n, d)
+    y, _ = _clustered(rng, m, d)
+    a = np.full(n, 1.0 / n, np.float32)
+    b = (rng.random(m) + 0.5).astype(np.float32)
+    b /= b.sum()
+    X, Y, A, B = dev(x, y, a, b)
+    kw = dict(blur=0.05, scaling=0.5, allow_tf32=False)
+    monkeypatch.setattr(solvers, "COARSE_TEST", False)
+    f0, g0 = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, **kw)
+    monkeypatch.setattr(solvers, "COARSE_TEST", None)
+    runs = []
+    for _ in range(2):
+        info = {}
+        f1, g1 = solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw)
+        st = info["prepared"].variant_state()
+        assert info["coarse"] == "auto"
+        # the last steps ran the coarse variant, and it had its three launches with counts
+        assert not st["plain_selected"] and st["decisions"] == 3, st
+        runs.append((f1, g1))
+    assert torch.equal(runs[0][0], runs[1][0]) and torch.equal(runs[0][1], runs[1][1])
+    assert rel_err(f1, f0.cpu().numpy()) < 2e-6 and rel_err(g1, g0.cpu().numpy()) < 2e-6
+    loss = SamplesLoss("sinkhorn", blur=0.05, debias=True, allow_tf32=False)
+    v1 = float(loss(X, Y))
+    monkeypatch.setattr(solvers, "COARSE_TEST", False)
+    v0 = float(loss(X, Y))
+    assert abs(v1 - v0) <= 1e-5 * abs(v0) + 1e-6
+
+
 def test_graph_replays_equal_eager_solves(monkeypatch):
     """Small solves are captured into a HIP graph on their second call and replayed afterwards.
     Every call (eager, capturing, replaying) is compared with the launch-by-launch solve of the
