@@ -26,8 +26,12 @@ the solve used, after the eight launches in which the rows' starting keys settle
                                  roofline.algorithmic_tflops = 4*n*m*d / launch time is what a
                                  user gets (it counts flop the coarse test never ran).
 The solver lets the device decide, from the share of tiles that end at the coarse test, which
-kernel variant runs; value_plain_kernel_ms is the same solve with the plain kernel on every
-tile, which is what a plan too flat for the test to end anything costs.
+kernel variant runs; value_plain_kernel_ms is the same solve with the plain variant on every
+tile, which is what a plan too flat for the test to end anything costs.  Once its potentials
+have settled the plain variant takes both sides' sums of a step from one sweep over the logits
+(lse_sweep_kernel, half the MFMA and exp2 work; roofline.other_launches.one_sweep_kernel);
+value_two_sided_kernel_ms is the same solve with that form switched off (lse2_kernel twice over
+the logits in every step).
 cpu_baseline: the numpy oracle's symmetric step (fp32) timed on the host cores on a
 bounded sample and scaled to the metric's unit.
 """
@@ -291,9 +295,11 @@ def main():
     fh, gh = (f - alpha).contiguous(), (g - beta).contiguous()
     ops = (X, Y, fh, gh, la, lb)
 
-    def launch_ms(mode, coarse=False, reps=20):
-        """(ms per launch, device counters of the coarse variant over the timed launches)"""
+    def launch_ms(mode, coarse=False, reps=20, sweep=True):
+        """(ms per launch, device counters of the coarse variant over the timed launches);
+        sweep=False: steps of the plain variant stay on the two-sided kernel"""
         set_mode(mode)
+        _lib.SWEEP = sweep
         prep = _lib.PreparedOperands(ops[0], ops[1], _lib.flags(True, False))
         kw = dict(cost_scale=1.0, allow_tf32=False, prepared=prep, coarse=coarse)
         steps = [(EPS, 0.5, 1.0, 1.0)] * reps
@@ -312,6 +318,8 @@ def main():
         counts = {k: (after[k] - before[k]) / reps
                   for k in ("tiles_ended", "tiles_tested", "tiles_skipped")}
         counts["plain_selected"] = after["plain_selected"]
+        counts["one_sweep"] = bool(after["sweep_next"]) and (coarse is False or after["plain_selected"])
+        _lib.SWEEP = True
         return e0.elapsed_time(e1) / reps, counts
 
     flop = 4.0 * n * m * d
@@ -338,6 +346,10 @@ def main():
             # on; its sparse form does not visit tiles whose carried margin still holds.
             products = 3.0 * tiles_all
             exps = 2.0 * n * m
+            if counts is not None and counts.get("one_sweep"):
+                # both sides from one sweep over the logits: half the tiles, half the exponentials
+                products, exps = products / 2, exps / 2
+                r["kernel"] = r["kernel"].replace("lse2_kernel", "lse_sweep_kernel")
             if counts is not None and counts["tiles_tested"] > 0 and not counts["plain_selected"]:
                 went_on = 1.0 - counts["tiles_ended"] / counts["tiles_tested"]
                 visited = 1.0 - counts["tiles_skipped"] / counts["tiles_tested"]
@@ -397,15 +409,29 @@ def main():
         forced = solvers.COARSE_TEST
         solvers.COARSE_TEST = False
         line["value_plain_kernel_ms"], _ = timed_solves(max(2, args.steps // 2), 1)
+        # (value_two_sided_kernel_ms, below: the same without the one-sweep form)
         solvers.COARSE_TEST = forced
         # the 101-step variant (no extrapolation step) that the reference's README times
         line["value_without_last_extrapolation_ms"], _ = timed_solves(
             max(2, args.steps // 2), 1, last_extrapolation=False)
-        plain_ms, _ = launch_ms(args.mode)
+        solvers.COARSE_TEST = False
+        _lib.SWEEP = False
+        line["value_two_sided_kernel_ms"], _ = timed_solves(max(2, args.steps // 2), 1)
+        _lib.SWEEP = True
+        solvers.COARSE_TEST = forced
+        sweep_ms, sweep_counts = launch_ms(args.mode)
+        plain_ms, _ = launch_ms(args.mode, sweep=False)
         _lib.TILE_SKIP = False
-        every_exp_ms, _ = launch_ms(args.mode, reps=10)
+        every_exp_ms, _ = launch_ms(args.mode, reps=10, sweep=False)
         _lib.TILE_SKIP = True
         rf["other_launches"] = {
+            "one_sweep_kernel": {
+                "launch_ms": sweep_ms, "ran": sweep_counts["one_sweep"],
+                **{k: v for k, v in roofline_for(args.mode, sweep_ms, sweep_counts).items()
+                   if k in ("achieved", "frac", "algorithmic_tflops")},
+                "note": "plain variant on settled potentials: lse_sweep_kernel takes both sides' "
+                        "sums from one sweep over the logits (half the MFMA and exp2 work of the "
+                        "two-sided launch; achieved counts the executed half)"},
             "plain_kernel": {
                 "launch_ms": plain_ms, **{k: v for k, v in roofline_for(
                     args.mode, plain_ms, None).items() if k in ("achieved", "frac",

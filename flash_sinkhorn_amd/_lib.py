@@ -24,6 +24,7 @@ FS_FLAG_NO_TILE_SKIP = 32
 FS_FLAG_COARSE_TEST = 64
 FS_FLAG_COARSE_AUTO = 128
 FS_FLAG_START_PLAIN = 256
+FS_FLAG_NO_SWEEP = 512
 # Every call runs on the two-plane fp16 operands (fp32-grade accuracy, the fastest mode here),
 # whatever allow_tf32 says: permission to reduce precision is not an obligation.
 # STRICT_OPERANDS (or env FLASH_SINKHORN_STRICT_OPERANDS) = "fp32_mfma" makes allow_tf32=False
@@ -34,6 +35,9 @@ OP_LSE, OP_SYMMETRIC_STEP, OP_GRAD, OP_APPLY_VEC, OP_APPLY_MAT, OP_MAT5, OP_C_TR
 # d <= 128 log-sum-exp kernel: leave out the exponentials of logits tiles that lie 2^40 below
 # the running row maxima (no effect on fp32 sums); False computes every exponential.
 TILE_SKIP = os.environ.get("FLASH_SINKHORN_TILE_SKIP", "1") != "0"
+# Two-sided steps on prepared planes compute both sides' sums from one sweep over the logits
+# once the potentials move little from step to step (FS_FLAG_NO_SWEEP switches that off)
+SWEEP = os.environ.get("FLASH_SINKHORN_SWEEP", "1") != "0"
 _lib: Optional[ctypes.CDLL] = None
 
 _P = ctypes.c_void_p
@@ -124,6 +128,8 @@ def flags(use_exp2: bool, allow_tf32: bool) -> int:
     f = FS_FLAG_EXP2 if use_exp2 else 0
     if not TILE_SKIP:
         f |= FS_FLAG_NO_TILE_SKIP
+    if not SWEEP:
+        f |= FS_FLAG_NO_SWEEP
     if STRICT_OPERANDS not in _STRICT_FLAGS:
         raise ValueError(f"STRICT_OPERANDS must be one of {sorted(_STRICT_FLAGS)}")
     if allow_tf32:
@@ -132,6 +138,7 @@ def flags(use_exp2: bool, allow_tf32: bool) -> int:
 
 
 _STRICT_FLAGS = {"fp16x2": 0, "fp32_mfma": FS_FLAG_FP32_MFMA}
+_SEL_SWEEP = 247  # word of the variant-choice state that permits the one-sweep step (kSelSweep)
 
 
 class PreparedOperands:
@@ -183,16 +190,19 @@ class PreparedOperands:
         32 x 32 logits tiles of the coarse variant ended at its test."""
         if self.state_offset == 0:
             return {"plain_selected": True, "decisions": 0, "tiles_ended": 0, "tiles_tested": 0,
-                    "tiles_skipped": 0}
-        w = self.ws[self.state_offset:self.state_offset + 32].cpu().view(torch.int32).tolist()
+                    "tiles_skipped": 0, "sweep_next": False}
+        w = self.ws[self.state_offset:self.state_offset + 4 * _SEL_SWEEP + 4].cpu().view(torch.int32).tolist()
         u = [v & 0xFFFFFFFF for v in w]
+        # sweep_next: the next two-sided step under the same eps may take both sides' sums from
+        # one sweep over the logits
         return {"plain_selected": u[0] != 0, "decisions": u[1],
                 "tiles_ended": u[2] | (u[3] << 32), "tiles_tested": u[4] | (u[5] << 32),
-                "tiles_skipped": u[6] | (u[7] << 32)}
+                "tiles_skipped": u[6] | (u[7] << 32), "sweep_next": u[_SEL_SWEEP] != 0}
 
     def serves(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int) -> bool:
         # the workspace layout depends on the set of matrices, so the call must name the same set
-        same = ~FS_FLAG_REDUCED_OPERANDS  # the permission bit does not change the planes
+        # (the permission bit and the choice of kernels for a two-sided step do not change the planes)
+        same = ~(FS_FLAG_REDUCED_OPERANDS | FS_FLAG_NO_SWEEP)
         return ((flag_bits & same) == (self.flag_bits & same) and x.shape[1] == self.d
                 and {(x.data_ptr(), x.shape[0]), (y.data_ptr(), y.shape[0])} == self.keys)
 

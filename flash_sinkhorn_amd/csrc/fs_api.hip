@@ -47,7 +47,7 @@ constexpr int kPlanePadRowsApi = 512;  // must match kPlanePadRows of the plane-
 // after the planes: absmax partials [2][256], plane scales [4] (+4 spare), variant-choice state
 // (a multiple of 256 bytes: the margin entries, queues and their 64-bit slots come right behind)
 constexpr size_t kPlaneAuxBytes = ((2 * 256 + 8 + kSelWords) * sizeof(float) + 255) / 256 * 256;
-static_assert(kSelWords <= 256, "the state is cleared by one workgroup");
+static_assert(kSelWords <= 512, "the state is cleared by one workgroup");
 
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
@@ -239,6 +239,15 @@ size_t margin_slot_bytes(int64_t max_rows, const LseConfig& c) {
   // wavefront rows in whole workgroups of four: the last workgroup's spare wavefronts keep entries too
   const size_t b = (size_t)ceil_div(max_rows, 256) * 4 * (size_t)margin_stride_for(max_rows) * 8;
   return b <= ((size_t)128 << 20) ? b : 0;
+}
+
+// Column sums of lse_sweep_kernel: one row of sums (over the keys) per workgroup row group of
+// 256 query rows; problems with more row groups than this stay on the two-sided kernel.
+constexpr int kSweepMaxGroups = 256;
+size_t sweep_col_bytes(int64_t nq, int64_t nk) {
+  const int64_t groups = ceil_div(nq, 256);
+  if (groups > kSweepMaxGroups || nq < 2048 || nk < 2048) return 0;
+  return (((size_t)groups * (size_t)nk * 4) + 63) & ~(size_t)63;
 }
 
 // Piece counts of lse_sparse_kernel for one side of a launch: one byte per 64-row group and key
@@ -916,6 +925,19 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       aux_bytes[s] = coarse_aux_bytes(sides[s].nk);
       need += aux_bytes[s];
     }
+  // The one-sweep form of a two-sided step: the sides are the two orders of one pair of matrices
+  // on prepared planes (the permission to run it is state, like the variant choice), two row
+  // blocks per wavefront, keys split on both sides.
+  bool sweep = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && nsides == 2 && prepared && !coarse &&
+               !(flags & FS_FLAG_NO_SWEEP) && ps.n > 0 && rb == 2;
+  if (sweep) {
+    const Side &s0 = sides[0], &s1 = sides[1];
+    sweep = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
+            plans[0].rb == 2 && plans[1].rb == 2 && plans[0].splits > 1 && plans[1].splits > 1 &&
+            plans[0].igroups <= kSweepMaxGroups;
+  }
+  const size_t col_off = need;
+  if (sweep) need += sweep_col_bytes(sides[0].nq, sides[0].nk);
   if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
   float* wsp = reinterpret_cast<float*>(static_cast<char*>(ws) + need_planes_end);
   bool any_split = false;
@@ -1003,6 +1025,40 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   } else if (lse2) {
     rc = prepared ? FS_OK : launch_plane_set(ps, cfg, d, ws, st);
     a.skip_log2 = (flags & FS_FLAG_NO_TILE_SKIP) ? -3.0e38f : -40.0f;
+    if (sweep) {
+      // enqueued ahead of the two-sided kernel, which only runs when this one did not, or failed
+      a.sel = select_state(ps, ws);
+      a.sweep = auto_sel ? 2 : 1;
+      a.col_part = reinterpret_cast<float*>(static_cast<char*>(ws) + col_off);
+      auto bits = [](float v) { unsigned u; std::memcpy(&u, &v, 4); return u; };
+      unsigned t = 0x9e3779b9u * (unsigned)(1 + a.side[0].ps_q + 2 * a.side[0].ps_k);
+      for (int s = 0; s < 2; ++s)
+        for (unsigned w : {bits(a.side[s].qscale), bits(a.side[s].kc0), bits(a.side[s].kc1), bits(a.side[s].kc2),
+                           (unsigned)(a.side[s].kb1 != nullptr) + 2u * (unsigned)(a.side[s].kb2 != nullptr),
+                           (unsigned)a.side[s].nq})
+          t = (t ^ w) * 0x85ebca6bu + 0xc2b2ae35u;
+      a.sweep_tag = t | 1u;  // never 0, the cleared state
+      // Its own key split (it has half the workgroups of the two-sided launch): of the counts
+      // down to half of side 0's, the one that fills the last round of workgroups best (two
+      // workgroups per CU at a time)
+      {
+        const int nk = a.side[0].nk, ig = a.side[0].igroups, smax = a.side[0].splits;
+        double best = -1.0;
+        for (int s = smax; s >= std::max(1, smax / 2); --s) {
+          const int chunk = ceil_div(ceil_div(nk, s), 64) * 64;
+          const int real = ceil_div(nk, chunk);
+          if (real > smax) continue;
+          const double rounds = (double)ig * real / 512.0;
+          const double eff = rounds / std::ceil(rounds);
+          if (eff > best + 1e-9) {
+            best = eff;
+            a.sw_splits = real;
+            a.sw_chunk = chunk;
+          }
+        }
+      }
+      if (rc == FS_OK) rc = launch_lse_sweep(a, dp2, st);
+    }
     // device-chosen variant: both are enqueued, the one the state word names runs
     if (auto_sel) {
       a.sel = select_state(ps, ws);
@@ -1117,7 +1173,10 @@ const char* fs_error_string(int code) {
   return "unknown error";
 }
 
-size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
+}  // extern "C"
+
+// with_sweep: room for the column sums of lse_sweep_kernel (prepared planes only)
+static size_t workspace_bytes(int op, int64_t n, int64_t m, int64_t d, bool with_sweep) {
   if (bad_sizes(n, m, d) || d > kMaxSlicedD) return 0;
   const Family fam = family_for(d);
   const int dp = fam.dp;
@@ -1154,6 +1213,9 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
              margin_region_bytes(std::max(n, m), c);
   }
   if (mode == kLse && !fam.sliced) planes += coarse_aux_bytes(n) + coarse_aux_bytes(m);
+  // (the one-sweep form of the symmetric step: either matrix may hold the query rows)
+  if (op == FS_OP_SYMMETRIC_STEP && !fam.sliced && dp <= 64 && with_sweep)
+    planes += std::max(sweep_col_bytes(n, m), sweep_col_bytes(m, n));
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)
                     ? gemm_ws_bytes(n, m, d, both, either) : 0;
@@ -1164,6 +1226,12 @@ size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
   if (both) return std::max(a + b - planes + 64, gemm);
   if (either) return std::max(std::max(a, b) + 64, gemm);
   return std::max(a + 64, gemm);
+}
+
+extern "C" {
+
+size_t fs_workspace_bytes(int op, int64_t n, int64_t m, int64_t d) {
+  return workspace_bytes(op, n, m, d, true);
 }
 
 int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
@@ -1268,7 +1336,7 @@ int fs_symmetric_step_noalloc(const float* x, const float* y, const float* f_hat
                               uint32_t flags, void* stream) {
   if (bad_sizes(n, m, d)) return FS_ERR_BAD_SIZE;
   if (d > kMaxSlicedD) return FS_ERR_UNSUPPORTED;
-  const size_t need = fs_workspace_bytes(FS_OP_SYMMETRIC_STEP, n, m, d);
+  const size_t need = workspace_bytes(FS_OP_SYMMETRIC_STEP, n, m, d, false);
   if (need == 0 || need > kScratchBytes) return FS_ERR_SCRATCH_TOO_SMALL;
   void* buf = nullptr;
   const int rc = scratch_on_current_device(&buf);

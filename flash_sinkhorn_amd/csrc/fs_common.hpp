@@ -152,6 +152,17 @@ struct LaunchArgs {
   // words per side and XCD, zeroed by coarse_bias_kernel before every launch)
   int blocks_sparse, sparse_sides;
   unsigned* queue;
+  // Two-sided steps whose sides are the two orders of one pair of matrices, on prepared planes:
+  // lse_sweep_kernel computes both sides' sums from one sweep over the logits when the state
+  // words allow it (sweep != 0: the step has such a launch; the two-sided kernel then only runs
+  // when that one did not, or failed).  col_part: [side[0].igroups][side[0].nk] sums over the
+  // query rows of a workgroup for every key.
+  int sweep;            // 1, or 2 when the variant is chosen on the device (the one-sweep form
+                        // then belongs to the plain variant)
+  int sw_splits, sw_chunk;  // key chunks of the one-sweep launch (its own: at most side[0].splits)
+  unsigned sweep_tag;   // what kSelSweep must hold for the one-sweep launch to run (never 0): names
+                        // the pairing, eps and the bias coefficients the permission was given under
+  float* col_part;
 };
 
 // Work queue of lse_sparse_kernel for one (side, XCD): word 0 counts the base items handed out,
@@ -196,8 +207,27 @@ constexpr int kSelHave = kSelDmax + 2 * kDmaxSlots;
 // the share of units the plain kernel left out in the first launch of its current stretch, in
 // 65536ths plus one (0: not taken yet)
 constexpr int kSelBase = kSelHave + 2;
-constexpr int kSelWords = kSelBase + 1;
-static_assert(kSelWords <= 256, "one workgroup clears the state block");
+// The one-sweep form of a two-sided step (lse_sweep_kernel): whether this step may run it (set by
+// the merge of the step before), whether its sums left the range it is exact in (the two-sided
+// kernel then redoes the step), the merge kernel's count of workgroups that are done, and the
+// step's largest and smallest log2 of a row or column sum (float bits of the largest and of minus
+// the smallest, by atomic max, spread over slots)
+constexpr int kSelSweep = kSelBase + 1, kSelSweepFail = kSelSweep + 1, kSelSweepDone = kSelSweep + 2;
+constexpr int kSweepSlots = 8;
+constexpr int kSelSweepHi = kSelSweep + 3, kSelSweepLo = kSelSweepHi + kSweepSlots;
+// which variant's kernels ran in the step under way (1: the plain one, one-sweep form included;
+// 0: the one with the coarse tile test), written by them for the merge kernel, whose first
+// workgroup may change kSelWord while the others still need to know
+constexpr int kSelRan = kSelSweepLo + kSweepSlots;
+constexpr int kSelWords = kSelRan + 1;
+static_assert(kSelWords <= 512, "one workgroup clears the state block, two words per thread");
+// log2 of the sums (each about a row's or column's weight times 2^(twice the change of its
+// potential in this step, in base-2 units)): the one-sweep form's exponentials have no running
+// maximum under them, so terms below 2^-126 are lost and sums above 2^127 overflow.  Its
+// results count while every sum lies in [2^-80, 2^60] (what is lost is then below 2^-29 of any
+// sum even with a million terms), and the step after a step whose sums all lie in [2^-56, 2^24]
+// may run it.
+constexpr float kSweepFailLo = -80.f, kSweepFailHi = 60.f, kSweepOkLo = -56.f, kSweepOkHi = 24.f;
 // lse_coarse_kernel leaves margin entries behind once a side's largest bias change is below this
 // many base-2 units (lse_sparse_kernel takes over below 256)
 constexpr float kSettleBelow = FS_SETTLE, kUnsettleAbove = 4.0f * FS_SETTLE;
@@ -316,6 +346,7 @@ __device__ __forceinline__ void state_after_launch(unsigned* st, int lane, int c
         st[kSelWord] = 0u;
         st[kSelDecisions] = 0u;
         st[kSelBase] = 0u;
+        st[kSelSweep] = 0u;  // (the one-sweep form's permission is not kept up by the other variant)
       }
     }
   }

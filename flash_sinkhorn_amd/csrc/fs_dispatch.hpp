@@ -42,5 +42,8 @@ int launch_transpose_planes(const float* src, const float* rowscale, unsigned* d
 int launch_plan_tile(const LaunchArgs& a, int mode, int dp, int rb, int blocks, hipStream_t st);
 int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, bool coarse, int blocks,
                 hipStream_t st);
+// Both sides of a two-sided step from one sweep over the logits (lse_sweep_kernel over side 0's
+// grid, then its merge); both run only when the state words at LaunchArgs::sel allow it.
+int launch_lse_sweep(const LaunchArgs& a, int dp, hipStream_t st);
 
 }  // namespace fs

@@ -123,8 +123,11 @@ __global__ __launch_bounds__(256) void split_planes_f16_kernel(
     if (scale_out2) *scale_out2 = sc;  // the same matrix plays both roles
   }
   // (start_plain: the variant choice begins with the plain kernel, see FS_FLAG_START_PLAIN)
-  if (blockIdx.x == 0 && clear_state != nullptr && threadIdx.x < kSelWords)
-    clear_state[threadIdx.x] = (threadIdx.x == kSelWord && start_plain) ? 1u : 0u;
+  if (blockIdx.x == 0 && clear_state != nullptr) {
+    if (threadIdx.x < kSelWords)
+      clear_state[threadIdx.x] = (threadIdx.x == kSelWord && start_plain) ? 1u : 0u;
+    if (threadIdx.x + 256 < kSelWords) clear_state[threadIdx.x + 256] = 0u;
+  }
 
   const int per_row = dp / 4;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -227,6 +230,9 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
+  // a step with a one-sweep launch: this kernel runs when that one did not, or failed
+  if (args.sweep && args.sel[kSelSweep] == args.sweep_tag && args.sel[kSelSweepFail] == 0u) return;
+  if (args.sweep && blockIdx.x == 0 && threadIdx.x == 0) args.sel[kSelRan] = 1u;
 
   int bid = blockIdx.x;
   const bool second = bid >= args.blocks0;

@@ -75,6 +75,7 @@ __global__ __launch_bounds__(64) void coarse_bias_kernel(const LaunchArgs args, 
                                                          int seed_blocks0, int dp) {
   // variant chosen on the device: nothing reads the records when the plain kernel runs
   if (args.sel_pred && args.sel[kSelWord] != 0u) return;
+  if (args.sweep && blockIdx.x == 0 && threadIdx.x == 0) args.sel[kSelRan] = 0u;
   if (args.queue != nullptr)  // lse_sparse_kernel's work queues start empty
     for (int i = blockIdx.x * 64 + threadIdx.x; i < 2 * 8 * kQueueWords; i += gridDim.x * 64)
       args.queue[i] = 0u;

@@ -463,6 +463,11 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
   }
 }
 
+template <bool HAS_O>
+__device__ __forceinline__ void finish_rows(const LaunchArgs& args, int dp, int items0, int items1,
+                                            float* sweep_l2);
+__device__ __forceinline__ void sweep_step_merge(const LaunchArgs& args, int items0, int items1);
+
 // Merge `splits` partial rows and run the epilogue.  One thread per output row
 // (scalar kinds) or per 4 output columns (matrix kinds); grid covers both sides.
 template <bool HAS_O>
@@ -484,6 +489,23 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
       state_after_launch(args.sel, threadIdx.x, commit_sides, role, ls);
     }
   }
+  if constexpr (!HAS_O) {
+    // a step with a one-sweep launch (see lse_sweep_kernel); with the variant chosen on the
+    // device that form belongs to the plain variant, and a step of the other one has nothing to
+    // do with it
+    if (args.sweep == 1 || (args.sweep == 2 && args.sel[kSelRan] == 1u)) {
+      sweep_step_merge(args, items0, items1);
+      return;
+    }
+  }
+  finish_rows<HAS_O>(args, dp, items0, items1, nullptr);
+}
+
+// The merge itself.  sweep_l2 (may be null): receives log2 of what the row's sum would be with
+// the row's own bias (as a key of the other side) inside the exponent, see lse_sweep_kernel.
+template <bool HAS_O>
+__device__ __forceinline__ void finish_rows(const LaunchArgs& args, int dp, int items0, int items1,
+                                            float* sweep_l2) {
   int it = blockIdx.x * 256 + threadIdx.x;
   if (it >= items0 + items1) return;  // the other side may have nothing to merge
   const bool second = it >= items0;
@@ -583,6 +605,87 @@ __global__ __launch_bounds__(256) void finish_kernel(const LaunchArgs args, int 
     if (keys && bj >= 0) sd.best_key[row] = bj;  // no chunk exceeded the starting value: the old key stays
     if (sd.m_prev != nullptr) sd.m_prev[row] = M;
     epilogue_scalar(sd.ep, row, M, s, o);
+    if (sweep_l2 != nullptr) {
+      const Side& so = second ? args.side[0] : args.side[1];
+      float b = so.kc0 * so.kb0[row];
+      if (so.kb1 != nullptr) b += so.kc1 * so.kb1[row];
+      if (so.kb2 != nullptr) b += so.kc2 * so.kb2[row];
+      *sweep_l2 = (M + log2f(s)) + fmaxf(b, kNegBig);
+    }
+  }
+}
+
+// log2 of a row or column sum joins the step's extremes (kSelSweepHi / kSelSweepLo: float bits of
+// non-negative numbers order like unsigned integers; anything that is not a number counts as
+// out of every range).  One atomic per wavefront and slot.
+__device__ __forceinline__ void sweep_note_sums(unsigned* st, float l2, bool live) {
+  float hi = live ? fmaxf(l2, 0.f) : 0.f, lo = live ? fmaxf(-l2, 0.f) : 0.f;
+  if (live && !(l2 == l2)) hi = lo = 3.0e38f;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    hi = fmaxf(hi, __shfl_xor(hi, o, 64));
+    lo = fmaxf(lo, __shfl_xor(lo, o, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    const int slot = (blockIdx.x * 4 + (threadIdx.x >> 6)) % kSweepSlots;
+    if (hi > 0.f) atomicMax(&st[kSelSweepHi + slot], __builtin_bit_cast(unsigned, hi));
+    if (lo > 0.f) atomicMax(&st[kSelSweepLo + slot], __builtin_bit_cast(unsigned, lo));
+  }
+}
+
+// Did lse_sweep_kernel and its merge produce this step's results?  (Asked in a step of the
+// plain variant only.)
+__device__ __forceinline__ bool sweep_done(const LaunchArgs& args) {
+  const unsigned* st = args.sel;
+  return st[kSelSweep] == args.sweep_tag && st[kSelSweepFail] == 0u;
+}
+
+// The last merge launch of a step that had a one-sweep launch.  If that launch produced the
+// step's results there is nothing left to merge; else the two-sided kernel ran and its rows are
+// merged here, each noting what its sum would have been in the one-sweep form.  The workgroup
+// that finishes last turns the step's extremes into the permission for the next step.
+__device__ __forceinline__ void sweep_step_merge(const LaunchArgs& args, int items0, int items1) {
+  unsigned* st = args.sel;
+  __shared__ int last;
+  if (!sweep_done(args)) {
+    float l2 = 0.f;
+    bool live = false;
+    {
+      float v = __builtin_bit_cast(float, 0x7fc00000u);  // stays so for rows that wrote nothing
+      const int it = blockIdx.x * 256 + threadIdx.x;
+      live = it < items0 + items1;
+      finish_rows<false>(args, 0, items0, items1, &v);
+      l2 = v;
+    }
+    sweep_note_sums(st, l2, live);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    last = atomicAdd(&st[kSelSweepDone], 1u) == gridDim.x - 1 ? 1 : 0;
+  }
+  __syncthreads();
+  if (last && threadIdx.x < 64) {
+    __threadfence();
+    const int lane = threadIdx.x;
+    unsigned hi = 0u, lo = 0u;
+    if (lane < kSweepSlots) {
+      hi = __hip_atomic_load(&st[kSelSweepHi + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      lo = __hip_atomic_load(&st[kSelSweepLo + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      st[kSelSweepHi + lane] = 0u;
+      st[kSelSweepLo + lane] = 0u;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      hi = max(hi, (unsigned)__shfl_xor((int)hi, o, 64));
+      lo = max(lo, (unsigned)__shfl_xor((int)lo, o, 64));
+    }
+    if (lane == 0) {
+      const bool ok = __builtin_bit_cast(float, hi) <= kSweepOkHi && __builtin_bit_cast(float, lo) <= -kSweepOkLo;
+      st[kSelSweep] = ok ? args.sweep_tag : 0u;
+      st[kSelSweepFail] = 0u;
+      st[kSelSweepDone] = 0u;
+    }
   }
 }
 

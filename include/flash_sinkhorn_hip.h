@@ -95,6 +95,7 @@ extern "C" {
 #define FS_FLAG_COARSE_TEST 64u
 #define FS_FLAG_COARSE_AUTO 128u
 #define FS_FLAG_START_PLAIN 256u
+#define FS_FLAG_NO_SWEEP 512u
 
 /* operation ids for fs_workspace_bytes */
 #define FS_OP_LSE 0

@@ -282,11 +282,16 @@ def test_prepared_operands_give_identical_results(n, m, d):
     assert torch.equal(o2, flashsinkhorn_lse_fused(X, Y, G, LB, 0.2, allow_tf32=False))
 
 @pytest.mark.parametrize("n,m,d", [(3000, 4100, 64), (129, 1000, 3), (5000, 300, 128), (260, 260, 32)])
-def test_launches_are_repeatable_on_one_workspace(n, m, d):
+def test_launches_are_repeatable_on_one_workspace(n, m, d, monkeypatch):
     """Split keys leave partial rows in the workspace between the streaming kernel and the merge:
     every launch on one prepared workspace must give the bits of the first, and of a call with
-    a fresh workspace (nothing carried over, no dependence on workgroup arrival order)."""
+    a fresh workspace (nothing carried over, no dependence on workgroup arrival order).  The one
+    thing that is carried on purpose, the permission to take both sides from one sweep, is
+    switched off for that and looked at afterwards: with it, launches on the same inputs give the
+    two-sided kernel's bits until the form is on, the same bits as each other from then on, and
+    the two-sided kernel's numbers to rounding."""
     from flash_sinkhorn_amd import _lib
+    monkeypatch.setattr(_lib, "SWEEP", False)
     from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
     x, y, a, b = inputs(47, n, m, d, scale=2.0 / np.sqrt(d))
     rng = np.random.default_rng(5)
@@ -301,6 +306,20 @@ def test_launches_are_repeatable_on_one_workspace(n, m, d):
     for _ in range(25):
         f1, g1 = _symmetric_step_raw(X, Y, F, G, LA, LB, 0.2, prepared=prep, **kw)
         assert torch.equal(f0, f1) and torch.equal(g0, g1)
+    monkeypatch.setattr(_lib, "SWEEP", True)
+    prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+    later = []
+    for it in range(12):
+        on = prep.variant_state()["sweep_next"]
+        f1, g1 = _symmetric_step_raw(X, Y, F, G, LA, LB, 0.2, prepared=prep, **kw)
+        if not on:
+            assert torch.equal(f0, f1) and torch.equal(g0, g1)
+        else:
+            later.append((f1, g1))
+            assert torch.equal(later[0][0], f1) and torch.equal(later[0][1], g1)
+            assert rel_err(f1, f0.cpu().numpy()) < 2e-6 and rel_err(g1, g0.cpu().numpy()) < 2e-6
+    assert (len(later) > 0) == (min(n, m) >= 2048 and d <= 64)
+    monkeypatch.setattr(_lib, "SWEEP", False)
     if n == m:  # the aliased self problem on its own prepared workspace
         s0, _ = _symmetric_step_raw(X, X, F, F, LA, LA, 0.2, **kw)
         prep = _lib.PreparedOperands(X, X, _lib.flags(True, False))
