@@ -242,8 +242,9 @@ size_t margin_slot_bytes(int64_t max_rows, const LseConfig& c) {
 }
 
 // Column sums of lse_sweep_kernel: one row of sums (over the keys) per workgroup row group of
-// 256 query rows; problems with more row groups than this stay on the two-sided kernel.
-constexpr int kSweepMaxGroups = 256;
+// 256 query rows (n = m = 50,000: 39 MB, read once by the merge); problems with more row groups
+// than this (262,144 rows: 1 GiB at as many keys) stay on the two-sided kernel.
+constexpr int kSweepMaxGroups = 1024;
 size_t sweep_col_bytes(int64_t nq, int64_t nk) {
   const int64_t groups = ceil_div(nq, 256);
   if (groups > kSweepMaxGroups || nq < 2048 || nk < 2048) return 0;
