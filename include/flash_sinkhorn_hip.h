@@ -40,13 +40,15 @@
  *    plan nearly every tile ends at the test, sorted rows or not.  Any content of that array
  *    leaves the results exact (indices are clamped into the key set); fs_prepare_operands
  *    resets it, and a row without a key starts from the largest logit of 64 keys sampled from
- *    the whole key set.  With prepared operands the workspace also carries, per 64 query rows
+ *    the whole key set.  With prepared operands the workspace also carries, per 32 query rows
  *    and 32 keys, by how much a tile that ended at the test stayed clear of mattering, together
  *    with the running sum of the largest key-bias changes of the launches so far: as long as
  *    twice the bias change accumulated since a tile's test is below its margin, the tile would
  *    end again, and the launch does not visit it.  The margins are dropped when the operands'
  *    pairing, eps or the bias coefficients change; overwritten keys only cost visits.  Once the
- *    potentials of a solve move little, nine tiles in ten are not visited on a peaked plan.
+ *    potentials of a solve move little, more than nine tiles in ten are not visited on a peaked
+ *    plan (the launch then runs as wavefronts that take lists of tiles to visit from work
+ *    queues in the same workspace).
  *    Results stay within fp32 rounding of the full computation.  On a flat plan, where every
  *    tile matters, the test costs about 20 %.  Ignored where it does not apply.
  *    FS_FLAG_COARSE_AUTO (with FS_FLAG_OPERANDS_PREPARED, same conditions) leaves that choice to
@@ -64,6 +66,16 @@
  *    knows that its first steps run at a large eps).  Nothing is read back or timed on the
  *    host: the same inputs take the same path on every run, and the calls can be captured into
  *    a graph.
+ *    One more form of a two-sided step lives in the same state (fs_symmetric_step(s) on prepared
+ *    operands, default operand mode, d <= 64, both matrices of 2048 rows or more): when the
+ *    sums of a step show that the potentials have settled, the next step under the same eps
+ *    and bias coefficients computes every logit once and takes both sides' sums from the same
+ *    exponentials (row sums and column sums of 2^(logit + both biases), no running maximum).
+ *    Its merge checks every sum against the range in which that is exact in fp32 and has the
+ *    two-sided kernel, enqueued behind it, redo the step otherwise: results stay within fp32
+ *    rounding of the two-sided step whatever a caller does to the potentials between steps,
+ *    and the same inputs give the same bits on every run.  FS_FLAG_NO_SWEEP keeps every step
+ *    two-sided.
  *    Every operation runs on the two-plane fp16 operands by default and on fp32 MFMA operands
  *    with FS_FLAG_FP32_MFMA (the c-transform at d > 128: fp16 planes in either case).
  */
@@ -127,11 +139,13 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
 
 /*
  * Byte offset, inside a workspace that fs_prepare_operands(x, y, ...) has filled, of the state
- * FS_FLAG_COARSE_AUTO keeps (0 when the configuration has none).  Eight 32-bit words a caller
+ * FS_FLAG_COARSE_AUTO keeps (0 when the configuration has none).  32-bit words a caller
  * may read for diagnostics once the stream has drained: [0] the variant the steps run now
  * (0: coarse tile test, 1: plain), [1] decisions taken so far, [2..3] a 64-bit count of the
- * 32 x 32 logits tiles that ended at the coarse test or were not visited at all, [4..5] of all
- * tiles of those launches, [6..7] of the tiles not visited (carried margins, part of [2..3]).
+ * 32 x 32 logits tiles that ended at the coarse test or were not visited at all (in launches of
+ * the plain variant: whose exponentials were left out), [4..5] of all tiles of those launches,
+ * [6..7] of the tiles not visited (carried margins, part of [2..3]); [247] non-zero: the next
+ * two-sided step under the same eps may take both sides' sums from one sweep.
  * Host arithmetic only.  No counterpart in the reference.
  */
 size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
