@@ -52,10 +52,10 @@ MODES = ["strict", "fp32_mfma"]
 FP32_MFMA_PEAK_TFLOPS = 157.3
 F16_MFMA_PEAK_TFLOPS = 2516.6
 EXP2_PER_S = 18.6e12  # v_exp_f32 lanes per second measured on the box (half rate)
-# Memory-side bytes per lse_coarse_kernel launch of the default workload, from two rocprofv3 --pmc
+# Memory-side bytes per lse_sparse_kernel launch of the default workload, from two rocprofv3 --pmc
 # runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each times the factor that the same
 # counter shows for the 256 MiB device copy of --copy-calibration); see profiles/.
-MEASURED_TRAFFIC_BYTES = {"strict": int((129000 * 2.0 + 28490) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"strict": int((134600 * 2.0 + 15550) * 1024)}
 
 
 def gmm_cloud(rng, n, d, k=8):

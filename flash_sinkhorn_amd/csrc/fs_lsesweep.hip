@@ -8,7 +8,9 @@ namespace fs {
 template <int DP>
 static int launch_sweep_dp(const LaunchArgs& a, hipStream_t st) {
   const Side& s0 = a.side[0];
-  hipLaunchKernelGGL((lse_sweep_kernel<DP>), dim3(s0.igroups * a.sw_splits), dim3(256), 0, st, a);
+  // (a multiple of 8 workgroups: each XCD takes an eighth of the work items)
+  const int per_xcd = (s0.igroups * a.sw_splits + 7) / 8;
+  hipLaunchKernelGGL((lse_sweep_kernel<DP>), dim3(8 * per_xcd), dim3(256), 0, st, a);
   if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
   const int rows = s0.nq + a.side[1].nq;
   hipLaunchKernelGGL((finish_sweep_kernel<0>), dim3((rows + 255) / 256), dim3(256), 0, st, a);
