@@ -138,7 +138,9 @@ def flags(use_exp2: bool, allow_tf32: bool) -> int:
 
 
 _STRICT_FLAGS = {"fp16x2": 0, "fp32_mfma": FS_FLAG_FP32_MFMA}
-_SEL_SWEEP = 247  # word of the variant-choice state that permits the one-sweep step (kSelSweep)
+# words of the variant-choice state: the permission for the one-sweep step (kSelSweep) and the
+# count of such steps that were redone (kSelSweepRedone)
+_SEL_SWEEP, _SEL_REDONE = 247, 269
 
 
 class PreparedOperands:
@@ -190,14 +192,15 @@ class PreparedOperands:
         32 x 32 logits tiles of the coarse variant ended at its test."""
         if self.state_offset == 0:
             return {"plain_selected": True, "decisions": 0, "tiles_ended": 0, "tiles_tested": 0,
-                    "tiles_skipped": 0, "sweep_next": False}
-        w = self.ws[self.state_offset:self.state_offset + 4 * _SEL_SWEEP + 4].cpu().view(torch.int32).tolist()
+                    "tiles_skipped": 0, "sweep_next": False, "sweep_redone": 0}
+        w = self.ws[self.state_offset:self.state_offset + 4 * _SEL_REDONE + 4].cpu().view(torch.int32).tolist()
         u = [v & 0xFFFFFFFF for v in w]
-        # sweep_next: the next two-sided step under the same eps may take both sides' sums from
-        # one sweep over the logits
+        # sweep_next: the next two-sided step may take both sides' sums from one sweep over the
+        # logits; sweep_redone: how many such steps the two-sided kernel had to redo so far
         return {"plain_selected": u[0] != 0, "decisions": u[1],
                 "tiles_ended": u[2] | (u[3] << 32), "tiles_tested": u[4] | (u[5] << 32),
-                "tiles_skipped": u[6] | (u[7] << 32), "sweep_next": u[_SEL_SWEEP] != 0}
+                "tiles_skipped": u[6] | (u[7] << 32), "sweep_next": u[_SEL_SWEEP] != 0,
+                "sweep_redone": u[_SEL_REDONE]}
 
     def serves(self, x: torch.Tensor, y: torch.Tensor, flag_bits: int) -> bool:
         # the workspace layout depends on the set of matrices, so the call must name the same set

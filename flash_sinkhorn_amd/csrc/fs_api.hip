@@ -1031,14 +1031,6 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       a.sel = select_state(ps, ws);
       a.sweep = auto_sel ? 2 : 1;
       a.col_part = reinterpret_cast<float*>(static_cast<char*>(ws) + col_off);
-      auto bits = [](float v) { unsigned u; std::memcpy(&u, &v, 4); return u; };
-      unsigned t = 0x9e3779b9u * (unsigned)(1 + a.side[0].ps_q + 2 * a.side[0].ps_k);
-      for (int s = 0; s < 2; ++s)
-        for (unsigned w : {bits(a.side[s].qscale), bits(a.side[s].kc0), bits(a.side[s].kc1), bits(a.side[s].kc2),
-                           (unsigned)(a.side[s].kb1 != nullptr) + 2u * (unsigned)(a.side[s].kb2 != nullptr),
-                           (unsigned)a.side[s].nq})
-          t = (t ^ w) * 0x85ebca6bu + 0xc2b2ae35u;
-      a.sweep_tag = t | 1u;  // never 0, the cleared state
       // Its own key split (it has half the workgroups of the two-sided launch): of the counts
       // down to half of side 0's, the one that fills the last round of workgroups best (two
       // workgroups per CU at a time)

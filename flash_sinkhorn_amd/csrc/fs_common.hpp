@@ -160,8 +160,6 @@ struct LaunchArgs {
   int sweep;            // 1, or 2 when the variant is chosen on the device (the one-sweep form
                         // then belongs to the plain variant)
   int sw_splits, sw_chunk;  // key chunks of the one-sweep launch (its own: at most side[0].splits)
-  unsigned sweep_tag;   // what kSelSweep must hold for the one-sweep launch to run (never 0): names
-                        // the pairing, eps and the bias coefficients the permission was given under
   float* col_part;
 };
 
@@ -219,14 +217,22 @@ constexpr int kSelSweepHi = kSelSweep + 3, kSelSweepLo = kSelSweepHi + kSweepSlo
 // 0: the one with the coarse tile test), written by them for the merge kernel, whose first
 // workgroup may change kSelWord while the others still need to know
 constexpr int kSelRan = kSelSweepLo + kSweepSlots;
-constexpr int kSelWords = kSelRan + 1;
+// the extremes of the last step of the plain variant (float bits of the largest log2 of a sum
+// and of minus the smallest), kept for the next step's permission and for diagnostics
+constexpr int kSelSweepLast = kSelRan + 1;
+// how many steps of the one-sweep form the two-sided kernel had to redo so far (diagnostics)
+constexpr int kSelSweepRedone = kSelSweepLast + 2;
+constexpr int kSelWords = kSelSweepRedone + 1;
 static_assert(kSelWords <= 512, "one workgroup clears the state block, two words per thread");
 // log2 of the sums (each about a row's or column's weight times 2^(twice the change of its
 // potential in this step, in base-2 units)): the one-sweep form's exponentials have no running
 // maximum under them, so terms below 2^-126 are lost and sums above 2^127 overflow.  Its
 // results count while every sum lies in [2^-80, 2^60] (what is lost is then below 2^-29 of any
 // sum even with a million terms), and the step after a step whose sums all lie in [2^-56, 2^24]
-// may run it.
+// may run it, under whatever eps that step comes with: on a flat plan (large eps) the sums
+// hardly move when eps changes, which is where a schedule of decreasing eps spends its first
+// steps; where they do move, the check above catches it and the permission is gone until a
+// two-sided step has given it again.
 constexpr float kSweepFailLo = -80.f, kSweepFailHi = 60.f, kSweepOkLo = -56.f, kSweepOkHi = 24.f;
 // lse_coarse_kernel leaves margin entries behind once a side's largest bias change is below this
 // many base-2 units (lse_sparse_kernel takes over below 256)

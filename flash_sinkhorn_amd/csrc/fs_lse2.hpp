@@ -231,7 +231,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
   // a step with a one-sweep launch: this kernel runs when that one did not, or failed
-  if (args.sweep && args.sel[kSelSweep] == args.sweep_tag && args.sel[kSelSweepFail] == 0u) return;
+  if (args.sweep && args.sel[kSelSweep] != 0u && args.sel[kSelSweepFail] == 0u) return;
   if (args.sweep && blockIdx.x == 0 && threadIdx.x == 0) args.sel[kSelRan] = 1u;
 
   int bid = blockIdx.x;

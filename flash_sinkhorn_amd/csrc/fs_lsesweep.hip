@@ -21,7 +21,7 @@ int launch_lse_sweep(const LaunchArgs& a, int dp, hipStream_t st) {
   // what the kernel takes for granted
   const Side& s0 = a.side[0];
   const Side& s1 = a.side[1];
-  if (a.sel == nullptr || a.col_part == nullptr || a.sweep_tag == 0u || s0.part_ms == nullptr ||
+  if (a.sel == nullptr || a.col_part == nullptr || s0.part_ms == nullptr ||
       a.sw_splits < 1 || a.sw_splits > s0.splits || a.sw_chunk % 64 != 0 || a.sw_chunk <= 0 ||
       (long long)a.sw_splits * a.sw_chunk < s0.nk || (long long)(a.sw_splits - 1) * a.sw_chunk >= s0.nk || s0.nq != s1.nk || s0.nk != s1.nq ||
       s0.qplanes == nullptr || s0.kplanes == nullptr || s1.kb0 == nullptr)

@@ -23,7 +23,7 @@
 // The merge kernel checks every sum against the range this is exact in (kSweepFailLo/Hi) and
 // has the two-sided kernel redo the step otherwise; whether a step may run this kernel at all is
 // decided by the merge of the step before (kSweepOkLo/Hi), so the first steps of a solve, steps
-// after a change of eps and problems with empty weights stay on the two-sided kernel.
+// on a plan that is moving fast and problems with empty weights stay on the two-sided kernel.
 #pragma once
 
 #include <type_traits>
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
   __shared__ __attribute__((aligned(16))) float lds_col[2][4][2][JT];  // [tile][wavefront][row of 16 lanes][key]
 
   // the step may not run this kernel, or the device chose another variant
-  if (args.sel[kSelSweep] != args.sweep_tag) return;
+  if (args.sel[kSelSweep] == 0u) return;
   if (args.sweep == 2 && args.sel[kSelWord] != 1u) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) args.sel[kSelRan] = 1u;
 
@@ -428,7 +428,7 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
 template <int T>
 __global__ __launch_bounds__(256) void finish_sweep_kernel(const LaunchArgs args) {
   unsigned* st = args.sel;
-  if (st[kSelSweep] != args.sweep_tag) return;
+  if (st[kSelSweep] == 0u) return;
   if (args.sweep == 2 && st[kSelWord] != 1u) return;
   const Side& s0 = args.side[0];
   const Side& s1 = args.side[1];

@@ -637,7 +637,7 @@ __device__ __forceinline__ void sweep_note_sums(unsigned* st, float l2, bool liv
 // plain variant only.)
 __device__ __forceinline__ bool sweep_done(const LaunchArgs& args) {
   const unsigned* st = args.sel;
-  return st[kSelSweep] == args.sweep_tag && st[kSelSweepFail] == 0u;
+  return st[kSelSweep] != 0u && st[kSelSweepFail] == 0u;
 }
 
 // The last merge launch of a step that had a one-sweep launch.  If that launch produced the
@@ -682,7 +682,10 @@ __device__ __forceinline__ void sweep_step_merge(const LaunchArgs& args, int ite
     }
     if (lane == 0) {
       const bool ok = __builtin_bit_cast(float, hi) <= kSweepOkHi && __builtin_bit_cast(float, lo) <= -kSweepOkLo;
-      st[kSelSweep] = ok ? args.sweep_tag : 0u;
+      st[kSelSweep] = ok ? 1u : 0u;
+      st[kSelSweepLast] = hi;
+      st[kSelSweepLast + 1] = lo;
+      if (st[kSelSweepFail] != 0u) st[kSelSweepRedone] += 1u;
       st[kSelSweepFail] = 0u;
       st[kSelSweepDone] = 0u;
     }

@@ -68,8 +68,8 @@
  *    a graph.
  *    One more form of a two-sided step lives in the same state (fs_symmetric_step(s) on prepared
  *    operands, default operand mode, d <= 64, both matrices of 2048 rows or more): when the
- *    sums of a step show that the potentials have settled, the next step under the same eps
- *    and bias coefficients computes every logit once and takes both sides' sums from the same
+ *    sums of a step show that the potentials have settled, the next step (under the same eps or
+ *    another: on a flat plan the sums hardly move with eps) computes every logit once and takes both sides' sums from the same
  *    exponentials (row sums and column sums of 2^(logit + both biases), no running maximum).
  *    Its merge checks every sum against the range in which that is exact in fp32 and has the
  *    two-sided kernel, enqueued behind it, redo the step otherwise: results stay within fp32
@@ -145,7 +145,8 @@ int fs_prepare_operands(const float* x, const float* y, int64_t n, int64_t m, in
  * 32 x 32 logits tiles that ended at the coarse test or were not visited at all (in launches of
  * the plain variant: whose exponentials were left out), [4..5] of all tiles of those launches,
  * [6..7] of the tiles not visited (carried margins, part of [2..3]); [247] non-zero: the next
- * two-sided step under the same eps may take both sides' sums from one sweep.
+ * two-sided step may take both sides' sums from one sweep; [269] how many such steps the
+ * two-sided kernel had to redo so far.
  * Host arithmetic only.  No counterpart in the reference.
  */
 size_t fs_variant_state_offset(const float* x, const float* y, int64_t n, int64_t m, int64_t d,
