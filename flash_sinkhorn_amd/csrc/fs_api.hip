@@ -404,7 +404,7 @@ GemmPlan gemm_plan(int64_t nq, int64_t nk, int total_igroups) {
 
 // Workspace: plane region (see above), then per side 2*bsplits partial (M, s) rows.
 int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& cfg, bool prepared,
-                 void* ws, size_t ws_bytes, hipStream_t st) {
+                 void* ws, size_t ws_bytes, hipStream_t st, uint32_t flags) {
   const bool vec = (mode == kVec);
   PlaneSet ps;
   int rc = side_plane_set(sides, nsides, cfg, ps);
@@ -423,6 +423,17 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
       need += (((size_t)2 * plans[s].bsplits * (size_t)sides[s].nq * sizeof(float)) + 15) & ~(size_t)15;
     }
   }
+  // The one-sweep form of a two-sided step (lse_gemm_kernel<3>): the sides are the two orders of
+  // one pair of matrices on prepared planes, whose state words hold the permission.
+  bool sweep = mode == kLse && nsides == 2 && prepared && !(flags & FS_FLAG_NO_SWEEP);
+  if (sweep) {
+    const Side &s0 = sides[0], &s1 = sides[1];
+    sweep = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
+            sweep_col_bytes(s0.nq, s0.nk) > 0;
+  }
+  need = (need + 63) & ~(size_t)63;
+  const size_t col_off = need;
+  if (sweep) need += sweep_col_bytes(sides[0].nq, sides[0].nk);
   if (need > ws_bytes || ws == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
   char* base = static_cast<char*>(ws);
 
@@ -452,6 +463,20 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
   if (total <= 0) return FS_OK;
 
   if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);
+  if (sweep) {
+    // enqueued ahead of the two-sided launch, which only runs when this one did not, or failed
+    a.sel = select_state(ps, ws);
+    a.sweep = 1;
+    a.col_part = reinterpret_cast<float*>(base + col_off);
+    // its own key split: one workgroup per CU where the keys allow, never more chunks than
+    // side 0 has partial rows for
+    int s = 1;
+    while (plans[0].igroups * s < 256 && sides[0].nk / (2 * s) >= kGemmTile && 2 * s <= plans[0].bsplits) s *= 2;
+    a.sw_chunk = ceil_div(ceil_div(sides[0].nk, s), kGemmTile) * kGemmTile;
+    a.sw_splits = 2 * ceil_div(sides[0].nk, a.sw_chunk);
+    if (rc == FS_OK) rc = launch_lse_gemm_sweep(a, st);
+    if (rc == FS_OK) rc = launch_finish_sweep(a, st);
+  }
   if (rc == FS_OK) rc = launch_lse_gemm(a, mode, total, st);
   if (rc != FS_OK) return rc;
   const int items0 = a.side[0].nq, items1 = (nsides == 2) ? a.side[1].nq : 0;
@@ -465,7 +490,7 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }
 
-size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
+size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bool with_sweep = false) {
   LseConfig c;
   c.gemm = true; c.prec = 3; c.dp = chunked_stride(d); c.np = 2;
   size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
@@ -474,7 +499,9 @@ size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either) {
     return (size_t)2 * p.bsplits * (size_t)nq * 3 * sizeof(float) + 32;  // (M, s) and a weighted sum
   };
   const int ig_n = ceil_div(n, kGemmTile), ig_m = ceil_div(m, kGemmTile);
-  if (both) return planes + part(n, m, ig_n + ig_m) + part(m, n, ig_n + ig_m) + 64;
+  // (the one-sweep form of a two-sided step: either matrix may hold the query rows)
+  const size_t col = with_sweep ? std::max(sweep_col_bytes(n, m), sweep_col_bytes(m, n)) + 64 : 0;
+  if (both) return planes + part(n, m, ig_n + ig_m) + part(m, n, ig_n + ig_m) + 64 + col;
   if (either) return planes + std::max(part(n, m, ig_n), part(m, n, ig_m)) + 64;
   return planes + part(n, m, ig_n) + 64;
 }
@@ -844,7 +871,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   const LseConfig cfg = lse_config(d, flags);
   const bool prepared = (flags & FS_FLAG_OPERANDS_PREPARED) != 0;
   if ((mode == kLse || mode == kVec || mode == kArgmax) && cfg.gemm)
-    return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
+    return run_lse_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st, flags);
   if (mode == kArgmax && fam.sliced) return FS_ERR_UNSUPPORTED;  // d > 128 runs on fp16 planes only
   if ((mode == kMat || mode == kMat5) && cfg.gemm)
     return run_plan_gemm(mode, sides, nsides, d, cfg, prepared, ws, ws_bytes, st);
@@ -1211,7 +1238,7 @@ static size_t workspace_bytes(int op, int64_t n, int64_t m, int64_t d, bool with
     planes += std::max(sweep_col_bytes(n, m), sweep_col_bytes(m, n));
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)
-                    ? gemm_ws_bytes(n, m, d, both, either) : 0;
+                    ? gemm_ws_bytes(n, m, d, both, either, with_sweep && op == FS_OP_SYMMETRIC_STEP) : 0;
   if ((mode == kMat || mode == kMat5) && fam.sliced)
     gemm = pg_ws_bytes(n, m, d, both, either, mode == kMat5);
   if ((mode == kMat || mode == kVec || mode == kArgmax || mode == kMat5) && !fam.sliced)

@@ -28,6 +28,9 @@ int launch_split_planes_f16(const float* src, unsigned* dst, int rows, int d, in
 // GEMM-style LSE kernel for 128 < d <= 1536 on chunked fp16 planes; Side::splits counts
 // partial rows (twice the workgroup-level key splits).
 int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st);  // kLse, kVec, kArgmax
+// Its one-sweep form (both sides of a two-sided step; side 0's grid with LaunchArgs::sw_splits
+// partial rows per query row and sw_chunk keys per workgroup); launch_finish_sweep follows.
+int launch_lse_gemm_sweep(const LaunchArgs& a, hipStream_t st);
 // Plan-matrix products (mat5: with the second stationary operand) for d > 128 on fp16 planes: cb column blocks per wavefront (2, 4 or 6),
 // LaunchArgs::nss column groups.  The value matrix (times an optional per-row scale) is
 // brought into operand order by launch_transpose_planes; partial needs 256 floats.
@@ -45,5 +48,8 @@ int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, bool co
 // Both sides of a two-sided step from one sweep over the logits (lse_sweep_kernel over side 0's
 // grid, then its merge); both run only when the state words at LaunchArgs::sel allow it.
 int launch_lse_sweep(const LaunchArgs& a, int dp, hipStream_t st);
+// The merge of a one-sweep launch alone (row sums from side 0's partial rows, column sums from
+// LaunchArgs::col_part).
+int launch_finish_sweep(const LaunchArgs& a, hipStream_t st);
 
 }  // namespace fs

@@ -5,6 +5,21 @@
 
 namespace fs {
 
+int launch_lse_gemm_sweep(const LaunchArgs& a, hipStream_t st) {
+  // what the kernel takes for granted
+  const Side& s0 = a.side[0];
+  const Side& s1 = a.side[1];
+  if (a.sel == nullptr || a.col_part == nullptr || s0.part_ms == nullptr || a.sw_splits < 2 ||
+      (a.sw_splits & 1) || a.sw_splits > s0.splits || a.sw_chunk <= 0 || a.sw_chunk % kGemmRows != 0 ||
+      (long long)(a.sw_splits / 2) * a.sw_chunk < s0.nk ||
+      (long long)(a.sw_splits / 2 - 1) * a.sw_chunk >= s0.nk || s0.nq != s1.nk || s0.nk != s1.nq ||
+      s0.igroups != (s0.nq + kGemmRows - 1) / kGemmRows || s0.qplanes == nullptr ||
+      s0.kplanes == nullptr || s1.kb0 == nullptr)
+    return FS_ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(lse_gemm_kernel<3>, dim3(s0.igroups * (a.sw_splits / 2)), dim3(512), 0, st, a);
+  return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
+}
+
 int launch_lse_gemm(const LaunchArgs& a, int mode, int blocks, hipStream_t st) {
   if (mode == kVec)
     hipLaunchKernelGGL(lse_gemm_kernel<1>, dim3(blocks), dim3(512), 0, st, a);

@@ -21,6 +21,7 @@
 // makes the ds_read_b128 of 16 consecutive rows at one piece index conflict free.
 #pragma once
 
+#include "fs_colsum.hpp"
 #include "fs_common.hpp"
 #include "fs_stream.hpp"
 
@@ -29,22 +30,42 @@ namespace fs {
 constexpr int kGemmRows = 256;   // query rows per workgroup = keys per tile
 constexpr int kGemmCols = 32;    // feature columns per k-step
 
-// GM: 0 log-sum-exp, 1 plan-vector (VEC), 2 running arg-max of the logits (c-transform).
+// GM: 0 log-sum-exp, 1 plan-vector (VEC), 2 running arg-max of the logits (c-transform),
+// 3 both sides of a two-sided log-sum-exp step from one sweep (SWP): side 0's grid only, the
+// bias of the query rows (as keys of side 1) joins the key bias in the fold, the exponentials
+// are taken without a running maximum and summed along the rows (lane-private, as for GM 0)
+// and along the columns (fs_colsum.hpp over the 32 lanes of a half-wave, then over the four
+// wavefronts of a key group through LDS; one row of column sums per workgroup in
+// LaunchArgs::col_part).  What makes that exact, who permits it and what happens when a sum
+// leaves the range is lse_sweep_kernel's story (fs_lsesweep.hpp); the merge is shared with it.
 template <int GM>
 __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args) {
   constexpr bool VEC = (GM == 1);
   constexpr bool AMAX = (GM == 2);
+  constexpr bool SWP = (GM == 3);
   __shared__ __attribute__((aligned(16))) unsigned lds[2][2 * kGemmRows * 32];
   __shared__ __attribute__((aligned(16))) float lds_v[2][VEC ? kGemmRows : 4];  // v of a key tile
+  // SWP: column sums of a tile, [wavefront][row of 16 lanes][key of the wavefront's 128]
+  __shared__ __attribute__((aligned(16))) float lds_col[SWP ? 8 : 1][2][SWP ? 128 : 1];
+
+  if constexpr (SWP) {
+    if (args.sel[kSelSweep] == 0u) return;  // the step before did not permit it
+  }
+  if constexpr (GM == 0) {
+    // a step with a one-sweep launch ahead of this one: nothing to do unless that launch did
+    // not run or its sums left the range
+    if (args.sweep != 0 && args.sel[kSelSweep] != 0u && args.sel[kSelSweepFail] == 0u) return;
+  }
 
   int bid = blockIdx.x;
-  const bool second = bid >= args.blocks0;
+  const bool second = !SWP && bid >= args.blocks0;
   if (second) bid -= args.blocks0;
   const Side& sd = second ? args.side[1] : args.side[0];
   const int dp = args.pstride;  // words per plane row pair
   const int nch = (args.d + kGemmCols - 1) / kGemmCols;
 
-  const int bsplits = sd.splits >> 1;  // workgroup-level key splits
+  const int bsplits = (SWP ? args.sw_splits : sd.splits) >> 1;  // workgroup-level key splits
+  const int chunk = SWP ? args.sw_chunk : sd.chunk;
   const int split = bid % bsplits;
   const int ig = bid / bsplits;
   const int tid = threadIdx.x;
@@ -55,8 +76,8 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   const int qg = wave & 3;
   const int kg = wave >> 2;
   const int row0 = ig * kGemmRows;
-  const int j_begin = split * sd.chunk;
-  const int j_end = min(sd.nk, j_begin + sd.chunk);
+  const int j_begin = split * chunk;
+  const int j_end = min(sd.nk, j_begin + chunk);
   const int ntiles = (j_end - j_begin + kGemmRows - 1) / kGemmRows;
 
   const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
@@ -99,6 +120,20 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   float run_m[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f}, run_o[2] = {0.f, 0.f};
   int best_j[2] = {0, 0};  // AMAX: run_m holds the largest raw value so far, best_j its key
   if constexpr (AMAX) run_m[0] = run_m[1] = -3.0e38f;
+  float rbias[2] = {0.f, 0.f};  // SWP: the rows' own bias (base 2), as keys of the other side
+  if constexpr (SWP) {
+    const Side& so = args.side[1];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const int row = row0 + qg * 64 + qb * 32 + li;
+      const int rr = min(row, sd.nq - 1);
+      float r = so.kc0 * so.kb0[rr];
+      if (so.kb1 != nullptr) r += so.kc1 * so.kb1[rr];
+      if (so.kb2 != nullptr) r += so.kc2 * so.kb2[rr];
+      // rows past the last one must not reach the column sums
+      rbias[qb] = row < sd.nq ? fmaxf(r, kNegBig) : kNegBig;
+    }
+  }
 
   auto swap_halves = [&](float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
@@ -166,6 +201,49 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
 #pragma unroll
     for (int st = 0; st < 4; ++st)
       ab[st] = h ? 1.0f : key_bias(sd, j0 + kg * 128 + st * 32 + li, j_end) * inv_lscale;
+    if constexpr (SWP) {
+      const float rq[2] = {h ? rbias[0] * inv_lscale : 1.0f, h ? rbias[1] * inv_lscale : 1.0f};
+      const int my_key = colsum_key(li, h);
+      float rs0[2] = {0.f, 0.f}, rs1[2] = {0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        float c[16];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+          acc[qb][st] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[st], rq[qb], acc[qb][st], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const float e00 = fast_exp2(acc[0][st][r] * lscale);
+          const float e01 = fast_exp2(acc[0][st][r + 1] * lscale);
+          const float e10 = fast_exp2(acc[1][st][r] * lscale);
+          const float e11 = fast_exp2(acc[1][st][r + 1] * lscale);
+          rs0[0] += e00;
+          rs1[0] += e01;
+          rs0[1] += e10;
+          rs1[1] += e11;
+          c[r] = e00 + e10;
+          c[r + 1] = e01 + e11;
+        }
+        lds_col[wave][li >> 4][st * 32 + my_key] = colsum_all(c, li);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[qb][st][r] = 0.f;
+      }
+      run_s[0] += rs0[0] + rs1[0];
+      run_s[1] += rs0[1] + rs1[1];
+      // the sums of the four wavefronts of a key group and of their two rows of 16 lanes, in a
+      // fixed order; the next tile's sums reach LDS only after the barriers of its k-loop
+      __syncthreads();
+      if (tid < kGemmRows) {
+        const int kgk = tid >> 7, kk = tid & 127;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) v += lds_col[kgk * 4 + w][0][kk] + lds_col[kgk * 4 + w][1][kk];
+        if (j0 + tid < j_end) args.col_part[(size_t)ig * (size_t)sd.nk + (size_t)(j0 + tid)] = v;
+      }
+      continue;
+    }
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       if constexpr (AMAX) {
@@ -262,6 +340,15 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
       continue;
     }
     const float s = run_s[qb] + xor32(run_s[qb]);
+    if constexpr (SWP) {
+      // every partial sum of a row is taken under the same offset, the row's own bias (a
+      // wavefront whose keys were all masked adds zero)
+      if (row < sd.nq && h == 0) {
+        const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(-rbias[qb], s);
+      }
+      continue;
+    }
     if (row < sd.nq && h == 0) {
       const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;
       *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =

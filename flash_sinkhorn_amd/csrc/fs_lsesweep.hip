@@ -5,6 +5,8 @@
 
 namespace fs {
 
+int launch_finish_sweep(const LaunchArgs& a, hipStream_t st);
+
 template <int DP>
 static int launch_sweep_dp(const LaunchArgs& a, hipStream_t st) {
   const Side& s0 = a.side[0];
@@ -12,7 +14,11 @@ static int launch_sweep_dp(const LaunchArgs& a, hipStream_t st) {
   const int per_xcd = (s0.igroups * a.sw_splits + 7) / 8;
   hipLaunchKernelGGL((lse_sweep_kernel<DP>), dim3(8 * per_xcd), dim3(256), 0, st, a);
   if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
-  const int rows = s0.nq + a.side[1].nq;
+  return launch_finish_sweep(a, st);
+}
+
+int launch_finish_sweep(const LaunchArgs& a, hipStream_t st) {
+  const int rows = a.side[0].nq + a.side[1].nq;
   hipLaunchKernelGGL((finish_sweep_kernel<0>), dim3((rows + 255) / 256), dim3(256), 0, st, a);
   return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
 }

@@ -28,6 +28,7 @@
 
 #include <type_traits>
 
+#include "fs_colsum.hpp"
 #include "fs_common.hpp"
 #include "fs_stream.hpp"
 
@@ -203,36 +204,15 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
 
   // ---- the exponentials of one unit (32 keys x 32 rows), in pieces between the MFMAs of the
   // next one ----
-  // Column sums: the 32 query columns of a key sit in the 32 lanes of a half-wave, 16 key
-  // registers per lane.  The sum over lanes goes in steps that pair lanes differing in one bit
-  // of li and halve the number of registers: of a pair of registers (A, B) a lane with the bit
-  // clear keeps A + A of its partner, a lane with the bit set B + B of its partner.  For bits 3
-  // and 2 the partner is the lane's mirror image in its row of 16 / its group of 8 lanes, the
-  // two kinds of lanes are whole banks of four, and a DPP add with a bank mask writes only one
-  // kind: two instructions per pair, in place.  These two steps are taken on every unit as its
-  // exponentials come out (16 -> 4 registers, which the second row block's unit adds to); the
-  // steps for bits 1 and 0 (within a quad: both sums, then a select) follow once per sub-tile.
-  // Lane li then holds register 8 b0 + 4 b1 + 2 b2 + b3 (b: the bits of li) summed over its row
-  // of 16 lanes; the two rows of a half-wave are added by the wavefront that writes the sums out.
+  // Column sums (see fs_colsum.hpp): the steps for bits 3 and 2 of the lane number are taken on
+  // every unit as its exponentials come out (16 -> 4 registers, which the second row block's
+  // unit adds to); the steps for bits 1 and 0 follow once per sub-tile.  The two rows of 16
+  // lanes of a half-wave are added by the wavefront that writes the sums out.
   float col[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) col[k] = 0.f;
   struct Stage {
     float t[16], e[16], ps0, ps1;
-  };
-  // (s_nop: a VALU result read through DPP needs two wait states, which the compiler does not
-  // insert inside an asm statement; without them the sums came out wrong)
-  auto step_bit3 = [&](float& a, const float& b) {
-    asm volatile("s_nop 1\n\t"
-                 "v_add_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0x3\n\t"
-                 "v_add_f32_dpp %0, %1, %1 row_mirror row_mask:0xf bank_mask:0xc"
-                 : "+v"(a) : "v"(b));
-  };
-  auto step_bit2 = [&](float& a, const float& b) {
-    asm volatile("s_nop 1\n\t"
-                 "v_add_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
-                 "v_add_f32_dpp %0, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa"
-                 : "+v"(a) : "v"(b));
   };
   auto soft_piece = [&](int p, Stage& s, const f32x16& a, int prb) {
     // values 2p, 2p + 1: fma at piece p, exp2 at p + 1, row sums and the step for bit 3 at
@@ -253,11 +233,11 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
       const int r = 2 * p - 4;
       s.ps0 += s.e[r];
       s.ps1 += s.e[r + 1];
-      step_bit3(s.e[r], s.e[r + 1]);  // e[r]: registers r (+1 where bit 3 is set)
+      colsum_step_bit3(s.e[r], s.e[r + 1]);  // e[r]: registers r (+1 where bit 3 is set)
     }
     if (p >= 3 && p < 10 && p % 2 == 1) {
       const int m = (p - 3) / 2;  // results e[4m], e[4m + 2]
-      step_bit2(s.e[4 * m], s.e[4 * m + 2]);
+      colsum_step_bit2(s.e[4 * m], s.e[4 * m + 2]);
       if (prb == 0) {
         col[m] = s.e[4 * m];
       } else {
@@ -273,32 +253,14 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
     soft_tail(s, prb);
   };
 
-  auto dpp_f32 = [](float v, auto ctrl) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
-                                                                 decltype(ctrl)::value, 0xf, 0xf, true));
-  };
-  using QuadXor2 = std::integral_constant<int, 0x4E>;  // quad_perm [2,3,0,1]
-  using QuadXor1 = std::integral_constant<int, 0xB1>;  // quad_perm [1,0,3,2]
-  const bool bit1 = (li & 2) != 0, bit0 = (li & 1) != 0;
   struct Red {
     float f[2], g;
   };
   auto red_piece = [&](int p, Red& R) {
-    if (p == 0 || p == 1) {
-      const float t = col[2 * p] + dpp_f32(col[2 * p], QuadXor2{});
-      const float u = col[2 * p + 1] + dpp_f32(col[2 * p + 1], QuadXor2{});
-      R.f[p] = bit1 ? u : t;
-    }
-    if (p == 2) {
-      const float t = R.f[0] + dpp_f32(R.f[0], QuadXor1{});
-      const float u = R.f[1] + dpp_f32(R.f[1], QuadXor1{});
-      R.g = bit0 ? u : t;
-    }
+    if (p == 0 || p == 1) R.f[p] = colsum_bit1(col[2 * p], col[2 * p + 1], li);
+    if (p == 2) R.g = colsum_bit0(R.f[0], R.f[1], li);
   };
-  // lane (li, h) holds, for its row of 16 lanes, the sum of key 8(r/4) + 4h + r%4 of the
-  // sub-tile, r as above
-  const int my_reg = 8 * (li & 1) + 4 * ((li >> 1) & 1) + 2 * ((li >> 2) & 1) + ((li >> 3) & 1);
-  const int my_key = 8 * (my_reg >> 2) + 4 * h + (my_reg & 3);
+  const int my_key = colsum_key(li, h);  // of the sub-tile
   auto red_store = [&](const Red& R, int tile, int js) {
     lds_col[tile & 1][wave][li >> 4][js * 32 + my_key] = R.g;
   };

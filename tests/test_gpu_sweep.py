@@ -108,6 +108,34 @@ def test_one_sweep_steps_equal_two_sided_steps(n, m, d):
     assert worst0 == 0.0 and not any(allowed0)
 
 
+@pytest.mark.parametrize("n,m,d", [(2300, 2100, 200), (2048, 4500, 136), (3000, 2500, 520)])
+def test_one_sweep_steps_at_more_than_128_columns(n, m, d):
+    """The GEMM-style kernel's one-sweep form (``lse_gemm_kernel<3>``): the same permission, range
+    check and fallback; key chunks whose last tile leaves a whole wavefront without keys."""
+    x, y, a, b = _problem(n + d, n, m, d)
+    worst, allowed, outs = _steps(x, y, a, b, [0.05] * 8, sweep=True, check_oracle_at=(4, 7))
+    assert not allowed[0] and allowed[-1] and sum(allowed) >= 4, allowed
+    assert worst < 2e-6 and outs.redone == 0, (worst, outs.redone)
+    worst0, allowed0, _ = _steps(x, y, a, b, [0.05] * 3, sweep=False)
+    assert worst0 == 0.0 and not any(allowed0)
+    # bit for bit the same on a second run
+    again = _steps(x, y, a, b, [0.05] * 8, sweep=True)[2]
+    for (f0, g0), (f1, g1) in zip(outs, again):
+        assert torch.equal(f0, f1) and torch.equal(g0, g1)
+
+
+def test_a_jump_is_redone_at_more_than_128_columns():
+    n, m, d = 2600, 2200, 256
+    x, y, a, b = _problem(29, n, m, d)
+    rng = np.random.default_rng(2)
+    eps = 0.05
+    jump = [t * 400.0 * eps for t in dev(rng.standard_normal(n).astype(np.float32),
+                                         rng.standard_normal(m).astype(np.float32))]
+    worst, allowed, outs = _steps(x, y, a, b, [eps] * 22, sweep=True, disturb={6: jump})
+    assert allowed[6] and not allowed[7] and allowed[-1], allowed
+    assert worst < 2e-6 and outs.redone == 1, (worst, outs.redone)
+
+
 def test_one_sweep_steps_are_repeatable_bit_for_bit():
     x, y, a, b = _problem(5, 4400, 5200, 64)
     runs = [_steps(x, y, a, b, [0.1] * 8, sweep=True) for _ in range(2)]
