@@ -460,6 +460,7 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
   if (nsides == 1) a.side[1] = a.side[0];
   a.blocks0 = blocks[0];
   const int total = blocks[0] + blocks[1];
+  a.blocks_all = total;
   if (total <= 0) return FS_OK;
 
   if (!prepared) rc = launch_plane_set(ps, cfg, d, ws, st);

@@ -134,6 +134,7 @@ struct Side {
 struct LaunchArgs {
   Side side[2];
   int blocks0;   // blocks belonging to side[0]; the rest belong to side[1]
+  int blocks_all;  // lse_gemm_kernel: work items of both sides (its grid is rounded up to 8 k)
   int d;         // true feature dimension
   int vec_ok;    // rows are 16-byte aligned (d % 4 == 0 and aligned bases)
   int nss;       // column-sliced kernels: super-slices of 1536 columns (1 unless d > 1536)

@@ -57,17 +57,29 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
     if (args.sweep != 0 && args.sel[kSelSweep] != 0u && args.sel[kSelSweepFail] == 0u) return;
   }
 
-  int bid = blockIdx.x;
-  const bool second = !SWP && bid >= args.blocks0;
-  if (second) bid -= args.blocks0;
+  // Work items: side 0's, then side 1's, each side in the order (block of 4 row groups, key
+  // chunk, row group of the block).  Workgroups are dealt round-robin to the 8 XCDs, and XCD x
+  // takes the x-th eighth of the items in that order, so the workgroups that share an L2 share
+  // few row groups AND few key chunks.  (With all row groups of one key chunk on an XCD every
+  // workgroup fetched its own query rows from memory once per key tile: 1.66 GB per one-sweep
+  // launch at 8192 x 8192 x 1536 instead of 0.6.)
+  const int sw_items = args.side[0].igroups * (args.sw_splits >> 1);
+  const int n_items = SWP ? sw_items : args.blocks_all;
+  const int per_xcd = (n_items + 7) / 8;
+  int item = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (((int)blockIdx.x >> 3) >= per_xcd || item >= n_items) return;  // (whole workgroup, before any barrier)
+  const bool second = !SWP && item >= args.blocks0;
+  if (second) item -= args.blocks0;
   const Side& sd = second ? args.side[1] : args.side[0];
   const int dp = args.pstride;  // words per plane row pair
   const int nch = (args.d + kGemmCols - 1) / kGemmCols;
 
   const int bsplits = (SWP ? args.sw_splits : sd.splits) >> 1;  // workgroup-level key splits
   const int chunk = SWP ? args.sw_chunk : sd.chunk;
-  const int split = bid % bsplits;
-  const int ig = bid / bsplits;
+  const int blk = item / (4 * bsplits), within = item % (4 * bsplits);
+  const int nb = min(4, sd.igroups - 4 * blk);
+  const int split = within / nb;
+  const int ig = 4 * blk + within % nb;
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;

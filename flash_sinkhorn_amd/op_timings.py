@@ -1,7 +1,9 @@
 """Per-operation timings at the benchmark shapes: ``python -m flash_sinkhorn_amd.op_timings [c1 c2 c3 c4 c5]``.
 
 Prints one JSON line per shape with the average launch time (HIP events on the current
-stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop),
+stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop; alone, and
+as a solver loop runs it: on planes converted once, where a step whose sums have settled takes
+both sides from one sweep over the logits and ``one_sweep`` says whether the timed steps did),
 one LSE half-update (2nmd), gradient of one side (4nmd), plan-vector (2nmd), plan-matrix
 (4nmd), mat5 (6nmd) and the hard c-transform (2nmd); at c3 also the gradient after a solve on clustered clouds,
 with and without the keys the solve carried; then end-to-end wall times of the five configurations
@@ -15,7 +17,7 @@ import time
 
 import torch
 
-from flash_sinkhorn_amd import SamplesLoss, c_transform_fwd
+from flash_sinkhorn_amd import SamplesLoss, _lib, c_transform_fwd
 from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating
 from flash_sinkhorn_amd.kernels.apply_flash import (apply_plan_mat_flashstyle,
                                                     apply_plan_vec_flashstyle)
@@ -89,6 +91,14 @@ def kernel_timings(name):
     for op, (k, fn) in ops.items():
         ms = _avg_ms(fn)
         out[op] = {"ms": round(ms, 4), "algorithmic_TFLOPs": round(k * nmd / ms / 1e9, 1)}
+    # the step inside a solver loop: planes converted once, a few more steps so that it settles
+    prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+    f2, g2 = fh, gh
+    for _ in range(6):
+        f2, g2 = _symmetric_step_raw(X, Y, f2, g2, la, lb, eps, prepared=prep, **kw)
+    ms = _avg_ms(lambda: _symmetric_step_raw(X, Y, f2, g2, la, lb, eps, prepared=prep, **kw))
+    out["symmetric_step_in_a_loop"] = {"ms": round(ms, 4), "algorithmic_TFLOPs": round(4 * nmd / ms / 1e9, 1),
+                                       "one_sweep": bool(prep.variant_state()["sweep_next"])}
     return out
 
 
