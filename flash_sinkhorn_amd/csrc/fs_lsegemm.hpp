@@ -21,11 +21,33 @@
 // makes the ds_read_b128 of 16 consecutive rows at one piece index conflict free.
 #pragma once
 
+#include <type_traits>
+#include <utility>
+
 #include "fs_colsum.hpp"
 #include "fs_common.hpp"
 #include "fs_stream.hpp"
 
 namespace fs {
+
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}) in order
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// 16 bytes from LDS at byte address addr + OFF (OFF < 65536), not visible to the compiler's
+// wait-count insertion: the consumer must sit behind an explicit wait
+template <int OFF>
+__device__ __forceinline__ u32x4 lds_read16(unsigned addr) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+  return v;
+}
 
 constexpr int kGemmRows = 256;   // query rows per workgroup = keys per tile
 constexpr int kGemmCols = 32;    // feature columns per k-step
@@ -117,9 +139,33 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
           (__attribute__((address_space(3))) void*)(dst + i * 8 * 32), 16, 0, 0);
   };
 
-  // ---- reader addresses (words): piece p of local row r at r*32 + ((p ^ ((r>>1)&7)) * 4) ----
-  auto lds_piece = [&](const unsigned* stage, int r, int p) {
-    return *reinterpret_cast<const u32x4*>(stage + r * 32 + ((p ^ ((r >> 1) & 7)) << 2));
+  // ---- reader addresses: piece p of local row r at word r*32 + ((p ^ ((r>>1)&7)) * 4) ----
+  // Stage reads are ds_read_b128 written out by hand: the compiler cannot tell a read of one
+  // stage buffer from the global->LDS loads filling the other and would make every read wait
+  // for the loads just issued (which is what it did: the prefetch of the next k-step was waited
+  // for before the current one was even read).  It does not see these reads either: their
+  // consumers sit behind wait_lds().  A lane reads the same four pieces (plane, 16-column half)
+  // of every row block; block and stage go into the instruction's offset and a toggled bit, so
+  // eight address registers serve all 24 reads of a k-step.
+  unsigned qaddr[2][2], kaddr[2][2];  // [plane][half]: byte addresses in the current stage
+  {
+    const unsigned base = (unsigned)(size_t)(const __attribute__((address_space(3))) unsigned*)&lds[0][0];
+    const int sw = (li >> 1) & 7;  // (row blocks start at multiples of 32 rows)
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int slot = (p * 4 + kk * 2 + h) ^ sw;
+        qaddr[p][kk] = base + (unsigned)(((qg * 64 + li) * 32 + slot * 4) * 4);
+        kaddr[p][kk] = base + (unsigned)(((kGemmRows + kg * 128 + li) * 32 + slot * 4) * 4);
+      }
+  }
+  static_assert(sizeof(lds[0]) == 65536, "the stages are one address bit apart");
+  auto wait_lds = [&](auto newer) {  // at most `newer` of the reads issued last are still in flight
+    constexpr int n = decltype(newer)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F | (n << 8));  // lgkmcnt(n)
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   f32x16 acc[2][4];
@@ -168,44 +214,57 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
       const bool wrap = (c + 1 == nch);
       if (!wrap || t + 1 < ntiles) issue_loads(buf ^ 1, wrap ? j0 + kGemmRows : j0, wrap ? 0 : c + 1);
 
-      const unsigned* stage = lds[buf];
       u32x4 qreg[2][2][2];  // [query block][plane][16-column half]
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
+      u32x4 kreg[2][2][2];  // [slot][plane][half]: sub-tile st in slot st % 2
+      static_for<2>([&](auto qb_) {
+        constexpr int qb = decltype(qb_)::value;
 #pragma unroll
         for (int p = 0; p < 2; ++p)
 #pragma unroll
-          for (int kk = 0; kk < 2; ++kk)
-            qreg[qb][p][kk] = lds_piece(stage, qg * 64 + qb * 32 + li, p * 4 + kk * 2 + h);
+          for (int kk = 0; kk < 2; ++kk) qreg[qb][p][kk] = lds_read16<qb * 32 * 128>(qaddr[p][kk]);
+      });
+      auto read_keys = [&](auto st_) {
+        constexpr int st = decltype(st_)::value;
 #pragma unroll
-      for (int sp = 0; sp < 2; ++sp) {
-        u32x4 kreg[2][2][2];  // [sub-tile of the pair][plane][half]
+        for (int p = 0; p < 2; ++p)
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int p = 0; p < 2; ++p)
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-              kreg[s2][p][kk] = lds_piece(stage, kGemmRows + kg * 128 + (sp * 2 + s2) * 32 + li,
-                                          p * 4 + kk * 2 + h);
-        // products lo*hi, hi*lo, hi*hi; four independent accumulators between dependent MFMAs
+          for (int kk = 0; kk < 2; ++kk) kreg[st % 2][p][kk] = lds_read16<st * 32 * 128>(kaddr[p][kk]);
+      };
+      read_keys(std::integral_constant<int, 0>{});
+      read_keys(std::integral_constant<int, 1>{});
+      // sub-tile st + 2 is requested into the registers of sub-tile st once its MFMAs are
+      // issued (they have read their operands by then), and lands while those of st + 1 run
+      static_for<4>([&](auto st_) {
+        constexpr int st = decltype(st_)::value;
+        if constexpr (st < 3) wait_lds(std::integral_constant<int, 4>{});
+        else wait_lds(std::integral_constant<int, 0>{});
+        // products lo*hi, hi*lo, hi*hi; the two query blocks alternate, so no MFMA waits for
+        // the one just before it
 #pragma unroll
         for (int prod = 0; prod < 3; ++prod)
 #pragma unroll
           for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-              for (int qb = 0; qb < 2; ++qb) {
-                const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
-                acc[qb][sp * 2 + s2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                    __builtin_bit_cast(f16x8, kreg[s2][pk][kk]),
-                    __builtin_bit_cast(f16x8, qreg[qb][pq][kk]), acc[qb][sp * 2 + s2], 0, 0, 0);
-              }
-      }
+            for (int qb = 0; qb < 2; ++qb) {
+              const int pk = (prod == 0) ? 1 : 0, pq = (prod == 1) ? 1 : 0;
+              acc[qb][st] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, kreg[st % 2][pk][kk]),
+                  __builtin_bit_cast(f16x8, qreg[qb][pq][kk]), acc[qb][st], 0, 0, 0);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (st < 2) read_keys(std::integral_constant<int, st + 2>{});
+      });
+      __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(0);  // this wavefront's direct loads have landed
       __syncthreads();
       buf ^= 1;
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          qaddr[p][kk] ^= 65536u;
+          kaddr[p][kk] ^= 65536u;
+        }
     }
 
     // ---- tile done: fold bias - M, lane-private online soft-max over the 4 sub-tiles ----
