@@ -957,16 +957,28 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   // The one-sweep form of a two-sided step: the sides are the two orders of one pair of matrices
   // on prepared planes (the permission to run it is state, like the variant choice), two row
   // blocks per wavefront, keys split on both sides.
-  bool sweep = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && nsides == 2 && prepared && !coarse &&
-               !(flags & FS_FLAG_NO_SWEEP) && ps.n > 0 && rb == 2;
-  if (sweep) {
+  const bool sweep_base = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && prepared && !coarse &&
+                          !(flags & FS_FLAG_NO_SWEEP) && ps.n > 0 && rb == 2;
+  bool sweep_pair = sweep_base && nsides == 2;
+  if (sweep_pair) {
     const Side &s0 = sides[0], &s1 = sides[1];
-    sweep = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
-            plans[0].rb == 2 && plans[1].rb == 2 && plans[0].splits > 1 && plans[1].splits > 1 &&
-            plans[0].igroups <= kSweepMaxGroups;
+    sweep_pair = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
+                 plans[0].rb == 2 && plans[1].rb == 2 && plans[0].splits > 1 && plans[1].splits > 1 &&
+                 plans[0].igroups <= kSweepMaxGroups && sweep_col_bytes(s0.nq, s0.nk) > 0;
   }
+  // ... or every side is a problem of a matrix with itself (the self problems of a debiased
+  // loss): a symmetric matrix of logits, of which the one-sweep launch visits the tiles on and
+  // above the diagonal of 256 x 256 blocks only
+  bool sweep_self = sweep_base && !sweep_pair;
+  for (int s = 0; s < nsides && sweep_self; ++s)
+    sweep_self = sides[s].q == sides[s].k && sides[s].nq == sides[s].nk && plans[s].rb == 2 &&
+                 plans[s].splits > 1 && plans[s].igroups <= kSweepMaxGroups &&
+                 sweep_col_bytes(sides[s].nq, sides[s].nk) > 0;
+  const bool sweep = sweep_pair || sweep_self;
   const size_t col_off = need;
   if (sweep) need += sweep_col_bytes(sides[0].nq, sides[0].nk);
+  const size_t col_off_b = need;
+  if (sweep_self && nsides == 2) need += sweep_col_bytes(sides[1].nq, sides[1].nk);
   if (need > ws_bytes || (need > 0 && ws == nullptr)) return FS_ERR_WORKSPACE_TOO_SMALL;
   float* wsp = reinterpret_cast<float*>(static_cast<char*>(ws) + need_planes_end);
   bool any_split = false;
@@ -1059,23 +1071,40 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       a.sel = select_state(ps, ws);
       a.sweep = auto_sel ? 2 : 1;
       a.col_part = reinterpret_cast<float*>(static_cast<char*>(ws) + col_off);
-      // Its own key split (it has half the workgroups of the two-sided launch): of the counts
-      // down to half of side 0's, the one that fills the last round of workgroups best (two
-      // workgroups per CU at a time)
-      {
-        const int nk = a.side[0].nk, ig = a.side[0].igroups, smax = a.side[0].splits;
+      // Its own key split (it has half the workgroups of the two-sided launch, or fewer): of
+      // the counts down to half of the side's, the one that fills the last round of workgroups
+      // best (two workgroups per CU at a time)
+      auto choose = [&](int sidx, int items_before, int& splits_out, int& chunk_out) {
+        const int nk = a.side[sidx].nk, ig = a.side[sidx].igroups, smax = a.side[sidx].splits;
         double best = -1.0;
+        int best_items = 0;
         for (int s = smax; s >= std::max(1, smax / 2); --s) {
           const int chunk = ceil_div(ceil_div(nk, s), 64) * 64;
           const int real = ceil_div(nk, chunk);
           if (real > smax) continue;
-          const double rounds = (double)ig * real / 512.0;
+          int items = ig * real;
+          if (sweep_self) {
+            items = 0;
+            for (int c = 0; c < real; ++c) items += self_groups_of_chunk(c, chunk, nk, ig);
+          }
+          const double rounds = (double)(items_before + items) / 512.0;
           const double eff = rounds / std::ceil(rounds);
           if (eff > best + 1e-9) {
             best = eff;
-            a.sw_splits = real;
-            a.sw_chunk = chunk;
+            splits_out = real;
+            chunk_out = chunk;
+            best_items = items;
           }
+        }
+        return best_items;
+      };
+      const int items0 = choose(0, 0, a.sw_splits, a.sw_chunk);
+      if (sweep_self) {
+        a.sweep_self = 1;
+        a.sw_items0 = a.sw_items = items0;
+        if (nsides == 2) {
+          a.sw_items += choose(1, items0, a.sw_splits_b, a.sw_chunk_b);
+          a.col_part_b = reinterpret_cast<float*>(static_cast<char*>(ws) + col_off_b);
         }
       }
       if (rc == FS_OK) rc = launch_lse_sweep(a, dp2, st);

@@ -162,7 +162,24 @@ struct LaunchArgs {
                         // then belongs to the plain variant)
   int sw_splits, sw_chunk;  // key chunks of the one-sweep launch (its own: at most side[0].splits)
   float* col_part;
+  // sweep_self: every side is a problem of a matrix with itself (q == k, a symmetric matrix of
+  // logits once both biases are inside): the one-sweep launch only visits key tiles at or beyond
+  // a workgroup's own 256 rows, a row's sum is its partial row sums plus the column sums that the
+  // row groups before its own took for it.  Side 1 (if any) has its own chunks and column sums;
+  // sw_items0 / sw_items: work items of side 0 / of the launch.
+  int sweep_self;
+  int sw_splits_b, sw_chunk_b;
+  float* col_part_b;
+  int sw_items0, sw_items;
 };
+
+// Row groups (of 256 rows) that have keys at or beyond their first row in key chunk s of a
+// matrix paired with itself.
+__host__ __device__ inline int self_groups_of_chunk(int s, int chunk, int n, int groups) {
+  const long long end = (long long)(s + 1) * chunk < n ? (long long)(s + 1) * chunk : n;
+  const int g = (int)((end + 255) / 256);
+  return g < groups ? g : groups;
+}
 
 // Work queue of lse_sparse_kernel for one (side, XCD): word 0 counts the base items handed out,
 // word 16 the remainders pushed, word 32 the remainders popped (one cache line each); from word

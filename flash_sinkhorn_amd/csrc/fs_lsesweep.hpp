@@ -66,27 +66,48 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
   if (args.sweep == 2 && args.sel[kSelWord] != 1u) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) args.sel[kSelRan] = 1u;
 
-  const Side& sd = args.side[0];
-  const Side& so = args.side[1];  // the other side: its key bias is the bias of this side's rows
   // Work items (key chunk, row group), key chunk slowest; workgroups are dealt round-robin to the
   // 8 XCDs, and XCD x takes the x-th eighth of the items in that order: the workgroups that run on
   // an XCD at any one time share one key chunk (two at a boundary), which stays in its L2
   // whatever the number of chunks.  (With chunk = id % chunks and 13 chunks every XCD streamed
   // the whole key matrix: 1.35 GB from beyond L2 per launch instead of 0.2.)
-  const int n_items = sd.igroups * args.sw_splits;
+  // sweep_self: side 0's items, then side 1's; a chunk only has items for the row groups that
+  // begin before its end.
+  const bool self = args.sweep_self != 0;
+  const int n_items = self ? args.sw_items : args.side[0].igroups * args.sw_splits;
   const int per_xcd = (n_items + 7) / 8;
-  const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if ((int)(blockIdx.x >> 3) >= per_xcd || item >= n_items) return;
-  const int split = item / sd.igroups;
-  const int ig = item % sd.igroups;
+  const bool second = self && item >= args.sw_items0;
+  if (second) item -= args.sw_items0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  // whose key bias is the bias of this side's rows: the other side's, or (self) its own
+  const Side& so = self ? sd : args.side[1];
+  const int sw_chunk = second ? args.sw_chunk_b : args.sw_chunk;
+  int split, ig;
+  if (self) {
+    split = 0;
+    for (;;) {  // (item < the number of items of this side: ends within its chunks)
+      const int g = self_groups_of_chunk(split, sw_chunk, sd.nk, sd.igroups);
+      if (item < g) break;
+      item -= g;
+      ++split;
+    }
+    ig = item;
+  } else {
+    split = item / sd.igroups;
+    ig = item % sd.igroups;
+  }
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
   const int li = lane & 31;
   const int h = lane >> 5;
   const int row0 = (ig * 4 + wave) * (32 * RB);
-  const int j_begin = split * args.sw_chunk;
-  const int j_end = min(sd.nk, j_begin + args.sw_chunk);
+  // (self: from the first row of this row group on; chunks and row groups are multiples of the
+  // 64 keys of a tile)
+  const int j_begin = self ? max(split * sw_chunk, ig * 256) : split * sw_chunk;
+  const int j_end = min(sd.nk, (split + 1) * sw_chunk);
   const int ntiles = (j_end - j_begin + JT - 1) / JT;
   if (ntiles <= 0) return;  // (whole workgroup: no barrier is left waiting)
 
@@ -265,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
     lds_col[tile & 1][wave][li >> 4][js * 32 + my_key] = R.g;
   };
   // one wavefront adds the four wavefronts' sums of a finished tile and writes them out
-  float* colp = args.col_part + (size_t)ig * (size_t)sd.nk;
+  float* colp = (second ? args.col_part_b : args.col_part) + (size_t)ig * (size_t)sd.nk;
   auto flush = [&](int tile) {
     const float* c = &lds_col[tile & 1][0][0][0];  // (a fixed order of additions: the same sums on every run)
     float v = c[lane] + c[JT + lane];
@@ -394,14 +415,32 @@ __global__ __launch_bounds__(256) void finish_sweep_kernel(const LaunchArgs args
   if (args.sweep == 2 && st[kSelWord] != 1u) return;
   const Side& s0 = args.side[0];
   const Side& s1 = args.side[1];
+  const bool self = args.sweep_self != 0;
+  const int rows1 = (self && args.sw_items == args.sw_items0) ? 0 : s1.nq;  // (self: side 1 may be absent)
   int it = blockIdx.x * 256 + threadIdx.x;
-  const bool live = it < s0.nq + s1.nq;
+  const bool live = it < s0.nq + rows1;
   float l2 = 0.f;
   if (live) {
     const bool second = it >= s0.nq;
     const int row = second ? it - s0.nq : it;
     float M, s = 0.f;
-    if (!second) {
+    if (self) {
+      // the row's partial sums over the chunks that reach its row group, and what the row
+      // groups before its own added to it as one of their keys
+      const Side& sd = second ? s1 : s0;
+      const int chunk = second ? args.sw_chunk_b : args.sw_chunk;
+      const int splits = second ? args.sw_splits_b : args.sw_splits;
+      const float* colp = second ? args.col_part_b : args.col_part;
+      const int g_own = row >> 8;
+      float b = sd.kc0 * sd.kb0[row];
+      if (sd.kb1 != nullptr) b += sd.kc1 * sd.kb1[row];
+      if (sd.kb2 != nullptr) b += sd.kc2 * sd.kb2[row];
+      M = -fmaxf(b, kNegBig);
+#pragma unroll 4
+      for (int sp = (g_own * 256) / chunk; sp < splits; ++sp) s += sd.part_ms[2 * ((size_t)sp * sd.nq + row) + 1];
+#pragma unroll 8
+      for (int g = 0; g < g_own; ++g) s += colp[(size_t)g * sd.nk + row];
+    } else if (!second) {
       M = s0.part_ms[2 * (size_t)row];
 #pragma unroll 8
       for (int sp = 0; sp < args.sw_splits; ++sp) s += s0.part_ms[2 * ((size_t)sp * s0.nq + row) + 1];

@@ -606,7 +606,9 @@ __device__ __forceinline__ void finish_rows(const LaunchArgs& args, int dp, int 
     if (sd.m_prev != nullptr) sd.m_prev[row] = M;
     epilogue_scalar(sd.ep, row, M, s, o);
     if (sweep_l2 != nullptr) {
-      const Side& so = second ? args.side[0] : args.side[1];
+      // (the row's own bias as a key: of the other side, or of its own in a problem of a
+      // matrix with itself)
+      const Side& so = args.sweep_self ? sd : (second ? args.side[0] : args.side[1]);
       float b = so.kc0 * so.kb0[row];
       if (so.kb1 != nullptr) b += so.kc1 * so.kb1[row];
       if (so.kb2 != nullptr) b += so.kc2 * so.kb2[row];

@@ -136,6 +136,79 @@ def test_a_jump_is_redone_at_more_than_128_columns():
     assert worst < 2e-6 and outs.redone == 1, (worst, outs.redone)
 
 
+def _self_steps(x, y, a, b, eps_list, *, sweep, alpha=0.5, pair=True):
+    """Steps of the self problems OT(x, x; a) and OT(y, y; b) on one set of prepared planes (the
+    pair in one launch per step, or with ``pair=False`` the first one alone through the
+    symmetric-step call); every step is also run by the two-sided kernel on the same inputs."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels._common import log_weights
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (_self_pair_steps_raw,
+                                                                         _symmetric_step_raw)
+    X, Y, A, B = dev(x, y, a, b)
+    la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
+    Fx, Fy = (-(X * X).sum(1)).contiguous(), (-(Y * Y).sum(1)).contiguous()
+    old = _lib.SWEEP
+    worst, allowed, outs = 0.0, [], []
+    try:
+        _lib.SWEEP = sweep
+        fl = _lib.flags(True, False)
+        prep = _lib.PreparedOperands(X, Y, fl, self_pair=True) if pair else _lib.PreparedOperands(X, X, fl)
+        for i, eps in enumerate(eps_list):
+            allowed.append(prep.variant_state()["sweep_next"])
+            al = 1.0 if i == 0 else alpha
+            if pair:
+                run = lambda p: _self_pair_steps_raw(X, Y, Fx, Fy, la, lb, [(eps, eps, al, 1.0, 1.0)],
+                                                     cost_scale=1.0, allow_tf32=False, prepared=p)
+            else:
+                run = lambda p: (_symmetric_step_raw(X, X, Fx, Fx, la, la, eps, cost_scale=1.0, alpha=al,
+                                                     damping_f=1.0, damping_g=1.0, allow_tf32=False,
+                                                     prepared=p)[0], Fy)
+            f1x, f1y = run(prep)
+            _lib.SWEEP = False
+            f0x, f0y = run(None)
+            _lib.SWEEP = sweep
+            for got, want in ((f1x, f0x), (f1y, f0y)):
+                err = float((got - want).abs().max()) / float(want.abs().max())
+                assert np.isfinite(err)
+                worst = max(worst, err / max(1.0, eps))
+            if i == len(eps_list) - 1:
+                for pts, F, lw, got in ((x, Fx, a, f1x),) + (((y, Fy, b, f1y),) if pair else ()):
+                    lwo = oracle.log_weights(lw)
+                    want = oracle.symmetric_step(pts, pts, F.cpu().numpy(), F.cpu().numpy(), lwo, lwo,
+                                                 eps, 1.0, al, 1.0, 1.0)[0]
+                    e = np.abs(got.cpu().numpy().astype(np.float64) - want).max() / np.abs(want).max()
+                    assert e < 1e-4, e
+            outs.append((f1x, f1y))
+            Fx, Fy = f1x, f1y
+        redone = prep.variant_state()["sweep_redone"]
+    finally:
+        _lib.SWEEP = old
+    return worst, allowed, _Outs(outs, redone)
+
+
+@pytest.mark.parametrize("n,m,d", [(4200, 3100, 32), (2048, 2500, 64), (5000, 6100, 16), (2300, 9000, 7)])
+def test_self_problems_take_the_tiles_on_and_above_the_diagonal(n, m, d):
+    """The two self problems of a debiased loss: the matrix of logits is symmetric once both
+    biases are inside the exponent, and the one-sweep launch visits only the key tiles at or
+    beyond a workgroup's own rows (row counts that are no multiple of the 256-row groups, a
+    cloud of exactly 2048 rows, clouds of different sizes sharing the launch)."""
+    x, y, a, b = _problem(n + m + d, n, m, d)
+    worst, allowed, outs = _self_steps(x, y, a, b, [0.05] * 9, sweep=True)
+    assert not allowed[0] and allowed[-1] and sum(allowed) >= 4, allowed
+    assert worst < 2e-6 and outs.redone == 0, (worst, outs.redone)
+    worst0, allowed0, _ = _self_steps(x, y, a, b, [0.05] * 3, sweep=False)
+    assert worst0 == 0.0 and not any(allowed0)
+    again = _self_steps(x, y, a, b, [0.05] * 9, sweep=True)[2]
+    for (f0, g0), (f1, g1) in zip(outs, again):
+        assert torch.equal(f0, f1) and torch.equal(g0, g1)
+
+
+def test_a_single_self_problem_takes_the_form_too():
+    x, y, a, b = _problem(31, 4700, 2100, 24)
+    worst, allowed, outs = _self_steps(x, y, a, b, [0.1] * 8, sweep=True, pair=False)
+    assert allowed[-1] and worst < 2e-6 and outs.redone == 0, (allowed, worst, outs.redone)
+
+
 def test_one_sweep_steps_are_repeatable_bit_for_bit():
     x, y, a, b = _problem(5, 4400, 5200, 64)
     runs = [_steps(x, y, a, b, [0.1] * 8, sweep=True) for _ in range(2)]
