@@ -387,6 +387,7 @@ int side_plane_set(const Side* sides, int nsides, const LseConfig& c, PlaneSet& 
 
 // ---- large-d LSE on chunked fp16 planes (lse_gemm_kernel) ----
 constexpr int kGemmTile = 256;  // query rows per workgroup and keys per tile
+constexpr int kGemmSweepSplits = 64;  // most key chunks of a one-sweep launch on a matrix with itself
 
 struct GemmPlan {
   int igroups, bsplits, chunk;
@@ -413,27 +414,74 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
   int total_ig = 0;
   for (int s = 0; s < nsides; ++s) total_ig += ceil_div(sides[s].nq, kGemmTile);
   GemmPlan plans[2];
+  for (int s = 0; s < nsides; ++s) plans[s] = gemm_plan(sides[s].nq, sides[s].nk, total_ig);
+  // The one-sweep form of a two-sided step (lse_gemm_kernel<3>) on prepared planes, whose state
+  // words hold the permission: the sides are the two orders of one pair of matrices ...
+  const bool sweep_base = mode == kLse && prepared && !(flags & FS_FLAG_NO_SWEEP);
+  bool sweep_pair = sweep_base && nsides == 2;
+  if (sweep_pair) {
+    const Side &s0 = sides[0], &s1 = sides[1];
+    sweep_pair = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
+                 sweep_col_bytes(s0.nq, s0.nk) > 0;
+  }
+  // ... or every side is a problem of a matrix with itself, of whose symmetric matrix of logits
+  // the launch visits the 256 x 256 tiles on and above the diagonal only
+  bool sweep_self = sweep_base && !sweep_pair;
+  for (int s = 0; s < nsides && sweep_self; ++s)
+    sweep_self = sides[s].q == sides[s].k && sides[s].nq == sides[s].nk &&
+                 sweep_col_bytes(sides[s].nq, sides[s].nk) > 0;
+  const bool sweep = sweep_pair || sweep_self;
+  // Key chunks of the one-sweep launch.  Pair: one workgroup per CU where the keys allow, never
+  // more chunks than side 0 has partial rows for.  Self: the number of items per chunk grows
+  // along the keys, so the chunks are made as small as fills the CUs' rounds best (down to one
+  // tile; at most kGemmSweepSplits chunks), all sides alike.
+  int sw_bs[2] = {0, 0}, sw_chunk[2] = {0, 0}, sw_items[2] = {0, 0};
+  if (sweep_pair) {
+    int s = 1;
+    while (plans[0].igroups * s < 256 && sides[0].nk / (2 * s) >= kGemmTile && 2 * s <= plans[0].bsplits) s *= 2;
+    sw_chunk[0] = ceil_div(ceil_div(sides[0].nk, s), kGemmTile) * kGemmTile;
+    sw_bs[0] = ceil_div(sides[0].nk, sw_chunk[0]);
+  } else if (sweep_self) {
+    double best = 0.0;
+    for (int tiles = 1; tiles <= 64; tiles *= 2) {
+      const int chunk = tiles * kGemmTile;
+      long long items = 0;
+      bool ok = true;
+      for (int s = 0; s < nsides; ++s) {
+        const int bs = ceil_div(sides[s].nk, chunk);
+        ok = ok && bs <= kGemmSweepSplits;
+        for (int c = 0; c < bs; ++c) items += self_groups_of_chunk(c, chunk, sides[s].nk, plans[s].igroups);
+      }
+      if (!ok) continue;
+      const double cost = std::ceil((double)items / 256.0) * tiles;  // rounds of one workgroup per CU
+      if (best == 0.0 || cost < best - 1e-9) {
+        best = cost;
+        for (int s = 0; s < nsides; ++s) {
+          sw_chunk[s] = chunk;
+          sw_bs[s] = ceil_div(sides[s].nk, chunk);
+        }
+      }
+    }
+    if (best == 0.0) return FS_ERR_UNSUPPORTED;  // (64 tiles x kGemmSweepSplits chunks cover every size accepted)
+    for (int s = 0; s < nsides; ++s)
+      for (int c = 0; c < sw_bs[s]; ++c)
+        sw_items[s] += self_groups_of_chunk(c, sw_chunk[s], sides[s].nk, plans[s].igroups);
+  }
   size_t part_off[2], part_o_off[2] = {0, 0};
   for (int s = 0; s < nsides; ++s) {
-    plans[s] = gemm_plan(sides[s].nq, sides[s].nk, total_ig);
+    const int prows = 2 * std::max(plans[s].bsplits, sweep_self ? sw_bs[s] : 0);  // partial rows per row
     part_off[s] = need;
-    need += (((size_t)2 * plans[s].bsplits * (size_t)sides[s].nq * 2 * sizeof(float)) + 15) & ~(size_t)15;
+    need += (((size_t)prows * (size_t)sides[s].nq * 2 * sizeof(float)) + 15) & ~(size_t)15;
     if (vec) {  // one weighted sum per partial row
       part_o_off[s] = need;
       need += (((size_t)2 * plans[s].bsplits * (size_t)sides[s].nq * sizeof(float)) + 15) & ~(size_t)15;
     }
   }
-  // The one-sweep form of a two-sided step (lse_gemm_kernel<3>): the sides are the two orders of
-  // one pair of matrices on prepared planes, whose state words hold the permission.
-  bool sweep = mode == kLse && nsides == 2 && prepared && !(flags & FS_FLAG_NO_SWEEP);
-  if (sweep) {
-    const Side &s0 = sides[0], &s1 = sides[1];
-    sweep = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
-            sweep_col_bytes(s0.nq, s0.nk) > 0;
-  }
   need = (need + 63) & ~(size_t)63;
   const size_t col_off = need;
   if (sweep) need += sweep_col_bytes(sides[0].nq, sides[0].nk);
+  const size_t col_off_b = need;
+  if (sweep_self && nsides == 2) need += sweep_col_bytes(sides[1].nq, sides[1].nk);
   if (need > ws_bytes || ws == nullptr) return FS_ERR_WORKSPACE_TOO_SMALL;
   char* base = static_cast<char*>(ws);
 
@@ -469,12 +517,19 @@ int run_lse_gemm(int mode, Side* sides, int nsides, int64_t d, const LseConfig& 
     a.sel = select_state(ps, ws);
     a.sweep = 1;
     a.col_part = reinterpret_cast<float*>(base + col_off);
-    // its own key split: one workgroup per CU where the keys allow, never more chunks than
-    // side 0 has partial rows for
-    int s = 1;
-    while (plans[0].igroups * s < 256 && sides[0].nk / (2 * s) >= kGemmTile && 2 * s <= plans[0].bsplits) s *= 2;
-    a.sw_chunk = ceil_div(ceil_div(sides[0].nk, s), kGemmTile) * kGemmTile;
-    a.sw_splits = 2 * ceil_div(sides[0].nk, a.sw_chunk);
+    a.sw_part_mult = 2;
+    a.sw_chunk = sw_chunk[0];
+    a.sw_splits = 2 * sw_bs[0];
+    if (sweep_self) {
+      a.sweep_self = 1;
+      a.sw_items0 = a.sw_items = sw_items[0];
+      if (nsides == 2) {
+        a.sw_chunk_b = sw_chunk[1];
+        a.sw_splits_b = 2 * sw_bs[1];
+        a.sw_items += sw_items[1];
+        a.col_part_b = reinterpret_cast<float*>(base + col_off_b);
+      }
+    }
     if (rc == FS_OK) rc = launch_lse_gemm_sweep(a, st);
     if (rc == FS_OK) rc = launch_finish_sweep(a, st);
   }
@@ -497,7 +552,9 @@ size_t gemm_ws_bytes(int64_t n, int64_t m, int64_t d, bool both, bool either, bo
   size_t planes = plane_bytes(n, c) + plane_bytes(m, c) + kPlaneAuxBytes;
   auto part = [&](int64_t nq, int64_t nk, int total_ig) {
     const GemmPlan p = gemm_plan(nq, nk, total_ig);
-    return (size_t)2 * p.bsplits * (size_t)nq * 3 * sizeof(float) + 32;  // (M, s) and a weighted sum
+    // (with_sweep: a matrix with itself may take up to kGemmSweepSplits chunks)
+    const int bs = (with_sweep && nq == nk) ? std::max(p.bsplits, kGemmSweepSplits) : p.bsplits;
+    return (size_t)2 * bs * (size_t)nq * 3 * sizeof(float) + 32;  // (M, s) and a weighted sum
   };
   const int ig_n = ceil_div(n, kGemmTile), ig_m = ceil_div(m, kGemmTile);
   // (the one-sweep form of a two-sided step: either matrix may hold the query rows)

@@ -171,6 +171,7 @@ struct LaunchArgs {
   int sw_splits_b, sw_chunk_b;
   float* col_part_b;
   int sw_items0, sw_items;
+  int sw_part_mult;  // partial rows per key chunk (2 for lse_gemm_kernel, else 1; 0 reads as 1)
 };
 
 // Row groups (of 256 rows) that have keys at or beyond their first row in key chunk s of a

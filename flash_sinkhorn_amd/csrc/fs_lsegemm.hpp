@@ -85,23 +85,40 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   // few row groups AND few key chunks.  (With all row groups of one key chunk on an XCD every
   // workgroup fetched its own query rows from memory once per key tile: 1.66 GB per one-sweep
   // launch at 8192 x 8192 x 1536 instead of 0.6.)
-  const int sw_items = args.side[0].igroups * (args.sw_splits >> 1);
-  const int n_items = SWP ? sw_items : args.blocks_all;
+  // SWP on problems of a matrix with itself (LaunchArgs::sweep_self): side 0's items, then side
+  // 1's, key chunk slowest; a chunk only has items for the row groups that begin before its end.
+  const bool self = SWP && args.sweep_self != 0;
+  const int n_items = SWP ? (self ? args.sw_items : args.side[0].igroups * (args.sw_splits >> 1))
+                          : args.blocks_all;
   const int per_xcd = (n_items + 7) / 8;
   int item = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
   if (((int)blockIdx.x >> 3) >= per_xcd || item >= n_items) return;  // (whole workgroup, before any barrier)
-  const bool second = !SWP && item >= args.blocks0;
-  if (second) item -= args.blocks0;
+  const int items0 = SWP ? args.sw_items0 : args.blocks0;
+  const bool second = (SWP ? self : true) && item >= items0;
+  if (second) item -= items0;
   const Side& sd = second ? args.side[1] : args.side[0];
   const int dp = args.pstride;  // words per plane row pair
   const int nch = (args.d + kGemmCols - 1) / kGemmCols;
 
-  const int bsplits = (SWP ? args.sw_splits : sd.splits) >> 1;  // workgroup-level key splits
-  const int chunk = SWP ? args.sw_chunk : sd.chunk;
-  const int blk = item / (4 * bsplits), within = item % (4 * bsplits);
-  const int nb = min(4, sd.igroups - 4 * blk);
-  const int split = within / nb;
-  const int ig = 4 * blk + within % nb;
+  // workgroup-level key splits
+  const int bsplits = (SWP ? (second ? args.sw_splits_b : args.sw_splits) : sd.splits) >> 1;
+  const int chunk = SWP ? (second ? args.sw_chunk_b : args.sw_chunk) : sd.chunk;
+  int split, ig;
+  if (self) {
+    split = 0;
+    for (;;) {  // (item < the number of items of this side: ends within its chunks)
+      const int g = self_groups_of_chunk(split, chunk, sd.nk, sd.igroups);
+      if (item < g) break;
+      item -= g;
+      ++split;
+    }
+    ig = item;
+  } else {
+    const int blk = item / (4 * bsplits), within = item % (4 * bsplits);
+    const int nb = min(4, sd.igroups - 4 * blk);
+    split = within / nb;
+    ig = 4 * blk + within % nb;
+  }
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
@@ -110,8 +127,9 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   const int qg = wave & 3;
   const int kg = wave >> 2;
   const int row0 = ig * kGemmRows;
-  const int j_begin = split * chunk;
-  const int j_end = min(sd.nk, j_begin + chunk);
+  // (self: from the first row of this row group on; chunks are multiples of the 256 keys of a tile)
+  const int j_begin = self ? max(split * chunk, ig * kGemmRows) : split * chunk;
+  const int j_end = min(sd.nk, (split + 1) * chunk);
   const int ntiles = (j_end - j_begin + kGemmRows - 1) / kGemmRows;
 
   const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
@@ -180,7 +198,7 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
   if constexpr (AMAX) run_m[0] = run_m[1] = -3.0e38f;
   float rbias[2] = {0.f, 0.f};  // SWP: the rows' own bias (base 2), as keys of the other side
   if constexpr (SWP) {
-    const Side& so = args.side[1];
+    const Side& so = self ? sd : args.side[1];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       const int row = row0 + qg * 64 + qb * 32 + li;
@@ -311,7 +329,8 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) v += lds_col[kgk * 4 + w][0][kk] + lds_col[kgk * 4 + w][1][kk];
-        if (j0 + tid < j_end) args.col_part[(size_t)ig * (size_t)sd.nk + (size_t)(j0 + tid)] = v;
+        float* colp = second ? args.col_part_b : args.col_part;
+        if (j0 + tid < j_end) colp[(size_t)ig * (size_t)sd.nk + (size_t)(j0 + tid)] = v;
       }
       continue;
     }

@@ -437,7 +437,8 @@ __global__ __launch_bounds__(256) void finish_sweep_kernel(const LaunchArgs args
       if (sd.kb2 != nullptr) b += sd.kc2 * sd.kb2[row];
       M = -fmaxf(b, kNegBig);
 #pragma unroll 4
-      for (int sp = (g_own * 256) / chunk; sp < splits; ++sp) s += sd.part_ms[2 * ((size_t)sp * sd.nq + row) + 1];
+      for (int sp = max(1, args.sw_part_mult) * ((g_own * 256) / chunk); sp < splits; ++sp)
+        s += sd.part_ms[2 * ((size_t)sp * sd.nq + row) + 1];
 #pragma unroll 8
       for (int g = 0; g < g_own; ++g) s += colp[(size_t)g * sd.nk + row];
     } else if (!second) {

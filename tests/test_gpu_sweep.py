@@ -186,7 +186,8 @@ def _self_steps(x, y, a, b, eps_list, *, sweep, alpha=0.5, pair=True):
     return worst, allowed, _Outs(outs, redone)
 
 
-@pytest.mark.parametrize("n,m,d", [(4200, 3100, 32), (2048, 2500, 64), (5000, 6100, 16), (2300, 9000, 7)])
+@pytest.mark.parametrize("n,m,d", [(4200, 3100, 32), (2048, 2500, 64), (5000, 6100, 16), (2300, 9000, 7),
+                                   (2300, 2100, 200), (2048, 3900, 136)])
 def test_self_problems_take_the_tiles_on_and_above_the_diagonal(n, m, d):
     """The two self problems of a debiased loss: the matrix of logits is symmetric once both
     biases are inside the exponent, and the one-sweep launch visits only the key tiles at or
