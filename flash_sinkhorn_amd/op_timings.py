@@ -3,7 +3,8 @@
 Prints one JSON line per shape with the average launch time (HIP events on the current
 stream) and the algorithmic rate of every C-ABI operation: symmetric step (4nmd flop; alone, and
 as a solver loop runs it: on planes converted once, where a step whose sums have settled takes
-both sides from one sweep over the logits and ``one_sweep`` says whether the timed steps did),
+both sides from one sweep over the logits and ``one_sweep`` says whether the timed steps did;
+likewise a step of the two self problems x-with-x and y-with-y, 2(n^2 + m^2)d flop),
 one LSE half-update (2nmd), gradient of one side (4nmd), plan-vector (2nmd), plan-matrix
 (4nmd), mat5 (6nmd) and the hard c-transform (2nmd); at c3 also the gradient after a solve on clustered clouds,
 with and without the keys the solve carried; then end-to-end wall times of the five configurations
@@ -22,7 +23,8 @@ from flash_sinkhorn_amd.kernels import sinkhorn_flashstyle_alternating
 from flash_sinkhorn_amd.kernels.apply_flash import (apply_plan_mat_flashstyle,
                                                     apply_plan_vec_flashstyle)
 from flash_sinkhorn_amd.kernels.apply_ott import mat5_sqeuclid
-from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (_symmetric_step_raw,
+from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import (_self_pair_steps_raw,
+                                                                     _symmetric_step_raw,
                                                                      flashsinkhorn_lse_fused)
 from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
     sinkhorn_geomloss_online_grad_sqeuclid)
@@ -99,6 +101,14 @@ def kernel_timings(name):
     ms = _avg_ms(lambda: _symmetric_step_raw(X, Y, f2, g2, la, lb, eps, prepared=prep, **kw))
     out["symmetric_step_in_a_loop"] = {"ms": round(ms, 4), "algorithmic_TFLOPs": round(4 * nmd / ms / 1e9, 1),
                                        "one_sweep": bool(prep.variant_state()["sweep_next"])}
+    # a step of the two self problems of a debiased loss (x with x, y with y), in a loop
+    prep2 = _lib.PreparedOperands(X, Y, _lib.flags(True, False), self_pair=True)
+    skw = dict(cost_scale=1.0, allow_tf32=False, prepared=prep2)
+    sx, sy = _self_pair_steps_raw(X, Y, -al, -be, la, lb, [(eps, eps, 1.0, 1.0, 1.0)] + [(eps, eps, 0.5, 1.0, 1.0)] * 7, **skw)
+    ms = _avg_ms(lambda: _self_pair_steps_raw(X, Y, sx, sy, la, lb, [(eps, eps, 0.5, 1.0, 1.0)] * 10, **skw), reps=2) / 10
+    out["self_pair_step_in_a_loop"] = {"ms": round(ms, 4),
+                                       "algorithmic_TFLOPs": round(2 * (float(n) * n + float(m) * m) * d / ms / 1e9, 1),
+                                       "one_sweep": bool(prep2.variant_state()["sweep_next"])}
     return out
 
 

@@ -66,16 +66,20 @@
  *    knows that its first steps run at a large eps).  Nothing is read back or timed on the
  *    host: the same inputs take the same path on every run, and the calls can be captured into
  *    a graph.
- *    One more form of a two-sided step lives in the same state (fs_symmetric_step(s) on prepared
- *    operands, default operand mode, d <= 64, both matrices of 2048 rows or more): when the
+ *    One more form of a two-sided step lives in the same state (fs_symmetric_step(s) and
+ *    fs_self_pair_steps on prepared operands, default operand mode, d <= 64 or d > 128, every
+ *    matrix of 2048 rows or more): when the
  *    sums of a step show that the potentials have settled, the next step (under the same eps or
  *    another: on a flat plan the sums hardly move with eps) computes every logit once and takes both sides' sums from the same
  *    exponentials (row sums and column sums of 2^(logit + both biases), no running maximum).
  *    Its merge checks every sum against the range in which that is exact in fp32 and has the
  *    two-sided kernel, enqueued behind it, redo the step otherwise: results stay within fp32
  *    rounding of the two-sided step whatever a caller does to the potentials between steps,
- *    and the same inputs give the same bits on every run.  FS_FLAG_NO_SWEEP keeps every step
- *    two-sided.
+ *    and the same inputs give the same bits on every run.  A problem of a matrix with itself
+ *    (fs_self_pair_steps, or fs_symmetric_step with x == y and aliased vectors) has a symmetric
+ *    matrix of logits: that form then visits only the tiles on and above the diagonal, a row's
+ *    sum being its row sums there plus the column sums the earlier rows took for it.
+ *    FS_FLAG_NO_SWEEP keeps every step two-sided.
  *    Every operation runs on the two-plane fp16 operands by default and on fp32 MFMA operands
  *    with FS_FLAG_FP32_MFMA (the c-transform at d > 128: fp16 planes in either case).
  */
