@@ -123,29 +123,46 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
   auto swz = [&](int r) {
     return PPR >= 16 ? (r & 15) : (PPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3));
   };
-  const unsigned* kp[PER_THREAD];
+  // (one wave-uniform running base and 32-bit lane offsets: four 64-bit pointers per lane are
+  // what tipped the matrix product at 64 columns into spilling inside the tile loop, and a
+  // reload from scratch there waits for every load in flight)
+  unsigned koff[PER_THREAD];
 #pragma unroll
   for (int c = 0; c < PER_THREAD; ++c) {
     const int idx = tid + 256 * c;
     const int r = idx / PPR;
     const int piece = (idx % PPR) ^ swz(r);
-    kp[c] = sd.kplanes + (size_t)(j_begin + r) * (size_t)ROWW + piece * 4;
+    koff[c] = (unsigned)((r * ROWW + piece * 4) * 4);
   }
+  const char* ktile = reinterpret_cast<const char*>(sd.kplanes + (size_t)j_begin * (size_t)ROWW);
   auto issue_tile = [&](int buf) {  // the next tile in sequence; the planes end in zero rows
 #pragma unroll
     for (int c = 0; c < PER_THREAD; ++c) {
       __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)kp[c],
+          (const __attribute__((address_space(1))) void*)(ktile + koff[c]),
           (__attribute__((address_space(3))) void*)(&lds_k[buf][(c * 256 + wave * 64) * 4]), 16, 0,
           0);
-      kp[c] += kPtKeys * ROWW;
     }
+    ktile += kPtKeys * ROWW * 4;
   };
   auto wait_newest_tile_only = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_THREAD & 15));
   };
   auto lds_piece = [&](const unsigned* tile, int r, int piece) {
     return *reinterpret_cast<const u32x4*>(tile + r * ROWW + ((piece ^ swz(r)) << 2));
+  };
+  // the same by hand (see the streamed logits below): invisible to the compiler's wait counts,
+  // the consumer sits behind wait_lds()
+  auto lds_read16 = [&](const unsigned* p) -> u32x4 {
+    u32x4 v;
+    const unsigned addr = (unsigned)(size_t)(const __attribute__((address_space(3))) unsigned*)p;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+  };
+  auto wait_lds = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
   };
   // Bias of key j (lanes with h == 0 feed it to the fp32 MFMA), in units of the raw products.
   // Its up to three terms are fetched raw, one tile ahead and without branches (absent terms
@@ -301,10 +318,23 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
         }
         // products lo*hi, hi*lo, hi*hi
         if constexpr (kStreamK) {
+          // the key operands of step kk + 1 are requested while the MFMAs of step kk run, by
+          // reads written out by hand: two steps' worth of registers instead of all of them
+          // (which is what the compiler made of plain loads, spilling around the tile loop),
+          // and no wait for the global->LDS loads in flight
+          u32x4 ks[2][2];  // [step parity][plane]
+          auto read_step = [&](int kk) {
+            const unsigned* row = tile + (js * 32 + li) * ROWW;
+            ks[kk & 1][0] = lds_read16(row + (((2 * kk + h) ^ swz(js * 32 + li)) << 2));
+            ks[kk & 1][1] = lds_read16(row + ((((DP / 8) + 2 * kk + h) ^ swz(js * 32 + li)) << 2));
+          };
+          read_step(0);
 #pragma unroll
           for (int kk = 0; kk < KK16; ++kk) {
-            const u32x4 k_hi = lds_piece(tile, js * 32 + li, 2 * kk + h);
-            const u32x4 k_lo = lds_piece(tile, js * 32 + li, (DP / 8) + 2 * kk + h);
+            wait_lds();
+            if (kk + 1 < KK16) read_step(kk + 1);
+            const u32x4 k_hi = ks[kk & 1][0];
+            const u32x4 k_lo = ks[kk & 1][1];
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, k_lo),
                                                          __builtin_bit_cast(f16x8, xq[rb][0][kk]),
                                                          acc, 0, 0, 0);
