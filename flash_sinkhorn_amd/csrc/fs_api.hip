@@ -957,16 +957,18 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   // the kernel variant with the coarse tile test: asked for, or left to the device.  The device's
   // choice lives in state that belongs to prepared planes (a call that writes its own planes
   // would start it afresh), so without them FS_FLAG_COARSE_AUTO means the plain kernel.
-  const bool can_coarse = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && !(flags & FS_FLAG_NO_TILE_SKIP);
+  // (rows of 65 .. 128 columns: lse_coarse128_kernel, without carried margins)
+  const bool can_coarse = lse2 && mode == kLse && prec == 3 && dp2 <= 128 && !(flags & FS_FLAG_NO_TILE_SKIP);
+  const bool wide = dp2 == 128;
   const bool coarse = (flags & FS_FLAG_COARSE_TEST) && can_coarse;
   const bool auto_sel = (flags & FS_FLAG_COARSE_AUTO) && can_coarse && !coarse && prepared;
   Family fam_plan = fam;
   // carried margins: prepared planes only (they are state)
-  bool margins = (coarse || auto_sel) && prepared;
+  bool margins = (coarse || auto_sel) && prepared && !wide;
   int min_splits[2] = {1, 1};
   if (coarse || auto_sel) {  // that kernel works on two row blocks per wavefront and 128-key tiles
-    rb = 2;
-    fam_plan.jt = 128;
+    rb = 2;                  // (64-key tiles at 128 columns)
+    fam_plan.jt = wide ? 64 : 128;
     for (int s = 0; s < nsides; ++s) {
       min_splits[s] = 2;  // the merge kernel carries the margins' state from launch to launch
       if (sides[s].nk < 2 * 128) margins = false;
@@ -1171,7 +1173,17 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       a.sel = select_state(ps, ws);
       a.sel_pred = 1;
       a.sel_want = 1u;
-      if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, false, false, total, st);
+      if (wide) {
+        // the plain kernel at 128 columns works on one row block per wavefront: the same key
+        // chunks and partial rows, twice the row groups
+        LaunchArgs ap = a;
+        int pb[2] = {0, 0};
+        for (int s = 0; s < nsides; ++s) pb[s] = ceil_div(a.side[s].nq, 128) * a.side[s].splits;
+        ap.blocks0 = pb[0];
+        if (rc == FS_OK) rc = launch_lse2(ap, dp2, 1, prec, false, false, pb[0] + pb[1], st);
+      } else if (rc == FS_OK) {
+        rc = launch_lse2(a, dp2, rb, prec, false, false, total, st);
+      }
       a.sel_want = 0u;
       if (rc == FS_OK) rc = launch_lse2(a, dp2, rb, prec, false, true, total, st);
     } else if (rc == FS_OK) {
@@ -1304,9 +1316,9 @@ static size_t workspace_bytes(int op, int64_t n, int64_t m, int64_t d, bool with
     size_t b = 0;  // the launch may settle on any rows-per-wave count: size for the largest
     for (int rb = 0; rb <= 3; ++rb)
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, fam, rb), nq, dp));
-    if (mode == kLse && !fam.sliced && dp <= 64) {  // the plans of lse_coarse_kernel
+    if (mode == kLse && !fam.sliced && dp <= 128) {  // the plans of lse_coarse_kernel / lse_coarse128_kernel
       Family f2 = fam;
-      f2.jt = 128;
+      f2.jt = dp <= 64 ? 128 : 64;
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, f2, 2), nq, dp));
       b = std::max(b, side_ws_floats(mode, plan_side(mode, nq, nk, f2, 2, 2), nq, dp));  // with carried margins
     }
@@ -1372,7 +1384,7 @@ size_t fs_best_keys_offset(const float* x, const float* y, int64_t n, int64_t m,
                            uint32_t flags, int which) {
   if (!x || !y || bad_sizes(n, m, d) || d > kMaxSlicedD || (which != 0 && which != 1)) return 0;
   const LseConfig cfg = lse_config(d, flags);
-  if (cfg.gemm || cfg.dp > 64) return 0;
+  if (cfg.gemm || cfg.dp > 128) return 0;
   const float* ptrs[2] = {x, y};
   const int rows[2] = {(int)n, (int)m};
   PlaneSet ps;

@@ -1,6 +1,7 @@
 // Instantiations and dispatch of the software-pipelined log-sum-exp kernel.
 #include "fs_lse2.hpp"
 #include "fs_lsecoarse.hpp"
+#include "fs_lsecoarse128.hpp"
 #include "fs_lsesparse.hpp"
 
 #include "fs_dispatch.hpp"
@@ -93,13 +94,17 @@ static int launch_coarse(const LaunchArgs& a, int dp, int rb, int blocks, hipStr
     case 16: return launch_coarse_dp<16>(a, blocks, st);
     case 32: return launch_coarse_dp<32>(a, blocks, st);
     case 64: return launch_coarse_dp<64>(a, blocks, st);
+    case 128:  // no carried margins, no sparse form
+      if (a.side[0].margins != nullptr) return FS_ERR_BAD_ARGUMENT;
+      hipLaunchKernelGGL((lse_coarse128_kernel<0>), dim3(blocks), dim3(256), 0, st, a);
+      return hipGetLastError() == hipSuccess ? FS_OK : FS_ERR_LAUNCH_FAILED;
   }
   return FS_ERR_UNSUPPORTED;
 }
 
 int launch_lse2(const LaunchArgs& a, int dp, int rb, int prec, bool vec, bool coarse, int blocks,
                 hipStream_t st) {
-  if (coarse && !vec && prec == kH3 && dp <= 64) return launch_coarse(a, dp, rb, blocks, st);
+  if (coarse && !vec && prec == kH3 && dp <= 128) return launch_coarse(a, dp, rb, blocks, st);
   if (vec) {  // plan-vector product: fp16 planes, rows of at most 64 columns
     return prec == kH3 ? launch_dp<kH3, true>(a, dp, rb, blocks, st) : FS_ERR_UNSUPPORTED;
   }

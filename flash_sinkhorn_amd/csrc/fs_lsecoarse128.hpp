@@ -1,0 +1,384 @@
+// Log-sum-exp kernel with the coarse tile test for rows of 65 .. 128 columns (fp16 planes).
+//
+// The test is the one of lse_coarse_kernel (fs_lsecoarse.hpp): the hi*hi plane product of a
+// 32 x 32 logits tile, plus the exact key bias and a per-row bound on the two cross products,
+// shows whether any logit of the tile lies within 2^40 of its row's running maximum; a tile
+// where none does ends there, after a third of its MFMAs and without a single exponential.
+// Rows start from their logit at the key that held their maximum in the launch before
+// (Side::seed, computed by coarse_bias_kernel's seed blocks from Side::best_key), so on a
+// peaked plan nearly every tile ends.
+//
+// A wavefront keeps both planes of its 64 query rows (two blocks of 32: 128 registers) and
+// walks its key chunk in tiles of 64 keys whose two planes sit in LDS (32 KiB, two buffers, the
+// next tile in flight; two workgroups per CU).  Per 32-key sub-tile the hi*hi products of both
+// row blocks are taken first (the key operands serve both), then each block's unit is tested;
+// a unit (32 keys x 32 rows) that goes on reads the keys' lo plane from LDS, adds the two cross
+// products and runs the online soft-max: nothing such a block computes outlives it except the
+// rows' running (maximum, sum) and the key of the maximum, and nothing in it waits for memory
+// (with the lo planes fetched from global memory on demand, the tenth of the units that goes on
+// at 20,000 x 30,000 x 128, eps 0.0025, cost more than all the tests).  There is no software
+// pipeline across units.  Carried margins and the sparse form of the 64-column kernel do not
+// exist here; the unit counters for the variant choice on the device do.
+//
+// Everything LDS-related is written out by hand (ds_read / ds_write / s_waitcnt / s_barrier):
+// key tiles arrive by direct global->LDS loads two tiles ahead, and the compiler, which cannot
+// tell a read of one ring buffer from the loads still filling another, would make every LDS
+// access wait for all of them.
+#pragma once
+
+#include "fs_common.hpp"
+#include "fs_stream.hpp"
+
+namespace fs {
+
+template <int T>
+__global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs args) {
+  constexpr int DP = 128, RB = 2, JT = 64, NSUB = JT / 32, KK16 = DP / 16;
+  constexpr int ROWW = DP;        // 32-bit words per two-plane row in global memory
+  constexpr int ROWH = DP / 2;    // words per hi-plane row in LDS
+  constexpr int PPRH = ROWH / 4;  // 16-byte pieces per hi-plane row
+  constexpr int PER_PLANE = JT * PPRH / 256;  // direct loads per lane and plane of a tile
+  static_assert(PPRH == 16 && PER_PLANE == 4, "64 keys x 16 pieces: four direct loads per lane and plane");
+
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[2][2][JT * ROWH];  // [buffer][plane]
+  __shared__ __attribute__((aligned(16))) float lds_b[2][JT];               // key bias, raw units
+
+  // variant chosen on the device: the launch of the variant that was not chosen ends here
+  if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
+
+  int bid = blockIdx.x;
+  const bool second = bid >= args.blocks0;
+  if (second) bid -= args.blocks0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const int split = bid % sd.splits;
+  const int ig = bid / sd.splits;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int h = lane >> 5;
+  const int row0 = (ig * 4 + wave) * (32 * RB);
+  const int j_begin = split * sd.chunk;
+  const int j_end = min(sd.nk, j_begin + sd.chunk);
+  const int ntiles = (j_end > j_begin) ? (j_end - j_begin + JT - 1) / JT : 0;
+
+  // MFMAs produce raw products of the scaled planes; lscale turns them into base-2 logits
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
+  const float inv_lscale = 1.0f / lscale;
+  const float skip_below = args.skip_log2 * inv_lscale;  // the 2^40 distance in raw units (< 0)
+
+  // ---- stationary planes of the query rows: [block][16-column step] ----
+  u32x4 xh[RB][KK16], xl[RB][KK16];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = min(row0 + rb * 32 + li, sd.nq - 1);
+    const unsigned* qrow = sd.qplanes + (size_t)row * (size_t)ROWW;
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) {
+      xh[rb][kk] = *reinterpret_cast<const u32x4*>(qrow + 8 * kk + 4 * h);
+      xl[rb][kk] = *reinterpret_cast<const u32x4*>(qrow + ROWH + 8 * kk + 4 * h);
+    }
+  }
+  // Bound on the two cross products of a row, in raw units (see lse_coarse_kernel): with X, Y
+  // the scaled matrices (|.| < 2^15), |Y_lo| <= 8 and |X_lo| <= 2^-11 |X_hi| (+ 2^-24), hence
+  //   sum_k |Y_lo X_hi| + |Y_hi X_lo| <= 24 (1 + 2^-10) sum_k |X_hi| + DP 2^-9;
+  // one base-2 unit of slack covers the fp32 roundings of the chain.
+  float corr[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float l1 = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) {
+      const f16x8 hv = __builtin_bit_cast(f16x8, xh[rb][kk]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) l1 += fabsf((float)hv[e]);
+    }
+    l1 += xor32(l1);
+    corr[rb] = 24.5f * l1 + (float)DP * 0x1p-9f + inv_lscale;
+  }
+
+  // ---- LDS access by hand ----
+  auto lds_addr = [](const void* p) {
+    return (unsigned)(size_t)(const __attribute__((address_space(3))) void*)p;
+  };
+  auto ds_read16 = [&](const unsigned* p) -> u32x4 {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+    return v;
+  };
+  auto ds_read4 = [&](const float* p) -> float {
+    float v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+    return v;
+  };
+  auto ds_write4 = [&](float* p, float v) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(lds_addr(p)), "v"(v) : "memory");
+  };
+  auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+  auto wait_lds = [&]() {  // lgkmcnt(0), and nothing moves across
+    fence();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    fence();
+  };
+  auto barrier = [&]() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  // ---- key tiles: lane idx of instruction c fills LDS slot idx of a plane's buffer and fetches
+  // the piece that belongs there (slot = piece ^ (row & 15)); the plane buffers end in zero
+  // rows, so tiles past the chunk are fetched like any other and masked by their bias ----
+  unsigned koff[PER_PLANE];
+#pragma unroll
+  for (int c = 0; c < PER_PLANE; ++c) {
+    const int idx = tid + 256 * c;
+    const int r = idx / PPRH;
+    const int piece = (idx % PPRH) ^ (r & 15);
+    koff[c] = (unsigned)((r * ROWW + piece * 4) * 4);
+  }
+  const char* ktile = reinterpret_cast<const char*>(sd.kplanes + (size_t)j_begin * (size_t)ROWW);
+  auto issue_tile = [&](int buf) {  // the next tile in sequence
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int c = 0; c < PER_PLANE; ++c)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(ktile + p * ROWH * 4 + koff[c]),
+            (__attribute__((address_space(3))) void*)(&lds_k[buf][p][(c * 256 + wave * 64) * 4]), 16, 0, 0);
+    ktile += JT * ROWW * 4;
+  };
+  // ---- key bias: lane tid < 64 of the workgroup fetches the terms of key j0 + tid by loads the
+  // compiler does not see (it would wait for the key tiles with them), two tiles ahead (ahead
+  // of the next tile's keys, so that they have landed when those have), and writes the combined
+  // value to LDS one tile ahead ----
+  const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
+  const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
+  const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
+  const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
+  float rb0 = 0.f, rb1 = 0.f, rb2 = 0.f, rpen = 0.f;
+  auto gload4 = [](const float* p) -> float {
+    float v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+  };
+  auto issue_bias = [&](int j0) {  // three loads per lane, every lane (the counts stay uniform)
+    const int j = max(0, min(j0 + (tid & 63), j_end - 1));
+    rb0 = gload4(sd.kb0 + j);
+    rb1 = gload4(kb1p + j);
+    rb2 = gload4(kb2p + j);
+    rpen = (j0 + (tid & 63) < j_end) ? 0.f : 1.0f;
+  };
+  auto store_bias = [&](int buf) {  // (after a wait that covers the three loads)
+    asm volatile("" : "+v"(rb0), "+v"(rb1), "+v"(rb2));
+    float b = kc0 * rb0 + (has_kb1 ? kc1 * rb1 : 0.f);
+    b += (has_kb2 ? kc2 * rb2 : 0.f);
+    b = (rpen == 0.f) ? fmaxf(b, kNegBig) : kNegBig;
+    if (wave == 0) ds_write4(&lds_b[buf][lane], fmaxf(b * inv_lscale, -3.0e38f));
+  };
+  // vmcnt(n): all but the newest n vector-memory operations of this wavefront have completed
+  auto wait_vm = [&](auto newer) {
+    constexpr int n = decltype(newer)::value;
+    fence();
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (n & 15) | ((n >> 4) << 14));
+    fence();
+  };
+
+  auto mfma16 = [](const u32x4& a, const u32x4& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  };
+  auto swap_halves = [&](float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  };
+  auto max16 = [](const f32x16& a) {
+    float m = fmaxf(a[0], a[1]);
+#pragma unroll
+    for (int r = 2; r < 16; ++r) m = fmaxf(m, a[r]);
+    return m;
+  };
+
+  // ---- running statistics: run_m in raw units (of the full logit with its key bias) ----
+  float run_m[RB], run_s[RB], best_v[RB];
+  int best_j[RB];
+  const bool track = sd.best_key != nullptr;
+  bool seeded = sd.seed != nullptr;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    run_m[rb] = 0.f;
+    run_s[rb] = 0.f;
+    best_v[rb] = -3.0e38f;
+    best_j[rb] = -1;
+    if (sd.seed != nullptr) {
+      run_m[rb] = sd.seed[min(row0 + rb * 32 + li, sd.nq - 1)];
+      seeded = seeded && run_m[rb] > -3.0e38f;
+    }
+  }
+  // (wavefront-uniform: without a starting value for every row the first unit sets the maxima)
+  seeded = __builtin_amdgcn_ballot_w64(seeded) == ~0ull;
+  bool started[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    started[rb] = seeded;
+    if (!seeded) run_m[rb] = 0.f;
+  }
+  unsigned n_ended = 0;
+
+  // ---- prologue: bias of tiles 0 and 1, tile 0 ----
+  if (ntiles > 0) {
+    issue_bias(j_begin);
+    wait_vm(std::integral_constant<int, 0>{});
+    store_bias(0);
+    issue_bias(j_begin + JT);  // consumed at the top of tile 0
+    issue_tile(0);
+    fence();
+    __builtin_amdgcn_s_waitcnt(0x0070);  // everything has landed, the bias store is done
+    fence();
+  }
+  barrier();
+
+  int buf = 0;
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = j_begin + t * JT;
+    const int nbuf = buf ^ 1;
+    // the bias terms of tile t + 1 were requested a tile ago, ahead of tile t's keys, which have
+    // landed; the other buffer was read during tile t - 1, which every wavefront has left
+    store_bias(nbuf);
+    issue_bias(j0 + 2 * JT);
+    issue_tile(nbuf);
+    fence();
+
+#pragma unroll
+    for (int js = 0; js < NSUB; ++js) {
+      const unsigned* yrow = lds_k[buf][0] + (js * 32 + li) * ROWH;
+      float kbias = ds_read4(&lds_b[buf][js * 32 + li]);
+      // hi*hi of both row blocks, the key operands one step ahead of their MFMAs
+      u32x4 ks[2];
+      ks[0] = ds_read16(yrow + (((0 + h) ^ (li & 15)) << 2));
+      f32x16 acc[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk) {
+        wait_lds();
+        if (kk + 1 < KK16) ks[(kk + 1) & 1] = ds_read16(yrow + (((2 * (kk + 1) + h) ^ (li & 15)) << 2));
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = mfma16(ks[kk & 1], xh[rb][kk], acc[rb]);
+      }
+      fence();
+      asm volatile("" : "+v"(kbias));  // (read before the first wait above)
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        // + key bias - running maximum: A = [bias_j, 1], B = [1, -M_i]
+        acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(h ? 1.0f : kbias, h ? -run_m[rb] : 1.0f,
+                                                       acc[rb], 0, 0, 0);
+        const float tmax = max16(acc[rb]);
+        // every logit of the unit at least 2^40 below its row's running maximum, whatever the
+        // cross products add: nothing of it could change the fp32 sums
+        if (started[rb] && !wave_any(tmax + corr[rb] > skip_below)) {
+          ++n_ended;
+          continue;
+        }
+        // ---- the unit goes on: cross products on the lo planes, then the online soft-max ----
+        {
+          // (both planes of the keys again from LDS, four steps at a time: the registers of the
+          // first pass are free by now)
+          const unsigned* ylo = lds_k[buf][1] + (js * 32 + li) * ROWH;
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            u32x4 kh[KK16 / 2], kl[KK16 / 2];
+#pragma unroll
+            for (int k4 = 0; k4 < KK16 / 2; ++k4) {
+              const int kk = half * (KK16 / 2) + k4;
+              kh[k4] = ds_read16(yrow + (((2 * kk + h) ^ (li & 15)) << 2));
+              kl[k4] = ds_read16(ylo + (((2 * kk + h) ^ (li & 15)) << 2));
+            }
+            wait_lds();
+#pragma unroll
+            for (int k4 = 0; k4 < KK16 / 2; ++k4) {
+              const int kk = half * (KK16 / 2) + k4;
+              acc[rb] = mfma16(kh[k4], xl[rb][kk], acc[rb]);
+              acc[rb] = mfma16(kl[k4], xh[rb][kk], acc[rb]);
+            }
+          }
+          float tm = max16(acc[rb]);
+          {
+            float a = tm, b = tm;
+            swap_halves(a, b);
+            tm = fmaxf(a, b);  // the row's largest logit of the unit, relative to run_m
+          }
+          // the key of the row's largest logit so far (absolute raw units; lane-private, the two
+          // half-waves are merged at the end)
+          if (track) {
+            const int jb = j0 + js * 32 + 4 * h;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float v = acc[rb][r] + run_m[rb];
+              if (v > best_v[rb]) {
+                best_v[rb] = v;
+                best_j[rb] = jb + 8 * (r / 4) + (r % 4);
+              }
+            }
+          }
+          const bool first = !started[rb];
+          const float delta = first ? tm : fmaxf(tm, 0.f);
+          const float cc = -delta * lscale;
+          float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            ps0 += fast_exp2(__builtin_fmaf(acc[rb][r], lscale, cc));
+            ps1 += fast_exp2(__builtin_fmaf(acc[rb][r + 1], lscale, cc));
+          }
+          const float resc = first ? 0.f : fast_exp2(cc);
+          run_s[rb] = run_s[rb] * resc + (ps0 + ps1);
+          run_m[rb] += delta;
+          started[rb] = true;
+        }
+      }
+    }
+
+    // tile t + 1 has landed (and with it the bias terms requested ahead of it), this wavefront's
+    // bias store is done; after the barrier both are visible and every wavefront is done
+    // reading tile t
+    fence();
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    fence();
+    barrier();
+    buf = nbuf;
+  }
+  fence();
+  __builtin_amdgcn_s_waitcnt(0x0070);  // what was fetched past the chunk: let it land before the end
+
+  // unit counts of this wavefront for the variant choice on the device
+  if (args.sel != nullptr && lane == 0 && ntiles > 0) {
+    const int slot = blockIdx.x % kSelSlots;
+    atomicAdd(&args.sel[kSelEnded + slot], n_ended);
+    atomicAdd(&args.sel[kSelUnits + slot], (unsigned)(ntiles * NSUB * RB));
+  }
+
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = row0 + rb * 32 + li;
+    const float s = run_s[rb] + xor32(run_s[rb]);
+    const float M2 = run_m[rb] * lscale;
+    float bv = best_v[rb];
+    int bj = best_j[rb];
+    const float ov = xor32(bv);
+    const int oj = __shfl_xor(bj, 32, 64);
+    if (ov > bv || (ov == bv && oj >= 0 && (bj < 0 || oj < bj))) bj = oj;
+    if (row < sd.nq && h == 0) {
+      if (sd.splits == 1) {
+        epilogue_scalar(sd.ep, row, M2, s, 0.f);
+        if (track && bj >= 0) sd.best_key[row] = bj;
+      } else {
+        const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+        *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
+        if (sd.part_best != nullptr) sd.part_best[pr] = bj;
+      }
+    }
+  }
+}
+
+}  // namespace fs

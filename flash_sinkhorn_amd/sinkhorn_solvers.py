@@ -35,6 +35,19 @@ COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_
 # 100,000: 1.4-1.8x); below, its start-up per key chunk outweighs what the test saves
 _COARSE_MIN_ROWS = 24000
 _COARSE_MIN_STEPS = 8
+# rows of 65 .. 128 columns (a kernel without carried margins, but with twice the matrix work per
+# tile to save): from fewer rows on
+_COARSE_MIN_ROWS_WIDE = 8000
+
+
+def _coarse_rows_ok(xf, yf):
+    """Clouds large enough, and rows narrow enough, for the variant with the coarse tile test."""
+    d = xf.shape[1]
+    if d > 128:
+        return False
+    need = _COARSE_MIN_ROWS if d <= 64 else _COARSE_MIN_ROWS_WIDE
+    return min(xf.shape[0], yf.shape[0]) >= need
+
 
 # Reference switches from the one-launch step to two launches at this n
 # (sinkhorn_solvers.py:463-468).  Both give the same numbers; here the one-launch
@@ -113,8 +126,7 @@ def sinkhorn_flashstyle_alternating(
     # the kernel variant with the coarse tile test (see COARSE_TEST): every half-update starts
     # its rows from the keys of the same half-update one iteration earlier
     coarse = False
-    if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
-            and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
+    if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and _coarse_rows_ok(xf, yf)
             and int(n_iters) >= _COARSE_MIN_STEPS):
         coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
     kw = dict(cost_scale=cost_scale, allow_tf32=allow_tf32, use_exp2=use_exp2,
@@ -222,8 +234,7 @@ def sinkhorn_flashstyle_symmetric(
     coarse = False
     fixed_eps = all(e == eps_list[0] for e in eps_list)
     if (fused and not use_labels and _lib.TILE_SKIP
-            and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
-            and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
+            and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and _coarse_rows_ok(xf, yf)
             and len(eps_list) >= _COARSE_MIN_STEPS):
         if fixed_eps:
             coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)
@@ -390,8 +401,7 @@ def sinkhorn_flashstyle_symmetric_self_pair(
     # the kernel variant with the coarse tile test, under the single-problem solver's conditions
     coarse = False
     fixed_eps = all(e == ex[0] for e in ex) and all(e == ey[0] for e in ey)
-    if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and xf.shape[1] <= 64
-            and min(xf.shape[0], yf.shape[0]) >= _COARSE_MIN_ROWS
+    if (_lib.TILE_SKIP and (allow_tf32 or _lib.STRICT_OPERANDS == "fp16x2") and _coarse_rows_ok(xf, yf)
             and min(len(ex), len(ey)) >= _COARSE_MIN_STEPS):
         if fixed_eps:
             coarse = "auto" if COARSE_TEST is None else bool(COARSE_TEST)

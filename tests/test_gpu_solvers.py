@@ -614,7 +614,8 @@ def _clustered(rng, n, d, k=8, spread=2.0):
 
 @pytest.mark.parametrize("n,m,d,eps,sort", [(3000, 4100, 64, 0.01, True), (3000, 4100, 64, 0.01, False),
                                             (2100, 2300, 20, 0.3, False), (129, 1000, 3, 0.05, True),
-                                            (40, 33, 16, 0.5, False)])
+                                            (40, 33, 16, 0.5, False), (2500, 3100, 128, 0.02, True),
+                                            (1100, 2300, 100, 0.3, False), (70, 200, 65, 0.1, False)])
 def test_coarse_tile_test_leaves_results_unchanged(n, m, d, eps, sort):
     """FS_FLAG_COARSE_TEST (tiles tested after their hi*hi plane product, running maximum started
     from 64 sampled keys) against the oracle and against the launch without the flag, on peaked
@@ -640,7 +641,8 @@ def test_coarse_tile_test_leaves_results_unchanged(n, m, d, eps, sort):
     assert rel_err(f1, f0.cpu().numpy()) < 2e-6 and rel_err(g1, g0.cpu().numpy()) < 2e-6
 
 
-@pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2100, 2300, 20, 0.3), (700, 5000, 33, 0.02)])
+@pytest.mark.parametrize("n,m,d,eps", [(3000, 4100, 64, 0.01), (2100, 2300, 20, 0.3), (700, 5000, 33, 0.02),
+                                       (2200, 3300, 128, 0.02), (900, 2600, 80, 0.1)])
 def test_coarse_test_starts_rows_from_the_keys_of_the_last_step(n, m, d, eps):
     """On prepared planes the kernel with the coarse tile test keeps, per row, the key that held
     the row's largest logit, and starts the next launch from the row's current logit at that key.
@@ -860,6 +862,53 @@ def test_solver_with_the_coarse_tile_test_equals_the_plain_solve(monkeypatch, va
         assert float((u - v).abs().max()) < 2e-6 * scale
     for u, v in zip(px, wu):
         assert float((u - v).abs().max()) < 2e-6 * scale
+
+
+@pytest.mark.parametrize("variant", [True, None])
+@pytest.mark.parametrize("d", [128, 100])
+def test_solvers_with_the_coarse_tile_test_on_rows_of_65_to_128_columns(monkeypatch, variant, d):
+    """``lse_coarse128_kernel``: the same test on wider rows (no carried margins), forced or
+    chosen on the device, in the symmetric solver, the alternating solver (balanced in the other
+    convention, and unbalanced) and the paired self problems; against the plain solves and, for
+    the symmetric solve, the fp64 oracle."""
+    import flash_sinkhorn_amd.sinkhorn_solvers as solvers
+    rng = np.random.default_rng(33 + d)
+    n, m = 2300, 2700
+    x, _ = _clustered(rng, n, d, spread=0.4)
+    y, _ = _clustered(rng, m, d, spread=0.4)
+    x, y = 0.3 * x, 0.3 * y
+    a = rng.random(n).astype(np.float32) + 0.5
+    b = rng.random(m).astype(np.float32) + 0.5
+    a, b = a / a.sum(), b / b.sum()
+    X, Y, A, B = dev(x, y, a, b)
+    kw = dict(use_epsilon_scaling=False, eps=0.05, n_iters=20, allow_tf32=False)
+    akw = [dict(eps=0.05, n_iters=10, allow_tf32=False, reach=1.5),
+           dict(eps=0.05, n_iters=10, allow_tf32=False, ott_convention=True)]
+    monkeypatch.setattr(solvers, "_COARSE_MIN_ROWS_WIDE", 2048)
+
+    def run(info):
+        return (solvers.sinkhorn_flashstyle_symmetric(X, Y, A, B, solve_info=info, **kw),
+                [solvers.sinkhorn_flashstyle_alternating(X, Y, A, B, **k) for k in akw],
+                solvers.sinkhorn_flashstyle_symmetric_self_pair(X, A, Y, B, **kw))
+
+    monkeypatch.setattr(solvers, "COARSE_TEST", False)
+    info0, info1 = {}, {}
+    want = run(info0)
+    assert info0["coarse"] is False
+    monkeypatch.setattr(solvers, "COARSE_TEST", variant)
+    got = run(info1)
+    assert info1["coarse"] == ("auto" if variant is None else variant)
+    assert info1["prepared"].variant_state()["tiles_tested"] > 0
+    scale = float((X * X).sum(dim=1).max())
+    for u, v in zip(got[0], want[0]):
+        assert float((u - v).abs().max()) < 2e-6 * scale
+    for g_alt, w_alt in zip(got[1], want[1]):
+        for u, v in zip(g_alt, w_alt):
+            assert float((u - v).abs().max()) < 2e-6 * scale
+    for u, v in zip(got[2][0] + got[2][1], want[2][0] + want[2][1]):
+        assert float((u - v).abs().max()) < 2e-6 * scale
+    wf, wg = oracle.sinkhorn_symmetric(x, y, a, b, eps=0.05, n_iters=20, use_epsilon_scaling=False)[:2]
+    assert rel_err(got[0][0], wf) < RTOL and rel_err(got[0][1], wg) < RTOL
 
 
 @pytest.mark.parametrize("extra", [dict(), dict(reach=1.5), dict(reach_x=0.8, reach_y=2.0)])
