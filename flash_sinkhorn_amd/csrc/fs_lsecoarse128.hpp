@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
   static_assert(PPRH == 16 && PER_PLANE == 4, "64 keys x 16 pieces: four direct loads per lane and plane");
 
   __shared__ __attribute__((aligned(16))) unsigned lds_k[2][2][JT * ROWH];  // [buffer][plane]
-  __shared__ __attribute__((aligned(16))) float lds_b[2][JT];               // key bias, raw units
+  __shared__ __attribute__((aligned(16))) float lds_b[2][3][JT];            // the key bias terms as given
 
   // variant chosen on the device: the launch of the variant that was not chosen ends here
   if (args.sel_pred && args.sel[kSelWord] != args.sel_want) return;
@@ -129,14 +129,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
   // ---- key tiles: lane idx of instruction c fills LDS slot idx of a plane's buffer and fetches
   // the piece that belongs there (slot = piece ^ (row & 15)); the plane buffers end in zero
   // rows, so tiles past the chunk are fetched like any other and masked by their bias ----
-  unsigned koff[PER_PLANE];
-#pragma unroll
-  for (int c = 0; c < PER_PLANE; ++c) {
-    const int idx = tid + 256 * c;
-    const int r = idx / PPRH;
-    const int piece = (idx % PPRH) ^ (r & 15);
-    koff[c] = (unsigned)((r * ROWW + piece * 4) * 4);
-  }
+  // (the four rounds of a plane are 16 rows apart and share the slot permutation)
+  const unsigned koff = (unsigned)(((tid / PPRH) * ROWW + (((tid % PPRH) ^ ((tid / PPRH) & 15)) * 4)) * 4);
   const char* ktile = reinterpret_cast<const char*>(sd.kplanes + (size_t)j_begin * (size_t)ROWW);
   auto issue_tile = [&](int buf) {  // the next tile in sequence
 #pragma unroll
@@ -144,46 +138,28 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
 #pragma unroll
       for (int c = 0; c < PER_PLANE; ++c)
         __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(ktile + p * ROWH * 4 + koff[c]),
+            (const __attribute__((address_space(1))) void*)(ktile + (p * ROWH + c * (256 / PPRH) * ROWW) * 4 + koff),
             (__attribute__((address_space(3))) void*)(&lds_k[buf][p][(c * 256 + wave * 64) * 4]), 16, 0, 0);
     ktile += JT * ROWW * 4;
   };
-  // ---- key bias: lane tid < 64 of the workgroup fetches the terms of key j0 + tid by loads the
-  // compiler does not see (it would wait for the key tiles with them), two tiles ahead (ahead
-  // of the next tile's keys, so that they have landed when those have), and writes the combined
-  // value to LDS one tile ahead ----
+  // ---- key bias: wavefront 0 brings the (up to three) terms of the tile's 64 keys into LDS as
+  // they are, by direct loads issued ahead of the tile's keys (the same wait covers both);
+  // absent terms re-read the first vector and are dropped when the terms are combined ----
   const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
   const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
   const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
   const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
-  float rb0 = 0.f, rb1 = 0.f, rb2 = 0.f, rpen = 0.f;
-  auto gload4 = [](const float* p) -> float {
-    float v;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
-    return v;
+  auto issue_bias = [&](int j0, int buf) {
+    if (wave == 0) {
+      const int j = max(0, min(j0 + lane, sd.nk - 1));
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sd.kb0 + j),
+                                       (__attribute__((address_space(3))) void*)(&lds_b[buf][0][0]), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb1p + j),
+                                       (__attribute__((address_space(3))) void*)(&lds_b[buf][1][0]), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb2p + j),
+                                       (__attribute__((address_space(3))) void*)(&lds_b[buf][2][0]), 4, 0, 0);
+    }
   };
-  auto issue_bias = [&](int j0) {  // three loads per lane, every lane (the counts stay uniform)
-    const int j = max(0, min(j0 + (tid & 63), j_end - 1));
-    rb0 = gload4(sd.kb0 + j);
-    rb1 = gload4(kb1p + j);
-    rb2 = gload4(kb2p + j);
-    rpen = (j0 + (tid & 63) < j_end) ? 0.f : 1.0f;
-  };
-  auto store_bias = [&](int buf) {  // (after a wait that covers the three loads)
-    asm volatile("" : "+v"(rb0), "+v"(rb1), "+v"(rb2));
-    float b = kc0 * rb0 + (has_kb1 ? kc1 * rb1 : 0.f);
-    b += (has_kb2 ? kc2 * rb2 : 0.f);
-    b = (rpen == 0.f) ? fmaxf(b, kNegBig) : kNegBig;
-    if (wave == 0) ds_write4(&lds_b[buf][lane], fmaxf(b * inv_lscale, -3.0e38f));
-  };
-  // vmcnt(n): all but the newest n vector-memory operations of this wavefront have completed
-  auto wait_vm = [&](auto newer) {
-    constexpr int n = decltype(newer)::value;
-    fence();
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (n & 15) | ((n >> 4) << 14));
-    fence();
-  };
-
   auto mfma16 = [](const u32x4& a, const u32x4& b, const f32x16& c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -224,15 +200,12 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
   }
   unsigned n_ended = 0;
 
-  // ---- prologue: bias of tiles 0 and 1, tile 0 ----
+  // ---- prologue: tile 0 and its bias terms ----
   if (ntiles > 0) {
-    issue_bias(j_begin);
-    wait_vm(std::integral_constant<int, 0>{});
-    store_bias(0);
-    issue_bias(j_begin + JT);  // consumed at the top of tile 0
+    issue_bias(j_begin, 0);
     issue_tile(0);
     fence();
-    __builtin_amdgcn_s_waitcnt(0x0070);  // everything has landed, the bias store is done
+    __builtin_amdgcn_s_waitcnt(0x0070);  // everything has landed
     fence();
   }
   barrier();
@@ -241,17 +214,17 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
   for (int t = 0; t < ntiles; ++t) {
     const int j0 = j_begin + t * JT;
     const int nbuf = buf ^ 1;
-    // the bias terms of tile t + 1 were requested a tile ago, ahead of tile t's keys, which have
-    // landed; the other buffer was read during tile t - 1, which every wavefront has left
-    store_bias(nbuf);
-    issue_bias(j0 + 2 * JT);
+    // the other buffer was read during tile t - 1, which every wavefront has left
+    issue_bias(j0 + JT, nbuf);
     issue_tile(nbuf);
     fence();
 
 #pragma unroll
     for (int js = 0; js < NSUB; ++js) {
       const unsigned* yrow = lds_k[buf][0] + (js * 32 + li) * ROWH;
-      float kbias = ds_read4(&lds_b[buf][js * 32 + li]);
+      float kb0r = ds_read4(&lds_b[buf][0][js * 32 + li]);
+      float kb1r = ds_read4(&lds_b[buf][1][js * 32 + li]);
+      float kb2r = ds_read4(&lds_b[buf][2][js * 32 + li]);
       // hi*hi of both row blocks, the key operands one step ahead of their MFMAs
       u32x4 ks[2];
       ks[0] = ds_read16(yrow + (((0 + h) ^ (li & 15)) << 2));
@@ -268,7 +241,11 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
         for (int rb = 0; rb < RB; ++rb) acc[rb] = mfma16(ks[kk & 1], xh[rb][kk], acc[rb]);
       }
       fence();
-      asm volatile("" : "+v"(kbias));  // (read before the first wait above)
+      asm volatile("" : "+v"(kb0r), "+v"(kb1r), "+v"(kb2r));  // (read before the first wait above)
+      float kbias = kc0 * kb0r + (has_kb1 ? kc1 * kb1r : 0.f);
+      kbias += (has_kb2 ? kc2 * kb2r : 0.f);
+      kbias = (j0 + js * 32 + li < j_end) ? fmaxf(kbias, kNegBig) : kNegBig;  // keys past the chunk are masked
+      kbias = fmaxf(kbias * inv_lscale, -3.0e38f);
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         // + key bias - running maximum: A = [bias_j, 1], B = [1, -M_i]
@@ -303,7 +280,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
               acc[rb] = mfma16(kl[k4], xh[rb][kk], acc[rb]);
             }
           }
-          float tm = max16(acc[rb]);
+          const float lane_max = max16(acc[rb]);
+          float tm = lane_max;
           {
             float a = tm, b = tm;
             swap_halves(a, b);
@@ -311,7 +289,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
           }
           // the key of the row's largest logit so far (absolute raw units; lane-private, the two
           // half-waves are merged at the end)
-          if (track) {
+          // (searched only when some lane's largest value of the unit beats what it has)
+          if (track && wave_any(lane_max + run_m[rb] > best_v[rb])) {
             const int jb = j0 + js * 32 + 4 * h;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -339,9 +318,8 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
       }
     }
 
-    // tile t + 1 has landed (and with it the bias terms requested ahead of it), this wavefront's
-    // bias store is done; after the barrier both are visible and every wavefront is done
-    // reading tile t
+    // tile t + 1 has landed (and with it the bias terms requested ahead of it); after the barrier
+    // both are visible and every wavefront is done reading tile t
     fence();
     __builtin_amdgcn_s_waitcnt(0x0070);
     fence();

@@ -36,8 +36,11 @@ COARSE_TEST = {"1": True, "0": False}.get(os.environ.get("FLASH_SINKHORN_COARSE_
 _COARSE_MIN_ROWS = 24000
 _COARSE_MIN_STEPS = 8
 # rows of 65 .. 128 columns (a kernel without carried margins, but with twice the matrix work per
-# tile to save): from fewer rows on
-_COARSE_MIN_ROWS_WIDE = 8000
+# tile to save): from fewer rows on (20 alternating iterations at d = 128, eps = 0.01: 8192 rows
+# per cloud 3.5 -> 3.8 ms, 12,000 rows 6.1 -> 5.1, 16,000 x 100 columns 9.3 -> 6.6, 30,000 rows
+# 28.6 -> 16.1; on a flat plan, eps = 0.5 at 16,000 rows, the device's way back to the plain
+# kernel costs 9.7 -> 11.1)
+_COARSE_MIN_ROWS_WIDE = 10000
 
 
 def _coarse_rows_ok(xf, yf):
