@@ -28,7 +28,8 @@
  *    The d <= 128 log-sum-exp kernel leaves out the exponentials of a 32 x 32 logits tile
  *    whose every entry lies more than 2^40 below its row's running maximum (they cannot
  *    change the fp32 row sums); FS_FLAG_NO_TILE_SKIP computes them all the same.
- *    FS_FLAG_COARSE_TEST (log-sum-exp entry points, default operand mode, d <= 64) applies the
+ *    FS_FLAG_COARSE_TEST (log-sum-exp entry points, default operand mode, d <= 128; the carried
+ *    margins described below exist at d <= 64 only) applies the
  *    same 2^40 criterion one stage earlier: the hi*hi plane product of a tile is tested
  *    against the running maximum, lowered by a per-row bound on the two cross products, and a
  *    tile that fails ends there (5 MFMAs instead of 13 at d = 64).  What the test can end
