@@ -1016,22 +1016,25 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
   // The one-sweep form of a two-sided step: the sides are the two orders of one pair of matrices
   // on prepared planes (the permission to run it is state, like the variant choice), two row
   // blocks per wavefront, keys split on both sides.
-  const bool sweep_base = lse2 && mode == kLse && prec == 3 && dp2 <= 64 && prepared && !coarse &&
-                          !(flags & FS_FLAG_NO_SWEEP) && ps.n > 0 && rb == 2;
+  // (rows of 65 .. 128 columns: lse_sweep128_kernel, whose workgroups take 256 query rows like
+  // lse_sweep_kernel's whatever the two-sided kernel's plan says)
+  const bool sweep_base = lse2 && mode == kLse && prec == 3 && dp2 <= 128 && prepared && !coarse &&
+                          !(flags & FS_FLAG_NO_SWEEP) && ps.n > 0 && (rb == 2 || wide);
+  auto groups256 = [&](int s) { return ceil_div(sides[s].nq, 256); };
   bool sweep_pair = sweep_base && nsides == 2;
   if (sweep_pair) {
     const Side &s0 = sides[0], &s1 = sides[1];
     sweep_pair = s0.q == s1.k && s0.k == s1.q && s0.nq == s1.nk && s0.nk == s1.nq && s0.qscale == s1.qscale &&
-                 plans[0].rb == 2 && plans[1].rb == 2 && plans[0].splits > 1 && plans[1].splits > 1 &&
-                 plans[0].igroups <= kSweepMaxGroups && sweep_col_bytes(s0.nq, s0.nk) > 0;
+                 (wide || (plans[0].rb == 2 && plans[1].rb == 2)) && plans[0].splits > 1 && plans[1].splits > 1 &&
+                 groups256(0) <= kSweepMaxGroups && sweep_col_bytes(s0.nq, s0.nk) > 0;
   }
   // ... or every side is a problem of a matrix with itself (the self problems of a debiased
   // loss): a symmetric matrix of logits, of which the one-sweep launch visits the tiles on and
   // above the diagonal of 256 x 256 blocks only
   bool sweep_self = sweep_base && !sweep_pair;
   for (int s = 0; s < nsides && sweep_self; ++s)
-    sweep_self = sides[s].q == sides[s].k && sides[s].nq == sides[s].nk && plans[s].rb == 2 &&
-                 plans[s].splits > 1 && plans[s].igroups <= kSweepMaxGroups &&
+    sweep_self = sides[s].q == sides[s].k && sides[s].nq == sides[s].nk && (wide || plans[s].rb == 2) &&
+                 plans[s].splits > 1 && groups256(s) <= kSweepMaxGroups &&
                  sweep_col_bytes(sides[s].nq, sides[s].nk) > 0;
   const bool sweep = sweep_pair || sweep_self;
   const size_t col_off = need;
@@ -1134,7 +1137,7 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
       // the counts down to half of the side's, the one that fills the last round of workgroups
       // best (two workgroups per CU at a time)
       auto choose = [&](int sidx, int items_before, int& splits_out, int& chunk_out) {
-        const int nk = a.side[sidx].nk, ig = a.side[sidx].igroups, smax = a.side[sidx].splits;
+        const int nk = a.side[sidx].nk, ig = groups256(sidx), smax = a.side[sidx].splits;
         double best = -1.0;
         int best_items = 0;
         for (int s = smax; s >= std::max(1, smax / 2); --s) {
@@ -1166,7 +1169,11 @@ int run_stream(int mode, bool sepv, Side* sides, int nsides, int64_t d, void* ws
           a.col_part_b = reinterpret_cast<float*>(static_cast<char*>(ws) + col_off_b);
         }
       }
-      if (rc == FS_OK) rc = launch_lse_sweep(a, dp2, st);
+      // (its row groups are of 256 rows; the two-sided kernel's may be of 128)
+      LaunchArgs asw = a;
+      for (int s = 0; s < nsides; ++s) asw.side[s].igroups = groups256(s);
+      if (nsides == 1) asw.side[1] = asw.side[0];
+      if (rc == FS_OK) rc = launch_lse_sweep(asw, dp2, st);
     }
     // device-chosen variant: both are enqueued, the one the state word names runs
     if (auto_sel) {
@@ -1333,7 +1340,7 @@ static size_t workspace_bytes(int op, int64_t n, int64_t m, int64_t d, bool with
   }
   if (mode == kLse && !fam.sliced) planes += coarse_aux_bytes(n) + coarse_aux_bytes(m);
   // (the one-sweep form of the symmetric step: either matrix may hold the query rows)
-  if (op == FS_OP_SYMMETRIC_STEP && !fam.sliced && dp <= 64 && with_sweep)
+  if (op == FS_OP_SYMMETRIC_STEP && !fam.sliced && dp <= 128 && with_sweep)
     planes += std::max(sweep_col_bytes(n, m), sweep_col_bytes(m, n));
   const size_t a = side_bytes(n, m) + planes, b = side_bytes(m, n) + planes;
   size_t gemm = ((mode == kLse || mode == kVec || mode == kArgmax) && fam.sliced)

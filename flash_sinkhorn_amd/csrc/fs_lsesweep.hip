@@ -59,6 +59,12 @@ int launch_lse_sweep(const LaunchArgs& a, int dp, hipStream_t st) {
     case 16: return launch_sweep_dp<16>(a, st);
     case 32: return launch_sweep_dp<32>(a, st);
     case 64: return launch_sweep_dp<64>(a, st);
+    case 128: {
+      const int items = a.sweep_self ? a.sw_items : s0.igroups * a.sw_splits;
+      hipLaunchKernelGGL((lse_sweep128_kernel<0>), dim3(8 * ((items + 7) / 8)), dim3(256), 0, st, a);
+      if (hipGetLastError() != hipSuccess) return FS_ERR_LAUNCH_FAILED;
+      return launch_finish_sweep(a, st);
+    }
   }
   return FS_ERR_UNSUPPORTED;
 }

@@ -403,6 +403,284 @@ __global__ __launch_bounds__(256, 2) void lse_sweep_kernel(const LaunchArgs args
   }
 }
 
+// The same for rows of 65 .. 128 columns.  Two row blocks of both planes are 128 registers of
+// stationary operands, which leaves no room for lse_sweep_kernel's software pipeline; this
+// kernel keeps its work-item mapping, its outputs and its merge, and does the rest plainly: a
+// workgroup of four wavefronts shares 64-key tiles with both planes in LDS (two buffers of
+// 32 KiB, the next tile and its bias terms arriving by direct loads; two workgroups per CU), a
+// wavefront takes, per 32-key sub-tile, the three plane products of both row blocks (key
+// operands one 16-column step ahead, read by hand), folds the key bias and the rows' own bias
+// in with one fp32 MFMA per block, and sums the exponentials along the rows (lane-private) and,
+// for both blocks together, along the columns (fs_colsum.hpp).  What hides the latencies is the
+// second wavefront of the SIMD.
+template <int T>
+__global__ __launch_bounds__(256, 2) void lse_sweep128_kernel(const LaunchArgs args) {
+  constexpr int DP = 128, RB = 2, JT = 64, NSUB = JT / 32, KK16 = DP / 16;
+  constexpr int ROWW = DP;        // 32-bit words per two-plane row in global memory
+  constexpr int ROWH = DP / 2;    // words per plane row in LDS
+  constexpr int PPRH = ROWH / 4;  // 16-byte pieces per plane row
+  constexpr int PER_PLANE = JT * PPRH / 256;
+  static_assert(PPRH == 16 && PER_PLANE == 4, "64 keys x 16 pieces: four direct loads per lane and plane");
+
+  __shared__ __attribute__((aligned(16))) unsigned lds_k[2][2][JT * ROWH];  // [buffer][plane]
+  __shared__ __attribute__((aligned(16))) float lds_b[2][3][JT];            // the key bias terms as given
+  __shared__ __attribute__((aligned(16))) float lds_col[2][4][2][JT];       // [tile parity][wavefront][row of 16 lanes][key]
+
+  // the step may not run this kernel, or the device chose another variant
+  if (args.sel[kSelSweep] == 0u) return;
+  if (args.sweep == 2 && args.sel[kSelWord] != 1u) return;
+  if (blockIdx.x == 0 && threadIdx.x == 0) args.sel[kSelRan] = 1u;
+
+  // work items as in lse_sweep_kernel
+  const bool self = args.sweep_self != 0;
+  const int n_items = self ? args.sw_items : args.side[0].igroups * args.sw_splits;
+  const int per_xcd = (n_items + 7) / 8;
+  int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= per_xcd || item >= n_items) return;
+  const bool second = self && item >= args.sw_items0;
+  if (second) item -= args.sw_items0;
+  const Side& sd = second ? args.side[1] : args.side[0];
+  const Side& so = self ? sd : args.side[1];
+  const int sw_chunk = second ? args.sw_chunk_b : args.sw_chunk;
+  int split, ig;
+  if (self) {
+    split = 0;
+    for (;;) {
+      const int g = self_groups_of_chunk(split, sw_chunk, sd.nk, sd.igroups);
+      if (item < g) break;
+      item -= g;
+      ++split;
+    }
+    ig = item;
+  } else {
+    split = item / sd.igroups;
+    ig = item % sd.igroups;
+  }
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int h = lane >> 5;
+  const int row0 = (ig * 4 + wave) * (32 * RB);
+  const int j_begin = self ? max(split * sw_chunk, ig * 256) : split * sw_chunk;
+  const int j_end = min(sd.nk, (split + 1) * sw_chunk);
+  const int ntiles = (j_end - j_begin + JT - 1) / JT;
+  if (ntiles <= 0) return;  // (whole workgroup: no barrier is left waiting)
+
+  const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
+  const float inv_lscale = 1.0f / lscale;
+
+  // ---- stationary planes of the query rows, and the rows' own bias (base 2) ----
+  u32x4 xh[RB][KK16], xl[RB][KK16];
+  float cx[RB], run_s[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = min(row0 + rb * 32 + li, sd.nq - 1);
+    const unsigned* qrow = sd.qplanes + (size_t)row * (size_t)ROWW;
+#pragma unroll
+    for (int kk = 0; kk < KK16; ++kk) {
+      xh[rb][kk] = *reinterpret_cast<const u32x4*>(qrow + 8 * kk + 4 * h);
+      xl[rb][kk] = *reinterpret_cast<const u32x4*>(qrow + ROWH + 8 * kk + 4 * h);
+    }
+    float r = so.kc0 * so.kb0[row];
+    if (so.kb1 != nullptr) r += so.kc1 * so.kb1[row];
+    if (so.kb2 != nullptr) r += so.kc2 * so.kb2[row];
+    // rows past the last one (they repeat it) must not reach the column sums
+    cx[rb] = (row0 + rb * 32 + li < sd.nq) ? fmaxf(r, kNegBig) : kNegBig;
+    run_s[rb] = 0.f;
+  }
+
+  // ---- LDS access by hand (the compiler cannot tell a read of one buffer from the direct loads
+  // filling the other and would make every access wait for them) ----
+  auto lds_addr = [](const void* p) {
+    return (unsigned)(size_t)(const __attribute__((address_space(3))) void*)p;
+  };
+  auto ds_read16 = [&](const unsigned* p) -> u32x4 {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+    return v;
+  };
+  auto ds_read4 = [&](const float* p) -> float {
+    float v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+    return v;
+  };
+  auto ds_write4 = [&](float* p, float v) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(lds_addr(p)), "v"(v) : "memory");
+  };
+  auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+  auto wait_lds = [&]() {  // lgkmcnt(0), and nothing moves across
+    fence();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    fence();
+  };
+  auto barrier = [&]() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  // ---- key tiles: lane tid of round c fills LDS slot tid of a plane's buffer and fetches the
+  // piece that belongs there (slot = piece ^ (row & 15); the four rounds of a plane are 16 rows
+  // apart and share the permutation); the planes end in zero rows, so tiles past the chunk are
+  // fetched like any other and masked by their bias ----
+  const unsigned koff = (unsigned)(((tid / PPRH) * ROWW + (((tid % PPRH) ^ ((tid / PPRH) & 15)) * 4)) * 4);
+  const char* ktile = reinterpret_cast<const char*>(sd.kplanes + (size_t)j_begin * (size_t)ROWW);
+  auto issue_tile = [&](int buf) {  // the next tile in sequence
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int c = 0; c < PER_PLANE; ++c)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(ktile + (p * ROWH + c * (256 / PPRH) * ROWW) * 4 + koff),
+            (__attribute__((address_space(3))) void*)(&lds_k[buf][p][(c * 256 + wave * 64) * 4]), 16, 0, 0);
+    ktile += JT * ROWW * 4;
+  };
+  // the (up to three) bias terms of the tile's keys as they are, by direct loads of wavefront 0
+  // ahead of the tile's keys; absent terms re-read the first vector and are dropped later
+  const float kc0 = sd.kc0, kc1 = sd.kc1, kc2 = sd.kc2;
+  const bool has_kb1 = sd.kb1 != nullptr, has_kb2 = sd.kb2 != nullptr;
+  const float* kb1p = has_kb1 ? sd.kb1 : sd.kb0;
+  const float* kb2p = has_kb2 ? sd.kb2 : sd.kb0;
+  auto issue_bias = [&](int j0, int buf) {
+    if (wave == 0) {
+      const int j = max(0, min(j0 + lane, sd.nk - 1));
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sd.kb0 + j),
+                                       (__attribute__((address_space(3))) void*)(&lds_b[buf][0][0]), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb1p + j),
+                                       (__attribute__((address_space(3))) void*)(&lds_b[buf][1][0]), 4, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb2p + j),
+                                       (__attribute__((address_space(3))) void*)(&lds_b[buf][2][0]), 4, 0, 0);
+    }
+  };
+  auto mfma16 = [](const u32x4& a, const u32x4& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  };
+  // the sums of a finished tile's keys over the four wavefronts and their two rows of 16 lanes,
+  // in a fixed order, by one wavefront
+  const int my_key = colsum_key(li, h);
+  float* colp = (second ? args.col_part_b : args.col_part) + (size_t)ig * (size_t)sd.nk;
+  auto flush = [&](int tile) {
+    const float* c = &lds_col[tile & 1][0][0][0];
+    float v[8];
+#pragma unroll
+    for (int w = 0; w < 8; ++w) v[w] = ds_read4(c + w * JT + lane);
+    wait_lds();
+    float sum = v[0] + v[1];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) sum += v[2 * w] + v[2 * w + 1];
+    const int j = j_begin + tile * JT + lane;
+    if (j < j_end) colp[j] = sum;
+  };
+
+  // ---- prologue: tile 0 and its bias terms ----
+  issue_bias(j_begin, 0);
+  issue_tile(0);
+  fence();
+  __builtin_amdgcn_s_waitcnt(0x0070);  // everything has landed
+  fence();
+  barrier();
+
+  int buf = 0;
+  for (int t = 0; t < ntiles; ++t) {
+    const int j0 = j_begin + t * JT;
+    const int nbuf = buf ^ 1;
+    // the other buffer was read during tile t - 1, which every wavefront has left
+    issue_bias(j0 + JT, nbuf);
+    issue_tile(nbuf);
+    fence();
+    // (every wavefront wrote its sums of tile t - 1 before the barrier it has just passed, and
+    // writes those of tile t + 1 only behind the next one)
+    if (t >= 1 && wave == (t & 3)) flush(t - 1);
+
+#pragma unroll
+    for (int js = 0; js < NSUB; ++js) {
+      const unsigned* yhi = lds_k[buf][0] + (js * 32 + li) * ROWH;
+      const unsigned* ylo = lds_k[buf][1] + (js * 32 + li) * ROWH;
+      float kb0r = ds_read4(&lds_b[buf][0][js * 32 + li]);
+      float kb1r = ds_read4(&lds_b[buf][1][js * 32 + li]);
+      float kb2r = ds_read4(&lds_b[buf][2][js * 32 + li]);
+      // the three plane products of both row blocks, the key operands one step ahead
+      u32x4 kh[2], kl[2];
+      kh[0] = ds_read16(yhi + (((0 + h) ^ (li & 15)) << 2));
+      kl[0] = ds_read16(ylo + (((0 + h) ^ (li & 15)) << 2));
+      f32x16 acc[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rb][r] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KK16; ++kk) {
+        wait_lds();
+        if (kk + 1 < KK16) {
+          kh[(kk + 1) & 1] = ds_read16(yhi + (((2 * (kk + 1) + h) ^ (li & 15)) << 2));
+          kl[(kk + 1) & 1] = ds_read16(ylo + (((2 * (kk + 1) + h) ^ (li & 15)) << 2));
+        }
+        // (plane products from the lowest weight to hi*hi; the two blocks alternate)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = mfma16(kl[kk & 1], xh[rb][kk], acc[rb]);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = mfma16(kh[kk & 1], xl[rb][kk], acc[rb]);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) acc[rb] = mfma16(kh[kk & 1], xh[rb][kk], acc[rb]);
+      }
+      fence();
+      asm volatile("" : "+v"(kb0r), "+v"(kb1r), "+v"(kb2r));  // (read before the first wait above)
+      float kbias = kc0 * kb0r + (has_kb1 ? kc1 * kb1r : 0.f);
+      kbias += (has_kb2 ? kc2 * kb2r : 0.f);
+      kbias = (j0 + js * 32 + li < j_end) ? fmaxf(kbias, kNegBig) : kNegBig;  // keys past the chunk are masked
+      kbias = fmaxf(kbias * inv_lscale, -3.0e38f);
+      float c[16];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        // + key bias + the row's own bias: A = [bias_j, 1], B = [1, r_i]
+        acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(h ? 1.0f : kbias, h ? fmaxf(cx[rb] * inv_lscale, -3.0e38f) : 1.0f,
+                                                       acc[rb], 0, 0, 0);
+        float ps0 = 0.f, ps1 = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const float e0 = fast_exp2(acc[rb][r] * lscale);
+          const float e1 = fast_exp2(acc[rb][r + 1] * lscale);
+          ps0 += e0;
+          ps1 += e1;
+          if (rb == 0) {
+            c[r] = e0;
+            c[r + 1] = e1;
+          } else {
+            c[r] += e0;
+            c[r + 1] += e1;
+          }
+        }
+        run_s[rb] += ps0 + ps1;
+      }
+      ds_write4(&lds_col[t & 1][wave][li >> 4][js * 32 + my_key], colsum_all(c, li));
+    }
+
+    // tile t + 1 has landed (and with it its bias terms), this wavefront's column sums are
+    // written; after the barrier all of it is visible and every wavefront is done reading tile t
+    fence();
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    fence();
+    barrier();
+    buf = nbuf;
+  }
+  fence();
+  __builtin_amdgcn_s_waitcnt(0x0070);  // what was fetched past the chunk: let it land before the end
+  fence();
+  if (wave == 0) flush(ntiles - 1);
+
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = row0 + rb * 32 + li;
+    const float s = run_s[rb] + xor32(run_s[rb]);
+    if (row < sd.nq && h == 0) {
+      const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
+      *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(-cx[rb], s);
+    }
+  }
+}
+
 // Merge after lse_sweep_kernel: rows of side 0 add their partial row sums over the key chunks
 // (all taken under the same offset, the row's own bias), rows of side 1 (the keys) add the
 // column sums of the workgroup row groups.  A sum outside [2^kSweepFailLo, 2^kSweepFailHi]

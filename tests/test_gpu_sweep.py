@@ -95,7 +95,7 @@ class _Outs(list):
 
 
 @pytest.mark.parametrize("n,m,d", [(5000, 4700, 64), (2100, 9000, 32), (9100, 2300, 16),
-                                   (4100, 4099, 5), (3000, 3300, 40)])
+                                   (4100, 4099, 5), (3000, 3300, 40), (3100, 2900, 128), (2048, 5100, 70)])
 def test_one_sweep_steps_equal_two_sided_steps(n, m, d):
     x, y, a, b = _problem(n + d, n, m, d)
     worst, allowed, outs = _steps(x, y, a, b, [0.05] * 10, sweep=True, check_oracle_at=(5, 9))
@@ -187,7 +187,7 @@ def _self_steps(x, y, a, b, eps_list, *, sweep, alpha=0.5, pair=True):
 
 
 @pytest.mark.parametrize("n,m,d", [(4200, 3100, 32), (2048, 2500, 64), (5000, 6100, 16), (2300, 9000, 7),
-                                   (2300, 2100, 200), (2048, 3900, 136)])
+                                   (2300, 2100, 200), (2048, 3900, 136), (2700, 3300, 128), (4500, 2100, 96)])
 def test_self_problems_take_the_tiles_on_and_above_the_diagonal(n, m, d):
     """The two self problems of a debiased loss: the matrix of logits is symmetric once both
     biases are inside the exponent, and the one-sweep launch visits only the key tiles at or
