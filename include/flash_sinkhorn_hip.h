@@ -68,11 +68,11 @@
  *    host: the same inputs take the same path on every run, and the calls can be captured into
  *    a graph.
  *    One more form of a two-sided step lives in the same state (fs_symmetric_step(s) and
- *    fs_self_pair_steps on prepared operands, default operand mode, d <= 64 or d > 128, every
- *    matrix of 2048 rows or more): when the
- *    sums of a step show that the potentials have settled, the next step (under the same eps or
- *    another: on a flat plan the sums hardly move with eps) computes every logit once and takes both sides' sums from the same
- *    exponentials (row sums and column sums of 2^(logit + both biases), no running maximum).
+ *    fs_self_pair_steps on prepared operands, default operand mode, every matrix of 2048 rows
+ *    or more): when the sums of a step show that the potentials have settled, the next step
+ *    (under the same eps or another: on a flat plan the sums hardly move with eps) computes
+ *    every logit once and takes both sides' sums from the same exponentials (row sums and
+ *    column sums of 2^(logit + both biases), no running maximum).
  *    Its merge checks every sum against the range in which that is exact in fp32 and has the
  *    two-sided kernel, enqueued behind it, redo the step otherwise: results stay within fp32
  *    rounding of the two-sided step whatever a caller does to the potentials between steps,
