@@ -9,6 +9,10 @@ one LSE half-update (2nmd), gradient of one side (4nmd), plan-vector (2nmd), pla
 (4nmd), mat5 (6nmd) and the hard c-transform (2nmd); at c3 also the gradient after a solve on clustered clouds,
 with and without the keys the solve carried; then end-to-end wall times of the five configurations
 through the public API (solver loops, autograd, CG included).
+
+``python -m flash_sinkhorn_amd.op_timings clocks`` instead runs four operations in a loop for a
+few seconds each and prints the shader clock that ``rocm-smi`` reports meanwhile (the clock the
+chip sustains under that load, against the one it reaches for a plain device copy).
 """
 from __future__ import annotations
 
@@ -186,7 +190,81 @@ def gradient_after_solve(name):
     return out
 
 
+def clocks_under_load(seconds=4.0):
+    """Shader clock (rocm-smi, sampled every 0.15 s from a second thread) while one operation
+    runs back to back: the large-d plan-matrix and plan-vector products, the two-sided
+    symmetric step at the benchmark size, and a 1 GiB device copy for comparison."""
+    import re
+    import subprocess
+    import threading
+
+    def sclk():
+        try:
+            out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True,
+                                 timeout=10).stdout
+            hit = re.search(r"sclk clock level[^(]*\((\d+)Mhz\)", out)
+            return int(hit.group(1)) if hit else None
+        except (OSError, subprocess.SubprocessError):
+            return None
+
+    def measure(label, fn):
+        fn()
+        torch.cuda.synchronize()
+        stop, samples = [False], []
+
+        def poll():
+            while not stop[0]:
+                samples.append(sclk())
+                time.sleep(0.15)
+        th = threading.Thread(target=poll)
+        th.start()
+        t0, launches = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            launches += 20
+        dt = time.perf_counter() - t0
+        stop[0] = True
+        th.join()
+        got = sorted(v for v in samples[2:-1] if v is not None)
+        return {"operation": label, "ms_per_launch": round(dt / launches * 1e3, 3),
+                "sclk_mhz_min_median_max": [got[0], got[len(got) // 2], got[-1]] if got else None,
+                "samples": len(got)}
+
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    n, m, d, eps = SHAPES["c5"]
+    X = torch.randn(n, d, device="cuda", generator=gen) * (2.0 / d ** 0.5)
+    Y = torch.randn(m, d, device="cuda", generator=gen) * (2.0 / d ** 0.5)
+    la = torch.full((n,), 1.0 / n, device="cuda").log()
+    lb = torch.full((m,), 1.0 / m, device="cuda").log()
+    f, g = -(X * X).sum(1), -(Y * Y).sum(1)
+    V = torch.randn(m, d, device="cuda", generator=gen)
+    v = torch.randn(m, device="cuda", generator=gen)
+    out = [measure("c5 plan-matrix product (plan_gemm_kernel)", lambda: apply_plan_mat_flashstyle(
+        X, Y, f, g, la, lb, V, eps=eps, axis=1, allow_tf32=False))]
+    out.append(measure("c5 plan-vector product (lse_gemm_kernel)", lambda: apply_plan_vec_flashstyle(
+        X, Y, f, g, la, lb, v, eps=eps, axis=1, allow_tf32=False)))
+    n, m, d, eps = SHAPES["c3"]
+    X = torch.randn(n, d, device="cuda", generator=gen) * (2.0 / d ** 0.5)
+    Y = torch.randn(m, d, device="cuda", generator=gen) * (2.0 / d ** 0.5)
+    la = torch.full((n,), 1.0 / n, device="cuda").log()
+    lb = torch.full((m,), 1.0 / m, device="cuda").log()
+    fh, gh = -(X * X).sum(1), -(Y * Y).sum(1)
+    kw = dict(cost_scale=1.0, alpha=0.5, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    out.append(measure("c3 symmetric step alone (two-sided lse2_kernel, planes converted in the call)",
+                       lambda: _symmetric_step_raw(X, Y, fh, gh, la, lb, eps, **kw)))
+    src = torch.empty(1 << 28, device="cuda")
+    dst = torch.empty_like(src)
+    out.append(measure("1 GiB device copy", lambda: dst.copy_(src)))
+    return out
+
+
 def main(argv):
+    if "clocks" in argv:
+        for line in clocks_under_load():
+            print(json.dumps(line), flush=True)
+        return
     names = [a for a in argv if a in SHAPES] or list(SHAPES)
     for name in names:
         print(json.dumps(kernel_timings(name)), flush=True)
