@@ -290,3 +290,26 @@ def test_solver_results_do_not_depend_on_the_form(monkeypatch):
     wf, wg = oracle.sinkhorn_symmetric(x, y, a, b, eps=0.1, n_iters=30, use_epsilon_scaling=False)[:2]
     for got, want in ((f1, wf), (g1, wg)):
         assert np.abs(got.cpu().numpy() - want).max() / np.abs(want).max() < 1e-4
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_shapes_take_the_form_without_changing_results(seed):
+    """Seeded random shapes on both sides of each kernel family's width limits (64, 128), row
+    counts from one workgroup's worth down to a single row, zero weights now and then: steps of
+    xy pairs, of the pair of self problems and of a single one.  eps stays below 0.3: at large eps
+    a self problem's potentials nearly cancel against |x|^2, and an error measured against the
+    largest potential says little."""
+    rng = np.random.default_rng(4000 + seed)
+    widths = [1, 3, 16, 17, 33, 63, 64, 65, 70, 96, 127, 128, 129, 136, 200, 257, 300]
+    for case in range(14):
+        d = int(rng.choice(widths))
+        n, m = int(rng.integers(1, 2600)), int(rng.integers(1, 2600))
+        eps = float(10 ** rng.uniform(-1.7, -0.55))
+        steps = int(rng.integers(3, 8))
+        kind = int(rng.integers(0, 3))  # xy pair, pair of self problems, one self problem
+        x, y, a, b = _problem(int(rng.integers(0, 1 << 30)), n, m, d, zero_weights=bool(rng.random() < 0.3))
+        if kind == 0:
+            worst, allowed, outs = _steps(x, y, a, b, [eps] * steps, sweep=True)
+        else:
+            worst, allowed, outs = _self_steps(x, y, a, b, [eps] * steps, sweep=True, pair=(kind == 1))
+        assert worst < 2e-6, (seed, case, n, m, d, eps, steps, kind, worst)
