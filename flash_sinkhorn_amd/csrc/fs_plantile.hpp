@@ -201,12 +201,15 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
   };
 
   f32x16 oacc[kHasO ? RB : 1][kHasO ? NCB : 1];
-  float run_m[RB], run_s[RB], run_o[RB];
-  int best_j[RB];  // kArgmax: run_m is the largest raw value so far, best_j its key
+  // run_m: (kArgmax) the largest raw value so far, best_j its key; run_c: the constant of the
+  // exponentials, kPtUp minus the running maximum in base-2 units
+  float run_m[RB], run_c[RB], run_s[RB], run_o[RB];
+  int best_j[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     best_j[rb] = 0;
     run_m[rb] = (MODE == kArgmax) ? -3.0e38f : 0.f;
+    run_c[rb] = kPtUp;
     run_s[rb] = 0.f;
     run_o[rb] = 0.f;
     if constexpr (kHasO) {
@@ -234,7 +237,7 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
       seeded = __builtin_amdgcn_ballot_w64(ok) == ~0ull;
       if (seeded) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) run_m[rb] = sv[rb];
+        for (int rb = 0; rb < RB; ++rb) run_c[rb] = __builtin_fmaf(-sv[rb], lscale, kPtUp);
       }
     }
   }
@@ -392,25 +395,30 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
           }
           continue;
         }
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
+        // + key bias.  The logits stay in absolute raw units and the running maximum enters in
+        // the exponent only (run_c): a maximum far below the unit's logits (a first
+        // tile of keys without weight, a hint that names such a key) then costs no digits,
+        // which its subtraction here would
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
 
-        // ---- lazy lane-private soft-max (the two half-waves of a query share run_m) ----
+        // ---- lazy lane-private soft-max (the two half-waves of a query share run_c) ----
         float tmax = fmaxf(acc[0], acc[1]);
 #pragma unroll
         for (int r = 2; r < 16; ++r) tmax = fmaxf(tmax, acc[r]);
         const bool first = (t == 0 && js == 0 && !seeded);
+        // the unit's largest exponent: kPtUp above its distance to the running maximum
+        const float trel = __builtin_fmaf(tmax, lscale, run_c[rb]);
         // every logit of the unit 2^40 below the running maximum (itself never above the row's
         // largest logit): its exponentials could not change the fp32 sums
-        if (!first && !wave_any(tmax * lscale > skip_below)) continue;
-        float cc = 0.f;
-        if (first || wave_any(tmax * lscale > kPtLazyThresh)) {
+        if (!first && !wave_any(trel > skip_below + kPtUp)) continue;
+        if (first || wave_any(trel > kPtLazyThresh + kPtUp)) {
           float a = tmax, b = tmax;
           swap_halves(a, b);
           const float tm = fmaxf(a, b);
-          const float delta = (first || tm * lscale > kPtLazyThresh) ? tm : 0.f;
-          cc = -delta * lscale;
-          const float resc = first ? 0.f : fast_exp2(cc);
-          run_m[rb] += delta;
+          const bool up = first || __builtin_fmaf(tm, lscale, run_c[rb]) > kPtLazyThresh + kPtUp;
+          const float c_new = up ? __builtin_fmaf(-tm, lscale, kPtUp) : run_c[rb];
+          const float resc = first ? 0.f : fast_exp2(c_new - run_c[rb]);
+          run_c[rb] = c_new;
           run_s[rb] *= resc;
           run_o[rb] *= resc;
           if constexpr (kHasO) {
@@ -422,10 +430,9 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
         }
         float p[16];
         float ps = 0.f;
-        const float ccu = cc + kPtUp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, ccu));
+          p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, run_c[rb]));
           ps += p[r];
         }
         run_s[rb] += ps;
@@ -507,7 +514,7 @@ __global__ __launch_bounds__(256, (MODE == kMat5 && DP == 128) ? 1 : 2) void pla
       }
       continue;
     }
-    const float M = (ntiles > 0) ? run_m[rb] * lscale - kPtUp : kNegBig;
+    const float M = (ntiles > 0) ? -run_c[rb] : kNegBig;
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float o = run_o[rb] + xor32(run_o[rb]);
     if (sd.splits == 1) {
