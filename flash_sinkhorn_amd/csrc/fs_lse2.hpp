@@ -293,9 +293,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     }
   }
 
-  // run_m: running max in accumulator units; run_c (BIASC): -run_m * lscale as rounded once,
-  // the offset every exponent of the row uses, so that rescaling by differences of run_c is
-  // consistent with the exponents already summed
+  // The logits stay in absolute accumulator units in every configuration (a running maximum
+  // subtracted inside the accumulator costs the logits their digits whenever it lies far below
+  // them: after a first tile of keys without weight, say).  run_m: the running maximum in those
+  // units; run_c: -run_m * lscale as rounded once, the offset every exponent of the row uses, so
+  // that rescaling by differences of run_c is consistent with the exponents already summed
   float run_m[RB], run_s[RB], run_c[RB], run_o[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -405,49 +407,34 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     swap_halves(a, b);
     return fmaxf(a, b);
   };
-  // classic online soft-max step; acc holds (logit - M)/lscale for the current M = run_m[rb]
+  // classic online soft-max step; acc holds logit / lscale
   auto softmax = [&](const f32x16& acc, int rb, const f32x16& v16) {
-    if constexpr (BIASC) {  // acc holds logit/lscale itself
-      const float m_new = fmaxf(column_max(acc), run_m[rb]);
-      // rounded once, on purpose: the exponents below, the rescale and the value handed to the
-      // merge must all see the same number.  The empty asm hides the product from the
-      // compiler: fused into the subtraction below (fp contraction) it would rescale by
-      // 2^(rounding residual) on every tile, which adds up over a long key chunk.
-      float c_new = -m_new * lscale;
-      asm volatile("" : "+v"(c_new));
-      float ps0 = 0.f, ps1 = 0.f, po = 0.f;
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const float e0 = fast_exp2(__builtin_fmaf(acc[r], lscale, c_new));
-        const float e1 = fast_exp2(__builtin_fmaf(acc[r + 1], lscale, c_new));
-        ps0 += e0;
-        ps1 += e1;
-        if constexpr (VEC) po = __builtin_fmaf(e0, v16[r], __builtin_fmaf(e1, v16[r + 1], po));
-      }
-      const float resc = fast_exp2(c_new - run_c[rb]);
-      run_s[rb] = run_s[rb] * resc + (ps0 + ps1);
-      if constexpr (VEC) run_o[rb] = run_o[rb] * resc + po;
-      run_m[rb] = m_new;
-      run_c[rb] = c_new;
-      return;
-    }
-    const float delta = fmaxf(column_max(acc), 0.f);
-    // the max actually applied is what fp32 can represent next to the old one
-    const float m_new = run_m[rb] + delta;
-    const float c = -(m_new - run_m[rb]) * lscale;
-    float ps0 = 0.f, ps1 = 0.f;
+    const float m_new = fmaxf(column_max(acc), run_m[rb]);
+    // rounded once, on purpose: the exponents below, the rescale and the value handed to the
+    // merge must all see the same number.  The empty asm hides the product from the
+    // compiler: fused into the subtraction below (fp contraction) it would rescale by
+    // 2^(rounding residual) on every tile, which adds up over a long key chunk.
+    float c_new = -m_new * lscale;
+    asm volatile("" : "+v"(c_new));
+    float ps0 = 0.f, ps1 = 0.f, po = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
-      ps0 += fast_exp2(__builtin_fmaf(acc[r], lscale, c));
-      ps1 += fast_exp2(__builtin_fmaf(acc[r + 1], lscale, c));
+      const float e0 = fast_exp2(__builtin_fmaf(acc[r], lscale, c_new));
+      const float e1 = fast_exp2(__builtin_fmaf(acc[r + 1], lscale, c_new));
+      ps0 += e0;
+      ps1 += e1;
+      if constexpr (VEC) po = __builtin_fmaf(e0, v16[r], __builtin_fmaf(e1, v16[r + 1], po));
     }
-    run_s[rb] = run_s[rb] * fast_exp2(c) + (ps0 + ps1);
+    const float resc = fast_exp2(c_new - run_c[rb]);
+    run_s[rb] = run_s[rb] * resc + (ps0 + ps1);
+    if constexpr (VEC) run_o[rb] = run_o[rb] * resc + po;
     run_m[rb] = m_new;
+    run_c[rb] = c_new;
   };
   auto softmax_first = [&](const f32x16& acc, int rb, const f32x16& v16) {
     const float delta = column_max(acc);
     float c = -delta * lscale;
-    if constexpr (BIASC) asm volatile("" : "+v"(c));
+    asm volatile("" : "+v"(c));
     float ps = 0.f, po = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -480,20 +467,12 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
       swap_halves(s.aa, s.bb);
     }
     if (p == 3) {
-      if constexpr (BIASC) {
-        const float m_new = fmaxf(fmaxf(s.aa, s.bb), run_m[rb]);
-        s.cx = -m_new * lscale;
-        asm volatile("" : "+v"(s.cx));  // see softmax(): the rounded product, nothing fused
-        s.c = s.cx - run_c[rb];
-        run_m[rb] = m_new;
-        run_c[rb] = s.cx;
-      } else {
-        const float delta = fmaxf(fmaxf(s.aa, s.bb), 0.f);
-        const float m_new = run_m[rb] + delta;
-        s.c = -(m_new - run_m[rb]) * lscale;
-        s.cx = s.c;
-        run_m[rb] = m_new;
-      }
+      const float m_new = fmaxf(fmaxf(s.aa, s.bb), run_m[rb]);
+      s.cx = -m_new * lscale;
+      asm volatile("" : "+v"(s.cx));  // see softmax(): the rounded product, nothing fused
+      s.c = s.cx - run_c[rb];
+      run_m[rb] = m_new;
+      run_c[rb] = s.cx;
       s.ps0 = 0.f;
       s.ps1 = 0.f;
       s.po = 0.f;
@@ -650,10 +629,10 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     for (int k = 0; k < NMAIN; ++k) acc = mfma_k(k, acc, kr, rb);
     return acc;
   };
-  // The bias MFMA (fp32 operands in every mode): adds kbias_j - M_i with the freshest M.
+  // The bias MFMA (fp32 operands in every mode): adds kbias_j.
   auto add_bias = [&](f32x16 acc, const KeyRegs& kr, int rb) -> f32x16 {
     if constexpr (BIASC) return acc;  // the chain started from the bias
-    return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(kr.ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
   };
 
   KeyRegs K[KPF ? 2 : 1];
@@ -822,7 +801,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         // Every logit of the previous unit more than 2^40 (LaunchArgs::skip_log2) below its
         // row's running maximum: its exponentials would not change the fp32 row sums, so
         // they are not computed.
-        const float mx_rel = BIASC ? st.mx - run_m[prev_rb] : st.mx;
+        const float mx_rel = st.mx - run_m[prev_rb];
         const bool soft = wave_any(mx_rel > skip_below);
         n_left_out += soft ? 0u : 1u;
         if constexpr (BIASC) {
@@ -872,7 +851,7 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
     const int row = row0 + rb * 32 + li;
     const float s = run_s[rb] + xor32(run_s[rb]);
     const float o = VEC ? run_o[rb] + xor32(run_o[rb]) : 0.f;
-    const float M2 = BIASC ? -run_c[rb] : run_m[rb] * lscale;
+    const float M2 = -run_c[rb];
     if (row < sd.nq && h == 0) {
       if (sd.splits == 1) {
         epilogue_scalar(sd.ep, row, M2, s, o);

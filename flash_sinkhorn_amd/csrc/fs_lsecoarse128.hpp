@@ -65,7 +65,6 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
   // MFMAs produce raw products of the scaled planes; lscale turns them into base-2 logits
   const float lscale = sd.qscale / (sd.plane_scale[sd.ps_q] * sd.plane_scale[sd.ps_k]);
   const float inv_lscale = 1.0f / lscale;
-  const float skip_below = args.skip_log2 * inv_lscale;  // the 2^40 distance in raw units (< 0)
 
   // ---- stationary planes of the query rows: [block][16-column step] ----
   u32x4 xh[RB][KK16], xl[RB][KK16];
@@ -174,20 +173,24 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
     return m;
   };
 
-  // ---- running statistics: run_m in raw units (of the full logit with its key bias) ----
-  float run_m[RB], run_s[RB], best_v[RB];
+  // ---- running statistics.  The logits stay in absolute raw units (of the full logit with
+  // its key bias); the running maximum M is kept as run_c = -M * lscale, rounded once: the
+  // constant of the exponentials and what the test compares with (subtracted inside the
+  // accumulator, M would cost the logits their digits whenever it lies far below them) ----
+  float run_c[RB], run_s[RB], best_v[RB];
   int best_j[RB];
   const bool track = sd.best_key != nullptr;
   bool seeded = sd.seed != nullptr;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    run_m[rb] = 0.f;
+    run_c[rb] = 0.f;
     run_s[rb] = 0.f;
     best_v[rb] = -3.0e38f;
     best_j[rb] = -1;
     if (sd.seed != nullptr) {
-      run_m[rb] = sd.seed[min(row0 + rb * 32 + li, sd.nq - 1)];
-      seeded = seeded && run_m[rb] > -3.0e38f;
+      const float sv = sd.seed[min(row0 + rb * 32 + li, sd.nq - 1)];
+      seeded = seeded && sv > -3.0e38f;
+      run_c[rb] = -sv * lscale;
     }
   }
   // (wavefront-uniform: without a starting value for every row the first unit sets the maxima)
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     started[rb] = seeded;
-    if (!seeded) run_m[rb] = 0.f;
+    if (!seeded) run_c[rb] = 0.f;
   }
   unsigned n_ended = 0;
 
@@ -248,13 +251,13 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
       kbias = fmaxf(kbias * inv_lscale, -3.0e38f);
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        // + key bias - running maximum: A = [bias_j, 1], B = [1, -M_i]
-        acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(h ? 1.0f : kbias, h ? -run_m[rb] : 1.0f,
+        // + key bias: A = [bias_j, 1], B = [1, 0]
+        acc[rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(h ? 1.0f : kbias, h ? 0.0f : 1.0f,
                                                        acc[rb], 0, 0, 0);
         const float tmax = max16(acc[rb]);
         // every logit of the unit at least 2^40 below its row's running maximum, whatever the
         // cross products add: nothing of it could change the fp32 sums
-        if (started[rb] && !wave_any(tmax + corr[rb] > skip_below)) {
+        if (started[rb] && !wave_any(__builtin_fmaf(tmax + corr[rb], lscale, run_c[rb]) > args.skip_log2)) {
           ++n_ended;
           continue;
         }
@@ -285,16 +288,16 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
           {
             float a = tm, b = tm;
             swap_halves(a, b);
-            tm = fmaxf(a, b);  // the row's largest logit of the unit, relative to run_m
+            tm = fmaxf(a, b);  // the row's largest logit of the unit
           }
           // the key of the row's largest logit so far (absolute raw units; lane-private, the two
           // half-waves are merged at the end)
           // (searched only when some lane's largest value of the unit beats what it has)
-          if (track && wave_any(lane_max + run_m[rb] > best_v[rb])) {
+          if (track && wave_any(lane_max > best_v[rb])) {
             const int jb = j0 + js * 32 + 4 * h;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const float v = acc[rb][r] + run_m[rb];
+              const float v = acc[rb][r];
               if (v > best_v[rb]) {
                 best_v[rb] = v;
                 best_j[rb] = jb + 8 * (r / 4) + (r % 4);
@@ -302,17 +305,18 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
             }
           }
           const bool first = !started[rb];
-          const float delta = first ? tm : fmaxf(tm, 0.f);
-          const float cc = -delta * lscale;
+          float cc = -tm * lscale;
+          asm volatile("" : "+v"(cc));  // the exponents, the rescale and the result see one number
+          cc = first ? cc : fminf(cc, run_c[rb]);
           float ps0 = 0.f, ps1 = 0.f;
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
             ps0 += fast_exp2(__builtin_fmaf(acc[rb][r], lscale, cc));
             ps1 += fast_exp2(__builtin_fmaf(acc[rb][r + 1], lscale, cc));
           }
-          const float resc = first ? 0.f : fast_exp2(cc);
+          const float resc = first ? 0.f : fast_exp2(cc - run_c[rb]);
           run_s[rb] = run_s[rb] * resc + (ps0 + ps1);
-          run_m[rb] += delta;
+          run_c[rb] = cc;
           started[rb] = true;
         }
       }
@@ -340,7 +344,7 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
   for (int rb = 0; rb < RB; ++rb) {
     const int row = row0 + rb * 32 + li;
     const float s = run_s[rb] + xor32(run_s[rb]);
-    const float M2 = run_m[rb] * lscale;
+    const float M2 = -run_c[rb];
     float bv = best_v[rb];
     int bj = best_j[rb];
     const float ov = xor32(bv);

@@ -193,7 +193,11 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
     for (int st = 0; st < 4; ++st)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[qb][st][r] = 0.f;
-  float run_m[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f}, run_o[2] = {0.f, 0.f};
+  // run_c: minus the running maximum in base-2 units as rounded once, the constant of the
+  // exponentials (the logits stay in absolute raw units: a running maximum subtracted inside
+  // the accumulator costs them their digits whenever it lies far below them, after a first
+  // tile of keys without weight, say)
+  float run_m[2] = {0.f, 0.f}, run_c[2] = {0.f, 0.f}, run_s[2] = {0.f, 0.f}, run_o[2] = {0.f, 0.f};
   int best_j[2] = {0, 0};  // AMAX: run_m holds the largest raw value so far, best_j its key
   if constexpr (AMAX) run_m[0] = run_m[1] = -3.0e38f;
   float rbias[2] = {0.f, 0.f};  // SWP: the rows' own bias (base 2), as keys of the other side
@@ -355,11 +359,11 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
         }
         continue;
       }
-      const float negm = h ? -run_m[qb] : 1.0f;
       float m = -3.0e38f;
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
-        acc[qb][st] = __builtin_amdgcn_mfma_f32_32x32x2f32(ab[st], negm, acc[qb][st], 0, 0, 0);
+        acc[qb][st] =
+            __builtin_amdgcn_mfma_f32_32x32x2f32(ab[st], h ? 0.0f : 1.0f, acc[qb][st], 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 16; ++r) m = fmaxf(m, acc[qb][st][r]);
       }
@@ -367,9 +371,9 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
       swap_halves(a, b);
       m = fmaxf(a, b);
       const bool first = (t == 0);
-      const float delta = first ? m : fmaxf(m, 0.f);
-      const float m_new = run_m[qb] + delta;
-      const float cc = -(m_new - run_m[qb]) * lscale;
+      float cc = -m * lscale;
+      asm volatile("" : "+v"(cc));  // the exponents, the rescale and the result see one number
+      cc = first ? cc : fminf(cc, run_c[qb]);
       float ps0 = 0.f, ps1 = 0.f, po0 = 0.f, po1 = 0.f;
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
@@ -396,10 +400,10 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
           }
         }
       }
-      const float resc = first ? 0.f : fast_exp2(cc);
+      const float resc = first ? 0.f : fast_exp2(cc - run_c[qb]);
       run_s[qb] = run_s[qb] * resc + (ps0 + ps1);
       if constexpr (VEC) run_o[qb] = run_o[qb] * resc + (po0 + po1);
-      run_m[qb] = m_new;
+      run_c[qb] = cc;
 #pragma unroll
       for (int st = 0; st < 4; ++st)
 #pragma unroll
@@ -442,7 +446,7 @@ __global__ __launch_bounds__(512, 1) void lse_gemm_kernel(const LaunchArgs args)
     if (row < sd.nq && h == 0) {
       const size_t pr = (size_t)(split * 2 + kg) * (size_t)sd.nq + (size_t)row;
       *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) =
-          has_keys ? make_float2(run_m[qb] * lscale, s) : make_float2(kNegBig, 0.f);
+          has_keys ? make_float2(-run_c[qb], s) : make_float2(kNegBig, 0.f);
     }
     if constexpr (VEC) {
       const float o = run_o[qb] + xor32(run_o[qb]);

@@ -259,7 +259,9 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   for (int i = 0; i < CB; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-  float run_m = 0.f, run_s = 0.f;  // run_m in units of the raw dot products
+  // run_c: the constant of the exponentials, kPgUp minus the running maximum in base-2 units
+  // (the logits stay in absolute raw units: see plan_tile_kernel)
+  float run_c = kPgUp, run_s = 0.f;
 
   auto swap_halves = [&](float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
           h ? 1.0f : fmaxf(key_bias(sd, j0 + wave * 32 + li, j_end) * inv_lscale, -3.0e38f);
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] += acc2[r];
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m : 1.0f, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
     }
     float m = acc[0];
 #pragma unroll
@@ -383,13 +385,11 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
 #pragma unroll
     for (int w = 1; w < 8; ++w) tm = fmaxf(tm, lds_x[w][li]);
     const bool first = (t == 0);
-    const bool up = first || (tm * lscale > kPgLazyThresh);
-    float cc = 0.f;
+    const bool up = first || (__builtin_fmaf(tm, lscale, run_c) > kPgLazyThresh + kPgUp);
     if (first || wave_any(up)) {  // the same lanes vote in every wavefront
-      const float delta = up ? tm : 0.f;
-      cc = -delta * lscale;
-      const float resc = first ? 0.f : fast_exp2(cc);
-      run_m += delta;
+      const float c_new = up ? __builtin_fmaf(-tm, lscale, kPgUp) : run_c;
+      const float resc = first ? 0.f : fast_exp2(c_new - run_c);
+      run_c = c_new;
       run_s *= resc;
 #pragma unroll
       for (int i = 0; i < CB; ++i)
@@ -398,10 +398,9 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
     }
     float p[16];
     float ps = 0.f;
-    const float ccu = cc + kPgUp;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, ccu));
+      p[r] = fast_exp2(__builtin_fmaf(acc[r], lscale, run_c));
       ps += p[r];
     }
     run_s += ps;
@@ -470,7 +469,7 @@ __global__ __launch_bounds__(512, 1) void plan_gemm_kernel(const LaunchArgs args
   float s = 0.f;
 #pragma unroll
   for (int w = 0; w < 8; ++w) s += lds_x[w][li];
-  const float M = (ntiles > 0) ? run_m * lscale - kPgUp : kNegBig;
+  const float M = (ntiles > 0) ? -run_c : kNegBig;
   float inv_vs = 1.0f / sd.vplane_scale[0];
   if constexpr (MAT5) inv_vs /= t_unit * sd.q2plane_scale[0] * sd.kplane_scale[0];
   const bool live = row < sd.nq;

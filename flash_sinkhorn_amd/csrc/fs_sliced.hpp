@@ -124,7 +124,8 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
     }
     if (wave == 0) {
       const float ab = h ? 1.0f : key_bias(sd, j0 + li, j_end);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m : 1.0f, acc, 0, 0, 0);
+      // (+ key bias; the running maximum is taken off in the exponent: see stream_kernel)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
     }
 
     // ---- sum the NW partial tiles through LDS ----
@@ -168,15 +169,13 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
 #pragma unroll
     for (int r = 2; r < 16; ++r) tmax = fmaxf(tmax, acc[r]);
     const bool first = (t == 0);
-    if (first || wave_any(tmax > kLazyThresh)) {
+    if (first || wave_any(tmax - run_m > kLazyThresh)) {
       const float tm = fmaxf(tmax, xor32(tmax));
-      const float delta = (first || tm > kLazyThresh) ? tm : 0.f;
-      const float resc = first ? 0.f : fast_exp2(-delta);
-      run_m += delta;
+      const float m_new = (first || tm - run_m > kLazyThresh) ? tm : run_m;
+      const float resc = first ? 0.f : fast_exp2(run_m - m_new);
+      run_m = m_new;
       run_s *= resc;
       run_o *= resc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] -= delta;
       if constexpr (kHasO) {
 #pragma unroll
         for (int db = 0; db < NSL; ++db)
@@ -188,7 +187,7 @@ __global__ __launch_bounds__(NW * 64) void sliced_kernel(const LaunchArgs args) 
     float ps = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      p[r] = fast_exp2(acc[r]);
+      p[r] = fast_exp2(acc[r] - run_m);
       ps += p[r];
     }
     run_s += ps;

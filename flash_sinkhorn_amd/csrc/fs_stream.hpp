@@ -317,7 +317,10 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
           }
           continue;
         }
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? -run_m[rb] : 1.0f, acc, 0, 0, 0);
+        // + key bias; the logits stay absolute and the running maximum is taken off in the
+        // exponent (inside the accumulator it would cost them their digits whenever it lies far
+        // below them, after a first tile of keys without weight, say)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ab, h ? 0.0f : 1.0f, acc, 0, 0, 0);
 
         f32x16 tacc;
         if constexpr (MODE == kMat5) {
@@ -333,15 +336,13 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
         for (int r = 2; r < 16; ++r) tmax = fmaxf(tmax, acc[r]);
 
         const bool first = (t == 0 && js == 0);
-        if (first || wave_any(tmax > kLazyThresh)) {
+        if (first || wave_any(tmax - run_m[rb] > kLazyThresh)) {
           const float tm = fmaxf(tmax, xor32(tmax));
-          const float delta = (first || tm > kLazyThresh) ? tm : 0.f;
-          const float resc = first ? 0.f : fast_exp2(-delta);
-          run_m[rb] += delta;
+          const float m_new = (first || tm - run_m[rb] > kLazyThresh) ? tm : run_m[rb];
+          const float resc = first ? 0.f : fast_exp2(run_m[rb] - m_new);
+          run_m[rb] = m_new;
           run_s[rb] *= resc;
           run_o[rb] *= resc;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[r] -= delta;
           if constexpr (kHasO) {
 #pragma unroll
             for (int db = 0; db < G::NDB; ++db)
@@ -352,7 +353,7 @@ __global__ __launch_bounds__(256) void stream_kernel(const LaunchArgs args) {
 
         float p[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) p[r] = fast_exp2(acc[r]);
+        for (int r = 0; r < 16; ++r) p[r] = fast_exp2(acc[r] - run_m[rb]);
 
         if constexpr (MODE != kMat5) {
           float ps = 0.f;

@@ -461,3 +461,71 @@ def test_far_tail_of_the_plan_survives_the_fp16_probability_split(n, m, d):
     want = oracle.apply_plan_mat(x[rows], y, f_hat[rows], g_hat, la[rows], lb, y, eps, axis=1)
     got = apply_plan_mat_flashstyle(X, Y, *dev(f_hat, g_hat, la, lb), Y, eps=eps, axis=1)
     assert rel_err(got[rows], want) < RTOL
+
+
+@pytest.mark.parametrize("mode", ["fp16x2", "fp32_mfma"])
+@pytest.mark.parametrize("d", [16, 64, 100, 128, 200])
+@pytest.mark.parametrize("lead", [70, 300])
+def test_leading_keys_without_weight(monkeypatch, d, lead, mode):
+    """The first keys of both clouds carry no weight (log weight -100000, as the reference maps
+    them): whole first tiles of every kernel family see logits a hundred thousand base-2 units
+    below the rest.  A running maximum subtracted inside the accumulator cost the tiles after
+    them their digits (errors of 1e-3); every operation against the fp64 oracle.  Also the two
+    ways a key without weight can become a row's starting key: a caller's hint, and the key
+    array of prepared planes."""
+    from flash_sinkhorn_amd import _lib
+    from flash_sinkhorn_amd.kernels._common import log_weights
+    from flash_sinkhorn_amd.kernels.apply_flash import (apply_plan_mat_flashstyle,
+                                                        apply_plan_vec_flashstyle)
+    from flash_sinkhorn_amd.kernels.sinkhorn_flashstyle_sqeuclid import _symmetric_step_raw
+    from flash_sinkhorn_amd.kernels.sinkhorn_triton_grad_sqeuclid import (
+        sinkhorn_geomloss_online_grad_sqeuclid as grad)
+    monkeypatch.setattr(_lib, "STRICT_OPERANDS", mode)  # the default planes, or fp32 MFMA operands
+    rng = np.random.default_rng(7 * d + lead)
+    n, m, eps = 1100, 900, 0.05
+    x = (rng.standard_normal((n, d)) / np.sqrt(d)).astype(np.float32)
+    y = (rng.standard_normal((m, d)) / np.sqrt(d) + 0.1).astype(np.float32)
+    a = rng.random(n).astype(np.float32) + 0.5
+    b = rng.random(m).astype(np.float32) + 0.5
+    a[:lead] = 0
+    b[:lead // 2] = 0
+    a, b = a / a.sum(), b / b.sum()
+    wf, wg = oracle.sinkhorn_symmetric(x, y, a, b, eps=eps, n_iters=6, use_epsilon_scaling=False)[:2]
+    X, Y, A, B = dev(x, y, a, b)
+    f, g = dev(wf.astype(np.float32), wg.astype(np.float32))
+    Fh, Gh = (f - (X * X).sum(1)).contiguous(), (g - (Y * Y).sum(1)).contiguous()
+    la, lb = log_weights(A).contiguous(), log_weights(B).contiguous()
+    ola, olb = oracle.log_weights(a), oracle.log_weights(b)
+    fh, gh = Fh.cpu().numpy(), Gh.cpu().numpy()
+    kw = dict(cost_scale=1.0, alpha=1.0, damping_f=1.0, damping_g=1.0, allow_tf32=False)
+    want = oracle.symmetric_step(x, y, fh, gh, ola, olb, eps, 1.0, 1.0, 1.0, 1.0)
+    tol = 2e-5
+
+    def check(got, exp, what):
+        for u, v in zip(got, exp):
+            assert rel_err(u, v) < tol, (what, rel_err(u, v))
+
+    check(_symmetric_step_raw(X, Y, Fh, Gh, la, lb, eps, coarse=False, **kw), want, "step")
+    planes = mode == "fp16x2"
+    if d <= 128 and planes:
+        for keys in (None, 0):  # no keys yet; every row's key is key 0, which has no weight
+            prep = _lib.PreparedOperands(X, Y, _lib.flags(True, False))
+            if keys is not None:
+                prep.best_keys(0).fill_(keys)
+                prep.best_keys(1).fill_(keys)
+            check(_symmetric_step_raw(X, Y, Fh, Gh, la, lb, eps, coarse=True, prepared=prep, **kw), want,
+                  ("coarse step", keys))
+    wgrad = oracle.grad_barycentric(x, y, a, b, wf.astype(np.float32), wg.astype(np.float32), eps)[:2]
+    check(grad(X, Y, A, B, f, g, eps=eps, allow_tf32=False), wgrad, "gradient")
+    if d <= 128 and planes:
+        hints = (torch.zeros(n, dtype=torch.int32, device="cuda"), torch.zeros(m, dtype=torch.int32, device="cuda"))
+        check(grad(X, Y, A, B, f, g, eps=eps, allow_tf32=False, _seed_keys=hints), wgrad, "hinted gradient")
+    V = rng.standard_normal((m, d)).astype(np.float32)
+    W = rng.standard_normal((n, d)).astype(np.float32)
+    v = rng.standard_normal(m).astype(np.float32)
+    check([apply_plan_mat_flashstyle(X, Y, Fh, Gh, la, lb, dev(V)[0], eps=eps, axis=1, allow_tf32=False)],
+          [oracle.apply_plan_mat(x, y, fh, gh, ola, olb, V, eps, 1)], "plan.mat")
+    check([apply_plan_mat_flashstyle(X, Y, Fh, Gh, la, lb, dev(W)[0], eps=eps, axis=0, allow_tf32=False)],
+          [oracle.apply_plan_mat(x, y, fh, gh, ola, olb, W, eps, 0)], "plan^T.mat")
+    check([apply_plan_vec_flashstyle(X, Y, Fh, Gh, la, lb, dev(v)[0], eps=eps, axis=1, allow_tf32=False)],
+          [oracle.apply_plan_vec(x, y, fh, gh, ola, olb, v, eps, 1)], "plan.vec")
