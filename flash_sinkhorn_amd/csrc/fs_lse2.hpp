@@ -859,6 +859,11 @@ __global__ __launch_bounds__(256, 2) void lse2_kernel(const LaunchArgs args) {
         const size_t pr = (size_t)split * (size_t)sd.nq + (size_t)row;
         *reinterpret_cast<float2*>(&sd.part_ms[2 * pr]) = make_float2(M2, s);
         if constexpr (VEC) sd.part_o[pr] = o;
+        // this kernel follows no keys: the merge must not take what an earlier launch (or an
+        // earlier user of the workspace) left in the array for one
+        if constexpr (!VEC) {
+          if (sd.part_best != nullptr) sd.part_best[pr] = -1;
+        }
       }
     }
   }
