@@ -263,26 +263,33 @@ __global__ __launch_bounds__(256, 2) void lse_coarse128_kernel(const LaunchArgs 
         }
         // ---- the unit goes on: cross products on the lo planes, then the online soft-max ----
         {
-          // (both planes of the keys again from LDS, four steps at a time: the registers of the
-          // first pass are free by now)
+          // (both planes of the keys again from LDS, two steps at a time: the registers of the
+          // first pass are free by now.  The cross products are summed on their own, where they
+          // are small, and join the logits with one addition: added one by one to logits of a
+          // few thousand base-2 units they would each be rounded to those logits' last place.)
           const unsigned* ylo = lds_k[buf][1] + (js * 32 + li) * ROWH;
+          f32x16 cr;
 #pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            u32x4 kh[KK16 / 2], kl[KK16 / 2];
+          for (int r = 0; r < 16; ++r) cr[r] = 0.f;
 #pragma unroll
-            for (int k4 = 0; k4 < KK16 / 2; ++k4) {
-              const int kk = half * (KK16 / 2) + k4;
-              kh[k4] = ds_read16(yrow + (((2 * kk + h) ^ (li & 15)) << 2));
-              kl[k4] = ds_read16(ylo + (((2 * kk + h) ^ (li & 15)) << 2));
+          for (int part = 0; part < KK16 / 2; ++part) {
+            u32x4 kh[2], kl[2];
+#pragma unroll
+            for (int k2 = 0; k2 < 2; ++k2) {
+              const int kk = part * 2 + k2;
+              kh[k2] = ds_read16(yrow + (((2 * kk + h) ^ (li & 15)) << 2));
+              kl[k2] = ds_read16(ylo + (((2 * kk + h) ^ (li & 15)) << 2));
             }
             wait_lds();
 #pragma unroll
-            for (int k4 = 0; k4 < KK16 / 2; ++k4) {
-              const int kk = half * (KK16 / 2) + k4;
-              acc[rb] = mfma16(kh[k4], xl[rb][kk], acc[rb]);
-              acc[rb] = mfma16(kl[k4], xh[rb][kk], acc[rb]);
+            for (int k2 = 0; k2 < 2; ++k2) {
+              const int kk = part * 2 + k2;
+              cr = mfma16(kh[k2], xl[rb][kk], cr);
+              cr = mfma16(kl[k2], xh[rb][kk], cr);
             }
           }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[rb][r] += cr[r];
           const float lane_max = max16(acc[rb]);
           float tm = lane_max;
           {

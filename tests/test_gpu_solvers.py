@@ -902,12 +902,13 @@ def test_solvers_with_the_coarse_tile_test_on_rows_of_65_to_128_columns(monkeypa
     scale = float((X * X).sum(dim=1).max())
     for u, v in zip(got[0], want[0]):
         assert float((u - v).abs().max()) < 2e-6 * scale
-    # (alternating half-updates feed on each other: the two kernels round a row's largest
-    # logit differently by the same amount in every iteration, x.y does not change, so the
-    # difference of the solves grows with the iterations until the contraction holds it)
+    # (alternating half-updates feed on each other: where two kernels round a row's largest
+    # logit differently they do so by the same amount in every iteration, x.y does not change,
+    # and the difference of the solves grows with the iterations until the contraction holds
+    # it; the wide kernel therefore sums its cross products apart from the large terms)
     for g_alt, w_alt in zip(got[1], want[1]):
         for u, v in zip(g_alt, w_alt):
-            assert float((u - v).abs().max()) < 4e-6 * scale
+            assert float((u - v).abs().max()) < 2e-6 * scale
     for u, v in zip(got[2][0] + got[2][1], want[2][0] + want[2][1]):
         assert float((u - v).abs().max()) < 2e-6 * scale
     wf, wg = oracle.sinkhorn_symmetric(x, y, a, b, eps=0.05, n_iters=20, use_epsilon_scaling=False)[:2]
